@@ -1,0 +1,192 @@
+/* C ABI of libisoexec_hip.so: the gfx950 kernels of the batch-invariant token-logprob path.
+ *
+ * The reference (zanderjiang/SkyRL-IsoExec) has no C ABI on this path; its operator interface is
+ * Python (op functions + aten overrides + _register.py declarations) over Triton/CUDA kernels.
+ * Each entry point below names the reference function whose arithmetic it replaces; paths are
+ * relative to skyrl/backends/skyrl_train/isoexec/ in the reference tree.
+ *
+ * Conventions
+ *   - plain pointers and sizes only; every pointer is DEVICE memory unless stated otherwise;
+ *   - the caller owns all memory, outputs and workspaces included; no entry point allocates,
+ *     frees, synchronises the device or reads device memory back to the host;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *   - return value: 0 = launched, > 0 = declined (shape/dtype outside the envelope: nothing
+ *     was launched, the caller decides), < 0 = error (bad argument or launch failure);
+ *   - dtype codes: IX_DT_F32 = 0, IX_DT_BF16 = 1; bf16 values are raw uint16 bit patterns;
+ *   - results never depend on batch size, token count, tile choice or launch shape: arguments
+ *     named `tile`, `force_shape`, `time_tile`, `BM` choose who computes an element, not how.
+ */
+#ifndef ISOEXEC_HIP_H
+#define ISOEXEC_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define IX_ABI_VERSION 1
+
+#ifndef IX_OK
+#define IX_OK 0
+#define IX_DECLINED 1
+#define IX_ERR_ARG (-1)
+#define IX_ERR_LAUNCH (-2)
+#define IX_DT_F32 0
+#define IX_DT_BF16 1
+#endif
+
+/* primitive codes for ix_prim_unary */
+#define IX_PRIM_EXP 0
+#define IX_PRIM_LOG 1
+#define IX_PRIM_EXP_FAST 2
+#define IX_PRIM_SIGMOID 3
+#define IX_PRIM_SILU_DIV 4
+#define IX_PRIM_SOFTPLUS 5
+#define IX_PRIM_RSQRT_IEEE 6
+#define IX_PRIM_ROUND_BF16 7
+#define IX_PRIM_COUNT 8
+
+int ix_abi_version(void);
+const char* ix_arch_tag(void); /* "gfx950"; counterpart of core/arch.py:27-51 detect_arch() tags */
+
+/* y[i] = prim(x[i]) with the device's own exp/log/... as the kernels use them. A checker plugs
+ * these into the CPU restatement so that order-of-operations parity is bit-exact. No
+ * counterpart in the reference (its probes compare kernels against eager torch on device). */
+int ix_prim_unary(int op, const float* x, float* y, long n, void* stream);
+
+/* ---- log-softmax + target gather: ops/logprobs/rowinv.py ---------------------------------- */
+
+/* Workspace the split launch shape needs (bytes); 0 on invalid arguments. */
+size_t ix_logprob_workspace_bytes(long rows, long V, int G);
+
+/* rowinv_sampled_logprobs (rowinv.py:666-712; kernels leaf_sum_exp :136-154, finalize_rows
+ * :156-191) at world size 1. logits [rows, V] (row pitch row_stride elements), target int64
+ * [rows] (out of range -> logprob 0), G leaves (power of two, V % G == 0 else declined).
+ * out_logprob fp32 [rows]; out_lse fp32 [rows] or NULL. force_shape: 0 auto, 1 one workgroup
+ * per row, 2 split rows (needs the workspace). */
+int ix_logprob_rowinv_sampled(const void* logits, int dtype, long rows, long V, long row_stride,
+                              const int64_t* target, int G, float* out_logprob, float* out_lse,
+                              void* workspace, size_t workspace_bytes, int force_shape, void* stream);
+
+/* rowinv_full_logprobs (rowinv.py:796-875; kernel full_row_logprobs :193-245): the whole row
+ * (x - m) - log S into out_full fp32 [rows, V] (pitch out_stride). */
+int ix_logprob_rowinv_full(const void* logits, int dtype, long rows, long V, long row_stride, int G,
+                           float* out_full, long out_stride, float* out_lse, void* workspace,
+                           size_t workspace_bytes, int force_shape, void* stream);
+
+/* ---- norms: ops/norms/fused_outnorm.py, zero_centered_norm.py, fused_add_rmsnorm.py -------- */
+
+/* fused_rms_norm_gamma (fused_outnorm.py:159-185) / ZeroCenteredTorchRMSNorm.forward
+ * (zero_centered_norm.py:36-37). x, out bf16 [M, N]; weight bf16 [N]; zero_centered != 0 uses
+ * gamma = bf16(1 + weight), else gamma = weight. */
+int ix_rmsnorm_gamma(const void* x, const void* weight, void* out, long M, long N, float eps,
+                     int zero_centered, void* stream);
+
+/* fused_gated_out_norm (fused_outnorm.py:235-271) / _eager_apply_gated_norm
+ * (runtimes/megatron/gdn_fla_shim.py:390-425). x, out bf16 [T*HV, N]; gate bf16 viewed
+ * [T, HV, N] with token pitch gate_stride_t. */
+int ix_gated_out_norm(const void* x, const void* gate, long gate_stride_t, const void* weight, void* out,
+                      long T, long HV, long N, float eps, int zero_centered, void* stream);
+
+/* residual add + norm (fused_add_rmsnorm.py:1-25): h = bf16(x + residual) -> h_out, then the
+ * norm chain of ix_rmsnorm_gamma on h -> out. */
+int ix_add_rmsnorm_gamma(const void* x, const void* residual, const void* weight, void* out, void* h_out,
+                         long M, long N, float eps, int zero_centered, void* stream);
+
+/* ---- dense matmuls: ops/moe/moe_batch_invariant.py:422-473 (aten mm/addmm/bmm override),
+ *      ops/mm/mm_tiles.py:127-158, ops/mm/csrc/cublaslt_pinned.cpp:319-327 mm(x, w, out, slot) - */
+
+/* C[M,N] = A[M,K] . W[N,K]^T (+ bias[N]), bf16 in/out, fp32 accumulate in a fixed K order, no
+ * split-K. lda/ldw/ldc are row pitches in elements. bias may be NULL. tile: 0 auto. */
+int ix_gemm_bf16_nt(const void* A, long lda, const void* W, long ldw, const void* bias, void* C, long ldc,
+                    long M, long N, long K, int tile, void* stream);
+
+/* Router gating GEMM (moe/_register.py:59-66): C fp32 [M,N] = A[M,K] . W[N,K]^T with W fp32 and
+ * A fp32 or bf16 (a_dtype), fp32 accumulate in a fixed K order. */
+int ix_gemm_f32_nt(const void* A, int a_dtype, long lda, const void* W, long ldw, void* C, long ldc, long M,
+                   long N, long K, void* stream);
+
+/* ---- GatedDeltaNet: ops/gdn/gdn_ops.py ----------------------------------------------------- */
+
+/* gdn_recurrent_kernel (gdn_ops.py:400-441): the delta-rule scan over packed tokens, state pool
+ * advanced in place. q,k [tokens, H, K] and v [tokens, HV, V] with token pitches q_pitch,
+ * k_pitch, v_pitch (elements; heads contiguous inside a token, so slices of one projection
+ * buffer need no copy); o [tokens, HV, V] contiguous; g fp32 [tokens, HV]; beta [tokens, HV];
+ * q/k/v/beta/o share io_dtype. state_pool fp32 [rows, HV, V, K]. cu_seqlens int32
+ * [N+1]. state_indices int32: pool row for (sequence n, token t) at [n*stride + t]; column 0
+ * loads, a positive entry at column t stores after token t, row index <= 0 at column 0 skips
+ * the sequence. HV % H == 0 (GQA: head hv reads q/k head hv / (HV/H)). K in {32,64,128,256}.
+ * time_tile: tokens staged per LDS fill (<= 64, 0 = default); does not change results. */
+int ix_gdn_scan(const void* q, const void* k, const void* v, const float* g, const void* beta, void* o,
+                int io_dtype, long q_pitch, long k_pitch, long v_pitch, float* state_pool,
+                const int* cu_seqlens, const int* state_indices, long state_indices_stride, long N, long H,
+                long HV, long K, long V, float scale, int time_tile, void* stream);
+
+/* gdn_l2norm (gdn_ops.py:202-213): y = x * (1/sqrt(sum x^2 + eps)) over rows of K.
+ * x [tokens, H, K] with token pitch x_pitch; y [tokens, H, K] contiguous. */
+int ix_gdn_l2norm(const void* x, long x_pitch, void* y, int io_dtype, long tokens, long H, long K, float eps,
+                  void* stream);
+
+/* gdn_gate_and_beta (gdn_ops.py:1197-1210) in the fp32 form of the fused core (gdn/_register.py:33-55):
+ * g = -exp(A_log[hv]) * softplus(a + dt_bias[hv]) fp32; beta = sigmoid(b) in io_dtype.
+ * a, b [tokens, HV]; A_log, dt_bias fp32 [HV]. */
+int ix_gdn_gate(const void* a, const void* b, const float* A_log, const float* dt_bias, float* g, void* beta,
+                int io_dtype, long tokens, long HV, void* stream);
+
+/* gdn_causal_conv / gdn_causal_conv_batched (gdn_ops.py:74-170) over packed tokens, and the
+ * engine's window-slide update (gdn_recurrent_state.py:686-707,814-825) when every sequence has
+ * one token. x,y bf16 [tokens, D]; weight bf16 [D, W]; bias bf16 [D] or NULL; conv_pool bf16
+ * [rows, D, W-1] oldest first. state_rows_in[n] <= 0 (or NULL) = no history; state_rows_out[n]
+ * > 0 stores the last W-1 inputs to that row (may equal the input row). */
+int ix_gdn_conv(const void* x, const void* weight, const void* bias, void* y, void* conv_pool,
+                const int* cu_seqlens, const int* state_rows_in, const int* state_rows_out, long N,
+                long total_tokens, long D, long W, int silu, void* stream);
+
+/* ---- MoE: ops/moe ------------------------------------------------------------------------- */
+
+/* fused_router_dense / ref_router_dense (moe_router_o2_kernel.py:272-311,369-386) with mode 0;
+ * mode 1 is softmax over all experts, top-k on the probabilities, renormalise. logits fp32
+ * [T, E] (pitch ld). Outputs: topk_idx int32 [T,k] and topk_prob fp32 [T,k] in rank order
+ * (score desc, index asc on ties); dense_probs fp32 [T,E] / dense_map uint8 [T,E] optional.
+ * k must be a power of two <= 16, E <= 512 (else declined). scaling 0 = none. */
+int ix_moe_router_topk(const float* logits, long ld, long T, long E, long k, int mode, float scaling,
+                       int* topk_idx, float* topk_prob, float* dense_probs, uint8_t* dense_map, void* stream);
+
+/* Sizing helpers (host arithmetic only). */
+long ix_moe_max_tiles(long T, long k, long E, long BM);   /* ceil(T*k/BM) + E */
+size_t ix_moe_permute_scratch_ints(long T, long E);
+int ix_moe_pick_bm(long T, long k, long E);               /* 32, 128 or 256 */
+
+/* fused_permute_index / ref_permute_index (moe_router_o2_kernel.py:313-351,389-397) plus the
+ * block map (moe_fused_experts.py:156-205) and the inverse permutation of
+ * moe_combine_rows_kernel.py. Integer work only.
+ *   counts int32 [E] tokens per expert; offsets int32 [E+1]; sorted_token int32 [T*k]
+ *   (expert-major, token ascending); permuted_prob fp32 [T*k]; combine_rows int32 [T,k] = the
+ *   token's rows in ascending expert order; tile_meta int32 [1 + 3*max_tiles] = {n_tiles,
+ *   tile_expert[], tile_row0[], tile_nrows[]} for row tiles of BM; scratch int32
+ *   [ix_moe_permute_scratch_ints]. */
+int ix_moe_permute(const int* topk_idx, const float* topk_prob, long T, long E, long k, long BM, int* counts,
+                   int* offsets, int* sorted_token, float* permuted_prob, int* combine_rows, int* tile_meta,
+                   long max_tiles, int* scratch, void* stream);
+
+/* _batched_experts_forward / _fused_forward (moe_batched_experts.py:301-531,
+ * moe_fused_experts.py:292-503): grouped fc1 + SwiGLU + prob epilogue, then grouped fc2.
+ * x bf16 [T, Hd] (pitch ldx) gathered through sorted_token; W1 bf16 [E, 2F, Hd] (gate rows
+ * then up rows); W2 bf16 [E, Hd, F]; inter bf16 [rows, F]; expert_out bf16 [rows, Hd];
+ * rows = T*k. BM must be the value given to ix_moe_permute. */
+int ix_moe_experts(const void* x, long ldx, const int* sorted_token, const float* permuted_prob,
+                   const void* W1, const void* W2, const int* tile_meta, long max_tiles, long BM, void* inter,
+                   void* expert_out, long rows, long Hd, long F, void* stream);
+
+/* _fixed_order_combine / _combine_topk_kernel (moe_batch_invariant.py:276-320,
+ * moe_combine_kernel.py:36-76): out bf16 [T, Hd] = the token's k rows of expert_out summed in
+ * ascending expert order; fp32_acc 0 = bf16 adds (a round per add), 1 = fp32 sum, one round. */
+int ix_moe_combine(const void* expert_out, const int* combine_rows, void* out, long T, long Hd, long k,
+                   int fp32_acc, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ISOEXEC_HIP_H */

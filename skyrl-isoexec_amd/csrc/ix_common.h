@@ -1,0 +1,134 @@
+// Shared device helpers for the gfx950 kernels: bf16 bit handling, fixed-order reductions,
+// the transcendental primitives every kernel variant of one op must share, launch checks.
+//
+// Determinism rules used throughout this library:
+//   * compiled with -ffp-contract=off: a fused multiply-add happens only where __builtin_fmaf
+//     is written, so the rounding points of every expression are the ones in the source;
+//   * no atomics, no split-K, no reduction whose shape depends on a batch dimension;
+//   * every reduction is one of two named orders (ix_tree8, ix_lane_tree) or a plain
+//     left-to-right loop.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define IX_OK 0
+#define IX_DECLINED 1
+#define IX_ERR_ARG (-1)
+#define IX_ERR_LAUNCH (-2)
+
+#define IX_DT_F32 0
+#define IX_DT_BF16 1
+
+typedef uint16_t bf16_t;
+
+#define IX_WAVE 64
+#define IX_LOG2E 1.44269504088896340736f
+#define IX_NEG_INF (-__builtin_huge_valf())
+
+__device__ __forceinline__ float ix_bf2f(bf16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+
+// Round-to-nearest-even fp32 -> bf16, NaN canonicalised to 0x7fc0 (the rule torch's CPU and
+// GPU casts use), written with integer ops so the rounding is the same everywhere it is used.
+__device__ __forceinline__ bf16_t ix_f2bf(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)0x7fc0;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+// bf16-round a float and widen it back (the "x.to(bf16).float()" of the eager expressions).
+__device__ __forceinline__ float ix_rbf(float f) { return ix_bf2f(ix_f2bf(f)); }
+
+__device__ __forceinline__ uint32_t ix_pack_bf2(float lo, float hi) {
+  return (uint32_t)ix_f2bf(lo) | ((uint32_t)ix_f2bf(hi) << 16);
+}
+
+// ---- the transcendental primitives -------------------------------------------------------
+// One definition each; every kernel of an op family calls these and nothing else, so prefill
+// and decode, M=1 and M=4096, see the same function. ix_prim_unary (ix_prims.hip) exports
+// them elementwise so a host-side checker can evaluate the same functions.
+__device__ __forceinline__ float ix_exp(float x) { return expf(x); }        // ocml, <=1 ulp
+__device__ __forceinline__ float ix_log(float x) { return logf(x); }        // ocml, <=1 ulp
+__device__ __forceinline__ float ix_log1p(float x) { return log1pf(x); }    // ocml
+// Fast exp for the vocabulary sum: one multiply and one v_exp_f32. Argument is always <= 0.
+__device__ __forceinline__ float ix_exp_fast(float x) { return __builtin_amdgcn_exp2f(x * IX_LOG2E); }
+// IEEE divide and square root (correctly rounded; hipcc's default for fp32), so 1/sqrt is
+// reproducible on any IEEE host.
+__device__ __forceinline__ float ix_rsqrt_ieee(float x) { return 1.0f / sqrtf(x); }
+__device__ __forceinline__ float ix_sigmoid(float x) { return 1.0f / (1.0f + ix_exp(-x)); }
+// ATen's fp32 SiLU form x / (1 + exp(-x)).
+__device__ __forceinline__ float ix_silu_div(float x) { return x / (1.0f + ix_exp(-x)); }
+// softplus with torch's threshold 20: x > 20 -> x, else log1p(exp(x)).
+__device__ __forceinline__ float ix_softplus(float x) { return x > 20.0f ? x : ix_log1p(ix_exp(x)); }
+
+// ---- fixed-order reductions --------------------------------------------------------------
+// ix_tree8: ((a0+a1)+(a2+a3))+((a4+a5)+(a6+a7))
+__device__ __forceinline__ float ix_tree8(const float (&a)[8]) {
+  return ((a[0] + a[1]) + (a[2] + a[3])) + ((a[4] + a[5]) + (a[6] + a[7]));
+}
+__device__ __forceinline__ float ix_tree8_max(const float (&a)[8]) {
+  return fmaxf(fmaxf(fmaxf(a[0], a[1]), fmaxf(a[2], a[3])), fmaxf(fmaxf(a[4], a[5]), fmaxf(a[6], a[7])));
+}
+
+// ix_lane_tree<L>: adjacent-pairwise binary tree over L consecutive lanes (L a power of two,
+// group aligned to L). Step s adds lane^s; fp add is commutative, so both partners hold the
+// same bits after each step and every lane of the group ends with the tree's root:
+//   level 1: p[2i]+p[2i+1], level 2: those pairs, ...
+template <int L>
+__device__ __forceinline__ float ix_lane_tree(float v) {
+#pragma unroll
+  for (int s = 1; s < L; s <<= 1) v = v + __shfl_xor(v, s, IX_WAVE);
+  return v;
+}
+template <int L>
+__device__ __forceinline__ float ix_lane_max(float v) {
+#pragma unroll
+  for (int s = 1; s < L; s <<= 1) v = fmaxf(v, __shfl_xor(v, s, IX_WAVE));
+  return v;
+}
+
+// ---- 8-element group loads ----------------------------------------------------------------
+// Load 8 consecutive elements starting at p, of which the first `valid` (may be <=0 or >=8)
+// exist; the others read as `fill`. `vec` says p is 16-byte aligned for bf16 / 32 for fp32.
+__device__ __forceinline__ void ix_load8(const bf16_t* __restrict__ p, long valid, bool vec, float fill,
+                                         float (&o)[8]) {
+  if (vec && valid >= 8) {
+    uint4 u = *reinterpret_cast<const uint4*>(p);
+    o[0] = __uint_as_float(u.x << 16); o[1] = __uint_as_float(u.x & 0xffff0000u);
+    o[2] = __uint_as_float(u.y << 16); o[3] = __uint_as_float(u.y & 0xffff0000u);
+    o[4] = __uint_as_float(u.z << 16); o[5] = __uint_as_float(u.z & 0xffff0000u);
+    o[6] = __uint_as_float(u.w << 16); o[7] = __uint_as_float(u.w & 0xffff0000u);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = (i < valid) ? ix_bf2f(p[i]) : fill;
+  }
+}
+__device__ __forceinline__ void ix_load8(const float* __restrict__ p, long valid, bool vec, float fill,
+                                         float (&o)[8]) {
+  if (vec && valid >= 8) {
+    float4 a = *reinterpret_cast<const float4*>(p);
+    float4 b = *reinterpret_cast<const float4*>(p + 4);
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = (i < valid) ? p[i] : fill;
+  }
+}
+
+__device__ __forceinline__ void ix_store8_bf16(bf16_t* __restrict__ p, long valid, bool vec, const float (&v)[8]) {
+  if (vec && valid >= 8) {
+    uint4 u;
+    u.x = ix_pack_bf2(v[0], v[1]); u.y = ix_pack_bf2(v[2], v[3]);
+    u.z = ix_pack_bf2(v[4], v[5]); u.w = ix_pack_bf2(v[6], v[7]);
+    *reinterpret_cast<uint4*>(p) = u;
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (i < valid) p[i] = ix_f2bf(v[i]);
+  }
+}
+
+static inline int ix_launch_status() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? IX_OK : IX_ERR_LAUNCH;
+}
+static inline bool ix_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }

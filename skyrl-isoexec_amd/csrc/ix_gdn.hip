@@ -1,0 +1,387 @@
+// GatedDeltaNet: the gated delta-rule scan, its l2norm/gating preparation and the causal
+// depthwise short conv.
+//
+// Scan (one function for varlen prefill and T=1 decode; reference call sites
+// skyrl/backends/skyrl_train/isoexec/ops/gdn/gdn_ops.py:400-441 and :513-558):
+//   per (sequence, value head hv), state S [V, K] fp32, for each token t in order
+//     S      <- S * exp(g_t)
+//     kv[v]   = sum_k S[v,k] * k_t[k]
+//     d[v]    = (v_t[v] - kv[v]) * beta_t
+//     S[v,k] <- S[v,k] + d[v] * k_t[k]
+//     o_t[v]  = sum_k S[v,k] * (q_t[k] * scale)
+//   state loaded from pool row idx[n,0], stored to pool row idx[n,t] after token t when that
+//   index is > 0; a sequence whose idx[n,0] <= 0 is skipped (its outputs are written as 0).
+//
+// Each state row S[v,:] evolves independently, so the work is N*HV*V row recurrences. A row is
+// owned by KS = K/8 consecutive lanes, lane s holding k = 8s..8s+7 in registers for the whole
+// sequence. The two dot products use one fixed order: in-lane, two fused-multiply-add chains
+// (even k, odd k) joined by one add; across the KS lanes, the adjacent-pairwise tree. The
+// same device function runs for every token of a prefill and for a decode step, and a "chunk"
+// is only how many tokens of q/k/v/g/beta are staged per LDS fill, so chunk length, the
+// prefill/decode split and batch composition cannot move a bit.
+#include "ix_common.h"
+#include "../../include/isoexec_hip.h"
+
+__device__ __forceinline__ float ix_ld(const float* p) { return *p; }
+__device__ __forceinline__ float ix_ld(const bf16_t* p) { return ix_bf2f(*p); }
+__device__ __forceinline__ void ix_st(float* p, float v) { *p = v; }
+__device__ __forceinline__ void ix_st(bf16_t* p, float v) { *p = ix_f2bf(v); }
+
+// dot of the lane's 8-element slices: (chain over k = 0,2,4,6) + (chain over k = 1,3,5,7)
+__device__ __forceinline__ float ix_dot8(const float (&s)[8], const float (&x)[8]) {
+  float pa = s[0] * x[0];
+  float pb = s[1] * x[1];
+  pa = __builtin_fmaf(s[2], x[2], pa);
+  pb = __builtin_fmaf(s[3], x[3], pb);
+  pa = __builtin_fmaf(s[4], x[4], pa);
+  pb = __builtin_fmaf(s[5], x[5], pb);
+  pa = __builtin_fmaf(s[6], x[6], pa);
+  pb = __builtin_fmaf(s[7], x[7], pb);
+  return pa + pb;
+}
+
+// One token of one state-row slice. Returns o (valid in every lane of the row's group).
+template <int KS>
+__device__ __forceinline__ float ix_gdn_step(float (&S)[8], const float (&kk)[8], const float (&qs)[8], float vv,
+                                             float eg, float bt) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) S[i] = S[i] * eg;
+  const float kv = ix_lane_tree<KS>(ix_dot8(S, kk));
+  const float d = (vv - kv) * bt;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) S[i] = __builtin_fmaf(d, kk[i], S[i]);
+  return ix_lane_tree<KS>(ix_dot8(S, qs));
+}
+
+template <int KS, typename TIO>
+__global__ __launch_bounds__(256) void k_gdn_scan(const TIO* __restrict__ q, const TIO* __restrict__ k,
+                                                  const TIO* __restrict__ v, const float* __restrict__ g,
+                                                  const TIO* __restrict__ beta, TIO* __restrict__ o,
+                                                  float* __restrict__ state, const int* __restrict__ cu,
+                                                  const int* __restrict__ sidx, long sidx_stride, long q_pitch,
+                                                  long k_pitch, long v_pitch, int H, int HV, int V, float scale,
+                                                  int TT) {
+  constexpr int K = KS * 8;
+  constexpr int R = 256 / KS;  // state rows per workgroup
+  extern __shared__ __align__(16) char ix_lds[];
+  float* kf = reinterpret_cast<float*>(ix_lds);  // [TT][K]
+  float* qf = kf + TT * K;                       // [TT][K], pre-scaled
+  float* vf = qf + TT * K;                       // [TT][R]
+  float* of = vf + TT * R;                       // [TT][R]
+  float* egf = of + TT * R;                      // [TT]
+  float* btf = egf + TT;                         // [TT]
+  int* sif = reinterpret_cast<int*>(btf + TT);   // [TT]
+
+  const int VB = V / R;
+  long bid = blockIdx.x;
+  const int vb = (int)(bid % VB);
+  bid /= VB;
+  const int hv = (int)(bid % HV);
+  const int n = (int)(bid / HV);
+  const int h = hv / (HV / H);
+  const int tid = threadIdx.x;
+  const int sub = tid % KS, r = tid / KS;
+  const int vrow = vb * R + r;
+
+  const int t_begin = cu[n], t_end = cu[n + 1];
+  const int len = t_end - t_begin;
+  if (len <= 0) return;
+  const int row0 = sidx[n * sidx_stride];
+  if (row0 <= 0) {  // null lane: no state, outputs defined as zero
+    for (int i = tid; i < len * R; i += 256) {
+      const int tt = i / R, rr = i % R;
+      ix_st(o + ((long)(t_begin + tt) * HV + hv) * V + vb * R + rr, 0.0f);
+    }
+    return;
+  }
+
+  float S[8];
+  {
+    const float* sp = state + (((long)row0 * HV + hv) * V + vrow) * K + sub * 8;
+    const float4 a = *reinterpret_cast<const float4*>(sp);
+    const float4 b = *reinterpret_cast<const float4*>(sp + 4);
+    S[0] = a.x; S[1] = a.y; S[2] = a.z; S[3] = a.w; S[4] = b.x; S[5] = b.y; S[6] = b.z; S[7] = b.w;
+  }
+
+  for (int t0 = 0; t0 < len; t0 += TT) {
+    const int nt = min(TT, len - t0);
+    __syncthreads();
+    for (int i = tid; i < nt * K; i += 256) {
+      const int tt = i / K, kk = i % K;
+      const long tok = t_begin + t0 + tt;
+      kf[i] = ix_ld(k + tok * k_pitch + h * K + kk);
+      qf[i] = ix_ld(q + tok * q_pitch + h * K + kk) * scale;
+    }
+    for (int i = tid; i < nt * R; i += 256) {
+      const int tt = i / R, rr = i % R;
+      vf[i] = ix_ld(v + (long)(t_begin + t0 + tt) * v_pitch + (long)hv * V + vb * R + rr);
+    }
+    for (int i = tid; i < nt; i += 256) {
+      const long src = (long)(t_begin + t0 + i) * HV + hv;
+      egf[i] = ix_exp(g[src]);
+      btf[i] = ix_ld(beta + src);
+      sif[i] = sidx[n * sidx_stride + t0 + i];
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      float kk[8], qs[8];
+      {
+        const float4 a = *reinterpret_cast<const float4*>(kf + tt * K + sub * 8);
+        const float4 b = *reinterpret_cast<const float4*>(kf + tt * K + sub * 8 + 4);
+        kk[0] = a.x; kk[1] = a.y; kk[2] = a.z; kk[3] = a.w; kk[4] = b.x; kk[5] = b.y; kk[6] = b.z; kk[7] = b.w;
+        const float4 c = *reinterpret_cast<const float4*>(qf + tt * K + sub * 8);
+        const float4 d = *reinterpret_cast<const float4*>(qf + tt * K + sub * 8 + 4);
+        qs[0] = c.x; qs[1] = c.y; qs[2] = c.z; qs[3] = c.w; qs[4] = d.x; qs[5] = d.y; qs[6] = d.z; qs[7] = d.w;
+      }
+      const float ov = ix_gdn_step<KS>(S, kk, qs, vf[tt * R + r], egf[tt], btf[tt]);
+      if (sub == 0) of[tt * R + r] = ov;
+      const int si = sif[tt];
+      if (si > 0) {
+        float* sp = state + (((long)si * HV + hv) * V + vrow) * K + sub * 8;
+        *reinterpret_cast<float4*>(sp) = make_float4(S[0], S[1], S[2], S[3]);
+        *reinterpret_cast<float4*>(sp + 4) = make_float4(S[4], S[5], S[6], S[7]);
+      }
+    }
+    __syncthreads();
+    for (int i = tid; i < nt * R; i += 256) {
+      const int tt = i / R, rr = i % R;
+      ix_st(o + ((long)(t_begin + t0 + tt) * HV + hv) * V + vb * R + rr, of[i]);
+    }
+  }
+}
+
+static size_t ix_gdn_lds_bytes(int K, int R, int TT) {
+  return (size_t)TT * (2 * K + 2 * R + 3) * sizeof(float);
+}
+
+template <int KS, typename TIO>
+static int ix_gdn_scan_launch(const void* q, const void* k, const void* v, const float* g, const void* beta,
+                              void* o, float* state, const int* cu, const int* sidx, long sidx_stride,
+                              long q_pitch, long k_pitch, long v_pitch, long N, int H, int HV, int V, float scale,
+                              int TT, hipStream_t st) {
+  constexpr int R = 256 / KS;
+  if (V % R != 0) return IX_DECLINED;
+  const long grid = N * HV * (V / R);
+  if (grid > 0x7fffffffL) return IX_DECLINED;
+  const size_t lds = ix_gdn_lds_bytes(KS * 8, R, TT);
+  auto kern = k_gdn_scan<KS, TIO>;
+  if (lds > 48 * 1024) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return IX_ERR_LAUNCH;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, st, (const TIO*)q, (const TIO*)k, (const TIO*)v, g,
+                     (const TIO*)beta, (TIO*)o, state, cu, sidx, sidx_stride, q_pitch, k_pitch, v_pitch, H, HV, V,
+                     scale, TT);
+  return ix_launch_status();
+}
+
+extern "C" int ix_gdn_scan(const void* q, const void* k, const void* v, const float* g, const void* beta, void* o,
+                           int io_dtype, long q_pitch, long k_pitch, long v_pitch, float* state_pool,
+                           const int* cu_seqlens, const int* state_indices, long state_indices_stride, long N,
+                           long H, long HV, long K, long V, float scale, int time_tile, void* stream) {
+  if (!q || !k || !v || !g || !beta || !o || !state_pool || !cu_seqlens || !state_indices) return IX_ERR_ARG;
+  if (N < 0 || H <= 0 || HV <= 0 || K <= 0 || V <= 0 || HV % H != 0 || state_indices_stride < 0) return IX_ERR_ARG;
+  if (q_pitch < H * K || k_pitch < H * K || v_pitch < HV * V) return IX_ERR_ARG;
+  if (io_dtype != IX_DT_F32 && io_dtype != IX_DT_BF16) return IX_DECLINED;
+  if (N == 0) return IX_OK;
+  if (!ix_aligned(state_pool, 16)) return IX_DECLINED;
+  int TT = time_tile <= 0 ? 32 : time_tile;
+  if (TT > 64) TT = 64;
+  hipStream_t st = (hipStream_t)stream;
+#define IX_SCAN_CASE(KSV)                                                                                         \
+  if (K == KSV * 8) {                                                                                             \
+    if (io_dtype == IX_DT_BF16)                                                                                   \
+      return ix_gdn_scan_launch<KSV, bf16_t>(q, k, v, g, beta, o, state_pool, cu_seqlens, state_indices,         \
+                                             state_indices_stride, q_pitch, k_pitch, v_pitch, N, (int)H,         \
+                                             (int)HV, (int)V, scale, TT, st);                                    \
+    return ix_gdn_scan_launch<KSV, float>(q, k, v, g, beta, o, state_pool, cu_seqlens, state_indices,            \
+                                          state_indices_stride, q_pitch, k_pitch, v_pitch, N, (int)H, (int)HV,   \
+                                          (int)V, scale, TT, st);                                                \
+  }
+  IX_SCAN_CASE(4)
+  IX_SCAN_CASE(8)
+  IX_SCAN_CASE(16)
+  IX_SCAN_CASE(32)
+#undef IX_SCAN_CASE
+  return IX_DECLINED;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Preparation (gdn_ops.py:173-213 l2norm, :1197-1210 gating; fused form gdn_ops.py:513-558):
+//   qn = io(x * (1 / sqrt(sum_k x_k^2 + 1e-6)))   sum: ix_tree8 over a lane's 8 squares, then the
+//                                                 adjacent-pairwise tree over the K/8 lanes
+//   g    = -exp(A_log[hv]) * softplus(a + dt_bias[hv])        fp32
+//   beta = io(sigmoid(b))
+template <int KS, typename TIO>
+__global__ __launch_bounds__(256) void k_gdn_l2norm(const TIO* __restrict__ x, TIO* __restrict__ y, long rows,
+                                                    int H, long x_pitch, float eps) {
+  constexpr int K = KS * 8;
+  constexpr int RPB = 256 / KS;
+  const int sub = threadIdx.x % KS;
+  const long row = (long)blockIdx.x * RPB + threadIdx.x / KS;
+  const long rrow = row < rows ? row : rows - 1;
+  float xv[8], sq[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    xv[i] = ix_ld(x + (rrow / H) * x_pitch + (rrow % H) * K + sub * 8 + i);
+    sq[i] = xv[i] * xv[i];
+  }
+  const float s = ix_lane_tree<KS>(ix_tree8(sq));
+  const float rn = ix_rsqrt_ieee(s + eps);
+  if (row >= rows) return;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ix_st(y + row * K + sub * 8 + i, xv[i] * rn);
+}
+
+template <typename TIO>
+__global__ __launch_bounds__(256) void k_gdn_gate(const TIO* __restrict__ a, const TIO* __restrict__ b,
+                                                  const float* __restrict__ A_log,
+                                                  const float* __restrict__ dt_bias, float* __restrict__ g,
+                                                  TIO* __restrict__ beta, long n, int HV) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const int hv = (int)(i % HV);
+  const float sp = ix_softplus(ix_ld(a + i) + dt_bias[hv]);
+  const float neg_ea = -ix_exp(A_log[hv]);
+  g[i] = neg_ea * sp;
+  ix_st(beta + i, ix_sigmoid(ix_ld(b + i)));
+}
+
+extern "C" int ix_gdn_l2norm(const void* x, long x_pitch, void* y, int io_dtype, long tokens, long H, long K,
+                             float eps, void* stream) {
+  if (!x || !y || tokens < 0 || H <= 0 || K <= 0 || x_pitch < H * K) return IX_ERR_ARG;
+  const long rows = tokens * H;
+  if (io_dtype != IX_DT_F32 && io_dtype != IX_DT_BF16) return IX_DECLINED;
+  if (rows == 0) return IX_OK;
+  hipStream_t st = (hipStream_t)stream;
+#define IX_L2_CASE(KSV)                                                                                          \
+  if (K == KSV * 8) {                                                                                            \
+    const long grid = (rows + (256 / KSV) - 1) / (256 / KSV);                                                    \
+    if (grid > 0x7fffffffL) return IX_DECLINED;                                                                  \
+    if (io_dtype == IX_DT_BF16)                                                                                  \
+      hipLaunchKernelGGL((k_gdn_l2norm<KSV, bf16_t>), dim3((unsigned)grid), dim3(256), 0, st, (const bf16_t*)x, \
+                         (bf16_t*)y, rows, (int)H, x_pitch, eps);                                                \
+    else                                                                                                         \
+      hipLaunchKernelGGL((k_gdn_l2norm<KSV, float>), dim3((unsigned)grid), dim3(256), 0, st, (const float*)x,   \
+                         (float*)y, rows, (int)H, x_pitch, eps);                                                 \
+    return ix_launch_status();                                                                                   \
+  }
+  IX_L2_CASE(4)
+  IX_L2_CASE(8)
+  IX_L2_CASE(16)
+  IX_L2_CASE(32)
+#undef IX_L2_CASE
+  return IX_DECLINED;
+}
+
+extern "C" int ix_gdn_gate(const void* a, const void* b, const float* A_log, const float* dt_bias, float* g,
+                           void* beta, int io_dtype, long tokens, long HV, void* stream) {
+  if (!a || !b || !A_log || !dt_bias || !g || !beta || tokens < 0 || HV <= 0) return IX_ERR_ARG;
+  if (io_dtype != IX_DT_F32 && io_dtype != IX_DT_BF16) return IX_DECLINED;
+  const long n = tokens * HV;
+  if (n == 0) return IX_OK;
+  const long grid = (n + 255) / 256;
+  if (grid > 0x7fffffffL) return IX_DECLINED;
+  hipStream_t st = (hipStream_t)stream;
+  if (io_dtype == IX_DT_BF16)
+    hipLaunchKernelGGL((k_gdn_gate<bf16_t>), dim3((unsigned)grid), dim3(256), 0, st, (const bf16_t*)a,
+                       (const bf16_t*)b, A_log, dt_bias, g, (bf16_t*)beta, n, (int)HV);
+  else
+    hipLaunchKernelGGL((k_gdn_gate<float>), dim3((unsigned)grid), dim3(256), 0, st, (const float*)a,
+                       (const float*)b, A_log, dt_bias, g, (float*)beta, n, (int)HV);
+  return ix_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Causal depthwise conv of width W <= 8 over packed tokens (gdn_ops.py:74-170):
+//   acc = 0; for i = 0..W-1: acc = acc + w[d,i] * xp[t+i]   (multiply rounded, add rounded)
+//   acc = acc + bias[d]; acc = acc * sigmoid(acc); y = bf16(acc)
+// xp = [W-1 previous inputs (oldest first), from the state pool row or zeros] ++ x. A decode
+// step is the same kernel with one token per sequence. The final state (the last W-1 inputs)
+// is written by a second kernel so an in-place pool row is never read and written in one launch.
+__device__ __forceinline__ int ix_seq_of(const int* __restrict__ cu, int N, int t) {
+  int lo = 0, hi = N;  // largest n with cu[n] <= t
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cu[mid] <= t) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+__device__ __forceinline__ float ix_conv_xp(const bf16_t* __restrict__ x, const bf16_t* __restrict__ pool,
+                                            int srow, int t_begin, int rel, long D, int d, int W) {
+  // rel: position relative to the sequence start; negative -> history slot W-1+rel
+  if (rel >= 0) return ix_bf2f(x[(long)(t_begin + rel) * D + d]);
+  if (srow <= 0) return 0.0f;
+  return ix_bf2f(pool[((long)srow * D + d) * (W - 1) + (W - 1 + rel)]);
+}
+
+__global__ __launch_bounds__(256) void k_gdn_conv(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                  const bf16_t* __restrict__ bias, bf16_t* __restrict__ y,
+                                                  const bf16_t* __restrict__ pool, const int* __restrict__ cu,
+                                                  const int* __restrict__ rows_in, int N, long D, int W,
+                                                  int silu, long total) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int t = (int)(i / D);
+  const int d = (int)(i % D);
+  const int n = ix_seq_of(cu, N, t);
+  const int t_begin = cu[n];
+  const int rel = t - t_begin;
+  const int srow = rows_in ? rows_in[n] : 0;
+  float acc = 0.0f;
+  for (int j = 0; j < W; ++j) {
+    const float xv = ix_conv_xp(x, pool, srow, t_begin, rel - (W - 1) + j, D, d, W);
+    const float p = ix_bf2f(w[(long)d * W + j]) * xv;
+    acc = acc + p;
+  }
+  if (bias) acc = acc + ix_bf2f(bias[d]);
+  if (silu) acc = acc * ix_sigmoid(acc);
+  y[i] = ix_f2bf(acc);
+}
+
+__global__ __launch_bounds__(256) void k_gdn_conv_state(const bf16_t* __restrict__ x, bf16_t* __restrict__ pool,
+                                                        const int* __restrict__ cu,
+                                                        const int* __restrict__ rows_in,
+                                                        const int* __restrict__ rows_out, int N, long D, int W) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (long)N * D) return;
+  const int n = (int)(i / D);
+  const int d = (int)(i % D);
+  const int orow = rows_out[n];
+  if (orow <= 0) return;
+  const int t_begin = cu[n], len = cu[n + 1] - t_begin;
+  const int srow = rows_in ? rows_in[n] : 0;
+  bf16_t tmp[8];
+  for (int j = 0; j < W - 1; ++j) {
+    // new history slot j holds the input at relative position len - (W-1) + j
+    const float xv = ix_conv_xp(x, pool, srow, t_begin, len - (W - 1) + j, D, d, W);
+    tmp[j] = ix_f2bf(xv);  // exact: the value is a bf16 already
+  }
+  for (int j = 0; j < W - 1; ++j) pool[((long)orow * D + d) * (W - 1) + j] = tmp[j];
+}
+
+extern "C" int ix_gdn_conv(const void* x, const void* weight, const void* bias, void* y, void* conv_pool,
+                           const int* cu_seqlens, const int* state_rows_in, const int* state_rows_out, long N,
+                           long total_tokens, long D, long W, int silu, void* stream) {
+  if (!x || !weight || !y || !cu_seqlens || N < 0 || total_tokens < 0 || D <= 0) return IX_ERR_ARG;
+  if (W < 1 || W > 8) return IX_DECLINED;
+  if ((state_rows_in || state_rows_out) && !conv_pool) return IX_ERR_ARG;
+  if (total_tokens > 0x7fffffffL || N > 0x7fffffffL) return IX_DECLINED;
+  hipStream_t st = (hipStream_t)stream;
+  const long total = total_tokens * D;
+  if (total > 0 && N > 0) {
+    const long grid = (total + 255) / 256;
+    if (grid > 0x7fffffffL) return IX_DECLINED;
+    hipLaunchKernelGGL(k_gdn_conv, dim3((unsigned)grid), dim3(256), 0, st, (const bf16_t*)x, (const bf16_t*)weight,
+                       (const bf16_t*)bias, (bf16_t*)y, (const bf16_t*)conv_pool, cu_seqlens, state_rows_in, (int)N,
+                       D, (int)W, silu, total);
+  }
+  if (state_rows_out && N > 0 && W > 1) {
+    const long grid = (N * D + 255) / 256;
+    if (grid > 0x7fffffffL) return IX_DECLINED;
+    hipLaunchKernelGGL(k_gdn_conv_state, dim3((unsigned)grid), dim3(256), 0, st, (const bf16_t*)x,
+                       (bf16_t*)conv_pool, cu_seqlens, state_rows_in, state_rows_out, (int)N, D, (int)W);
+  }
+  return ix_launch_status();
+}

@@ -1,0 +1,197 @@
+// Batch-invariant dense matmuls: the bf16 GEMM behind every linear layer and the LM head, and
+// the fp32 GEMM behind the MoE router. Counterpart of the reference's global aten mm/addmm
+// override (ops/moe/moe_batch_invariant.py:422-473, ops/mm/mm_tiles.py:127-158) and of its
+// pinned non-split-K provider (ops/mm/csrc/cublaslt_pinned.cpp:1-36).
+#include "ix_gemm_core.h"
+#include "../../include/isoexec_hip.h"
+
+// Workgroup -> tile map. Hardware hands consecutive workgroup ids to the 8 XCDs round-robin,
+// and each XCD has its own L2: all M-tiles of one weight tile go to one XCD so a weight tile
+// is fetched from HBM by exactly one L2, while the (small) activation matrix is shared
+// through the memory-side cache.
+__device__ __forceinline__ bool ix_tile_of_block(long bid, int nb_m, int nb_n, int* tm, int* tn) {
+  const int xcd = (int)(bid & 7);
+  const long idx = bid >> 3;
+  const long nloc = idx / nb_m;
+  *tm = (int)(idx - nloc * nb_m);
+  *tn = (int)(nloc * 8 + xcd);
+  return *tn < nb_n;
+}
+
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void k_gemm_bf16_nt(const bf16_t* __restrict__ A, long lda,
+                                                              const bf16_t* __restrict__ W, long ldw,
+                                                              const bf16_t* __restrict__ bias,
+                                                              bf16_t* __restrict__ C, long ldc, int M, int N,
+                                                              int K, int nb_m, int nb_n) {
+  using Cfg = IxGemmCfg<BM, BN, WM, WN>;
+  extern __shared__ __align__(16) char ix_lds[];
+  int tm, tn;
+  if (!ix_tile_of_block(blockIdx.x, nb_m, nb_n, &tm, &tn)) return;
+  const long m0 = (long)tm * BM;
+  const long n0 = (long)tn * BN;
+
+  ix_f32x16 acc[Cfg::MI][Cfg::NI];
+#pragma unroll
+  for (int mi = 0; mi < Cfg::MI; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < Cfg::NI; ++ni)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mi][ni][i] = 0.0f;
+
+  IxRowsPlain rows{A, lda, 0, (long)M};
+  const int n_valid = (int)min((long)BN, (long)N - n0);
+  IxWRowsPlain wrows{W + n0 * ldw, ldw, n_valid};
+  ix_gemm_mainloop<Cfg, BM, BN, WM, WN>(rows, m0, wrows, K, ix_lds, acc);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+#pragma unroll
+  for (int ni = 0; ni < Cfg::NI; ++ni) {
+    const long n = n0 + wn * Cfg::TN + ni * 32 + (lane & 31);
+    if (n >= N) continue;
+    // addmm: the bias joins in fp32 before the single bf16 round.
+    const float b = bias ? ix_bf2f(bias[n]) : 0.0f;
+#pragma unroll
+    for (int mi = 0; mi < Cfg::MI; ++mi) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const long m = m0 + wm * Cfg::TM + mi * 32 + ix_acc_row(i, lane);
+        if (m < M) {
+          float v = acc[mi][ni][i];
+          if (bias) v = v + b;
+          C[m * ldc + n] = ix_f2bf(v);
+        }
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int WM, int WN>
+static int ix_gemm_bf16_launch(const bf16_t* A, long lda, const bf16_t* W, long ldw, const bf16_t* bias, bf16_t* C,
+                               long ldc, long M, long N, long K, hipStream_t st) {
+  using Cfg = IxGemmCfg<BM, BN, WM, WN>;
+  const long nb_m = (M + BM - 1) / BM, nb_n = (N + BN - 1) / BN;
+  const long grid = 8 * nb_m * ((nb_n + 7) / 8);
+  if (grid > 0x7fffffffL) return IX_DECLINED;
+  auto kern = k_gemm_bf16_nt<BM, BN, WM, WN>;
+  static bool attr_set = false;  // per instantiation
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES) !=
+        hipSuccess)
+      return IX_ERR_LAUNCH;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(Cfg::NT), Cfg::LDS_BYTES, st, A, lda, W, ldw, bias, C, ldc,
+                     (int)M, (int)N, (int)K, (int)nb_m, (int)nb_n);
+  return ix_launch_status();
+}
+
+extern "C" int ix_gemm_bf16_nt(const void* A, long lda, const void* W, long ldw, const void* bias, void* C,
+                               long ldc, long M, long N, long K, int tile, void* stream) {
+  if (!A || !W || !C || M < 0 || N <= 0 || K <= 0) return IX_ERR_ARG;
+  if (lda < K || ldw < K || ldc < N) return IX_ERR_ARG;
+  // 16-byte row chunks: every row start and K itself must be a multiple of 8 elements.
+  if ((K % 8) || (lda % 8) || (ldw % 8) || !ix_aligned(A, 16) || !ix_aligned(W, 16)) return IX_DECLINED;
+  if (M > 0x7fffffffL || N > 0x7fffffffL || K > 0x7fffffffL) return IX_DECLINED;
+  if (M == 0) return IX_OK;
+  hipStream_t st = (hipStream_t)stream;
+  const bf16_t *a = (const bf16_t*)A, *w = (const bf16_t*)W, *b = (const bf16_t*)bias;
+  bf16_t* c = (bf16_t*)C;
+  // `tile` only picks which workgroup owns an element (0 = by M); the bits do not depend on it.
+  if (tile == 0) tile = (M <= 32) ? 1 : (M <= 128) ? 2 : 3;
+  switch (tile) {
+    case 1: return ix_gemm_bf16_launch<32, 256, 1, 4>(a, lda, w, ldw, b, c, ldc, M, N, K, st);
+    case 2: return ix_gemm_bf16_launch<128, 128, 2, 2>(a, lda, w, ldw, b, c, ldc, M, N, K, st);
+    case 3: return ix_gemm_bf16_launch<256, 256, 2, 4>(a, lda, w, ldw, b, c, ldc, M, N, K, st);
+    case 4: return ix_gemm_bf16_launch<256, 256, 2, 2>(a, lda, w, ldw, b, c, ldc, M, N, K, st);
+    case 5: return ix_gemm_bf16_launch<128, 256, 2, 4>(a, lda, w, ldw, b, c, ldc, M, N, K, st);
+    default: return IX_ERR_ARG;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// fp32 GEMM (router gating): C[m, n] = sum_k A[m, k] * W[n, k], A bf16 (widened exactly) or
+// fp32, W fp32, C fp32. One instruction, v_mfma_f32_32x32x2_f32; instruction j consumes
+// k = 2j (lane group 0) and 2j+1 (lane group 1); instructions accumulate left to right.
+#define IX_F32_BM 64
+#define IX_F32_BN 128
+#define IX_F32_BK 32
+#define IX_F32_PITCH 33
+
+template <typename TA>
+__global__ __launch_bounds__(256) void k_gemm_f32_nt(const TA* __restrict__ A, long lda,
+                                                     const float* __restrict__ W, long ldw,
+                                                     float* __restrict__ C, long ldc, int M, int N, int K) {
+  __shared__ float sA[IX_F32_BM * IX_F32_PITCH];
+  __shared__ float sW[IX_F32_BN * IX_F32_PITCH];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;  // 2 x 2 waves, wave tile 32 x 64
+  const long m0 = (long)blockIdx.x * IX_F32_BM;
+  const long n0 = (long)blockIdx.y * IX_F32_BN;
+  ix_f32x16 acc[2];
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[ni][i] = 0.0f;
+
+  for (int k0 = 0; k0 < K; k0 += IX_F32_BK) {
+    // stage A: 64 rows x 32 k, W: 128 rows x 32 k; one element per thread per pass
+    for (int q = tid; q < IX_F32_BM * IX_F32_BK; q += 256) {
+      const int r = q >> 5, c = q & 31;
+      const long m = m0 + r;
+      float v = 0.0f;
+      if (m < M && k0 + c < K) {
+        if constexpr (sizeof(TA) == 2) v = ix_bf2f(A[m * lda + k0 + c]);
+        else v = A[m * lda + k0 + c];
+      }
+      sA[r * IX_F32_PITCH + c] = v;
+    }
+    for (int q = tid; q < IX_F32_BN * IX_F32_BK; q += 256) {
+      const int r = q >> 5, c = q & 31;
+      const long n = n0 + r;
+      sW[r * IX_F32_PITCH + c] = (n < N && k0 + c < K) ? W[n * ldw + k0 + c] : 0.0f;
+    }
+    __syncthreads();
+    const int fr = lane & 31, fg = lane >> 5;
+#pragma unroll
+    for (int j = 0; j < IX_F32_BK / 2; ++j) {
+      const float a = sA[(wm * 32 + fr) * IX_F32_PITCH + 2 * j + fg];
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni) {
+        const float b = sW[(wn * 64 + ni * 32 + fr) * IX_F32_PITCH + 2 * j + fg];
+        acc[ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[ni], 0, 0, 0);
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni) {
+    const long n = n0 + wn * 64 + ni * 32 + (lane & 31);
+    if (n >= N) continue;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const long m = m0 + wm * 32 + ix_acc_row(i, lane);
+      if (m < M) C[m * ldc + n] = acc[ni][i];
+    }
+  }
+}
+
+extern "C" int ix_gemm_f32_nt(const void* A, int a_dtype, long lda, const void* W, long ldw, void* C, long ldc,
+                              long M, long N, long K, void* stream) {
+  if (!A || !W || !C || M < 0 || N <= 0 || K <= 0) return IX_ERR_ARG;
+  if (lda < K || ldw < K || ldc < N) return IX_ERR_ARG;
+  if (a_dtype != IX_DT_F32 && a_dtype != IX_DT_BF16) return IX_DECLINED;
+  if (M > 0x7fffffffL || N > 0x7fffffffL || K > 0x7fffffffL) return IX_DECLINED;
+  if (M == 0) return IX_OK;
+  const long gm = (M + IX_F32_BM - 1) / IX_F32_BM, gn = (N + IX_F32_BN - 1) / IX_F32_BN;
+  if (gn > 65535) return IX_DECLINED;
+  hipStream_t st = (hipStream_t)stream;
+  if (a_dtype == IX_DT_BF16)
+    hipLaunchKernelGGL((k_gemm_f32_nt<bf16_t>), dim3((unsigned)gm, (unsigned)gn), dim3(256), 0, st,
+                       (const bf16_t*)A, lda, (const float*)W, ldw, (float*)C, ldc, (int)M, (int)N, (int)K);
+  else
+    hipLaunchKernelGGL((k_gemm_f32_nt<float>), dim3((unsigned)gm, (unsigned)gn), dim3(256), 0, st,
+                       (const float*)A, lda, (const float*)W, ldw, (float*)C, ldc, (int)M, (int)N, (int)K);
+  return ix_launch_status();
+}

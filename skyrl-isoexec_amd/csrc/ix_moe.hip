@@ -1,0 +1,474 @@
+// Mixture-of-experts FFN: router top-k, expert-major permutation and block map, grouped
+// fc1 + SwiGLU + prob epilogue, grouped fc2, fixed-order combine.
+//
+// Per-token function (skyrl/backends/skyrl_train/isoexec/ops/moe/moe_router_o2_kernel.py:87-174,369-386,
+// moe_batched_experts.py:496-503, moe_batch_invariant.py:276-320, moe_combine_kernel.py:36-76):
+//   router : k winners by (score desc, expert index asc); NaN scores count as -inf
+//            mode 0: p = softmax over the k winning logits            (top-k then softmax)
+//            mode 1: softmax over all E, top-k on the probabilities, renormalise by their sum
+//            both sums over the k winners: adjacent-pairwise tree in rank order
+//   expert : inter = bf16(x W1^T); gate/up halves; s = bf16(gate / (1 + exp(-gate)));
+//            h = bf16(s * up); a = bf16(h * prob); y = bf16(a W2^T)
+//   combine: the token's k rows added in ascending expert order; bf16 adds (a round per add)
+//            or one fp32 sum and a single round.
+// Nothing a token sees depends on the other tokens of the batch: the permutation and the block
+// map are integer-only and only decide which workgroup computes a row; the GEMM core's K order
+// is fixed (ix_gemm_core.h).
+#include "ix_gemm_core.h"
+#include "../../include/isoexec_hip.h"
+
+#define IX_MOE_KMAX 16
+#define IX_MOE_EC 8  // experts per lane: E <= 512
+#define IX_MOE_TILE_T 256
+
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ bool ix_beats(float av, int ai, float bv, int bi, int sentinel) {
+  // does candidate a beat candidate b?  sentinel index = "no candidate"
+  if (ai == sentinel) return false;
+  if (bi == sentinel) return true;
+  return (av > bv) || (av == bv && ai < bi);
+}
+
+__device__ __forceinline__ float ix_tree_k(float (&t)[IX_MOE_KMAX], int k) {
+#pragma unroll
+  for (int s = 1; s < IX_MOE_KMAX; s <<= 1) {
+    if (s < k) {
+#pragma unroll
+      for (int i = 0; i < IX_MOE_KMAX; i += 2 * s)
+        if (i + s < k) t[i] = t[i] + t[i + s];
+    }
+  }
+  return t[0];
+}
+
+__global__ __launch_bounds__(256) void k_moe_router(const float* __restrict__ logits, long ld, int T, int E, int k,
+                                                    int mode, float scaling, int* __restrict__ topk_idx,
+                                                    float* __restrict__ topk_prob, float* __restrict__ dense_probs,
+                                                    uint8_t* __restrict__ dense_map) {
+  const int lane = threadIdx.x & 63;
+  const long t = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T) return;
+  float s[IX_MOE_EC];
+  bool live[IX_MOE_EC];
+#pragma unroll
+  for (int c = 0; c < IX_MOE_EC; ++c) {
+    const int e = lane + 64 * c;
+    live[c] = e < E;
+    float v = live[c] ? logits[t * ld + e] : IX_NEG_INF;
+    if (v != v) v = IX_NEG_INF;
+    s[c] = v;
+  }
+  if (mode == 1) {
+    float m = IX_NEG_INF;
+#pragma unroll
+    for (int c = 0; c < IX_MOE_EC; ++c) m = fmaxf(m, s[c]);
+    m = ix_lane_max<64>(m);
+    float z = 0.0f;
+#pragma unroll
+    for (int c = 0; c < IX_MOE_EC; ++c) {
+      s[c] = live[c] ? ix_exp(s[c] - m) : 0.0f;
+      z = z + s[c];
+    }
+    z = ix_lane_tree<64>(z);
+#pragma unroll
+    for (int c = 0; c < IX_MOE_EC; ++c) s[c] = s[c] / z;
+  }
+  float vals[IX_MOE_KMAX];
+  int idxs[IX_MOE_KMAX];
+#pragma unroll
+  for (int j = 0; j < IX_MOE_KMAX; ++j) {
+    vals[j] = 0.0f;
+    idxs[j] = 0;
+    if (j < k) {
+      float bv = 0.0f;
+      int bi = E;
+#pragma unroll
+      for (int c = 0; c < IX_MOE_EC; ++c) {
+        const int e = lane + 64 * c;
+        if (live[c] && ix_beats(s[c], e, bv, bi, E)) { bv = s[c]; bi = e; }
+      }
+#pragma unroll
+      for (int st = 1; st < 64; st <<= 1) {
+        const float ov = __shfl_xor(bv, st, IX_WAVE);
+        const int oi = __shfl_xor(bi, st, IX_WAVE);
+        if (ix_beats(ov, oi, bv, bi, E)) { bv = ov; bi = oi; }
+      }
+      bi = min(bi, E - 1);
+      vals[j] = bv;
+      idxs[j] = bi;
+#pragma unroll
+      for (int c = 0; c < IX_MOE_EC; ++c)
+        if (lane + 64 * c == bi) live[c] = false;
+    }
+  }
+  float p[IX_MOE_KMAX], tmp[IX_MOE_KMAX];
+  if (mode == 0) {
+    const float m = vals[0];
+#pragma unroll
+    for (int j = 0; j < IX_MOE_KMAX; ++j) { p[j] = (j < k) ? ix_exp(vals[j] - m) : 0.0f; tmp[j] = p[j]; }
+  } else {
+#pragma unroll
+    for (int j = 0; j < IX_MOE_KMAX; ++j) { p[j] = (j < k) ? vals[j] : 0.0f; tmp[j] = p[j]; }
+  }
+  const float den = ix_tree_k(tmp, k);
+#pragma unroll
+  for (int j = 0; j < IX_MOE_KMAX; ++j) {
+    p[j] = p[j] / den;
+    if (scaling != 0.0f) p[j] = p[j] * scaling;
+  }
+#pragma unroll
+  for (int j = 0; j < IX_MOE_KMAX; ++j) {
+    if (j < k && lane == j) {
+      topk_idx[t * k + j] = idxs[j];
+      topk_prob[t * k + j] = p[j];
+    }
+  }
+  if (dense_probs || dense_map) {
+#pragma unroll
+    for (int c = 0; c < IX_MOE_EC; ++c) {
+      const int e = lane + 64 * c;
+      if (e < E) {
+        float dp = 0.0f;
+        uint8_t dm = 0;
+#pragma unroll
+        for (int j = 0; j < IX_MOE_KMAX; ++j)
+          if (j < k && idxs[j] == e) { dp = p[j]; dm = 1; }
+        if (dense_probs) dense_probs[t * E + e] = dp;
+        if (dense_map) dense_map[t * E + e] = dm;
+      }
+    }
+  }
+}
+
+extern "C" int ix_moe_router_topk(const float* logits, long ld, long T, long E, long k, int mode, float scaling,
+                                  int* topk_idx, float* topk_prob, float* dense_probs, uint8_t* dense_map,
+                                  void* stream) {
+  if (!logits || !topk_idx || !topk_prob || T < 0 || E <= 0 || k <= 0 || ld < E) return IX_ERR_ARG;
+  if (k > E || k > IX_MOE_KMAX || (k & (k - 1)) != 0) return IX_DECLINED;  // pow2 k: padding would re-associate
+  if (E > 64 * IX_MOE_EC) return IX_DECLINED;
+  if (mode != 0 && mode != 1) return IX_ERR_ARG;
+  if (T == 0) return IX_OK;
+  const long grid = (T + 3) / 4;
+  if (grid > 0x7fffffffL) return IX_DECLINED;
+  hipLaunchKernelGGL(k_moe_router, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, logits, ld, (int)T,
+                     (int)E, (int)k, mode, scaling, topk_idx, topk_prob, dense_probs, dense_map);
+  return ix_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Permutation (integer only). Token tiles of 256; thread e of a tile walks the tile's (token,
+// slot) pairs in order, so each expert's rows come out token-ascending with no atomics.
+__global__ __launch_bounds__(256) void k_moe_tile_counts(const int* __restrict__ topk_idx, int T, int E, int k,
+                                                         int* __restrict__ tile_counts) {
+  __shared__ int s_idx[IX_MOE_TILE_T * IX_MOE_KMAX];
+  const int tile = blockIdx.x;
+  const int t0 = tile * IX_MOE_TILE_T;
+  const int nt = min(IX_MOE_TILE_T, T - t0);
+  for (int i = threadIdx.x; i < nt * k; i += 256) s_idx[i] = topk_idx[(long)t0 * k + i];
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += 256) {
+    int c = 0;
+    for (int i = 0; i < nt * k; ++i) c += (s_idx[i] == e);
+    tile_counts[(long)tile * E + e] = c;
+  }
+}
+
+// meta layout: [0] = number of m-tiles, then tile_expert[max_tiles], tile_row0[max_tiles],
+// tile_nrows[max_tiles].
+__global__ __launch_bounds__(256) void k_moe_offsets(const int* __restrict__ tile_counts, int ntiles, int E,
+                                                     int BM, int max_tiles, int* __restrict__ tile_base,
+                                                     int* __restrict__ counts, int* __restrict__ offsets,
+                                                     int* __restrict__ meta) {
+  for (int e = threadIdx.x; e < E; e += 256) {
+    int run = 0;
+    for (int tile = 0; tile < ntiles; ++tile) {
+      tile_base[(long)tile * E + e] = run;
+      run += tile_counts[(long)tile * E + e];
+    }
+    counts[e] = run;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0, nt = 0;
+    int* tile_expert = meta + 1;
+    int* tile_row0 = tile_expert + max_tiles;
+    int* tile_nrows = tile_row0 + max_tiles;
+    for (int e = 0; e < E; ++e) {
+      offsets[e] = run;
+      const int c = counts[e];
+      for (int r0 = 0; r0 < c && nt < max_tiles; r0 += BM) {
+        tile_expert[nt] = e;
+        tile_row0[nt] = run + r0;
+        tile_nrows[nt] = min(BM, c - r0);
+        ++nt;
+      }
+      run += c;
+    }
+    offsets[E] = run;
+    meta[0] = nt;
+  }
+}
+
+__global__ __launch_bounds__(256) void k_moe_scatter(const int* __restrict__ topk_idx,
+                                                     const float* __restrict__ topk_prob, int T, int E, int k,
+                                                     const int* __restrict__ tile_base,
+                                                     const int* __restrict__ offsets, int* __restrict__ sorted_token,
+                                                     float* __restrict__ permuted_prob,
+                                                     int* __restrict__ combine_rows) {
+  __shared__ int s_idx[IX_MOE_TILE_T * IX_MOE_KMAX];
+  __shared__ float s_prob[IX_MOE_TILE_T * IX_MOE_KMAX];
+  const int tile = blockIdx.x;
+  const int t0 = tile * IX_MOE_TILE_T;
+  const int nt = min(IX_MOE_TILE_T, T - t0);
+  for (int i = threadIdx.x; i < nt * k; i += 256) {
+    s_idx[i] = topk_idx[(long)t0 * k + i];
+    s_prob[i] = topk_prob[(long)t0 * k + i];
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += 256) {
+    int pos = offsets[e] + tile_base[(long)tile * E + e];
+    for (int tt = 0; tt < nt; ++tt) {
+      for (int j = 0; j < k; ++j) {
+        if (s_idx[tt * k + j] == e) {
+          int rank = 0;
+          for (int j2 = 0; j2 < k; ++j2) rank += (s_idx[tt * k + j2] < e);
+          const long t = t0 + tt;
+          sorted_token[pos] = (int)t;
+          permuted_prob[pos] = s_prob[tt * k + j];
+          combine_rows[t * k + rank] = pos;
+          ++pos;
+        }
+      }
+    }
+  }
+}
+
+extern "C" long ix_moe_max_tiles(long T, long k, long E, long BM) {
+  if (T < 0 || k <= 0 || E <= 0 || BM <= 0) return 0;
+  return (T * k + BM - 1) / BM + E;
+}
+
+extern "C" size_t ix_moe_permute_scratch_ints(long T, long E) {
+  if (T < 0 || E <= 0) return 0;
+  const long ntiles = (T + IX_MOE_TILE_T - 1) / IX_MOE_TILE_T;
+  return (size_t)(2 * ntiles * E);
+}
+
+extern "C" int ix_moe_pick_bm(long T, long k, long E) {
+  const long avg = (T * k) / (E > 0 ? E : 1);
+  return avg >= 192 ? 256 : (avg >= 48 ? 128 : 32);
+}
+
+extern "C" int ix_moe_permute(const int* topk_idx, const float* topk_prob, long T, long E, long k, long BM,
+                              int* counts, int* offsets, int* sorted_token, float* permuted_prob,
+                              int* combine_rows, int* tile_meta, long max_tiles, int* scratch, void* stream) {
+  if (!topk_idx || !topk_prob || !counts || !offsets || !sorted_token || !permuted_prob || !combine_rows ||
+      !tile_meta || !scratch)
+    return IX_ERR_ARG;
+  if (T < 0 || E <= 0 || k <= 0 || k > IX_MOE_KMAX || BM <= 0) return IX_ERR_ARG;
+  if (max_tiles < ix_moe_max_tiles(T, k, E, BM)) return IX_ERR_ARG;
+  if (T * k > 0x7fffffffL) return IX_DECLINED;
+  hipStream_t st = (hipStream_t)stream;
+  const long ntiles = (T + IX_MOE_TILE_T - 1) / IX_MOE_TILE_T;
+  int* tile_counts = scratch;
+  int* tile_base = scratch + ntiles * E;
+  if (ntiles > 0)
+    hipLaunchKernelGGL(k_moe_tile_counts, dim3((unsigned)ntiles), dim3(256), 0, st, topk_idx, (int)T, (int)E, (int)k,
+                       tile_counts);
+  hipLaunchKernelGGL(k_moe_offsets, dim3(1), dim3(256), 0, st, tile_counts, (int)ntiles, (int)E, (int)BM,
+                     (int)max_tiles, tile_base, counts, offsets, tile_meta);
+  if (ntiles > 0)
+    hipLaunchKernelGGL(k_moe_scatter, dim3((unsigned)ntiles), dim3(256), 0, st, topk_idx, topk_prob, (int)T, (int)E,
+                       (int)k, tile_base, offsets, sorted_token, permuted_prob, combine_rows);
+  return ix_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Grouped GEMMs over the block map. A workgroup past the device-side tile count exits at once,
+// so the host never reads the routing back.
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void k_moe_fc1_glu(const bf16_t* __restrict__ x, long ldx,
+                                                             const int* __restrict__ sorted_token,
+                                                             const float* __restrict__ permuted_prob,
+                                                             const bf16_t* __restrict__ W1,
+                                                             const int* __restrict__ meta, int max_tiles,
+                                                             bf16_t* __restrict__ inter, int Hd, int F, int nb_n) {
+  using Cfg = IxGemmCfg<BM, BN, WM, WN>;
+  static_assert(Cfg::NI == 2, "a wave must hold one gate tile and its up tile");
+  extern __shared__ __align__(16) char ix_lds[];
+  const int mt = blockIdx.x / nb_n, nt = blockIdx.x % nb_n;
+  if (mt >= meta[0]) return;
+  const int e = meta[1 + mt];
+  const long row0 = meta[1 + max_tiles + mt];
+  const long nrows = meta[1 + 2 * max_tiles + mt];
+  const int n0h = nt * (BN / 2);
+
+  ix_f32x16 acc[Cfg::MI][2];
+#pragma unroll
+  for (int mi = 0; mi < Cfg::MI; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mi][ni][i] = 0.0f;
+
+  IxRowsGather rows{x, ldx, sorted_token, row0, row0 + nrows};
+  IxWRowsGlu wrows{W1 + (long)e * 2 * F * Hd, (long)Hd, n0h, F};
+  ix_gemm_mainloop<Cfg, BM, BN, WM, WN>(rows, row0, wrows, Hd, ix_lds, acc);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  const int col = n0h + wn * 32 + (lane & 31);
+  if (col >= F) return;
+#pragma unroll
+  for (int mi = 0; mi < Cfg::MI; ++mi) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const long m = row0 + wm * Cfg::TM + mi * 32 + ix_acc_row(i, lane);
+      if (m < row0 + nrows) {
+        const float gate = ix_rbf(acc[mi][0][i]);
+        const float up = ix_rbf(acc[mi][1][i]);
+        const float s = ix_rbf(ix_silu_div(gate));
+        const float h = ix_rbf(s * up);
+        inter[m * F + col] = ix_f2bf(h * permuted_prob[m]);
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void k_moe_fc2(const bf16_t* __restrict__ inter,
+                                                         const bf16_t* __restrict__ W2,
+                                                         const int* __restrict__ meta, int max_tiles,
+                                                         bf16_t* __restrict__ out, int Hd, int F, int nb_n) {
+  using Cfg = IxGemmCfg<BM, BN, WM, WN>;
+  extern __shared__ __align__(16) char ix_lds[];
+  const int mt = blockIdx.x / nb_n, nt = blockIdx.x % nb_n;
+  if (mt >= meta[0]) return;
+  const int e = meta[1 + mt];
+  const long row0 = meta[1 + max_tiles + mt];
+  const long nrows = meta[1 + 2 * max_tiles + mt];
+  const long n0 = (long)nt * BN;
+
+  ix_f32x16 acc[Cfg::MI][Cfg::NI];
+#pragma unroll
+  for (int mi = 0; mi < Cfg::MI; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < Cfg::NI; ++ni)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mi][ni][i] = 0.0f;
+
+  IxRowsPlain rows{inter, (long)F, row0, row0 + nrows};
+  IxWRowsPlain wrows{W2 + ((long)e * Hd + n0) * F, (long)F, (int)min((long)BN, (long)Hd - n0)};
+  ix_gemm_mainloop<Cfg, BM, BN, WM, WN>(rows, row0, wrows, F, ix_lds, acc);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+#pragma unroll
+  for (int ni = 0; ni < Cfg::NI; ++ni) {
+    const long n = n0 + wn * Cfg::TN + ni * 32 + (lane & 31);
+    if (n >= Hd) continue;
+#pragma unroll
+    for (int mi = 0; mi < Cfg::MI; ++mi) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const long m = row0 + wm * Cfg::TM + mi * 32 + ix_acc_row(i, lane);
+        if (m < row0 + nrows) out[m * Hd + n] = ix_f2bf(acc[mi][ni][i]);
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int WM, int WN>
+static int ix_moe_experts_launch(const bf16_t* x, long ldx, const int* sorted_token, const float* permuted_prob,
+                                 const bf16_t* W1, const bf16_t* W2, const int* meta, long max_tiles,
+                                 bf16_t* inter, bf16_t* out, int Hd, int F, hipStream_t st) {
+  using Cfg = IxGemmCfg<BM, BN, WM, WN>;
+  auto k1 = k_moe_fc1_glu<BM, BN, WM, WN>;
+  auto k2 = k_moe_fc2<BM, BN, WM, WN>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES) !=
+            hipSuccess ||
+        hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES) !=
+            hipSuccess)
+      return IX_ERR_LAUNCH;
+    attr_set = true;
+  }
+  const long nb1 = (F + BN / 2 - 1) / (BN / 2);
+  const long nb2 = (Hd + BN - 1) / BN;
+  if (max_tiles * nb1 > 0x7fffffffL || max_tiles * nb2 > 0x7fffffffL) return IX_DECLINED;
+  hipLaunchKernelGGL(k1, dim3((unsigned)(max_tiles * nb1)), dim3(Cfg::NT), Cfg::LDS_BYTES, st, x, ldx, sorted_token,
+                     permuted_prob, W1, meta, (int)max_tiles, inter, Hd, F, (int)nb1);
+  hipLaunchKernelGGL(k2, dim3((unsigned)(max_tiles * nb2)), dim3(Cfg::NT), Cfg::LDS_BYTES, st, inter, W2, meta,
+                     (int)max_tiles, out, Hd, F, (int)nb2);
+  return ix_launch_status();
+}
+
+extern "C" int ix_moe_experts(const void* x, long ldx, const int* sorted_token, const float* permuted_prob,
+                              const void* W1, const void* W2, const int* tile_meta, long max_tiles, long BM,
+                              void* inter, void* expert_out, long rows, long Hd, long F, void* stream) {
+  if (!x || !sorted_token || !permuted_prob || !W1 || !W2 || !tile_meta || !inter || !expert_out)
+    return IX_ERR_ARG;
+  if (rows < 0 || Hd <= 0 || F <= 0 || max_tiles < 0 || ldx < Hd) return IX_ERR_ARG;
+  if ((Hd % 8) || (F % 8) || (ldx % 8) || !ix_aligned(x, 16) || !ix_aligned(W1, 16) || !ix_aligned(W2, 16) ||
+      !ix_aligned(inter, 16))
+    return IX_DECLINED;
+  if (rows == 0 || max_tiles == 0) return IX_OK;
+  hipStream_t st = (hipStream_t)stream;
+  const bf16_t *xx = (const bf16_t*)x, *w1 = (const bf16_t*)W1, *w2 = (const bf16_t*)W2;
+  bf16_t *it = (bf16_t*)inter, *eo = (bf16_t*)expert_out;
+  switch (BM) {
+    case 32:
+      return ix_moe_experts_launch<32, 256, 1, 4>(xx, ldx, sorted_token, permuted_prob, w1, w2, tile_meta,
+                                                  max_tiles, it, eo, (int)Hd, (int)F, st);
+    case 128:
+      return ix_moe_experts_launch<128, 256, 2, 4>(xx, ldx, sorted_token, permuted_prob, w1, w2, tile_meta,
+                                                   max_tiles, it, eo, (int)Hd, (int)F, st);
+    case 256:
+      return ix_moe_experts_launch<256, 256, 2, 4>(xx, ldx, sorted_token, permuted_prob, w1, w2, tile_meta,
+                                                   max_tiles, it, eo, (int)Hd, (int)F, st);
+    default: return IX_ERR_ARG;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_moe_combine(const bf16_t* __restrict__ expert_out,
+                                                     const int* __restrict__ combine_rows,
+                                                     bf16_t* __restrict__ out, long T, int Hd, int k, int fp32_acc,
+                                                     int vec) {
+  const int groups = (Hd + 7) / 8;
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= T * groups) return;
+  const long t = i / groups;
+  const int c0 = (int)(i % groups) * 8;
+  float acc[8];
+  for (int r = 0; r < k; ++r) {
+    const long row = combine_rows[t * k + r];
+    float xv[8];
+    ix_load8(expert_out + row * Hd + c0, Hd - c0, vec != 0, 0.0f, xv);
+    if (r == 0) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] = xv[j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float sum = acc[j] + xv[j];
+        acc[j] = fp32_acc ? sum : ix_rbf(sum);
+      }
+    }
+  }
+  ix_store8_bf16(out + t * Hd + c0, Hd - c0, vec != 0, acc);
+}
+
+extern "C" int ix_moe_combine(const void* expert_out, const int* combine_rows, void* out, long T, long Hd, long k,
+                              int fp32_acc, void* stream) {
+  if (!expert_out || !combine_rows || !out || T < 0 || Hd <= 0 || k <= 0) return IX_ERR_ARG;
+  if (T == 0) return IX_OK;
+  const long groups = (Hd + 7) / 8;
+  const long grid = (T * groups + 255) / 256;
+  if (grid > 0x7fffffffL) return IX_DECLINED;
+  const int vec = (Hd % 8 == 0) && ix_aligned(expert_out, 16) && ix_aligned(out, 16);
+  hipLaunchKernelGGL(k_moe_combine, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream,
+                     (const bf16_t*)expert_out, combine_rows, (bf16_t*)out, T, (int)Hd, (int)k, fp32_acc, vec);
+  return ix_launch_status();
+}

@@ -1,0 +1,150 @@
+// Zero-centred RMSNorm, the GatedDeltaNet gated output norm and the residual add + norm.
+//
+// Down-cast chain (skyrl/backends/skyrl_train/isoexec/ops/norms/fused_outnorm.py:16-29,113-232;
+// eager form ops/norms/zero_centered_norm.py:36-37 and runtimes/megatron/gdn_fla_shim.py:390-425):
+//   s    = sum_j x_j^2 in fp32          rstd = 1 / sqrt(s / N + eps)   (IEEE divide and sqrt)
+//   nb   = bf16(x * rstd)
+//   gam  = bf16(1 + w)  (zero-centred)   or  w
+//   y    = bf16(nb * gam)
+//   gated: out = bf16(y * (g / (1 + exp(-g))))   in fp32, one round
+//   add : h = bf16(x + r) (fp32 add, one round), then the chain on h; h is also returned.
+//
+// The reduction order is a function of N alone. A row is owned by LPR = min(64, pow2ceil(N/8))
+// consecutive lanes; lane l, slot i holds columns c*LPR*8 + l*8 + i; slot sums run left to right
+// over chunks c (multiply rounded, then add rounded: no fused multiply-add), then ix_tree8 over
+// the 8 slots, then the adjacent-pairwise lane tree over the LPR lanes. Rows only pick the grid.
+#include "ix_common.h"
+#include "../../include/isoexec_hip.h"
+
+template <int LPR>
+__device__ __forceinline__ float ix_row_sumsq(const bf16_t* __restrict__ xr, const bf16_t* __restrict__ rr,
+                                              int N, int sub, bool vec) {
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int off = sub * 8; off < N; off += LPR * 8) {
+    float x[8];
+    ix_load8(xr + off, N - off, vec, 0.0f, x);
+    if (rr) {
+      float r[8];
+      ix_load8(rr + off, N - off, vec, 0.0f, r);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = ix_rbf(x[i] + r[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float sq = x[i] * x[i];
+      acc[i] = acc[i] + sq;
+    }
+  }
+  return ix_lane_tree<LPR>(ix_tree8(acc));
+}
+
+// MODE 0: plain; 1: gated (gate strided by token); 2: residual add (writes h too).
+template <int LPR, int MODE>
+__global__ __launch_bounds__(256) void k_rmsnorm(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                 bf16_t* __restrict__ out, long M, int N, float eps,
+                                                 int zero_centered, const bf16_t* __restrict__ aux,
+                                                 long aux_stride_t, int HV, bf16_t* __restrict__ h_out,
+                                                 int vec) {
+  constexpr int RPB = 256 / LPR;  // rows per workgroup
+  const int tid = threadIdx.x;
+  const int sub = tid % LPR;
+  const long row = (long)blockIdx.x * RPB + tid / LPR;
+  // Lanes of rows past M still run the shuffles (their row pointer is clamped), never store.
+  const bool live = row < M;
+  const long rrow = live ? row : (M - 1);
+  const bf16_t* xr = x + rrow * N;
+  const bf16_t* rr = nullptr;
+  if (MODE == 2) rr = aux + rrow * N;
+  const float s = ix_row_sumsq<LPR>(xr, rr, N, sub, vec != 0);
+  const float ms = s / (float)N;
+  const float rstd = ix_rsqrt_ieee(ms + eps);
+  const bf16_t* gr = nullptr;
+  if (MODE == 1) {
+    const long t = rrow / HV, hh = rrow % HV;
+    gr = aux + t * aux_stride_t + hh * N;
+  }
+  if (!live) return;
+  bf16_t* orow = out + row * N;
+  for (int off = sub * 8; off < N; off += LPR * 8) {
+    float xv[8], wv[8], o[8];
+    ix_load8(xr + off, N - off, vec != 0, 0.0f, xv);
+    ix_load8(w + off, N - off, vec != 0, 0.0f, wv);
+    if (MODE == 2) {
+      float r[8];
+      ix_load8(rr + off, N - off, vec != 0, 0.0f, r);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) xv[i] = ix_rbf(xv[i] + r[i]);
+      ix_store8_bf16(h_out + row * N + off, N - off, vec != 0, xv);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float nb = ix_rbf(xv[i] * rstd);
+      const float gam = zero_centered ? ix_rbf(1.0f + wv[i]) : wv[i];
+      o[i] = ix_rbf(nb * gam);
+    }
+    if (MODE == 1) {
+      float g[8];
+      ix_load8(gr + off, N - off, vec != 0 && (aux_stride_t % 8 == 0), 0.0f, g);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) o[i] = o[i] * ix_silu_div(g[i]);
+    }
+    ix_store8_bf16(orow + off, N - off, vec != 0, o);
+  }
+}
+
+static int ix_lpr_for(int N) {
+  int groups = (N + 7) / 8, l = 1;
+  while (l < groups && l < 64) l <<= 1;
+  return l;
+}
+
+template <int MODE>
+static int ix_norm_launch(const bf16_t* x, const bf16_t* w, bf16_t* out, long M, int N, float eps, int zc,
+                          const bf16_t* aux, long aux_stride_t, int HV, bf16_t* h_out, hipStream_t st) {
+  if (M == 0) return IX_OK;
+  const int lpr = ix_lpr_for(N);
+  int vec = (N % 8 == 0) && ix_aligned(x, 16) && ix_aligned(w, 16) && ix_aligned(out, 16);
+  if (MODE != 0) vec = vec && ix_aligned(aux, 16);
+  if (MODE == 2) vec = vec && ix_aligned(h_out, 16);
+  const long rpb = 256 / lpr;
+  const long grid = (M + rpb - 1) / rpb;
+  if (grid > 0x7fffffffL) return IX_DECLINED;
+#define IX_NORM_CASE(L)                                                                                          \
+  case L:                                                                                                        \
+    hipLaunchKernelGGL((k_rmsnorm<L, MODE>), dim3((unsigned)grid), dim3(256), 0, st, x, w, out, M, N, eps, zc,   \
+                       aux, aux_stride_t, HV, h_out, vec);                                                       \
+    break;
+  switch (lpr) {
+    IX_NORM_CASE(1) IX_NORM_CASE(2) IX_NORM_CASE(4) IX_NORM_CASE(8) IX_NORM_CASE(16) IX_NORM_CASE(32)
+    IX_NORM_CASE(64)
+    default: return IX_ERR_ARG;
+  }
+#undef IX_NORM_CASE
+  return ix_launch_status();
+}
+
+extern "C" int ix_rmsnorm_gamma(const void* x, const void* weight, void* out, long M, long N, float eps,
+                                int zero_centered, void* stream) {
+  if (!x || !weight || !out || M < 0 || N <= 0) return IX_ERR_ARG;
+  if (N > (1 << 20)) return IX_DECLINED;
+  return ix_norm_launch<0>((const bf16_t*)x, (const bf16_t*)weight, (bf16_t*)out, M, (int)N, eps, zero_centered,
+                           nullptr, 0, 1, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int ix_gated_out_norm(const void* x, const void* gate, long gate_stride_t, const void* weight,
+                                 void* out, long T, long HV, long N, float eps, int zero_centered, void* stream) {
+  if (!x || !gate || !weight || !out || T < 0 || HV <= 0 || N <= 0) return IX_ERR_ARG;
+  if (N > (1 << 20) || HV > (1 << 20)) return IX_DECLINED;
+  if (gate_stride_t < HV * N) return IX_ERR_ARG;
+  return ix_norm_launch<1>((const bf16_t*)x, (const bf16_t*)weight, (bf16_t*)out, T * HV, (int)N, eps,
+                           zero_centered, (const bf16_t*)gate, gate_stride_t, (int)HV, nullptr,
+                           (hipStream_t)stream);
+}
+
+extern "C" int ix_add_rmsnorm_gamma(const void* x, const void* residual, const void* weight, void* out,
+                                    void* h_out, long M, long N, float eps, int zero_centered, void* stream) {
+  if (!x || !residual || !weight || !out || !h_out || M < 0 || N <= 0) return IX_ERR_ARG;
+  if (N > (1 << 20)) return IX_DECLINED;
+  return ix_norm_launch<2>((const bf16_t*)x, (const bf16_t*)weight, (bf16_t*)out, M, (int)N, eps, zero_centered,
+                           (const bf16_t*)residual, 0, 1, (bf16_t*)h_out, (hipStream_t)stream);
+}

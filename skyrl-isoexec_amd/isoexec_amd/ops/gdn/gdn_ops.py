@@ -1,0 +1,255 @@
+"""GatedDeltaNet op functions on the HIP kernels.
+
+Same names, argument meaning and error behaviour as the reference's ``ops/gdn/gdn_ops.py``:
+``gdn_recurrent_kernel`` (:400-441), ``gdn_native_core_kernel`` (:513-558), ``gdn_causal_conv``
+(:74-129), ``gdn_causal_conv_batched`` (:132-170), ``gdn_l2norm`` (:202-213),
+``gdn_gate_and_beta`` (:1197-1210), ``gdn_recurrent`` (:997-1027), ``gdn_native_core``
+(:702-716), ``gdn_core`` (:1118-1194). Forward only: the trainer's VJP is out of scope.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ... import _lib
+
+L2NORM_EPS = 1e-6  # gdn_ops.py:173
+
+
+def _token_pitch(t: torch.Tensor) -> int:
+    """Element pitch between tokens of a ``[..., heads, dim]`` tensor whose heads are contiguous."""
+    if t.stride(-1) != 1 or t.stride(-2) != t.shape[-1]:
+        raise RuntimeError(f"[isoexec-amd] heads must be contiguous inside a token, got strides {t.stride()}")
+    return t.stride(-3)
+
+
+def _flatten_tokens(t: torch.Tensor, tail: int) -> torch.Tensor:
+    """``[B, T, *tail]`` -> a view ``[B*T, *tail]`` (copying only if B and T cannot be merged)."""
+    lead = t.shape[: t.ndim - tail]
+    if len(lead) == 1:
+        return t
+    if len(lead) != 2:
+        raise RuntimeError(f"[isoexec-amd] expected [B, T, ...], got {tuple(t.shape)}")
+    b, n = lead
+    if b == 1:
+        return t[0]
+    if t.stride(0) == n * t.stride(1):
+        return t.as_strided((b * n, *t.shape[2:]), (t.stride(1), *t.stride()[2:]), t.storage_offset())
+    return t.reshape(b * n, *t.shape[2:])
+
+
+def gdn_recurrent_kernel(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    g: torch.Tensor,
+    beta: torch.Tensor,
+    *,
+    ssm_state: torch.Tensor,
+    state_indices: torch.Tensor,
+    cu_seqlens: torch.Tensor | None = None,
+    time_tile: int = 0,
+) -> torch.Tensor:
+    """The delta-rule scan. Advances ``ssm_state`` IN PLACE. Returns ``o`` shaped like ``v``.
+
+    ``q, k``: ``[B, T, H, K]`` already L2-normalised (H may be GQA-compressed: ``HV % H == 0``);
+    ``v``: ``[B, T, HV, V]``; ``g`` (fp32), ``beta``: ``[B, T, HV]``; ``ssm_state`` fp32 pool
+    ``[S, HV, V, K]``; ``state_indices`` ``[N]`` (one-token decode) or ``[N, Tmax]``; ``cu_seqlens``
+    ``[N+1]`` int32 for a packed batch (then ``B == 1``), ``None`` for ``[B, T, ...]``.
+    """
+    _lib.require_device(q, k, v, g, beta, ssm_state, state_indices, cu_seqlens)
+    if q.ndim != 4 or v.ndim != 4:
+        raise RuntimeError(f"[isoexec-amd] gdn_recurrent_kernel expects [B,T,H,K]/[B,T,HV,V], got {tuple(q.shape)}")
+    B, T, H, K = q.shape
+    HV, V = v.shape[-2], v.shape[-1]
+    if ssm_state.dtype is not torch.float32 or not ssm_state.is_contiguous():
+        raise RuntimeError("[isoexec-amd] ssm_state must be a contiguous fp32 pool [S, HV, V, K]")
+    if tuple(ssm_state.shape[1:]) != (HV, V, K):
+        raise RuntimeError(f"[isoexec-amd] ssm_state {tuple(ssm_state.shape)} != [S,{HV},{V},{K}]")
+    io = v.dtype
+    if q.dtype is not io or k.dtype is not io:
+        raise RuntimeError("[isoexec-amd] q/k/v must share a dtype")
+    dev = q.device
+    if cu_seqlens is None:
+        cu = torch.arange(0, (B + 1) * T, T, dtype=torch.int32, device=dev)
+        n_seq = B
+    else:
+        if B != 1:
+            raise RuntimeError("[isoexec-amd] a packed batch (cu_seqlens) needs B == 1")
+        cu = cu_seqlens.to(torch.int32).contiguous()
+        n_seq = cu.numel() - 1
+    qf, kf, vf = _flatten_tokens(q, 2), _flatten_tokens(k, 2), _flatten_tokens(v, 2)
+    gf = _flatten_tokens(g, 1).to(torch.float32).contiguous()
+    bf = _flatten_tokens(beta, 1).to(io).contiguous()
+    idx = state_indices.to(torch.int32)
+    if idx.ndim == 1:
+        idx = idx.contiguous()
+        idx_stride = 1
+    else:
+        if idx.stride(1) != 1:
+            idx = idx.contiguous()
+        idx_stride = idx.stride(0)
+    if idx.shape[0] != n_seq:
+        raise RuntimeError(f"[isoexec-amd] state_indices has {idx.shape[0]} rows for {n_seq} sequences")
+    o = torch.empty(qf.shape[0], HV, V, dtype=io, device=dev)
+    if time_tile == 0 and cu_seqlens is None and T == 1:
+        time_tile = 1
+    rc = _lib.check(
+        _lib.lib().ix_gdn_scan(
+            qf.data_ptr(), kf.data_ptr(), vf.data_ptr(), gf.data_ptr(), bf.data_ptr(), o.data_ptr(),
+            _lib.dtype_code(io), _token_pitch(qf), _token_pitch(kf), _token_pitch(vf), ssm_state.data_ptr(),
+            cu.data_ptr(), idx.data_ptr(), idx_stride, n_seq, H, HV, K, V, float(K) ** -0.5, time_tile,
+            _lib.current_stream(dev)), "ix_gdn_scan")
+    if rc != _lib.IX_OK:
+        raise RuntimeError(f"[isoexec-amd] ix_gdn_scan declined K={K} V={V} dtype={io}")
+    return o.view(B, T, HV, V) if cu_seqlens is None else o.unsqueeze(0)
+
+
+def gdn_l2norm(x: torch.Tensor) -> torch.Tensor:
+    """Row-local L2 normalisation ``x * rsqrt(sum x^2 + 1e-6)`` over the last dim; ``[..., H, K]``."""
+    _lib.require_device(x)
+    if x.ndim < 2:
+        raise RuntimeError("[isoexec-amd] gdn_l2norm expects [..., H, K]")
+    xf = x if x.ndim == 3 else x.reshape(-1, x.shape[-2], x.shape[-1])
+    tokens, H, K = xf.shape
+    y = torch.empty(tokens, H, K, dtype=x.dtype, device=x.device)
+    rc = _lib.check(
+        _lib.lib().ix_gdn_l2norm(xf.data_ptr(), _token_pitch(xf), y.data_ptr(), _lib.dtype_code(x.dtype), tokens, H,
+                                 K, L2NORM_EPS, _lib.current_stream(x.device)), "ix_gdn_l2norm")
+    if rc != _lib.IX_OK:
+        raise RuntimeError(f"[isoexec-amd] ix_gdn_l2norm declined K={K}")
+    return y.view(x.shape)
+
+
+def gdn_gate_and_beta(a: torch.Tensor, b: torch.Tensor, A_log: torch.Tensor, dt_bias: torch.Tensor):
+    """``g = -exp(A_log) * softplus(a + dt_bias)`` in fp32; ``beta = sigmoid(b)``. Elementwise."""
+    _lib.require_device(a, b, A_log, dt_bias)
+    HV = a.shape[-1]
+    ac, bc = a.contiguous(), b.contiguous()
+    g = torch.empty(a.shape, dtype=torch.float32, device=a.device)
+    beta = torch.empty_like(bc)
+    _lib.check(
+        _lib.lib().ix_gdn_gate(ac.data_ptr(), bc.data_ptr(), A_log.float().contiguous().data_ptr(),
+                               dt_bias.float().contiguous().data_ptr(), g.data_ptr(), beta.data_ptr(),
+                               _lib.dtype_code(a.dtype), ac.numel() // HV, HV, _lib.current_stream(a.device)),
+        "ix_gdn_gate")
+    return g, beta
+
+
+def conv_packed(x, weight, bias, *, cu_seqlens, conv_state=None, rows_in=None, rows_out=None, activation="silu"):
+    """Packed varlen conv: ``x [T, D]`` -> ``y [T, D]``; optional pool rows for history in/out."""
+    _lib.require_device(x, weight, bias, cu_seqlens, conv_state, rows_in, rows_out)
+    if activation not in (None, "silu", "swish"):
+        raise ValueError(f"unsupported activation {activation!r}")
+    if x.dtype is not torch.bfloat16:
+        raise RuntimeError("[isoexec-amd] conv serves bf16 only")
+    T, D = x.shape
+    W = weight.shape[-1]
+    if weight.shape[0] != D:
+        raise ValueError(f"weight {tuple(weight.shape)} incompatible with x dim {D}")
+    xc, wc = x.contiguous(), weight.contiguous()
+    y = torch.empty_like(xc)
+    n_seq = cu_seqlens.numel() - 1
+    rc = _lib.check(
+        _lib.lib().ix_gdn_conv(xc.data_ptr(), wc.data_ptr(), _lib.ptr(None if bias is None else bias.contiguous()),
+                               y.data_ptr(), _lib.ptr(conv_state), cu_seqlens.data_ptr(), _lib.ptr(rows_in),
+                               _lib.ptr(rows_out), n_seq, T, D, W, int(activation is not None),
+                               _lib.current_stream(x.device)), "ix_gdn_conv")
+    if rc != _lib.IX_OK:
+        raise RuntimeError(f"[isoexec-amd] ix_gdn_conv declined W={W}")
+    return y
+
+
+def gdn_causal_conv(x, weight, bias=None, *, initial_state=None, activation="silu", return_final_state=False):
+    """Width-W causal depthwise conv over one sequence ``x [T, D]`` (gdn_ops.py:74-129)."""
+    if x.ndim != 2:
+        raise ValueError(f"gdn_causal_conv expects x=[T, D], got {tuple(x.shape)}")
+    T, D = x.shape
+    W = weight.shape[-1]
+    if initial_state is not None and tuple(initial_state.shape) != (D, W - 1):
+        raise ValueError(f"initial_state must be [D, W-1]={(D, W - 1)}, got {tuple(initial_state.shape)}")
+    dev = x.device
+    pool = torch.zeros(2, D, W - 1, dtype=x.dtype, device=dev)
+    if initial_state is not None:
+        pool[1] = initial_state.to(x.dtype)
+    one = torch.ones(1, dtype=torch.int32, device=dev)
+    cu = torch.tensor([0, T], dtype=torch.int32, device=dev)
+    y = conv_packed(x, weight, bias, cu_seqlens=cu, conv_state=pool,
+                    rows_in=one if initial_state is not None else None,
+                    rows_out=one if return_final_state else None, activation=activation)
+    if not return_final_state:
+        return y
+    return y, pool[1].clone()
+
+
+def gdn_causal_conv_batched(x, weight, bias=None, *, initial_state=None, activation="silu"):
+    """Batched conv ``x [N, T, D]``, ``initial_state [N, D, W-1]`` -> ``y [N, T, D]`` (gdn_ops.py:132-170)."""
+    if x.ndim != 3:
+        raise ValueError(f"gdn_causal_conv_batched expects x=[N, T, D], got {tuple(x.shape)}")
+    N, T, D = x.shape
+    W = weight.shape[-1]
+    dev = x.device
+    cu = torch.arange(0, (N + 1) * T, T, dtype=torch.int32, device=dev)
+    pool = rows = None
+    if initial_state is not None:
+        if tuple(initial_state.shape) != (N, D, W - 1):
+            raise ValueError(f"initial_state must be [N, D, W-1]={(N, D, W - 1)}, got {tuple(initial_state.shape)}")
+        pool = torch.cat([torch.zeros(1, D, W - 1, dtype=x.dtype, device=dev), initial_state.to(x.dtype)], dim=0)
+        rows = torch.arange(1, N + 1, dtype=torch.int32, device=dev)
+    y = conv_packed(x.reshape(N * T, D), weight, bias, cu_seqlens=cu, conv_state=pool, rows_in=rows,
+                    activation=activation)
+    return y.view(N, T, D)
+
+
+def _recurrent_scratch_state(q, v, cu_seqlens):
+    """A throwaway pool + index map for a stateless forward (gdn_ops.py:444-464): row 0 unused,
+    sequence n at row n+1, only column 0 of the map set."""
+    if cu_seqlens is not None:
+        N = cu_seqlens.numel() - 1
+        Tmax = q.shape[1]
+    else:
+        N, Tmax = q.shape[0], q.shape[1]
+    HV, V, K = v.shape[-2], v.shape[-1], q.shape[-1]
+    ssm_state = torch.zeros(N + 1, HV, V, K, dtype=torch.float32, device=q.device)
+    idx = torch.zeros(N, max(Tmax, 1), dtype=torch.int32, device=q.device)
+    idx[:, 0] = torch.arange(1, N + 1, dtype=torch.int32, device=q.device)
+    return ssm_state, idx
+
+
+def gdn_recurrent(q, k, v, g, beta, *, initial_state=None, output_final_state=False, cu_seqlens=None):
+    """Stateless (training / prefill-from-zero) entry: ``(o, None)`` (gdn_ops.py:997-1027)."""
+    if initial_state is not None or output_final_state:
+        raise NotImplementedError(
+            "isoexec GDN: gdn_recurrent is the stateless (training/prefill-from-zero) entry point. "
+            "The engine carries state through gdn_recurrent_kernel + a real state pool.")
+    with torch.no_grad():
+        ssm_state, idx = _recurrent_scratch_state(q, v, cu_seqlens)
+        o = gdn_recurrent_kernel(q, k, v, g, beta, ssm_state=ssm_state, state_indices=idx, cu_seqlens=cu_seqlens)
+    return o, None
+
+
+def gdn_core(q, k, v, g, beta, *, initial_state=None, output_final_state=False, cu_seqlens=None):
+    """The trainer's door (gdn_ops.py:1118-1194). One kernel mode exists here: recurrent."""
+    return gdn_recurrent(q, k, v, g, beta, initial_state=initial_state, output_final_state=output_final_state,
+                         cu_seqlens=cu_seqlens)
+
+
+def gdn_native_core_kernel(q, k, v, a, b, A_log, dt_bias, *, ssm_state, state_indices, cu_seqlens):
+    """Raw ``q, k [B, T, H, K]`` (GQA-compressed or expanded), raw gating inputs ``a, b [T, HV]``:
+    l2norm, GQA map and fp32 gating folded in front of the scan (gdn_ops.py:513-558). The
+    composition is the same three kernels in every call shape, so one varlen call equals T decode
+    calls bitwise."""
+    qn, kn = gdn_l2norm(q), gdn_l2norm(k)
+    HV = v.shape[-2]
+    g, beta = gdn_gate_and_beta(a.reshape(-1, HV), b.reshape(-1, HV), A_log, dt_bias)
+    lead = v.shape[:2]
+    return gdn_recurrent_kernel(qn, kn, v, g.view(*lead, HV), beta.view(*lead, HV), ssm_state=ssm_state,
+                                state_indices=state_indices, cu_seqlens=cu_seqlens)
+
+
+def gdn_native_core(q, k, v, a, b, A_log, dt_bias, *, cu_seqlens=None):
+    """Stateless entry for the native composition (gdn_ops.py:702-716)."""
+    with torch.no_grad():
+        ssm_state, idx = _recurrent_scratch_state(q, v, cu_seqlens)
+        return gdn_native_core_kernel(q, k, v, a, b, A_log, dt_bias, ssm_state=ssm_state, state_indices=idx,
+                                      cu_seqlens=cu_seqlens)

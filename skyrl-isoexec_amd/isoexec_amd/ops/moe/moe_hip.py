@@ -1,0 +1,136 @@
+"""MoE FFN on the HIP kernels: router, permutation, grouped experts, fixed-order combine.
+
+Function names follow the reference: ``fused_router_dense`` / ``fused_permute_index``
+(``ops/moe/moe_router_o2_kernel.py:272-351``), the batched expert forward
+(``ops/moe/moe_batched_experts.py:301-531``), the deterministic unpermute
+(``ops/moe/moe_batch_invariant.py:276-385``). ``moe_ffn_forward`` chains them the way
+``MoELayer.forward`` does on both runtimes.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ... import _lib
+from ..mm.mm_hip import linear_f32_nt
+
+
+def router_topk(logits: torch.Tensor, k: int, *, pre_softmax: bool = False, scaling_factor: float | None = None,
+                dense: bool = False):
+    """Top-k routing. Returns ``(topk_idx [T,k] int32, topk_prob [T,k] fp32, dense_probs, dense_map)``."""
+    _lib.require_device(logits)
+    if logits.dtype is not torch.float32 or logits.ndim != 2:
+        raise RuntimeError("[isoexec-amd] router logits must be fp32 [T, E]")
+    lg = logits if logits.stride(1) == 1 else logits.contiguous()
+    T, E = lg.shape
+    dev = lg.device
+    idx = torch.empty(T, k, dtype=torch.int32, device=dev)
+    prob = torch.empty(T, k, dtype=torch.float32, device=dev)
+    dprob = torch.empty(T, E, dtype=torch.float32, device=dev) if dense else None
+    dmap = torch.empty(T, E, dtype=torch.uint8, device=dev) if dense else None
+    rc = _lib.check(
+        _lib.lib().ix_moe_router_topk(lg.data_ptr(), lg.stride(0), T, E, k, int(pre_softmax),
+                                      float(scaling_factor or 0.0), idx.data_ptr(), prob.data_ptr(),
+                                      _lib.ptr(dprob), _lib.ptr(dmap), _lib.current_stream(dev)),
+        "ix_moe_router_topk")
+    if rc != _lib.IX_OK:
+        raise RuntimeError(f"[isoexec-amd] router declined E={E} k={k} (k must be a power of two <= 16, E <= 512)")
+    return idx, prob, dprob, (dmap.view(torch.bool) if dmap is not None else None)
+
+
+def fused_router_dense(logits: torch.Tensor, k: int, *, scaling_factor: float | None = None):
+    """``(routing_probs [T,E] fp32, routing_map [T,E] bool)`` (moe_router_o2_kernel.py:272-311)."""
+    _, _, dprob, dmap = router_topk(logits, k, scaling_factor=scaling_factor, dense=True)
+    return dprob, dmap
+
+
+class Permutation:
+    """Device-side routing plan: everything the grouped GEMMs and the combine need."""
+
+    __slots__ = ("T", "E", "k", "BM", "counts", "offsets", "sorted_token", "permuted_prob", "combine_rows",
+                 "tile_meta", "max_tiles")
+
+
+def permute(topk_idx: torch.Tensor, topk_prob: torch.Tensor, E: int, *, BM: int | None = None) -> Permutation:
+    """Expert-major, token-ascending permutation + block map (integer only, no host sync)."""
+    _lib.require_device(topk_idx, topk_prob)
+    T, k = topk_idx.shape
+    dev = topk_idx.device
+    L = _lib.lib()
+    p = Permutation()
+    p.T, p.E, p.k = T, E, k
+    p.BM = int(BM or L.ix_moe_pick_bm(T, k, E))
+    p.max_tiles = int(L.ix_moe_max_tiles(T, k, E, p.BM))
+    i32 = dict(dtype=torch.int32, device=dev)
+    p.counts = torch.empty(E, **i32)
+    p.offsets = torch.empty(E + 1, **i32)
+    p.sorted_token = torch.empty(T * k, **i32)
+    p.permuted_prob = torch.empty(T * k, dtype=torch.float32, device=dev)
+    p.combine_rows = torch.empty(T, k, **i32)
+    p.tile_meta = torch.empty(1 + 3 * p.max_tiles, **i32)
+    scratch = torch.empty(max(1, int(L.ix_moe_permute_scratch_ints(T, E))), **i32)
+    _lib.check(
+        L.ix_moe_permute(topk_idx.contiguous().data_ptr(), topk_prob.contiguous().data_ptr(), T, E, k, p.BM,
+                         p.counts.data_ptr(), p.offsets.data_ptr(), p.sorted_token.data_ptr(),
+                         p.permuted_prob.data_ptr(), p.combine_rows.data_ptr(), p.tile_meta.data_ptr(), p.max_tiles,
+                         scratch.data_ptr(), _lib.current_stream(dev)), "ix_moe_permute")
+    return p
+
+
+def fused_permute_index(routing_map: torch.Tensor, routing_probs: torch.Tensor, topk: int):
+    """``(sorted_indices [T*k] int64, permuted_probs [T*k], tokens_per_expert [E] int64)`` from the
+    dense routing tensors (moe_router_o2_kernel.py:313-351)."""
+    T, E = routing_map.shape
+    idx = routing_map.to(torch.int32).argsort(dim=1, descending=True, stable=True)[:, :topk].to(torch.int32)
+    prob = torch.gather(routing_probs, 1, idx.long())
+    p = permute(idx.contiguous(), prob.contiguous(), E)
+    return p.sorted_token.long(), p.permuted_prob, p.counts.long()
+
+
+def experts_forward(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, p: Permutation):
+    """Grouped fc1 + SwiGLU + prob epilogue + fc2 over the permuted rows. ``x [T, H]`` bf16,
+    ``w1 [E, 2F, H]``, ``w2 [E, H, F]``. Returns ``expert_out [T*k, H]`` in permuted order."""
+    _lib.require_device(x, w1, w2)
+    if x.dtype is not torch.bfloat16 or w1.dtype is not torch.bfloat16 or w2.dtype is not torch.bfloat16:
+        raise RuntimeError("[isoexec-amd] experts serve bf16 only")
+    T, H = x.shape
+    E, F2, _ = w1.shape
+    F = F2 // 2
+    rows = T * p.k
+    dev = x.device
+    inter = torch.empty(rows, F, dtype=torch.bfloat16, device=dev)
+    out = torch.empty(rows, H, dtype=torch.bfloat16, device=dev)
+    xc = x if x.stride(1) == 1 else x.contiguous()
+    rc = _lib.check(
+        _lib.lib().ix_moe_experts(xc.data_ptr(), xc.stride(0), p.sorted_token.data_ptr(),
+                                  p.permuted_prob.data_ptr(), w1.contiguous().data_ptr(),
+                                  w2.contiguous().data_ptr(), p.tile_meta.data_ptr(), p.max_tiles, p.BM,
+                                  inter.data_ptr(), out.data_ptr(), rows, H, F, _lib.current_stream(dev)),
+        "ix_moe_experts")
+    if rc != _lib.IX_OK:
+        raise RuntimeError(f"[isoexec-amd] ix_moe_experts declined H={H} F={F}")
+    return out
+
+
+def combine(expert_out: torch.Tensor, p: Permutation, *, fp32_acc: bool = False) -> torch.Tensor:
+    """Per token, the sum of its k rows in ascending expert order (moe_batch_invariant.py:276-320)."""
+    H = expert_out.shape[1]
+    out = torch.empty(p.T, H, dtype=torch.bfloat16, device=expert_out.device)
+    _lib.check(
+        _lib.lib().ix_moe_combine(expert_out.data_ptr(), p.combine_rows.data_ptr(), out.data_ptr(), p.T, H, p.k,
+                                  int(fp32_acc), _lib.current_stream(expert_out.device)), "ix_moe_combine")
+    return out
+
+
+def moe_ffn_forward(x: torch.Tensor, router_weight: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, k: int, *,
+                    pre_softmax: bool = False, logit_bias: torch.Tensor | None = None,
+                    scaling_factor: float | None = None, fp32_combine: bool = False, BM: int | None = None):
+    """Router GEMM (fp32) -> top-k -> permutation -> grouped experts -> combine. ``x [T, H]`` bf16."""
+    logits = linear_f32_nt(x, router_weight.float())
+    if logits is None:
+        raise RuntimeError("[isoexec-amd] router GEMM declined")
+    if logit_bias is not None:
+        logits = logits + logit_bias  # elementwise, per token
+    idx, prob, _, _ = router_topk(logits, k, pre_softmax=pre_softmax, scaling_factor=scaling_factor)
+    p = permute(idx, prob, router_weight.shape[0], BM=BM)
+    return combine(experts_forward(x, w1, w2, p), p, fp32_acc=fp32_combine)

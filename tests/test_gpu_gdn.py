@@ -1,0 +1,255 @@
+"""GPU parity: GatedDeltaNet scan, preparation and conv (configs 0 and 2, reduced where stated)."""
+
+import numpy as np
+import pytest
+import torch
+
+from _util import DevicePrims, bf16_to_np, cpu_gen, np_bits, np_to_bf16, same_bits
+from oracle import gdn as o_gdn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def dprims():
+    return DevicePrims(DEV)
+
+
+def make_inputs(B, T, H, HV, K, V, seed, dtype=torch.float32):
+    """Config-0 style inputs: q,k randn then L2-normalised per head, v randn, beta = sigmoid(randn),
+    g = -softplus(randn)."""
+    g = cpu_gen(seed)
+    q = torch.randn(B, T, H, K, generator=g)
+    k = torch.randn(B, T, H, K, generator=g)
+    q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6)
+    k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+    v = torch.randn(B, T, HV, V, generator=g)
+    beta = torch.sigmoid(torch.randn(B, T, HV, generator=g))
+    gate = -torch.nn.functional.softplus(torch.randn(B, T, HV, generator=g))
+    return q.to(dtype), k.to(dtype), v.to(dtype), gate.float(), beta.to(dtype)
+
+
+def oracle_scan(q, k, v, g, beta, prims, io_bf16, state=None):
+    """Per-sequence oracle over a [B, T, ...] batch. Returns (o, final_states)."""
+    B = q.shape[0]
+    HV, V, K = v.shape[2], v.shape[3], q.shape[3]
+    outs, finals = [], []
+    for b in range(B):
+        st = np.zeros((HV, V, K), np.float32) if state is None else state[b].copy()
+        f = lambda t: t[b].float().numpy()
+        outs.append(o_gdn.scan(f(q), f(k), f(v), f(g), f(beta), st, io_bf16=io_bf16, prims=prims))
+        finals.append(st)
+    return np.stack(outs), np.stack(finals)
+
+
+def run_scan(q, k, v, g, beta, pool, idx, cu=None, time_tile=0):
+    from isoexec_amd.ops.gdn.gdn_ops import gdn_recurrent_kernel
+
+    return gdn_recurrent_kernel(q, k, v, g, beta, ssm_state=pool, state_indices=idx, cu_seqlens=cu,
+                                time_tile=time_tile)
+
+
+def test_config0_scan_bit_exact_and_chunk_invariant(dprims):
+    """Config 0: B=2, T=256, 4 heads, d_k=d_v=64, fp32. Oracle bit-exact; bitwise equal across
+    time tiles {16, 32, 64} and prefill/decode splits, state included."""
+    B, T, H, K, V = 2, 256, 4, 64, 64
+    q, k, v, g, beta = make_inputs(B, T, H, H, K, V, seed=0)
+    want_o, want_s = oracle_scan(q, k, v, g, beta, dprims, io_bf16=False)
+    d = lambda t: t.to(DEV)
+    idx = torch.zeros(B, T, dtype=torch.int32)
+    idx[:, 0] = torch.arange(1, B + 1)
+    idx[:, T - 1] = torch.arange(1, B + 1)
+    results = []
+    for tt in (16, 32, 64):
+        pool = torch.zeros(B + 1, H, V, K, device=DEV)
+        o = run_scan(d(q), d(k), d(v), d(g), d(beta), pool, d(idx), time_tile=tt)
+        results.append((o, pool))
+    o0, p0 = results[0]
+    assert np.array_equal(np_bits(o0.cpu().numpy()), np_bits(want_o))
+    assert np.array_equal(np_bits(p0[1:].cpu().numpy()), np_bits(want_s))
+    for o, p in results[1:]:
+        assert same_bits(o, o0) and same_bits(p, p0)
+    # tolerance against the textbook float64 recurrence
+    o64, _ = o_gdn.scan_fp64(q[0].numpy(), k[0].numpy(), v[0].numpy(), g[0].numpy(), beta[0].numpy())
+    assert np.abs(o0[0].cpu().numpy() - o64).max() <= 2e-5
+    # prefill to t, then token-by-token decode: identical bits and identical final state
+    for split in (0, 1, 63, 64, 65, 127, 255):
+        pool = torch.zeros(B + 1, H, V, K, device=DEV)
+        rows = torch.arange(1, B + 1, dtype=torch.int32, device=DEV)
+        outs = []
+        if split > 0:
+            ip = torch.zeros(B, split, dtype=torch.int32)
+            ip[:, 0] = torch.arange(1, B + 1)
+            ip[:, split - 1] = torch.arange(1, B + 1)
+            outs.append(run_scan(d(q[:, :split]), d(k[:, :split]), d(v[:, :split]), d(g[:, :split]),
+                                 d(beta[:, :split]), pool, d(ip)))
+        stop = min(T, split + 40)  # 40 decode steps are enough to expose any drift
+        for t in range(split, stop):
+            outs.append(run_scan(d(q[:, t:t + 1]), d(k[:, t:t + 1]), d(v[:, t:t + 1]), d(g[:, t:t + 1]),
+                                 d(beta[:, t:t + 1]), pool, rows))
+        got = torch.cat(outs, dim=1)
+        assert same_bits(got, o0[:, :stop]), split
+
+
+def test_scan_bf16_gqa_varlen_cross_sequence_and_null_lanes(dprims):
+    """Config-2 head geometry (K=V=128, GQA 2 v-heads per k-head) at reduced head count, bf16 io,
+    packed varlen with the reference's lengths [150, 37, 64, 201] (gdn_batch_invariant.py:141-215)."""
+    H, HV, K, V = 2, 4, 128, 128
+    lens = [150, 37, 64, 201]
+    total = sum(lens)
+    q, k, v, g, beta = make_inputs(1, total, H, HV, K, V, seed=2, dtype=torch.bfloat16)
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    N = len(lens)
+    idx = torch.zeros(N, max(lens), dtype=torch.int32)
+    for n, L in enumerate(lens):
+        idx[n, 0] = n + 1
+        idx[n, L - 1] = n + 1
+    d = lambda t: t.to(DEV)
+    pool = torch.zeros(N + 1, HV, V, K, device=DEV)
+    o = run_scan(d(q), d(k), d(v), d(g), d(beta), pool, d(idx), cu=d(cu))[0]
+    # oracle per sequence
+    for n, L in enumerate(lens):
+        s, e = int(cu[n]), int(cu[n + 1])
+        st = np.zeros((HV, V, K), np.float32)
+        f = lambda t: t[0, s:e].float().numpy()
+        want = o_gdn.scan(f(q), f(k), f(v), f(g), f(beta), st, io_bf16=True, prims=dprims)
+        assert same_bits(o[s:e].cpu(), np_to_bf16(want)), n
+        assert np.array_equal(np_bits(pool[n + 1].cpu().numpy()), np_bits(st)), n
+    # each sequence alone == inside the packed batch (cross-sequence invariance)
+    for n, L in enumerate(lens):
+        s, e = int(cu[n]), int(cu[n + 1])
+        p1 = torch.zeros(2, HV, V, K, device=DEV)
+        i1 = torch.zeros(1, L, dtype=torch.int32)
+        i1[0, 0] = 1
+        alone = run_scan(d(q[:, s:e]), d(k[:, s:e]), d(v[:, s:e]), d(g[:, s:e]), d(beta[:, s:e]), p1, d(i1))[0]
+        assert same_bits(alone, o[s:e])
+    # null lane: sequence 1 mapped to row 0 is skipped: zero output, pool untouched
+    idx2 = idx.clone()
+    idx2[1] = 0
+    pool2 = torch.zeros(N + 1, HV, V, K, device=DEV)
+    o2 = run_scan(d(q), d(k), d(v), d(g), d(beta), pool2, d(idx2), cu=d(cu))[0]
+    s, e = int(cu[1]), int(cu[2])
+    assert float(o2[s:e].float().abs().max()) == 0.0 and float(pool2[2].abs().max()) == 0.0
+    assert same_bits(o2[:s], o[:s]) and same_bits(o2[e:], o[e:])
+    # mid-sequence store: a positive index at column t stores the state after token t
+    idx3 = torch.zeros(1, 64, dtype=torch.int32)
+    idx3[0, 0] = 1
+    idx3[0, 9] = 2
+    idx3[0, 63] = 1
+    s, e = int(cu[2]), int(cu[3])
+    pool3 = torch.zeros(3, HV, V, K, device=DEV)
+    run_scan(d(q[:, s:e]), d(k[:, s:e]), d(v[:, s:e]), d(g[:, s:e]), d(beta[:, s:e]), pool3, d(idx3))
+    st = np.zeros((HV, V, K), np.float32)
+    f = lambda t: t[0, s:e].float().numpy()
+    _, snap = o_gdn.scan(f(q), f(k), f(v), f(g), f(beta), st, io_bf16=True, prims=dprims, snapshots=True)
+    assert np.array_equal(np_bits(pool3[2].cpu().numpy()), np_bits(snap[9]))
+    assert np.array_equal(np_bits(pool3[1].cpu().numpy()), np_bits(snap[63]))
+
+
+def test_scan_closed_forms():
+    """beta = 0: pure decay S_T = exp(sum g) S_0 (o = S q). g = 0, beta = 1, orthonormal keys:
+    the state is an associative memory and o_t = v_t for q_t = k_t * sqrt(K)."""
+    H, K, V, T = 1, 64, 64, 48
+    g = cpu_gen(3)
+    eye = torch.eye(K)[:T]  # orthonormal keys
+    k = eye.view(1, T, 1, K)
+    q = k * (K ** 0.5)
+    v = torch.randn(1, T, H, V, generator=g)
+    zeros = torch.zeros(1, T, H)
+    ones = torch.ones(1, T, H)
+    d = lambda t: t.to(DEV)
+    idx = torch.zeros(1, T, dtype=torch.int32)
+    idx[0, 0] = 1
+    pool = torch.zeros(2, H, V, K, device=DEV)
+    o = run_scan(d(q), d(k), d(v), d(zeros), d(ones), pool, d(idx))
+    assert torch.equal(o.cpu(), v)  # exact: products with 0/1 and a scale of 8 * 0.125
+    s0 = torch.randn(H, V, K, generator=g)
+    gg = -torch.rand(1, T, H, generator=g)
+    pool = torch.zeros(2, H, V, K, device=DEV)
+    pool[1] = s0.to(DEV)
+    idx[0, T - 1] = 1
+    run_scan(d(q), d(k), d(v), d(gg), d(zeros), pool, d(idx))
+    want = s0.double() * torch.exp(gg.double().sum())
+    assert (pool[1].cpu().double() - want).abs().max().item() <= 1e-5
+
+
+def test_l2norm_and_gate_bit_exact(dprims):
+    from isoexec_amd.ops.gdn.gdn_ops import gdn_gate_and_beta, gdn_l2norm
+
+    g = cpu_gen(4)
+    for dtype in (torch.bfloat16, torch.float32):
+        proj = (2 * torch.randn(50, 2 * 2 * 128 + 4 * 128, generator=g)).to(dtype)
+        x = proj[:, 256:512].view(50, 2, 128)  # a strided slice of the conv output
+        want = o_gdn.l2norm(x.float().numpy(), io_bf16=dtype is torch.bfloat16)
+        pd = proj.to(DEV)
+        got = gdn_l2norm(pd[:, 256:512].view(50, 2, 128))
+        assert np.array_equal(np_bits(got.float().cpu().numpy()), np_bits(want))
+        a = (2 * torch.randn(50, 4, generator=g)).to(dtype)
+        b = (2 * torch.randn(50, 4, generator=g)).to(dtype)
+        a[0, 0] = 30.0  # softplus threshold branch
+        A_log = 0.2 * torch.randn(4, generator=g)
+        dt_bias = 0.2 * torch.randn(4, generator=g)
+        wg, wb = o_gdn.gate_and_beta(a.float().numpy(), b.float().numpy(), A_log.numpy(), dt_bias.numpy(),
+                                     io_bf16=dtype is torch.bfloat16, prims=dprims)
+        gg, bb = gdn_gate_and_beta(a.to(DEV), b.to(DEV), A_log.to(DEV), dt_bias.to(DEV))
+        # softplus is evaluated as one device primitive; exp(A_log) and the product are IEEE
+        assert np.array_equal(np_bits(gg.cpu().numpy()), np_bits(wg))
+        assert np.array_equal(np_bits(bb.float().cpu().numpy()), np_bits(wb))
+
+
+def test_conv_bit_exact_prefill_decode_and_state(dprims):
+    from isoexec_amd.ops.gdn.gdn_ops import gdn_causal_conv, gdn_causal_conv_batched
+
+    g = cpu_gen(5)
+    T, D, W = 70, 384, 4
+    x = torch.randn(T, D, generator=g).to(torch.bfloat16)
+    w = (0.5 * torch.randn(D, W, generator=g)).to(torch.bfloat16)
+    b = (0.1 * torch.randn(D, generator=g)).to(torch.bfloat16)
+    for bias in (None, b):
+        bn = None if bias is None else bf16_to_np(bias)
+        want_y, want_s = o_gdn.causal_conv(bf16_to_np(x), bf16_to_np(w), bn, prims=dprims)
+        y, s = gdn_causal_conv(x.to(DEV), w.to(DEV), None if bias is None else bias.to(DEV),
+                               return_final_state=True)
+        assert same_bits(y.cpu(), np_to_bf16(want_y)) and same_bits(s.cpu(), np_to_bf16(want_s))
+    # split anywhere == unsplit, chained through the returned state (incl. a 2-token first chunk)
+    for cut in (1, 2, 3, 33):
+        y1, s1 = gdn_causal_conv(x[:cut].to(DEV), w.to(DEV), b.to(DEV), return_final_state=True)
+        y2, s2 = gdn_causal_conv(x[cut:].to(DEV), w.to(DEV), b.to(DEV), initial_state=s1, return_final_state=True)
+        assert same_bits(torch.cat([y1, y2]), y) and same_bits(s2, s)
+    # token-by-token batched decode == prefill
+    state = torch.zeros(1, D, W - 1, dtype=torch.bfloat16, device=DEV)
+    outs = []
+    for t in range(12):
+        xt = x[t:t + 1].to(DEV)
+        outs.append(gdn_causal_conv_batched(xt.view(1, 1, D), w.to(DEV), b.to(DEV), initial_state=state)[0])
+        state = torch.cat([state[..., 1:], xt.view(1, D, 1)], dim=-1)
+    assert same_bits(torch.cat(outs), y[:12])
+
+
+def test_native_core_varlen_equals_decode_steps():
+    """The fused-front composition (raw q/k, raw a/b): one varlen call == T sequential decode calls,
+    state included (gdn_native_kernel_parity_test_gpu.py T1-T4)."""
+    from isoexec_amd.ops.gdn.gdn_ops import gdn_native_core_kernel
+
+    g = cpu_gen(6)
+    T, H, HV, K, V = 24, 2, 4, 128, 128
+    q = torch.randn(1, T, H, K, generator=g).to(torch.bfloat16).to(DEV)
+    k = torch.randn(1, T, H, K, generator=g).to(torch.bfloat16).to(DEV)
+    v = torch.randn(1, T, HV, V, generator=g).to(torch.bfloat16).to(DEV)
+    a = torch.randn(T, HV, generator=g).to(torch.bfloat16).to(DEV)
+    b = torch.randn(T, HV, generator=g).to(torch.bfloat16).to(DEV)
+    A_log = (0.2 * torch.randn(HV, generator=g)).to(DEV)
+    dt_bias = (0.2 * torch.randn(HV, generator=g)).to(DEV)
+    idx = torch.zeros(1, T, dtype=torch.int32, device=DEV)
+    idx[0, 0] = 1
+    idx[0, T - 1] = 1
+    pool = torch.zeros(2, HV, V, K, device=DEV)
+    cu = torch.tensor([0, T], dtype=torch.int32, device=DEV)
+    o = gdn_native_core_kernel(q, k, v, a, b, A_log, dt_bias, ssm_state=pool, state_indices=idx, cu_seqlens=cu)
+    pool2 = torch.zeros(2, HV, V, K, device=DEV)
+    one = torch.ones(1, dtype=torch.int32, device=DEV)
+    outs = [gdn_native_core_kernel(q[:, t:t + 1], k[:, t:t + 1], v[:, t:t + 1], a[t:t + 1], b[t:t + 1], A_log,
+                                   dt_bias, ssm_state=pool2, state_indices=one, cu_seqlens=None)
+            for t in range(T)]
+    assert same_bits(torch.cat(outs, dim=1), o) and same_bits(pool2, pool)

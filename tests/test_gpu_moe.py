@@ -1,0 +1,160 @@
+"""GPU parity: MoE router, permutation, grouped experts and combine (config 3, reduced where stated)."""
+
+import numpy as np
+import pytest
+import torch
+
+from _util import DevicePrims, bf16_to_np, cpu_gen, np_bits, np_to_bf16, same_bits
+from oracle import moe as o_moe
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def dprims():
+    return DevicePrims(DEV)
+
+
+def make_moe(T, H, E, F, seed):
+    g = cpu_gen(seed)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    wr = (0.02 * torch.randn(E, H, generator=g)).to(torch.bfloat16)
+    w1 = (0.02 * torch.randn(E, 2 * F, H, generator=g)).to(torch.bfloat16)
+    w2 = (0.02 * torch.randn(E, H, F, generator=g)).to(torch.bfloat16)
+    return x, wr, w1, w2
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("E,k", [(128, 8), (16, 4), (60, 2), (200, 1)])
+def test_router_bit_exact_ties_and_nan(mode, E, k, dprims):
+    from isoexec_amd.ops.moe.moe_hip import router_topk
+
+    g = cpu_gen(E + k)
+    logits = 2 * torch.randn(64, E, generator=g)
+    logits[1, :] = 0.5  # all tied: lowest indices win
+    logits[2, 3] = float("nan")  # NaN counts as -inf
+    logits[3, 5] = logits[3, 9] = 7.0  # a tied pair at the top
+    logits[4, :] = -1e4
+    logits[4, 7] = 80.0  # outlier: the other exp terms underflow
+    idx, prob, dprob, dmap = router_topk(logits.to(DEV), k, pre_softmax=bool(mode), dense=True)
+    widx, wprob = o_moe.router_topk(logits.numpy(), k, mode, prims=dprims)
+    assert np.array_equal(idx.cpu().numpy(), widx)
+    assert np.array_equal(np_bits(prob.cpu().numpy()), np_bits(wprob))
+    assert idx[1].tolist() == list(range(k))
+    if E > 3 and k < E:
+        assert 3 not in idx[2].tolist() or k >= E
+    wd, wm = o_moe.dense_from_topk(widx, wprob, E)
+    assert np.array_equal(np_bits(dprob.cpu().numpy()), np_bits(wd)) and np.array_equal(dmap.cpu().numpy(), wm)
+    # library check: torch.topk membership and softmax values (libm exp) within 1e-6
+    lt = torch.nan_to_num(logits, nan=float("-inf"))
+    if mode == 0:
+        tv, _ = torch.topk(lt, k, dim=1)
+        ref = torch.softmax(tv, dim=-1)
+    else:
+        tv, _ = torch.topk(torch.softmax(lt, dim=-1), k, dim=1)
+        ref = tv / tv.sum(-1, keepdim=True)
+    assert (prob.cpu() - ref).abs().max().item() <= 2e-6
+    # row invariance
+    i1, p1, _, _ = router_topk(logits[5:6].to(DEV), k, pre_softmax=bool(mode))
+    assert torch.equal(i1, idx[5:6]) and same_bits(p1, prob[5:6])
+
+
+@pytest.mark.parametrize("T,E,k", [(1, 128, 8), (33, 128, 8), (700, 16, 4), (513, 128, 8)])
+def test_permutation_exact(T, E, k):
+    from isoexec_amd.ops.moe.moe_hip import permute, router_topk
+
+    g = cpu_gen(T)
+    logits = torch.randn(T, E, generator=g)
+    logits[:, :4] += 3.0  # skewed load
+    idx, prob, _, _ = router_topk(logits.to(DEV), k)
+    for BM in (32, 128, 256):
+        p = permute(idx, prob, E, BM=BM)
+        counts, st, pp, cr = o_moe.permute(idx.cpu().numpy(), prob.cpu().numpy(), E)
+        assert np.array_equal(p.counts.cpu().numpy(), counts)
+        assert np.array_equal(p.sorted_token.cpu().numpy(), st)
+        assert np.array_equal(np_bits(p.permuted_prob.cpu().numpy()), np_bits(pp))
+        assert np.array_equal(p.combine_rows.cpu().numpy(), cr)
+        assert np.array_equal(p.offsets.cpu().numpy(), np.concatenate([[0], np.cumsum(counts)]))
+        meta = p.tile_meta.cpu().numpy()
+        nt = int(meta[0])
+        te, r0, nr = (meta[1 + i * p.max_tiles: 1 + i * p.max_tiles + nt] for i in range(3))
+        assert nt == int(sum(-(-c // BM) for c in counts)) and nr.sum() == T * k
+        off = np.concatenate([[0], np.cumsum(counts)])
+        for e_, r_, n_ in zip(te, r0, nr):
+            assert off[e_] <= r_ and r_ + n_ <= off[e_ + 1] and 0 < n_ <= BM
+
+
+def test_moe_ffn_parity_and_batch_invariance(dprims):
+    """Reduced config 3 (hidden 256, 16 experts, top-4, inter 128): the full chain against the
+    oracle (device router logits fed to the oracle so the discrete choice is compared like for
+    like), then every token alone == co-batched == co-batched under skewed routing, for every BM."""
+    from isoexec_amd.ops.mm.mm_hip import linear_f32_nt
+    from isoexec_amd.ops.moe.moe_hip import combine, experts_forward, moe_ffn_forward, permute, router_topk
+
+    T, H, E, F, k = 300, 256, 16, 128, 4
+    x, wr, w1, w2 = make_moe(T, H, E, F, seed=1)
+    xd, wrd, w1d, w2d = (t.to(DEV) for t in (x, wr, w1, w2))
+    for mode in (0, 1):
+        logits = linear_f32_nt(xd, wrd.float())
+        idx, prob, _, _ = router_topk(logits, k, pre_softmax=bool(mode))
+        p = permute(idx, prob, E)
+        eo = experts_forward(xd, w1d, w2d, p)
+        out = combine(eo, p)
+        # oracle with float64 matmuls: each bf16 round may differ by an ulp where the fp32 sum
+        # lands near a rounding boundary, so compare with a tolerance in bf16 ulps of the scale
+        mm64 = lambda a, w: (a.astype(np.float64) @ w.astype(np.float64).T).astype(np.float32)
+        counts, st, pp, cr = o_moe.permute(idx.cpu().numpy(), prob.cpu().numpy(), E)
+        weo, _ = o_moe.expert_chain(bf16_to_np(x), bf16_to_np(w1), bf16_to_np(w2), st, pp, counts, prims=dprims,
+                                    matmul=mm64)
+        got = bf16_to_np(eo)
+        scale = np.abs(weo).max()
+        assert np.abs(got - weo).max() <= 2.0 ** -7 * scale, (np.abs(got - weo).max(), scale)
+        assert (got != weo).mean() < 0.05
+        # combine is exact given the expert rows
+        assert same_bits(out.cpu(), np_to_bf16(o_moe.combine(got, cr)))
+        assert same_bits(combine(eo, p, fp32_acc=True).cpu(), np_to_bf16(o_moe.combine(got, cr, fp32_acc=True)))
+        assert same_bits(moe_ffn_forward(xd, wrd, w1d, w2d, k, pre_softmax=bool(mode)), out)
+    # invariance: alone vs co-batched vs skewed co-batch, all BM
+    ref = moe_ffn_forward(xd, wrd, w1d, w2d, k, BM=256)
+    for BM in (32, 128):
+        assert same_bits(moe_ffn_forward(xd, wrd, w1d, w2d, k, BM=BM), ref)
+    for t in (0, 17, 299):
+        assert same_bits(moe_ffn_forward(xd[t:t + 1], wrd, w1d, w2d, k), ref[t:t + 1])
+    assert same_bits(moe_ffn_forward(xd[:33], wrd, w1d, w2d, k), ref[:33])
+    # skew the OTHER tokens' routing (+3.0 on 4 experts): token 5 keeps its own logits
+    bias = torch.zeros(T, E, device=DEV)
+    bias[:, :4] = 3.0
+    bias[5] = 0.0
+    skew = moe_ffn_forward(xd, wrd, w1d, w2d, k, logit_bias=bias)
+    assert same_bits(skew[5:6], ref[5:6])
+
+
+def test_config3_shapes_small_T():
+    """Config 3 dimensions (hidden 2048, 128 experts, top-8, inter 768, softmax-then-topk with
+    renormalisation, +3.0 skew on 4 experts) at T in {1, 33, 512}: alone == co-batched bits."""
+    from isoexec_amd.ops.moe.moe_hip import moe_ffn_forward
+
+    T, H, E, F, k = 512, 2048, 128, 768, 8
+    x, wr, w1, w2 = make_moe(T, H, E, F, seed=3)
+    xd, wrd, w1d, w2d = (t.to(DEV) for t in (x, wr, w1, w2))
+    ref = moe_ffn_forward(xd, wrd, w1d, w2d, k, pre_softmax=True)
+    assert bool(torch.isfinite(ref.float()).all())
+    assert same_bits(moe_ffn_forward(xd[:1], wrd, w1d, w2d, k, pre_softmax=True), ref[:1])
+    assert same_bits(moe_ffn_forward(xd[:33], wrd, w1d, w2d, k, pre_softmax=True), ref[:33])
+    bias = torch.zeros(T, E, device=DEV)
+    bias[1:, :4] = 3.0
+    skew = moe_ffn_forward(xd, wrd, w1d, w2d, k, pre_softmax=True, logit_bias=bias)
+    assert same_bits(skew[:1], ref[:1])
+    # dense fp64 reference for token 0 (top-8 of softmax, renormalised)
+    lg = (x[:1].double() @ wr.double().T)
+    pr = torch.softmax(lg, -1)
+    tv, ti = torch.topk(pr, k)
+    tv = tv / tv.sum()
+    acc = torch.zeros(H, dtype=torch.float64)
+    for pj, ej in zip(tv[0], ti[0]):
+        h = x[0].double() @ w1[ej].double().T
+        a = torch.nn.functional.silu(h[:F]) * h[F:] * pj
+        acc += a @ w2[ej].double().T
+    err = (ref[0].double().cpu() - acc).abs().max().item()
+    assert err <= 0.03 * acc.abs().max().item() + 1e-3, err
