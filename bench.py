@@ -1,0 +1,242 @@
+"""Benchmark of the batch-invariant token-logprob hot path on one MI355X.
+
+Default workload (``dense_head``, BASELINE.json configs[1]): M = 4096 hidden states of width 4096
+-> zero-centred RMSNorm -> bf16 LM-head GEMM against [151936, 4096] -> bf16 logits -> row-invariant
+log-softmax + target gather. One step = one pass over the 4096 tokens; inputs are resident in HBM
+before the timed region. Prints ONE JSON line.
+
+Other workloads (``--workload gdn_decode | gdn_prefill | moe``) time configs[2] and configs[3] with
+the same contract; they are extra lines for profiling, not the headline.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "skyrl-isoexec_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+PEAK_MFMA_BF16_TFLOPS = 2500.0  # MI355X dense bf16
+PEAK_HBM_GBS = 8000.0
+
+
+class KernelTimer:
+    """HIP-event timing of one kernel family on torch's current stream (the stream every entry
+    point of the library is launched on)."""
+
+    def __init__(self):
+        self.pairs = []
+
+    def __call__(self, fn):
+        import torch
+
+        s = torch.cuda.Event(enable_timing=True)
+        e = torch.cuda.Event(enable_timing=True)
+        s.record()
+        out = fn()
+        e.record()
+        self.pairs.append((s, e))
+        return out
+
+    def mean_ms(self):
+        return sum(s.elapsed_time(e) for s, e in self.pairs) / max(1, len(self.pairs))
+
+
+def dense_head(args):
+    import torch
+
+    from isoexec_amd.ops.logprobs.rowinv import sampled_forward
+    from isoexec_amd.ops.mm.mm_hip import linear_nt
+    from isoexec_amd.ops.norms.fused_outnorm import fused_rms_norm_gamma
+
+    dev = "cuda:0"
+    M, K, V = args.tokens, 4096, 151936
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1)
+    h = torch.randn(M, K, device=dev, generator=gen).to(torch.bfloat16)
+    w_norm = (0.02 * torch.randn(K, device=dev, generator=gen)).to(torch.bfloat16)  # gamma = 1 + w
+    w_lm = torch.empty(V, K, device=dev, dtype=torch.bfloat16)
+    for s in range(0, V, 16384):  # chunked so the fp32 temporary stays small
+        e = min(V, s + 16384)
+        w_lm[s:e] = (0.02 * torch.randn(e - s, K, device=dev, generator=gen)).to(torch.bfloat16)
+    target = torch.randint(0, V, (M,), device=dev, generator=gen)
+
+    t_gemm, t_lp, t_norm = KernelTimer(), KernelTimer(), KernelTimer()
+
+    def step(timed):
+        wrap = (lambda t, f: t(f)) if timed else (lambda t, f: f())
+        x = wrap(t_norm, lambda: fused_rms_norm_gamma(h, w_norm, 1e-6))
+        logits = wrap(t_gemm, lambda: linear_nt(x, w_lm, tile=args.tile))
+        lp, _ = wrap(t_lp, lambda: sampled_forward(logits, target, 8))
+        return lp
+
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        lp = step(True)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert bool(torch.isfinite(lp).all())
+
+    gemm_ms = t_gemm.mean_ms()
+    flops = 2.0 * M * V * K
+    achieved = flops / (gemm_ms * 1e-3) / 1e12
+    lp_ms = t_lp.mean_ms()
+    out = {
+        "metric": "trainer-fwd & decode tokens/s at bitwise parity; % of HBM/MFMA roofline",
+        "value": M * args.steps / dt,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": dt / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "dense_head: RMSNorm(4096) + LM head [151936,4096] + log-softmax/gather",
+                   "tokens_per_step": M, "hidden": K, "vocab": V, "gemm_tile": args.tile},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_MFMA_BF16_TFLOPS, "traffic": None,
+                     "kernel": "k_gemm_bf16_nt", "kernel_ms": gemm_ms},
+        "kernels_ms": {"rmsnorm": t_norm.mean_ms(), "gemm": gemm_ms, "logprob": lp_ms},
+        "logprob_hbm": {"bound": "hbm", "achieved": M * V * 2 / (lp_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                        "unit": "GB/s", "frac": M * V * 2 / (lp_ms * 1e-3) / 1e9 / PEAK_HBM_GBS},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = dense_head_cpu(h, w_norm, w_lm, target, args.cpu_tokens)
+    return out
+
+
+def dense_head_cpu(h, w_norm, w_lm, target, m):
+    """The oracle (CPU restatement of the reference's eager path) on the first ``m`` tokens of the
+    same workload, timed on this box's host cores."""
+    import numpy as np
+    import torch
+
+    from oracle import logprobs as o_lp
+    from oracle import norms as o_norms
+    from oracle.prims import round_bf16
+
+    hn = h[:m].float().cpu().numpy()
+    wn = w_norm.float().cpu().numpy()
+    wl = w_lm.float().cpu()  # fp32 copy of the LM head (conversion not timed)
+    tn = target[:m].cpu().numpy()
+    threads = torch.get_num_threads()
+    t0 = time.perf_counter()
+    x = o_norms.rms_norm_gamma(hn, wn, 1e-6)
+    logits = round_bf16((torch.from_numpy(x) @ wl.T).numpy())
+    lp, _ = o_lp.rowinv_sampled(logits, tn, 8)
+    dt = time.perf_counter() - t0
+    assert np.isfinite(lp).all()
+    return {"value": m / dt, "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": f"first {m} tokens of the same dense_head workload ({dt:.1f} s of CPU work; "
+                      f"fp32 torch matmul + numpy oracle norm/logprob)"}
+
+
+def gdn_decode(args):
+    import torch
+
+    from isoexec_amd.ops.gdn.gdn_ops import gdn_recurrent_kernel
+
+    dev = "cuda:0"
+    B, H, HV, K, V = args.batch, 16, 32, 128, 128
+    q = torch.randn(B, 1, H, K, device=dev).to(torch.bfloat16)
+    k = torch.randn(B, 1, H, K, device=dev).to(torch.bfloat16)
+    q = q / q.float().norm(dim=-1, keepdim=True).to(torch.bfloat16)
+    k = k / k.float().norm(dim=-1, keepdim=True).to(torch.bfloat16)
+    v = torch.randn(B, 1, HV, V, device=dev).to(torch.bfloat16)
+    g = -torch.nn.functional.softplus(torch.randn(B, 1, HV, device=dev))
+    beta = torch.sigmoid(torch.randn(B, 1, HV, device=dev)).to(torch.bfloat16)
+    pool = torch.zeros(B + 1, HV, V, K, device=dev)
+    rows = torch.arange(1, B + 1, dtype=torch.int32, device=dev)
+    timer = KernelTimer()
+    fn = lambda: gdn_recurrent_kernel(q, k, v, g, beta, ssm_state=pool, state_indices=rows)
+    for _ in range(args.warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        timer(fn)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms = timer.mean_ms()
+    by = B * HV * V * K * 4 * 2
+    return {"metric": "gdn decode tokens/s", "value": B * args.steps / dt, "unit": "tokens/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": f"gdn_decode B={B} HV=32 K=V=128 (state R+W 4 MiB/seq/step)"},
+            "roofline": {"bound": "hbm", "achieved": by / (ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": by / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None, "kernel": "k_gdn_scan",
+                         "kernel_ms": ms}}
+
+
+def moe(args):
+    import torch
+
+    from isoexec_amd.ops.moe.moe_hip import moe_ffn_forward
+
+    dev = "cuda:0"
+    T, H, E, F, k = args.tokens, 2048, 128, 768, 8
+    x = torch.randn(T, H, device=dev).to(torch.bfloat16)
+    wr = (0.02 * torch.randn(E, H, device=dev)).to(torch.bfloat16)
+    w1 = (0.02 * torch.randn(E, 2 * F, H, device=dev)).to(torch.bfloat16)
+    w2 = (0.02 * torch.randn(E, H, F, device=dev)).to(torch.bfloat16)
+    fn = lambda: moe_ffn_forward(x, wr, w1, w2, k, pre_softmax=True)
+    timer = KernelTimer()
+    for _ in range(args.warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        timer(fn)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms = timer.mean_ms()
+    fl = T * 75.5e6
+    return {"metric": "moe ffn tokens/s", "value": T * args.steps / dt, "unit": "tokens/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": f"moe T={T} hidden 2048, 128 experts top-8, inter 768"},
+            "roofline": {"bound": "mfma", "achieved": fl / (ms * 1e-3) / 1e12, "peak": PEAK_MFMA_BF16_TFLOPS,
+                         "unit": "TFLOP/s", "frac": fl / (ms * 1e-3) / 1e12 / PEAK_MFMA_BF16_TFLOPS, "traffic": None,
+                         "kernel": "whole FFN (router + grouped GEMMs + combine)", "kernel_ms": ms}}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="dense_head", choices=["dense_head", "gdn_decode", "moe"])
+    ap.add_argument("--tokens", type=int, default=None)
+    ap.add_argument("--batch", type=int, default=256)
+    ap.add_argument("--tile", type=int, default=0)
+    ap.add_argument("--cpu-tokens", type=int, default=64)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (no collectives, no sharding); --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+    if args.tokens is None:
+        args.tokens = 4096
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    out = {"dense_head": dense_head, "gdn_decode": gdn_decode, "moe": moe}[args.workload](args)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

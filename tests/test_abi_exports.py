@@ -1,0 +1,61 @@
+"""The C-ABI library loads without a GPU and exports exactly what include/isoexec_hip.h declares."""
+
+import ctypes
+import os
+import re
+
+from isoexec_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "isoexec_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(r"^\s*(?:const\s+)?[a-z_0-9]+\*?\s+\*?(ix_[a-z0-9_]+)\s*\(", text, flags=re.M)
+
+
+def test_header_and_binding_table_agree():
+    names = declared_functions()
+    assert len(names) >= 20 and len(set(names)) == len(names)
+    assert set(names) == set(_lib.SIGNATURES), set(names) ^ set(_lib.SIGNATURES)
+
+
+def test_library_exports_every_declared_symbol():
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared_functions():
+        assert hasattr(handle, name), name
+
+
+def test_host_only_entry_points():
+    h = _lib.lib()
+    assert h.ix_abi_version() == 1 and h.ix_arch_tag() == b"gfx950"
+    assert h.ix_moe_max_tiles(16384, 8, 128, 256) == 16384 * 8 // 256 + 128
+    assert h.ix_moe_pick_bm(16384, 8, 128) == 256 and h.ix_moe_pick_bm(1, 8, 128) == 32
+    assert h.ix_logprob_workspace_bytes(4, 151936, 8) == 4 * (19 + 40 + 2) * 4
+    assert h.ix_logprob_workspace_bytes(4, 151937, 8) == 0
+
+
+def test_product_path_has_no_cpu_fallback():
+    import pytest
+    import torch
+
+    from isoexec_amd.ops.mm.mm_hip import linear_nt
+    from isoexec_amd.ops.norms.fused_outnorm import fused_rms_norm_gamma
+
+    x = torch.zeros(2, 64, dtype=torch.bfloat16)
+    with pytest.raises(_lib.IsoExecLibraryError):
+        fused_rms_norm_gamma(x, torch.zeros(64, dtype=torch.bfloat16), 1e-6)
+    with pytest.raises(_lib.IsoExecLibraryError):
+        linear_nt(x, x)
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "skyrl-isoexec_amd")
+    for base, _dirs, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(base, f)).read()
+                assert "oracle" not in text.replace("oracle/", "oracle/") or "import oracle" not in text
+                assert "from oracle" not in text and "import oracle" not in text, os.path.join(base, f)

@@ -1,0 +1,168 @@
+"""CPU: pins for the oracle's GatedDeltaNet and MoE restatements (config 0 runs here in full)."""
+
+import numpy as np
+import torch
+
+from oracle import gdn as o_gdn
+from oracle import moe as o_moe
+from oracle import prims as o_prims
+
+
+def config0(seed=0, B=2, T=256, H=4, K=64, V=64):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, T, H, K, generator=g)
+    k = torch.randn(B, T, H, K, generator=g)
+    q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6)
+    k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+    v = torch.randn(B, T, H, V, generator=g)
+    beta = torch.sigmoid(torch.randn(B, T, H, generator=g))
+    gate = -torch.nn.functional.softplus(torch.randn(B, T, H, generator=g))
+    return [t.numpy() for t in (q, k, v, gate, beta)]
+
+
+def test_config0_scan_against_fp64_recurrence_and_chunked_form():
+    q, k, v, g, beta = config0()
+    for b in range(2):
+        st = np.zeros((4, 64, 64), np.float32)
+        o = o_gdn.scan(q[b], k[b], v[b], g[b], beta[b], st)
+        o64, s64 = o_gdn.scan_fp64(q[b], k[b], v[b], g[b], beta[b])
+        assert np.abs(o - o64).max() <= 5e-6 and np.abs(st - s64).max() <= 5e-6
+        for chunk in (16, 32, 64):  # the chunked WY algorithm of gdn_ops.py:261-315 in float64
+            assert np.abs(o_gdn.chunk_fp64(q[b], k[b], v[b], g[b], beta[b], chunk) - o64).max() <= 1e-10
+
+
+def test_config0_prefill_decode_splits_are_bitwise_equal():
+    q, k, v, g, beta = config0()
+    b = 1
+    st = np.zeros((4, 64, 64), np.float32)
+    whole = o_gdn.scan(q[b], k[b], v[b], g[b], beta[b], st)
+    for split in (0, 1, 63, 64, 65, 127, 255):
+        s2 = np.zeros((4, 64, 64), np.float32)
+        parts = []
+        if split:
+            parts.append(o_gdn.scan(q[b, :split], k[b, :split], v[b, :split], g[b, :split], beta[b, :split], s2))
+        for t in range(split, 256):
+            parts.append(o_gdn.scan(q[b, t:t + 1], k[b, t:t + 1], v[b, t:t + 1], g[b, t:t + 1], beta[b, t:t + 1], s2))
+        got = np.concatenate(parts)
+        assert np.array_equal(got.view(np.uint32), whole.view(np.uint32))
+        assert np.array_equal(s2.view(np.uint32), st.view(np.uint32))
+
+
+def test_scan_closed_forms_and_gqa():
+    T, K, V = 32, 64, 16
+    k = np.eye(K, dtype=np.float32)[:T].reshape(T, 1, K)
+    q = k * np.float32(K ** 0.5)
+    rng = np.random.default_rng(1)
+    v = rng.standard_normal((T, 1, V)).astype(np.float32)
+    zeros, ones = np.zeros((T, 1), np.float32), np.ones((T, 1), np.float32)
+    st = np.zeros((1, V, K), np.float32)
+    assert np.array_equal(o_gdn.scan(q, k, v, zeros, ones, st), v)  # associative recall
+    s0 = rng.standard_normal((1, V, K)).astype(np.float32)
+    st = s0.copy()
+    gg = -rng.random((T, 1)).astype(np.float32)
+    o_gdn.scan(q, k, v, gg, zeros, st)  # beta = 0: pure decay
+    assert np.abs(st - s0 * np.exp(gg.astype(np.float64).sum())).max() <= 1e-5
+    # GQA: 2 value heads per key head == the expanded form
+    q2 = rng.standard_normal((T, 2, K)).astype(np.float32)
+    k2 = o_gdn.l2norm(rng.standard_normal((T, 2, K)).astype(np.float32), io_bf16=False)
+    v4 = rng.standard_normal((T, 4, V)).astype(np.float32)
+    g4 = -rng.random((T, 4)).astype(np.float32)
+    b4 = rng.random((T, 4)).astype(np.float32)
+    sa, sb = np.zeros((4, V, K), np.float32), np.zeros((4, V, K), np.float32)
+    oa = o_gdn.scan(q2, k2, v4, g4, b4, sa)
+    ob = o_gdn.scan(np.repeat(q2, 2, axis=1), np.repeat(k2, 2, axis=1), v4, g4, b4, sb)
+    assert np.array_equal(oa, ob) and np.array_equal(sa, sb)
+
+
+def test_l2norm_gate_and_conv_against_eager_expressions():
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(40, 3, 128, generator=g)
+    want = (x * torch.rsqrt((x * x).sum(-1, keepdim=True) + 1e-6)).numpy()
+    assert np.abs(o_gdn.l2norm(x.numpy(), io_bf16=False) - want).max() <= 2e-7
+    a, b = torch.randn(40, 4, generator=g) * 3, torch.randn(40, 4, generator=g)
+    a[0, 0] = 25.0
+    A_log, dt_bias = 0.2 * torch.randn(4, generator=g), 0.2 * torch.randn(4, generator=g)
+    gg, bb = o_gdn.gate_and_beta(a.numpy(), b.numpy(), A_log.numpy(), dt_bias.numpy(), io_bf16=False)
+    want_g = -A_log.exp() * torch.nn.functional.softplus(a + dt_bias)  # gdn_ops.py:1208
+    assert np.abs(gg - want_g.numpy()).max() <= 1e-6 * np.abs(want_g.numpy()).max()
+    assert np.abs(bb - torch.sigmoid(b).numpy()).max() <= 2e-7
+    # conv: brute-force loop over (t, d, tap) in float64, and the split-anywhere property
+    T, D, W = 19, 6, 4
+    xx = torch.randn(T, D, generator=g).to(torch.bfloat16).float().numpy()
+    w = torch.randn(D, W, generator=g).to(torch.bfloat16).float().numpy()
+    bias = torch.randn(D, generator=g).to(torch.bfloat16).float().numpy()
+    y, fs = o_gdn.causal_conv(xx, w, bias)
+    for t in range(T):
+        for d in range(D):
+            acc = sum(float(w[d, i]) * (float(xx[t - (W - 1) + i, d]) if t - (W - 1) + i >= 0 else 0.0)
+                      for i in range(W)) + float(bias[d])
+            ref = acc / (1.0 + np.exp(-acc))
+            assert abs(float(y[t, d]) - ref) <= 2.0 ** -7 * abs(ref) + 1e-6
+    assert np.array_equal(fs, xx[T - 3:].T)
+    y1, s1 = o_gdn.causal_conv(xx[:2], w, bias)
+    y2, s2 = o_gdn.causal_conv(xx[2:], w, bias, initial_state=s1)
+    assert np.array_equal(np.concatenate([y1, y2]), y) and np.array_equal(s2, fs)
+
+
+def test_router_against_torch_topk_softmax_and_tie_rules():
+    g = torch.Generator().manual_seed(3)
+    lg = 2 * torch.randn(50, 128, generator=g)
+    idx, p = o_moe.router_topk(lg.numpy(), 8, mode=0)
+    tv, ti = torch.topk(lg, 8, dim=1)
+    assert np.array_equal(idx, ti.numpy()) and np.abs(p - torch.softmax(tv, -1).numpy()).max() <= 2e-7
+    idx, p = o_moe.router_topk(lg.numpy(), 8, mode=1)  # HF form: softmax, top-k, renormalise
+    pr = torch.softmax(lg, -1)
+    tv, ti = torch.topk(pr, 8, dim=1)
+    assert np.array_equal(idx, ti.numpy()) and np.abs(p - (tv / tv.sum(-1, keepdim=True)).numpy()).max() <= 2e-7
+    tie = np.zeros((1, 16), np.float32)
+    tie[0, 9] = np.nan
+    idx, p = o_moe.router_topk(tie, 4, mode=0)
+    assert idx[0].tolist() == [0, 1, 2, 3] and np.allclose(p, 0.25)  # lowest index wins; NaN is -inf
+    idx, _ = o_moe.router_topk(np.full((1, 8), np.nan, np.float32), 2, mode=0)
+    assert idx[0].tolist() == [0, 1]
+
+
+def test_permutation_against_stable_argsort_and_combine_loop():
+    rng = np.random.default_rng(4)
+    T, E, k = 97, 16, 4
+    lg = rng.standard_normal((T, E)).astype(np.float32)
+    idx, prob = o_moe.router_topk(lg, k)
+    counts, st, pp, cr = o_moe.permute(idx, prob, E)
+    dp, dm = o_moe.dense_from_topk(idx, prob, E)
+    # ref_permute_index (moe_router_o2_kernel.py:389-397) on the dense tensors
+    rt = torch.from_numpy(dm).T.contiguous()
+    flat = rt.reshape(-1).to(torch.int8).argsort(descending=True, stable=True)[: T * k]
+    assert np.array_equal(st, (flat % T).numpy())
+    assert np.array_equal(pp, torch.from_numpy(dp).T.contiguous().reshape(-1)[flat].numpy())
+    assert np.array_equal(counts, dm.sum(0))
+    eo = o_prims.round_bf16(rng.standard_normal((T * k, 8)).astype(np.float32))
+    got = o_moe.combine(eo, cr)
+    for t in (0, 50, 96):
+        rows = sorted((int(st_e), r) for r, st_e in enumerate(np.repeat(np.arange(E), counts)) if st[r] == t)
+        acc = eo[rows[0][1]]
+        for _, r in rows[1:]:
+            acc = o_prims.round_bf16(acc + eo[r])
+        assert np.array_equal(got[t], acc)
+
+
+def test_expert_chain_against_brute_force():
+    rng = np.random.default_rng(5)
+    T, H, E, F, k = 12, 32, 4, 16, 2
+    bf = lambda a: o_prims.round_bf16(a.astype(np.float32))
+    x, w1, w2 = bf(rng.standard_normal((T, H))), bf(0.3 * rng.standard_normal((E, 2 * F, H))), \
+        bf(0.3 * rng.standard_normal((E, H, F)))
+    wr = bf(rng.standard_normal((E, H)))
+    out = o_moe.moe_ffn(x, wr, w1, w2, k)
+    lg = x @ wr.T
+    for t in range(T):
+        top = np.argsort(-lg[t], kind="stable")[:k]
+        p = np.exp(lg[t, top] - lg[t, top].max())
+        p = p / p.sum()
+        acc = np.zeros(H)
+        for e, pe in sorted(zip(top, p)):
+            h = x[t].astype(np.float64) @ w1[e].astype(np.float64).T
+            a = h[:F] / (1 + np.exp(-h[:F])) * h[F:] * pe
+            acc += a @ w2[e].astype(np.float64).T
+        assert np.abs(out[t] - acc).max() <= 0.03 * np.abs(acc).max() + 1e-3
+    one = o_moe.moe_ffn(x[3:4], wr, w1, w2, k)
+    assert np.array_equal(one[0], out[3])
