@@ -178,7 +178,7 @@ int ix_moe_permute(const int* topk_idx, const float* topk_prob, long T, long E, 
  * rows = T*k. BM must be the value given to ix_moe_permute. */
 int ix_moe_experts(const void* x, long ldx, const int* sorted_token, const float* permuted_prob,
                    const void* W1, const void* W2, const int* tile_meta, long max_tiles, long BM, void* inter,
-                   void* expert_out, long rows, long Hd, long F, void* stream);
+                   void* expert_out, long T, long rows, long Hd, long F, void* stream);
 
 /* _fixed_order_combine / _combine_topk_kernel (moe_batch_invariant.py:276-320,
  * moe_combine_kernel.py:36-76): out bf16 [T, Hd] = the token's k rows of expert_out summed in

@@ -23,45 +23,57 @@ __global__ __launch_bounds__(WM* WN * 64) void k_gemm_bf16_nt(const bf16_t* __re
                                                               const bf16_t* __restrict__ W, long ldw,
                                                               const bf16_t* __restrict__ bias,
                                                               bf16_t* __restrict__ C, long ldc, int M, int N,
-                                                              int K, int nb_m, int nb_n) {
+                                                              int K, int nb_m, int nb_n, int vec_store) {
   using Cfg = IxGemmCfg<BM, BN, WM, WN>;
   extern __shared__ __align__(16) char ix_lds[];
   int tm, tn;
   if (!ix_tile_of_block(blockIdx.x, nb_m, nb_n, &tm, &tn)) return;
   const long m0 = (long)tm * BM;
   const long n0 = (long)tn * BN;
+  const int m_valid = (int)min((long)BM, (long)M - m0);
+  const int n_valid = (int)min((long)BN, (long)N - n0);
+
+  // Tile-local buffer descriptors: rows past the matrix fall outside the range and read as 0.
+  const __amdgpu_buffer_rsrc_t x_rsrc = ix_make_rsrc(A + m0 * lda, (uint32_t)(((long)(m_valid - 1) * lda + K) * 2));
+  const __amdgpu_buffer_rsrc_t w_rsrc = ix_make_rsrc(W + n0 * ldw, (uint32_t)(((long)(n_valid - 1) * ldw + K) * 2));
+  const int kc = ix_fetch_kchunk();
+  uint32_t x_voff[Cfg::X_CH], w_voff[Cfg::W_CH];
+#pragma unroll
+  for (int j = 0; j < Cfg::X_CH; ++j) {
+    const int r = ix_fetch_row<Cfg>(j);
+    x_voff[j] = (r < m_valid) ? (uint32_t)(r * lda * 2 + kc * 16) : IX_OOB;
+  }
+#pragma unroll
+  for (int j = 0; j < Cfg::W_CH; ++j) {
+    const int r = ix_fetch_row<Cfg>(j);
+    w_voff[j] = (r < n_valid) ? (uint32_t)(r * ldw * 2 + kc * 16) : IX_OOB;
+  }
 
   ix_f32x16 acc[Cfg::MI][Cfg::NI];
-#pragma unroll
-  for (int mi = 0; mi < Cfg::MI; ++mi)
-#pragma unroll
-    for (int ni = 0; ni < Cfg::NI; ++ni)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[mi][ni][i] = 0.0f;
-
-  IxRowsPlain rows{A, lda, 0, (long)M};
-  const int n_valid = (int)min((long)BN, (long)N - n0);
-  IxWRowsPlain wrows{W + n0 * ldw, ldw, n_valid};
-  ix_gemm_mainloop<Cfg, BM, BN, WM, WN>(rows, m0, wrows, K, ix_lds, acc);
+  ix_acc_zero<Cfg>(acc);
+  ix_gemm_mainloop<Cfg>(x_rsrc, x_voff, w_rsrc, w_voff, K, ix_lds, acc);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WN, wn = wave % WN;
 #pragma unroll
-  for (int ni = 0; ni < Cfg::NI; ++ni) {
-    const long n = n0 + wn * Cfg::TN + ni * 32 + (lane & 31);
-    if (n >= N) continue;
-    // addmm: the bias joins in fp32 before the single bf16 round.
-    const float b = bias ? ix_bf2f(bias[n]) : 0.0f;
+  for (int mi = 0; mi < Cfg::MI; ++mi) {
+    const long m = m0 + wm * Cfg::TM + mi * 32 + (lane & 31);
+    if (m >= M) continue;
 #pragma unroll
-    for (int mi = 0; mi < Cfg::MI; ++mi) {
+    for (int ni = 0; ni < Cfg::NI; ++ni) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const long m = m0 + wm * Cfg::TM + mi * 32 + ix_acc_row(i, lane);
-        if (m < M) {
-          float v = acc[mi][ni][i];
-          if (bias) v = v + b;
-          C[m * ldc + n] = ix_f2bf(v);
+      for (int q = 0; q < 4; ++q) {
+        const long n = n0 + wn * Cfg::TN + ni * 32 + ix_acc_row(q * 4, lane);
+        const int valid = (int)min(4L, (long)N - n);
+        if (valid <= 0) continue;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] = acc[mi][ni][q * 4 + e];
+          // addmm: the bias joins in fp32 before the single bf16 round.
+          if (bias && e < valid) v[e] = v[e] + ix_bf2f(bias[n + e]);
         }
+        ix_store4_bf16(C + m * ldc + n, valid, vec_store != 0, v[0], v[1], v[2], v[3]);
       }
     }
   }
@@ -83,7 +95,7 @@ static int ix_gemm_bf16_launch(const bf16_t* A, long lda, const bf16_t* W, long 
     attr_set = true;
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(Cfg::NT), Cfg::LDS_BYTES, st, A, lda, W, ldw, bias, C, ldc,
-                     (int)M, (int)N, (int)K, (int)nb_m, (int)nb_n);
+                     (int)M, (int)N, (int)K, (int)nb_m, (int)nb_n, (int)((ldc % 4 == 0) && ix_aligned(C, 8)));
   return ix_launch_status();
 }
 
@@ -94,6 +106,7 @@ extern "C" int ix_gemm_bf16_nt(const void* A, long lda, const void* W, long ldw,
   // 16-byte row chunks: every row start and K itself must be a multiple of 8 elements.
   if ((K % 8) || (lda % 8) || (ldw % 8) || !ix_aligned(A, 16) || !ix_aligned(W, 16)) return IX_DECLINED;
   if (M > 0x7fffffffL || N > 0x7fffffffL || K > 0x7fffffffL) return IX_DECLINED;
+  if (lda * 2 * 256 >= 0x7fffffffL || ldw * 2 * 256 >= 0x7fffffffL) return IX_DECLINED;  // 32-bit tile offsets
   if (M == 0) return IX_OK;
   hipStream_t st = (hipStream_t)stream;
   const bf16_t *a = (const bf16_t*)A, *w = (const bf16_t*)W, *b = (const bf16_t*)bias;

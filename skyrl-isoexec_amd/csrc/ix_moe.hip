@@ -287,7 +287,7 @@ extern "C" int ix_moe_permute(const int* topk_idx, const float* topk_prob, long 
 // Grouped GEMMs over the block map. A workgroup past the device-side tile count exits at once,
 // so the host never reads the routing back.
 template <int BM, int BN, int WM, int WN>
-__global__ __launch_bounds__(WM* WN * 64) void k_moe_fc1_glu(const bf16_t* __restrict__ x, long ldx,
+__global__ __launch_bounds__(WM* WN * 64) void k_moe_fc1_glu(const bf16_t* __restrict__ x, long ldx, int T,
                                                              const int* __restrict__ sorted_token,
                                                              const float* __restrict__ permuted_prob,
                                                              const bf16_t* __restrict__ W1,
@@ -300,37 +300,55 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc1_glu(const bf16_t* __res
   if (mt >= meta[0]) return;
   const int e = meta[1 + mt];
   const long row0 = meta[1 + max_tiles + mt];
-  const long nrows = meta[1 + 2 * max_tiles + mt];
+  const int nrows = meta[1 + 2 * max_tiles + mt];
   const int n0h = nt * (BN / 2);
 
-  ix_f32x16 acc[Cfg::MI][2];
+  // activations: gathered token rows of x; weights: the expert's [2F, Hd] fc1 matrix with the
+  // tile's rows interleaved so that each wave holds a gate tile (ni = 0) and its up tile (ni = 1):
+  // tile row r -> wave r/64, half (r/32)&1, column n0h + 32*(r/64) + r%32.
+  const __amdgpu_buffer_rsrc_t x_rsrc = ix_make_rsrc(x, (uint32_t)(((long)(T - 1) * ldx + Hd) * 2));
+  const __amdgpu_buffer_rsrc_t w_rsrc = ix_make_rsrc(W1 + (long)e * 2 * F * Hd, (uint32_t)((long)2 * F * Hd * 2));
+  const int kc = ix_fetch_kchunk();
+  uint32_t x_voff[Cfg::X_CH], w_voff[Cfg::W_CH];
 #pragma unroll
-  for (int mi = 0; mi < Cfg::MI; ++mi)
+  for (int j = 0; j < Cfg::X_CH; ++j) {
+    const int r = ix_fetch_row<Cfg>(j);
+    x_voff[j] = (r < nrows) ? (uint32_t)((long)sorted_token[row0 + r] * ldx * 2 + kc * 16) : IX_OOB;
+  }
 #pragma unroll
-    for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[mi][ni][i] = 0.0f;
+  for (int j = 0; j < Cfg::W_CH; ++j) {
+    const int r = ix_fetch_row<Cfg>(j);
+    const int col = n0h + (r >> 6) * 32 + (r & 31);
+    w_voff[j] = (col < F) ? (uint32_t)(((long)((r >> 5) & 1) * F + col) * Hd * 2 + kc * 16) : IX_OOB;
+  }
 
-  IxRowsGather rows{x, ldx, sorted_token, row0, row0 + nrows};
-  IxWRowsGlu wrows{W1 + (long)e * 2 * F * Hd, (long)Hd, n0h, F};
-  ix_gemm_mainloop<Cfg, BM, BN, WM, WN>(rows, row0, wrows, Hd, ix_lds, acc);
+  ix_f32x16 acc[Cfg::MI][2];
+  ix_acc_zero<Cfg>(acc);
+  ix_gemm_mainloop<Cfg>(x_rsrc, x_voff, w_rsrc, w_voff, Hd, ix_lds, acc);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WN, wn = wave % WN;
-  const int col = n0h + wn * 32 + (lane & 31);
-  if (col >= F) return;
 #pragma unroll
   for (int mi = 0; mi < Cfg::MI; ++mi) {
+    const int r = wm * Cfg::TM + mi * 32 + (lane & 31);
+    if (r >= nrows) continue;
+    const long m = row0 + r;
+    const float prob = permuted_prob[m];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const long m = row0 + wm * Cfg::TM + mi * 32 + ix_acc_row(i, lane);
-      if (m < row0 + nrows) {
-        const float gate = ix_rbf(acc[mi][0][i]);
-        const float up = ix_rbf(acc[mi][1][i]);
+    for (int q = 0; q < 4; ++q) {
+      const int col = n0h + wn * 32 + ix_acc_row(q * 4, lane);
+      const int valid = min(4, F - col);
+      if (valid <= 0) continue;
+      float v[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const float gate = ix_rbf(acc[mi][0][q * 4 + c]);
+        const float up = ix_rbf(acc[mi][1][q * 4 + c]);
         const float s = ix_rbf(ix_silu_div(gate));
         const float h = ix_rbf(s * up);
-        inter[m * F + col] = ix_f2bf(h * permuted_prob[m]);
+        v[c] = h * prob;
       }
+      ix_store4_bf16(inter + m * F + col, valid, true, v[0], v[1], v[2], v[3]);
     }
   }
 }
@@ -346,40 +364,53 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc2(const bf16_t* __restric
   if (mt >= meta[0]) return;
   const int e = meta[1 + mt];
   const long row0 = meta[1 + max_tiles + mt];
-  const long nrows = meta[1 + 2 * max_tiles + mt];
+  const int nrows = meta[1 + 2 * max_tiles + mt];
   const long n0 = (long)nt * BN;
+  const int n_valid = (int)min((long)BN, (long)Hd - n0);
+
+  const __amdgpu_buffer_rsrc_t x_rsrc = ix_make_rsrc(inter + row0 * F, (uint32_t)((long)nrows * F * 2));
+  const __amdgpu_buffer_rsrc_t w_rsrc = ix_make_rsrc(W2 + ((long)e * Hd + n0) * F, (uint32_t)((long)n_valid * F * 2));
+  const int kc = ix_fetch_kchunk();
+  uint32_t x_voff[Cfg::X_CH], w_voff[Cfg::W_CH];
+#pragma unroll
+  for (int j = 0; j < Cfg::X_CH; ++j) {
+    const int r = ix_fetch_row<Cfg>(j);
+    x_voff[j] = (r < nrows) ? (uint32_t)(r * F * 2 + kc * 16) : IX_OOB;
+  }
+#pragma unroll
+  for (int j = 0; j < Cfg::W_CH; ++j) {
+    const int r = ix_fetch_row<Cfg>(j);
+    w_voff[j] = (r < n_valid) ? (uint32_t)(r * F * 2 + kc * 16) : IX_OOB;
+  }
 
   ix_f32x16 acc[Cfg::MI][Cfg::NI];
-#pragma unroll
-  for (int mi = 0; mi < Cfg::MI; ++mi)
-#pragma unroll
-    for (int ni = 0; ni < Cfg::NI; ++ni)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[mi][ni][i] = 0.0f;
-
-  IxRowsPlain rows{inter, (long)F, row0, row0 + nrows};
-  IxWRowsPlain wrows{W2 + ((long)e * Hd + n0) * F, (long)F, (int)min((long)BN, (long)Hd - n0)};
-  ix_gemm_mainloop<Cfg, BM, BN, WM, WN>(rows, row0, wrows, F, ix_lds, acc);
+  ix_acc_zero<Cfg>(acc);
+  ix_gemm_mainloop<Cfg>(x_rsrc, x_voff, w_rsrc, w_voff, F, ix_lds, acc);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WN, wn = wave % WN;
 #pragma unroll
-  for (int ni = 0; ni < Cfg::NI; ++ni) {
-    const long n = n0 + wn * Cfg::TN + ni * 32 + (lane & 31);
-    if (n >= Hd) continue;
+  for (int mi = 0; mi < Cfg::MI; ++mi) {
+    const int r = wm * Cfg::TM + mi * 32 + (lane & 31);
+    if (r >= nrows) continue;
+    const long m = row0 + r;
 #pragma unroll
-    for (int mi = 0; mi < Cfg::MI; ++mi) {
+    for (int ni = 0; ni < Cfg::NI; ++ni) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const long m = row0 + wm * Cfg::TM + mi * 32 + ix_acc_row(i, lane);
-        if (m < row0 + nrows) out[m * Hd + n] = ix_f2bf(acc[mi][ni][i]);
+      for (int q = 0; q < 4; ++q) {
+        const long n = n0 + wn * Cfg::TN + ni * 32 + ix_acc_row(q * 4, lane);
+        const int valid = (int)min(4L, (long)Hd - n);
+        if (valid <= 0) continue;
+        ix_store4_bf16(out + m * Hd + n, valid, true, acc[mi][ni][q * 4], acc[mi][ni][q * 4 + 1],
+                       acc[mi][ni][q * 4 + 2], acc[mi][ni][q * 4 + 3]);
       }
     }
   }
 }
 
 template <int BM, int BN, int WM, int WN>
-static int ix_moe_experts_launch(const bf16_t* x, long ldx, const int* sorted_token, const float* permuted_prob,
+static int ix_moe_experts_launch(const bf16_t* x, long ldx, int T, const int* sorted_token,
+                                 const float* permuted_prob,
                                  const bf16_t* W1, const bf16_t* W2, const int* meta, long max_tiles,
                                  bf16_t* inter, bf16_t* out, int Hd, int F, hipStream_t st) {
   using Cfg = IxGemmCfg<BM, BN, WM, WN>;
@@ -397,8 +428,8 @@ static int ix_moe_experts_launch(const bf16_t* x, long ldx, const int* sorted_to
   const long nb1 = (F + BN / 2 - 1) / (BN / 2);
   const long nb2 = (Hd + BN - 1) / BN;
   if (max_tiles * nb1 > 0x7fffffffL || max_tiles * nb2 > 0x7fffffffL) return IX_DECLINED;
-  hipLaunchKernelGGL(k1, dim3((unsigned)(max_tiles * nb1)), dim3(Cfg::NT), Cfg::LDS_BYTES, st, x, ldx, sorted_token,
-                     permuted_prob, W1, meta, (int)max_tiles, inter, Hd, F, (int)nb1);
+  hipLaunchKernelGGL(k1, dim3((unsigned)(max_tiles * nb1)), dim3(Cfg::NT), Cfg::LDS_BYTES, st, x, ldx, T,
+                     sorted_token, permuted_prob, W1, meta, (int)max_tiles, inter, Hd, F, (int)nb1);
   hipLaunchKernelGGL(k2, dim3((unsigned)(max_tiles * nb2)), dim3(Cfg::NT), Cfg::LDS_BYTES, st, inter, W2, meta,
                      (int)max_tiles, out, Hd, F, (int)nb2);
   return ix_launch_status();
@@ -406,12 +437,14 @@ static int ix_moe_experts_launch(const bf16_t* x, long ldx, const int* sorted_to
 
 extern "C" int ix_moe_experts(const void* x, long ldx, const int* sorted_token, const float* permuted_prob,
                               const void* W1, const void* W2, const int* tile_meta, long max_tiles, long BM,
-                              void* inter, void* expert_out, long rows, long Hd, long F, void* stream) {
+                              void* inter, void* expert_out, long T, long rows, long Hd, long F, void* stream) {
   if (!x || !sorted_token || !permuted_prob || !W1 || !W2 || !tile_meta || !inter || !expert_out)
     return IX_ERR_ARG;
-  if (rows < 0 || Hd <= 0 || F <= 0 || max_tiles < 0 || ldx < Hd) return IX_ERR_ARG;
+  if (T < 0 || rows < 0 || Hd <= 0 || F <= 0 || max_tiles < 0 || ldx < Hd) return IX_ERR_ARG;
+  // 32-bit buffer offsets: the activation matrix, one expert's weights and one row tile must fit
+  if (T * ldx * 2 >= 0x7fffffffL || 2 * F * Hd * 2 >= 0x7fffffffL || 256 * F * 2 >= 0x7fffffffL) return IX_DECLINED;
   if ((Hd % 8) || (F % 8) || (ldx % 8) || !ix_aligned(x, 16) || !ix_aligned(W1, 16) || !ix_aligned(W2, 16) ||
-      !ix_aligned(inter, 16))
+      !ix_aligned(inter, 16) || !ix_aligned(expert_out, 8))
     return IX_DECLINED;
   if (rows == 0 || max_tiles == 0) return IX_OK;
   hipStream_t st = (hipStream_t)stream;
@@ -419,13 +452,13 @@ extern "C" int ix_moe_experts(const void* x, long ldx, const int* sorted_token, 
   bf16_t *it = (bf16_t*)inter, *eo = (bf16_t*)expert_out;
   switch (BM) {
     case 32:
-      return ix_moe_experts_launch<32, 256, 1, 4>(xx, ldx, sorted_token, permuted_prob, w1, w2, tile_meta,
+      return ix_moe_experts_launch<32, 256, 1, 4>(xx, ldx, (int)T, sorted_token, permuted_prob, w1, w2, tile_meta,
                                                   max_tiles, it, eo, (int)Hd, (int)F, st);
     case 128:
-      return ix_moe_experts_launch<128, 256, 2, 4>(xx, ldx, sorted_token, permuted_prob, w1, w2, tile_meta,
+      return ix_moe_experts_launch<128, 256, 2, 4>(xx, ldx, (int)T, sorted_token, permuted_prob, w1, w2, tile_meta,
                                                    max_tiles, it, eo, (int)Hd, (int)F, st);
     case 256:
-      return ix_moe_experts_launch<256, 256, 2, 4>(xx, ldx, sorted_token, permuted_prob, w1, w2, tile_meta,
+      return ix_moe_experts_launch<256, 256, 2, 4>(xx, ldx, (int)T, sorted_token, permuted_prob, w1, w2, tile_meta,
                                                    max_tiles, it, eo, (int)Hd, (int)F, st);
     default: return IX_ERR_ARG;
   }

@@ -68,7 +68,7 @@ SIGNATURES = {
     ),
     "ix_moe_experts": (
         c_int,
-        [P, c_long, P, P, P, P, P, c_long, c_long, P, P, c_long, c_long, c_long, P],
+        [P, c_long, P, P, P, P, P, c_long, c_long, P, P, c_long, c_long, c_long, c_long, P],
     ),
     "ix_moe_combine": (c_int, [P, P, P, c_long, c_long, c_long, c_int, P]),
 }

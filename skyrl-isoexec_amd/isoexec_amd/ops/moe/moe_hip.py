@@ -105,7 +105,7 @@ def experts_forward(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, p: Perm
         _lib.lib().ix_moe_experts(xc.data_ptr(), xc.stride(0), p.sorted_token.data_ptr(),
                                   p.permuted_prob.data_ptr(), w1.contiguous().data_ptr(),
                                   w2.contiguous().data_ptr(), p.tile_meta.data_ptr(), p.max_tiles, p.BM,
-                                  inter.data_ptr(), out.data_ptr(), rows, H, F, _lib.current_stream(dev)),
+                                  inter.data_ptr(), out.data_ptr(), T, rows, H, F, _lib.current_stream(dev)),
         "ix_moe_experts")
     if rc != _lib.IX_OK:
         raise RuntimeError(f"[isoexec-amd] ix_moe_experts declined H={H} F={F}")
