@@ -72,8 +72,8 @@ def dense_head(args):
     def step(timed):
         wrap = (lambda t, f: t(f)) if timed else (lambda t, f: f())
         x = wrap(t_norm, lambda: fused_rms_norm_gamma(h, w_norm, 1e-6))
-        logits = wrap(t_gemm, lambda: linear_nt(x, w_lm, tile=args.tile))
-        lp, _ = wrap(t_lp, lambda: sampled_forward(logits, target, 8))
+        logits, row_max = wrap(t_gemm, lambda: linear_nt(x, w_lm, tile=args.tile, want_row_max=True))
+        lp, _ = wrap(t_lp, lambda: sampled_forward(logits, target, 8, row_max=row_max))
         return lp
 
     for _ in range(args.warmup):
@@ -221,7 +221,7 @@ def main():
     ap.add_argument("--tokens", type=int, default=None)
     ap.add_argument("--batch", type=int, default=256)
     ap.add_argument("--tile", type=int, default=0)
-    ap.add_argument("--cpu-tokens", type=int, default=64)
+    ap.add_argument("--cpu-tokens", type=int, default=2048)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:

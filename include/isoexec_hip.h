@@ -65,16 +65,22 @@ size_t ix_logprob_workspace_bytes(long rows, long V, int G);
  * :156-191) at world size 1. logits [rows, V] (row pitch row_stride elements), target int64
  * [rows] (out of range -> logprob 0), G leaves (power of two, V % G == 0 else declined).
  * out_logprob fp32 [rows]; out_lse fp32 [rows] or NULL. force_shape: 0 auto, 1 one workgroup
- * per row, 2 split rows (needs the workspace). */
+ * per row, 2 split rows (needs the workspace). row_max_in: NULL, or fp32 [rows] holding each
+ * row's exact maximum (e.g. ix_gemm_bf16_nt's row_max_parts reduced by ix_rowmax_reduce): the
+ * max pass is skipped and the logits are read once. The workspace is always required with it. */
 int ix_logprob_rowinv_sampled(const void* logits, int dtype, long rows, long V, long row_stride,
                               const int64_t* target, int G, float* out_logprob, float* out_lse,
-                              void* workspace, size_t workspace_bytes, int force_shape, void* stream);
+                              void* workspace, size_t workspace_bytes, int force_shape,
+                              const float* row_max_in, void* stream);
 
 /* rowinv_full_logprobs (rowinv.py:796-875; kernel full_row_logprobs :193-245): the whole row
  * (x - m) - log S into out_full fp32 [rows, V] (pitch out_stride). */
 int ix_logprob_rowinv_full(const void* logits, int dtype, long rows, long V, long row_stride, int G,
                            float* out_full, long out_stride, float* out_lse, void* workspace,
-                           size_t workspace_bytes, int force_shape, void* stream);
+                           size_t workspace_bytes, int force_shape, const float* row_max_in, void* stream);
+
+/* rowmax[r] = max_p parts[r*parts_ld + p], p < P (torch.amax of rowinv.py:479 over partials). */
+int ix_rowmax_reduce(const float* parts, long parts_ld, long P, long rows, float* rowmax, void* stream);
 
 /* ---- norms: ops/norms/fused_outnorm.py, zero_centered_norm.py, fused_add_rmsnorm.py -------- */
 
@@ -98,10 +104,16 @@ int ix_add_rmsnorm_gamma(const void* x, const void* residual, const void* weight
 /* ---- dense matmuls: ops/moe/moe_batch_invariant.py:422-473 (aten mm/addmm/bmm override),
  *      ops/mm/mm_tiles.py:127-158, ops/mm/csrc/cublaslt_pinned.cpp:319-327 mm(x, w, out, slot) - */
 
-/* C[M,N] = A[M,K] . W[N,K]^T (+ bias[N]), bf16 in/out, fp32 accumulate in a fixed K order, no
- * split-K. lda/ldw/ldc are row pitches in elements. bias may be NULL. tile: 0 auto. */
-int ix_gemm_bf16_nt(const void* A, long lda, const void* W, long ldw, const void* bias, void* C, long ldc,
-                    long M, long N, long K, int tile, void* stream);
+/* C[M,N] = A[M,K] . W[N,K]^T (+ bias[N]), bf16 operands, fp32 accumulate in a fixed K order, no
+ * split-K. C is bf16 (one round of the accumulator) or, with c_dtype = IX_DT_F32, the fp32
+ * accumulator itself (the router's fp32 gating product when its fp32 weight is bf16-exact).
+ * lda/ldw/ldc are row pitches in elements. bias (bf16 [N]) may be NULL. tile: 0 auto.
+ * row_max_parts: NULL, or fp32 [M, parts_ld] receiving per column tile the max of the stored
+ * values, parts_ld >= ix_gemm_bf16_n_tiles(M, N, tile). */
+int ix_gemm_bf16_nt(const void* A, long lda, const void* W, long ldw, const void* bias, void* C, int c_dtype,
+                    long ldc, long M, long N, long K, int tile, float* row_max_parts, long parts_ld,
+                    void* stream);
+long ix_gemm_bf16_n_tiles(long M, long N, int tile);
 
 /* Router gating GEMM (moe/_register.py:59-66): C fp32 [M,N] = A[M,K] . W[N,K]^T with W fp32 and
  * A fp32 or bf16 (a_dtype), fp32 accumulate in a fixed K order. */

@@ -18,12 +18,29 @@ __device__ __forceinline__ bool ix_tile_of_block(long bid, int nb_m, int nb_n, i
   return *tn < nb_n;
 }
 
-template <int BM, int BN, int WM, int WN>
+__device__ __forceinline__ void ix_store4(bf16_t* p, int valid, bool vec, const float (&v)[4]) {
+  ix_store4_bf16(p, valid, vec, v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void ix_store4(float* p, int valid, bool vec, const float (&v)[4]) {
+  if (vec && valid >= 4) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (e < valid) p[e] = v[e];
+  }
+}
+
+// TC = bf16_t: C is the bf16 round of the fp32 accumulator; TC = float: the accumulator itself.
+// row_max_parts (optional): [M, parts_ld] fp32, entry (m, tn) = max over the tile's columns of the
+// values stored to C (exact, order-free), so a consumer can skip its own max pass over C.
+template <int BM, int BN, int WM, int WN, typename TC>
 __global__ __launch_bounds__(WM* WN * 64) void k_gemm_bf16_nt(const bf16_t* __restrict__ A, long lda,
                                                               const bf16_t* __restrict__ W, long ldw,
                                                               const bf16_t* __restrict__ bias,
-                                                              bf16_t* __restrict__ C, long ldc, int M, int N,
-                                                              int K, int nb_m, int nb_n, int vec_store) {
+                                                              TC* __restrict__ C, long ldc, int M, int N, int K,
+                                                              int nb_m, int nb_n, int vec_store,
+                                                              float* __restrict__ row_max_parts, long parts_ld) {
   using Cfg = IxGemmCfg<BM, BN, WM, WN>;
   extern __shared__ __align__(16) char ix_lds[];
   int tm, tn;
@@ -55,38 +72,59 @@ __global__ __launch_bounds__(WM* WN * 64) void k_gemm_bf16_nt(const bf16_t* __re
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WN, wn = wave % WN;
+  float rmax[Cfg::MI];
 #pragma unroll
   for (int mi = 0; mi < Cfg::MI; ++mi) {
+    rmax[mi] = IX_NEG_INF;
     const long m = m0 + wm * Cfg::TM + mi * 32 + (lane & 31);
-    if (m >= M) continue;
 #pragma unroll
     for (int ni = 0; ni < Cfg::NI; ++ni) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const long n = n0 + wn * Cfg::TN + ni * 32 + ix_acc_row(q * 4, lane);
         const int valid = (int)min(4L, (long)N - n);
-        if (valid <= 0) continue;
+        if (valid <= 0 || m >= M) continue;
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           v[e] = acc[mi][ni][q * 4 + e];
           // addmm: the bias joins in fp32 before the single bf16 round.
           if (bias && e < valid) v[e] = v[e] + ix_bf2f(bias[n + e]);
+          if (e < valid) rmax[mi] = fmaxf(rmax[mi], v[e]);
         }
-        ix_store4_bf16(C + m * ldc + n, valid, vec_store != 0, v[0], v[1], v[2], v[3]);
+        ix_store4(C + m * ldc + n, valid, vec_store != 0, v);
       }
+    }
+  }
+  if (row_max_parts) {
+    float* s_max = reinterpret_cast<float*>(ix_lds);  // [WN][BM]
+    __syncthreads();                                  // every wave has left the main loop's LDS reads
+#pragma unroll
+    for (int mi = 0; mi < Cfg::MI; ++mi) {
+      float v = fmaxf(rmax[mi], __shfl_xor(rmax[mi], 32, IX_WAVE));
+      // rounding is monotonic: the max of the rounded values is the rounded max
+      if (sizeof(TC) == 2) v = ix_rbf(v);
+      if (lane < 32) s_max[wn * BM + wm * Cfg::TM + mi * 32 + lane] = v;
+    }
+    __syncthreads();
+    for (int r = threadIdx.x; r < m_valid; r += Cfg::NT) {
+      float v = s_max[r];
+#pragma unroll
+      for (int w = 1; w < WN; ++w) v = fmaxf(v, s_max[w * BM + r]);
+      row_max_parts[(m0 + r) * parts_ld + tn] = v;
     }
   }
 }
 
-template <int BM, int BN, int WM, int WN>
-static int ix_gemm_bf16_launch(const bf16_t* A, long lda, const bf16_t* W, long ldw, const bf16_t* bias, bf16_t* C,
-                               long ldc, long M, long N, long K, hipStream_t st) {
+template <int BM, int BN, int WM, int WN, typename TC>
+static int ix_gemm_bf16_launch(const bf16_t* A, long lda, const bf16_t* W, long ldw, const bf16_t* bias, TC* C,
+                               long ldc, long M, long N, long K, float* parts, long parts_ld, hipStream_t st) {
   using Cfg = IxGemmCfg<BM, BN, WM, WN>;
   const long nb_m = (M + BM - 1) / BM, nb_n = (N + BN - 1) / BN;
   const long grid = 8 * nb_m * ((nb_n + 7) / 8);
   if (grid > 0x7fffffffL) return IX_DECLINED;
-  auto kern = k_gemm_bf16_nt<BM, BN, WM, WN>;
+  if (parts && parts_ld < nb_n) return IX_ERR_ARG;
+  auto kern = k_gemm_bf16_nt<BM, BN, WM, WN, TC>;
   static bool attr_set = false;  // per instantiation
   if (!attr_set) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES) !=
@@ -94,15 +132,43 @@ static int ix_gemm_bf16_launch(const bf16_t* A, long lda, const bf16_t* W, long 
       return IX_ERR_LAUNCH;
     attr_set = true;
   }
+  const int vec = (ldc % 4 == 0) && ix_aligned(C, 4 * sizeof(TC));
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(Cfg::NT), Cfg::LDS_BYTES, st, A, lda, W, ldw, bias, C, ldc,
-                     (int)M, (int)N, (int)K, (int)nb_m, (int)nb_n, (int)((ldc % 4 == 0) && ix_aligned(C, 8)));
+                     (int)M, (int)N, (int)K, (int)nb_m, (int)nb_n, vec, parts, parts_ld);
   return ix_launch_status();
 }
 
+static int ix_gemm_tile_for(long M, int tile) {
+  if (tile != 0) return tile;
+  return (M <= 32) ? 1 : (M <= 128) ? 2 : 3;
+}
+
+extern "C" long ix_gemm_bf16_n_tiles(long M, long N, int tile) {
+  const int t = ix_gemm_tile_for(M, tile);
+  const long bn = (t == 2) ? 128 : 256;
+  return N <= 0 ? 0 : (N + bn - 1) / bn;
+}
+
+template <typename TC>
+static int ix_gemm_bf16_dispatch(const bf16_t* a, long lda, const bf16_t* w, long ldw, const bf16_t* b, TC* c,
+                                 long ldc, long M, long N, long K, int tile, float* parts, long parts_ld,
+                                 hipStream_t st) {
+  // `tile` only picks which workgroup owns an element (0 = by M); the bits do not depend on it.
+  switch (ix_gemm_tile_for(M, tile)) {
+    case 1: return ix_gemm_bf16_launch<32, 256, 1, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
+    case 2: return ix_gemm_bf16_launch<128, 128, 2, 2, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
+    case 3: return ix_gemm_bf16_launch<256, 256, 2, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
+    case 5: return ix_gemm_bf16_launch<128, 256, 2, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
+    default: return IX_ERR_ARG;
+  }
+}
+
 extern "C" int ix_gemm_bf16_nt(const void* A, long lda, const void* W, long ldw, const void* bias, void* C,
-                               long ldc, long M, long N, long K, int tile, void* stream) {
+                               int c_dtype, long ldc, long M, long N, long K, int tile, float* row_max_parts,
+                               long parts_ld, void* stream) {
   if (!A || !W || !C || M < 0 || N <= 0 || K <= 0) return IX_ERR_ARG;
   if (lda < K || ldw < K || ldc < N) return IX_ERR_ARG;
+  if (c_dtype != IX_DT_BF16 && c_dtype != IX_DT_F32) return IX_DECLINED;
   // 16-byte row chunks: every row start and K itself must be a multiple of 8 elements.
   if ((K % 8) || (lda % 8) || (ldw % 8) || !ix_aligned(A, 16) || !ix_aligned(W, 16)) return IX_DECLINED;
   if (M > 0x7fffffffL || N > 0x7fffffffL || K > 0x7fffffffL) return IX_DECLINED;
@@ -110,17 +176,9 @@ extern "C" int ix_gemm_bf16_nt(const void* A, long lda, const void* W, long ldw,
   if (M == 0) return IX_OK;
   hipStream_t st = (hipStream_t)stream;
   const bf16_t *a = (const bf16_t*)A, *w = (const bf16_t*)W, *b = (const bf16_t*)bias;
-  bf16_t* c = (bf16_t*)C;
-  // `tile` only picks which workgroup owns an element (0 = by M); the bits do not depend on it.
-  if (tile == 0) tile = (M <= 32) ? 1 : (M <= 128) ? 2 : 3;
-  switch (tile) {
-    case 1: return ix_gemm_bf16_launch<32, 256, 1, 4>(a, lda, w, ldw, b, c, ldc, M, N, K, st);
-    case 2: return ix_gemm_bf16_launch<128, 128, 2, 2>(a, lda, w, ldw, b, c, ldc, M, N, K, st);
-    case 3: return ix_gemm_bf16_launch<256, 256, 2, 4>(a, lda, w, ldw, b, c, ldc, M, N, K, st);
-    case 4: return ix_gemm_bf16_launch<256, 256, 2, 2>(a, lda, w, ldw, b, c, ldc, M, N, K, st);
-    case 5: return ix_gemm_bf16_launch<128, 256, 2, 4>(a, lda, w, ldw, b, c, ldc, M, N, K, st);
-    default: return IX_ERR_ARG;
-  }
+  if (c_dtype == IX_DT_BF16)
+    return ix_gemm_bf16_dispatch(a, lda, w, ldw, b, (bf16_t*)C, ldc, M, N, K, tile, row_max_parts, parts_ld, st);
+  return ix_gemm_bf16_dispatch(a, lda, w, ldw, b, (float*)C, ldc, M, N, K, tile, row_max_parts, parts_ld, st);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -242,6 +242,25 @@ __global__ __launch_bounds__(256) void k_lp_fullwrite(const T* __restrict__ x, l
   }
 }
 
+// rowmax[row] = max over P parts (exact; any order). One wave per row.
+__global__ __launch_bounds__(256) void k_lp_reduce_parts(const float* __restrict__ parts, long parts_ld, int P,
+                                                         long rows, float* __restrict__ rowmax) {
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const float m = ix_row_max_from_parts(parts + row * parts_ld, P, threadIdx.x & 63);
+  if ((threadIdx.x & 63) == 0) rowmax[row] = m;
+}
+
+extern "C" int ix_rowmax_reduce(const float* parts, long parts_ld, long P, long rows, float* rowmax, void* stream) {
+  if (!parts || !rowmax || rows < 0 || P <= 0 || parts_ld < P || P > 0x7fffffffL) return IX_ERR_ARG;
+  if (rows == 0) return IX_OK;
+  const long grid = (rows + 3) / 4;
+  if (grid > 0x7fffffffL) return IX_DECLINED;
+  hipLaunchKernelGGL(k_lp_reduce_parts, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, parts, parts_ld,
+                     (int)P, rows, rowmax);
+  return ix_launch_status();
+}
+
 // ---------------------------------------------------------------------------------------------
 static int ix_lp_check(const void* logits, int dtype, long rows, long V, long row_stride, int G) {
   if (!logits || rows < 0 || V <= 0 || row_stride < V) return IX_ERR_ARG;
@@ -266,11 +285,13 @@ extern "C" size_t ix_logprob_workspace_bytes(long rows, long V, int G) {
 template <typename T>
 static int ix_lp_launch(const T* x, long rows, long V, long row_stride, int G, const int64_t* target,
                         float* out_lp, float* out_lse, float* out_full, long full_stride, float* ws,
-                        size_t ws_bytes, int force_shape, hipStream_t st) {
+                        size_t ws_bytes, int force_shape, const float* row_max_in, hipStream_t st) {
   if (rows == 0) return IX_OK;
   const long L = V / G;
   const int vec = (ix_aligned(x, 8 * sizeof(T)) && (row_stride % 8 == 0) && (L % 8 == 0)) ? 1 : 0;
-  const bool split = force_shape == 2 || (force_shape == 0 && rows < IX_LP_SPLIT_BELOW);
+  // a caller-supplied row max (exact, e.g. from the producing GEMM's epilogue) removes the max
+  // pass: the row is then read from HBM once, by the block sums
+  const bool split = row_max_in || force_shape == 2 || (force_shape == 0 && rows < IX_LP_SPLIT_BELOW);
   if (!split) {
     hipLaunchKernelGGL((k_lp_row<T>), dim3((unsigned)rows), dim3(512), 0, st, x, row_stride, (int)V, G, target,
                        out_lp, out_lse, out_full, full_stride, vec);
@@ -279,47 +300,52 @@ static int ix_lp_launch(const T* x, long rows, long V, long row_stride, int G, c
   if (rows > 65535L * 1024) return IX_DECLINED;
   if (!ws || ws_bytes < ix_logprob_workspace_bytes(rows, V, G)) return IX_ERR_ARG;
   const int NB = (int)((L + IX_LP_BLOCK - 1) / IX_LP_BLOCK);
-  const int P = (int)((V + IX_LP_SEG - 1) / IX_LP_SEG);
+  const int PW = (int)((V + IX_LP_SEG - 1) / IX_LP_SEG);  // workspace layout always reserves PW parts
   const int U = G * NB;
-  float* pmax = ws;
-  float* bsum = pmax + rows * P;
+  float* ws_pmax = ws;
+  float* bsum = ws_pmax + rows * PW;
   float* fin = bsum + rows * U;
-  hipLaunchKernelGGL((k_lp_partmax<T>), dim3((unsigned)rows, P), dim3(256), 0, st, x, row_stride, (int)V, P, pmax,
-                     vec);
+  const int P = row_max_in ? 1 : PW;
+  const float* pmax = row_max_in ? row_max_in : ws_pmax;
+  if (!row_max_in)
+    hipLaunchKernelGGL((k_lp_partmax<T>), dim3((unsigned)rows, P), dim3(256), 0, st, x, row_stride, (int)V, P,
+                       ws_pmax, vec);
   hipLaunchKernelGGL((k_lp_blocksums<T>), dim3((unsigned)rows, (U + 3) / 4), dim3(256), 0, st, x, row_stride,
                      (int)V, G, P, pmax, bsum, vec);
   hipLaunchKernelGGL((k_lp_finalize<T>), dim3((unsigned)rows), dim3(64), 0, st, x, row_stride, (int)V, G, P, pmax,
                      bsum, fin, target, out_lp, out_lse);
   if (out_full)
-    hipLaunchKernelGGL((k_lp_fullwrite<T>), dim3((unsigned)rows, P), dim3(256), 0, st, x, row_stride, (int)V, fin,
+    hipLaunchKernelGGL((k_lp_fullwrite<T>), dim3((unsigned)rows, PW), dim3(256), 0, st, x, row_stride, (int)V, fin,
                        out_full, full_stride, vec);
   return ix_launch_status();
 }
 
 extern "C" int ix_logprob_rowinv_sampled(const void* logits, int dtype, long rows, long V, long row_stride,
                                          const int64_t* target, int G, float* out_logprob, float* out_lse,
-                                         void* workspace, size_t workspace_bytes, int force_shape, void* stream) {
+                                         void* workspace, size_t workspace_bytes, int force_shape,
+                                         const float* row_max_in, void* stream) {
   int rc = ix_lp_check(logits, dtype, rows, V, row_stride, G);
   if (rc != IX_OK) return rc;
   if (!target || !out_logprob) return IX_ERR_ARG;
   hipStream_t st = (hipStream_t)stream;
   if (dtype == IX_DT_BF16)
     return ix_lp_launch((const bf16_t*)logits, rows, V, row_stride, G, target, out_logprob, out_lse, nullptr, 0,
-                        (float*)workspace, workspace_bytes, force_shape, st);
+                        (float*)workspace, workspace_bytes, force_shape, row_max_in, st);
   return ix_lp_launch((const float*)logits, rows, V, row_stride, G, target, out_logprob, out_lse, nullptr, 0,
-                      (float*)workspace, workspace_bytes, force_shape, st);
+                      (float*)workspace, workspace_bytes, force_shape, row_max_in, st);
 }
 
 extern "C" int ix_logprob_rowinv_full(const void* logits, int dtype, long rows, long V, long row_stride, int G,
                                       float* out_full, long out_stride, float* out_lse, void* workspace,
-                                      size_t workspace_bytes, int force_shape, void* stream) {
+                                      size_t workspace_bytes, int force_shape, const float* row_max_in,
+                                      void* stream) {
   int rc = ix_lp_check(logits, dtype, rows, V, row_stride, G);
   if (rc != IX_OK) return rc;
   if (!out_full || out_stride < V) return IX_ERR_ARG;
   hipStream_t st = (hipStream_t)stream;
   if (dtype == IX_DT_BF16)
     return ix_lp_launch((const bf16_t*)logits, rows, V, row_stride, G, nullptr, nullptr, out_lse, out_full,
-                        out_stride, (float*)workspace, workspace_bytes, force_shape, st);
+                        out_stride, (float*)workspace, workspace_bytes, force_shape, row_max_in, st);
   return ix_lp_launch((const float*)logits, rows, V, row_stride, G, nullptr, nullptr, out_lse, out_full,
-                      out_stride, (float*)workspace, workspace_bytes, force_shape, st);
+                      out_stride, (float*)workspace, workspace_bytes, force_shape, row_max_in, st);
 }

@@ -20,6 +20,8 @@
 #define IX_MOE_KMAX 16
 #define IX_MOE_EC 8  // experts per lane: E <= 512
 #define IX_MOE_TILE_T 256
+#define IX_MOE_EMAX 512
+#define IX_MOE_SCAN_TILES 16
 
 // ---------------------------------------------------------------------------------------------
 __device__ __forceinline__ bool ix_beats(float av, int ai, float bv, int bi, int sentinel) {
@@ -156,56 +158,98 @@ extern "C" int ix_moe_router_topk(const float* logits, long ld, long T, long E, 
 }
 
 // ---------------------------------------------------------------------------------------------
-// Permutation (integer only). Token tiles of 256; thread e of a tile walks the tile's (token,
-// slot) pairs in order, so each expert's rows come out token-ascending with no atomics.
+// Permutation (integer only). Token tiles of 256. Per tile and expert, a 256-bit membership mask
+// is built in LDS with integer OR (order-free, so the mask is the same in any execution order);
+// a row's position inside its expert's segment is then a popcount of the mask below the token,
+// which makes every expert's rows token-ascending without any ordered loop or counter.
+__device__ __forceinline__ void ix_moe_build_masks(const int* __restrict__ topk_idx, int t0, int nt, int E, int k,
+                                                   uint32_t* s_mask /* [E][8] */, int* s_idx /* [256][k] */) {
+  for (int i = threadIdx.x; i < E * 8; i += 256) s_mask[i] = 0u;
+  for (int i = threadIdx.x; i < nt * k; i += 256) s_idx[i] = topk_idx[(long)t0 * k + i];
+  __syncthreads();
+  const int t = threadIdx.x;
+  if (t < nt) {
+    for (int j = 0; j < k; ++j) {
+      const int e = s_idx[t * k + j];
+      atomicOr(&s_mask[e * 8 + (t >> 5)], 1u << (t & 31));
+    }
+  }
+  __syncthreads();
+}
+
 __global__ __launch_bounds__(256) void k_moe_tile_counts(const int* __restrict__ topk_idx, int T, int E, int k,
                                                          int* __restrict__ tile_counts) {
   __shared__ int s_idx[IX_MOE_TILE_T * IX_MOE_KMAX];
+  __shared__ uint32_t s_mask[IX_MOE_EMAX * 8];
   const int tile = blockIdx.x;
   const int t0 = tile * IX_MOE_TILE_T;
   const int nt = min(IX_MOE_TILE_T, T - t0);
-  for (int i = threadIdx.x; i < nt * k; i += 256) s_idx[i] = topk_idx[(long)t0 * k + i];
-  __syncthreads();
+  ix_moe_build_masks(topk_idx, t0, nt, E, k, s_mask, s_idx);
   for (int e = threadIdx.x; e < E; e += 256) {
     int c = 0;
-    for (int i = 0; i < nt * k; ++i) c += (s_idx[i] == e);
+#pragma unroll
+    for (int w = 0; w < 8; ++w) c += __popc(s_mask[e * 8 + w]);
     tile_counts[(long)tile * E + e] = c;
   }
 }
 
 // meta layout: [0] = number of m-tiles, then tile_expert[max_tiles], tile_row0[max_tiles],
-// tile_nrows[max_tiles].
+// tile_nrows[max_tiles]. One workgroup: per-expert running sums over the token tiles (staged
+// through LDS 64 tiles at a time), an exclusive scan over the experts in LDS, then every expert
+// writes its own row tiles.
 __global__ __launch_bounds__(256) void k_moe_offsets(const int* __restrict__ tile_counts, int ntiles, int E,
                                                      int BM, int max_tiles, int* __restrict__ tile_base,
                                                      int* __restrict__ counts, int* __restrict__ offsets,
                                                      int* __restrict__ meta) {
-  for (int e = threadIdx.x; e < E; e += 256) {
-    int run = 0;
-    for (int tile = 0; tile < ntiles; ++tile) {
-      tile_base[(long)tile * E + e] = run;
-      run += tile_counts[(long)tile * E + e];
+  __shared__ int s_stage[IX_MOE_SCAN_TILES * IX_MOE_EMAX];
+  __shared__ int s_cnt[IX_MOE_EMAX], s_off[IX_MOE_EMAX + 1], s_toff[IX_MOE_EMAX + 1];
+  const int tid = threadIdx.x;
+  for (int e = tid; e < E; e += 256) s_cnt[e] = 0;
+  __syncthreads();
+  for (int t0 = 0; t0 < ntiles; t0 += IX_MOE_SCAN_TILES) {
+    const int nt = min(IX_MOE_SCAN_TILES, ntiles - t0);
+    for (int i = tid; i < nt * E; i += 256) s_stage[i] = tile_counts[(long)t0 * E + i];
+    __syncthreads();
+    for (int e = tid; e < E; e += 256) {
+      int run = s_cnt[e];
+      for (int t = 0; t < nt; ++t) {
+        const int c = s_stage[t * E + e];
+        s_stage[t * E + e] = run;
+        run += c;
+      }
+      s_cnt[e] = run;
     }
-    counts[e] = run;
+    __syncthreads();
+    for (int i = tid; i < nt * E; i += 256) tile_base[(long)t0 * E + i] = s_stage[i];
+    __syncthreads();
+  }
+  if (tid == 0) {
+    int run = 0, trun = 0;
+    for (int e = 0; e < E; ++e) {
+      s_off[e] = run;
+      s_toff[e] = trun;
+      run += s_cnt[e];
+      trun += (s_cnt[e] + BM - 1) / BM;
+    }
+    s_off[E] = run;
+    s_toff[E] = trun;
+    offsets[E] = run;
+    meta[0] = min(trun, max_tiles);
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int run = 0, nt = 0;
-    int* tile_expert = meta + 1;
-    int* tile_row0 = tile_expert + max_tiles;
-    int* tile_nrows = tile_row0 + max_tiles;
-    for (int e = 0; e < E; ++e) {
-      offsets[e] = run;
-      const int c = counts[e];
-      for (int r0 = 0; r0 < c && nt < max_tiles; r0 += BM) {
-        tile_expert[nt] = e;
-        tile_row0[nt] = run + r0;
-        tile_nrows[nt] = min(BM, c - r0);
-        ++nt;
-      }
-      run += c;
+  int* tile_expert = meta + 1;
+  int* tile_row0 = tile_expert + max_tiles;
+  int* tile_nrows = tile_row0 + max_tiles;
+  for (int e = tid; e < E; e += 256) {
+    const int c = s_cnt[e];
+    counts[e] = c;
+    offsets[e] = s_off[e];
+    int nt = s_toff[e];
+    for (int r0 = 0; r0 < c && nt < max_tiles; r0 += BM, ++nt) {
+      tile_expert[nt] = e;
+      tile_row0[nt] = s_off[e] + r0;
+      tile_nrows[nt] = min(BM, c - r0);
     }
-    offsets[E] = run;
-    meta[0] = nt;
   }
 }
 
@@ -216,30 +260,24 @@ __global__ __launch_bounds__(256) void k_moe_scatter(const int* __restrict__ top
                                                      float* __restrict__ permuted_prob,
                                                      int* __restrict__ combine_rows) {
   __shared__ int s_idx[IX_MOE_TILE_T * IX_MOE_KMAX];
-  __shared__ float s_prob[IX_MOE_TILE_T * IX_MOE_KMAX];
+  __shared__ uint32_t s_mask[IX_MOE_EMAX * 8];
   const int tile = blockIdx.x;
   const int t0 = tile * IX_MOE_TILE_T;
   const int nt = min(IX_MOE_TILE_T, T - t0);
-  for (int i = threadIdx.x; i < nt * k; i += 256) {
-    s_idx[i] = topk_idx[(long)t0 * k + i];
-    s_prob[i] = topk_prob[(long)t0 * k + i];
-  }
-  __syncthreads();
-  for (int e = threadIdx.x; e < E; e += 256) {
-    int pos = offsets[e] + tile_base[(long)tile * E + e];
-    for (int tt = 0; tt < nt; ++tt) {
-      for (int j = 0; j < k; ++j) {
-        if (s_idx[tt * k + j] == e) {
-          int rank = 0;
-          for (int j2 = 0; j2 < k; ++j2) rank += (s_idx[tt * k + j2] < e);
-          const long t = t0 + tt;
-          sorted_token[pos] = (int)t;
-          permuted_prob[pos] = s_prob[tt * k + j];
-          combine_rows[t * k + rank] = pos;
-          ++pos;
-        }
-      }
-    }
+  ix_moe_build_masks(topk_idx, t0, nt, E, k, s_mask, s_idx);
+  const int t = threadIdx.x;
+  if (t >= nt) return;
+  const long tg = t0 + t;
+  for (int j = 0; j < k; ++j) {
+    const int e = s_idx[t * k + j];
+    int local = __popc(s_mask[e * 8 + (t >> 5)] & ((1u << (t & 31)) - 1u));
+    for (int w = 0; w < (t >> 5); ++w) local += __popc(s_mask[e * 8 + w]);
+    int rank = 0;
+    for (int j2 = 0; j2 < k; ++j2) rank += (s_idx[t * k + j2] < e);
+    const int pos = offsets[e] + tile_base[(long)tile * E + e] + local;
+    sorted_token[pos] = (int)tg;
+    permuted_prob[pos] = topk_prob[tg * k + j];
+    combine_rows[tg * k + rank] = pos;
   }
 }
 
@@ -266,6 +304,7 @@ extern "C" int ix_moe_permute(const int* topk_idx, const float* topk_prob, long 
       !tile_meta || !scratch)
     return IX_ERR_ARG;
   if (T < 0 || E <= 0 || k <= 0 || k > IX_MOE_KMAX || BM <= 0) return IX_ERR_ARG;
+  if (E > IX_MOE_EMAX) return IX_DECLINED;
   if (max_tiles < ix_moe_max_tiles(T, k, E, BM)) return IX_ERR_ARG;
   if (T * k > 0x7fffffffL) return IX_DECLINED;
   hipStream_t st = (hipStream_t)stream;

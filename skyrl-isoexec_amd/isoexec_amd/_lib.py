@@ -39,16 +39,21 @@ SIGNATURES = {
     "ix_logprob_workspace_bytes": (c_size_t, [c_long, c_long, c_int]),
     "ix_logprob_rowinv_sampled": (
         c_int,
-        [P, c_int, c_long, c_long, c_long, P, c_int, P, P, P, c_size_t, c_int, P],
+        [P, c_int, c_long, c_long, c_long, P, c_int, P, P, P, c_size_t, c_int, P, P],
     ),
     "ix_logprob_rowinv_full": (
         c_int,
-        [P, c_int, c_long, c_long, c_long, c_int, P, c_long, P, P, c_size_t, c_int, P],
+        [P, c_int, c_long, c_long, c_long, c_int, P, c_long, P, P, c_size_t, c_int, P, P],
     ),
+    "ix_rowmax_reduce": (c_int, [P, c_long, c_long, c_long, P, P]),
     "ix_rmsnorm_gamma": (c_int, [P, P, P, c_long, c_long, c_float, c_int, P]),
     "ix_gated_out_norm": (c_int, [P, P, c_long, P, P, c_long, c_long, c_long, c_float, c_int, P]),
     "ix_add_rmsnorm_gamma": (c_int, [P, P, P, P, P, c_long, c_long, c_float, c_int, P]),
-    "ix_gemm_bf16_nt": (c_int, [P, c_long, P, c_long, P, P, c_long, c_long, c_long, c_long, c_int, P]),
+    "ix_gemm_bf16_nt": (
+        c_int,
+        [P, c_long, P, c_long, P, P, c_int, c_long, c_long, c_long, c_long, c_int, P, c_long, P],
+    ),
+    "ix_gemm_bf16_n_tiles": (c_long, [c_long, c_long, c_int]),
     "ix_gemm_f32_nt": (c_int, [P, c_int, c_long, P, c_long, P, c_long, c_long, c_long, c_long, P]),
     "ix_gdn_scan": (
         c_int,

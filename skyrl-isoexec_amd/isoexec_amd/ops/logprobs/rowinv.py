@@ -85,9 +85,11 @@ def _workspace(rows: int, vocab: int, g: int, device) -> torch.Tensor:
     return torch.empty(max(n, 4) // 4, dtype=torch.float32, device=device)
 
 
-def sampled_forward(x: torch.Tensor, t: torch.Tensor, g: int, *, force_shape: int = 0):
-    """Kernel call on a 2-D ``[rows, V]`` matrix. Returns ``(logprob [rows], lse [rows])``."""
-    _lib.require_device(x, t)
+def sampled_forward(x: torch.Tensor, t: torch.Tensor, g: int, *, force_shape: int = 0,
+                    row_max: torch.Tensor | None = None):
+    """Kernel call on a 2-D ``[rows, V]`` matrix. Returns ``(logprob [rows], lse [rows])``.
+    ``row_max`` (fp32 ``[rows]``, each row's exact maximum) lets the kernel skip its max pass."""
+    _lib.require_device(x, t, row_max)
     rows, vocab = x.shape
     t64 = t.to(torch.int64).contiguous()
     out = torch.empty(rows, dtype=torch.float32, device=x.device)
@@ -96,7 +98,8 @@ def sampled_forward(x: torch.Tensor, t: torch.Tensor, g: int, *, force_shape: in
     rc = _lib.check(
         _lib.lib().ix_logprob_rowinv_sampled(
             x.data_ptr(), _lib.dtype_code(x.dtype), rows, vocab, x.stride(0), t64.data_ptr(), g, out.data_ptr(),
-            lse.data_ptr(), ws.data_ptr(), ws.numel() * 4, force_shape, _lib.current_stream(x.device)),
+            lse.data_ptr(), ws.data_ptr(), ws.numel() * 4, force_shape, _lib.ptr(row_max),
+            _lib.current_stream(x.device)),
         "ix_logprob_rowinv_sampled")
     if rc != _lib.IX_OK:
         return None, None
@@ -111,7 +114,7 @@ def full_forward(x: torch.Tensor, g: int, *, force_shape: int = 0):
     rc = _lib.check(
         _lib.lib().ix_logprob_rowinv_full(
             x.data_ptr(), _lib.dtype_code(x.dtype), rows, vocab, x.stride(0), g, out.data_ptr(), out.stride(0),
-            None, ws.data_ptr(), ws.numel() * 4, force_shape, _lib.current_stream(x.device)),
+            None, ws.data_ptr(), ws.numel() * 4, force_shape, None, _lib.current_stream(x.device)),
         "ix_logprob_rowinv_full")
     return out if rc == _lib.IX_OK else None
 
@@ -211,3 +214,22 @@ def rowinv_full_logprobs(
     _S["tokens"] += rows
     _S["full_rows"] += rows
     return out
+
+
+def dense_head_logprobs(hidden: torch.Tensor, norm_weight: torch.Tensor, lm_head: torch.Tensor,
+                        target: torch.Tensor, *, eps: float = 1e-6, zero_centered: bool = True, g: int | None = None,
+                        tile: int = 0):
+    """Final norm -> LM head -> sampled logprobs for ``hidden [M, H]`` (the tail of both the trainer
+    scoring forward and the engine's ``compute_logits`` + logprob hook). The GEMM epilogue hands the
+    row maxima to the log-softmax kernel, so the bf16 logits are written once and read once. Same
+    bits as calling the three ops separately. Returns ``(logprob [M], logits [M, V])``."""
+    from ..mm.mm_hip import linear_nt
+    from ..norms.fused_outnorm import fused_rms_norm_gamma
+
+    x = fused_rms_norm_gamma(hidden, norm_weight, eps, zero_centered=zero_centered)
+    got = linear_nt(x, lm_head, tile=tile, want_row_max=True)
+    if got is None:
+        raise RuntimeError("[isoexec-amd] LM-head GEMM declined")
+    logits, row_max = got
+    lp, _ = sampled_forward(logits, target, g or leaves(), row_max=row_max)
+    return lp, logits

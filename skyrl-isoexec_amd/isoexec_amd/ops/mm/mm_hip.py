@@ -20,8 +20,13 @@ def stats() -> dict:
     return dict(_COUNTS)
 
 
-def linear_nt(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *, tile: int = 0):
-    """``x [M, K] @ weight [N, K]^T (+ bias)``, bf16 in/out, fp32 accumulate; ``None`` if declined."""
+def linear_nt(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *, tile: int = 0,
+              out_dtype: torch.dtype = torch.bfloat16, want_row_max: bool = False):
+    """``x [M, K] @ weight [N, K]^T (+ bias)``, bf16 operands, fp32 accumulate; ``None`` if declined.
+
+    ``out_dtype=torch.float32`` returns the fp32 accumulator unrounded. ``want_row_max`` also returns
+    each row's exact maximum over the N outputs (taken in the kernel's epilogue), as ``(out, row_max)``.
+    """
     _lib.require_device(x, weight, bias)
     if x.dtype is not torch.bfloat16 or weight.dtype is not torch.bfloat16:
         return None
@@ -31,14 +36,38 @@ def linear_nt(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None =
         return None
     m, k = x.shape
     n = weight.shape[0]
-    out = torch.empty(m, n, dtype=torch.bfloat16, device=x.device)
+    out = torch.empty(m, n, dtype=out_dtype, device=x.device)
     if bias is not None and (bias.dtype is not torch.bfloat16 or not bias.is_contiguous()):
         return None
+    L = _lib.lib()
+    parts = None
+    n_parts = 0
+    if want_row_max:
+        n_parts = int(L.ix_gemm_bf16_n_tiles(m, n, tile))
+        parts = torch.empty(m, n_parts, dtype=torch.float32, device=x.device)
+    stream = _lib.current_stream(x.device)
     rc = _lib.check(
-        _lib.lib().ix_gemm_bf16_nt(x.data_ptr(), x.stride(0), weight.data_ptr(), weight.stride(0), _lib.ptr(bias),
-                                   out.data_ptr(), out.stride(0), m, n, k, tile, _lib.current_stream(x.device)),
-        "ix_gemm_bf16_nt")
-    return out if rc == _lib.IX_OK else None
+        L.ix_gemm_bf16_nt(x.data_ptr(), x.stride(0), weight.data_ptr(), weight.stride(0), _lib.ptr(bias),
+                          out.data_ptr(), _lib.dtype_code(out_dtype), out.stride(0), m, n, k, tile,
+                          _lib.ptr(parts), n_parts, stream), "ix_gemm_bf16_nt")
+    if rc != _lib.IX_OK:
+        return None
+    if not want_row_max:
+        return out
+    row_max = torch.empty(m, dtype=torch.float32, device=x.device)
+    if m:
+        _lib.check(L.ix_rowmax_reduce(parts.data_ptr(), n_parts, n_parts, m, row_max.data_ptr(), stream),
+                   "ix_rowmax_reduce")
+    return out, row_max
+
+
+def router_gemm(x: torch.Tensor, weight: torch.Tensor):
+    """Router gating logits in fp32. A bf16 router weight (exactly what an fp32 cast of a bf16
+    checkpoint holds) multiplies exactly in the bf16 MFMA and is accumulated in fp32, so the bf16
+    core with an fp32 store IS the fp32 gating product; an fp32 weight takes the fp32 kernel."""
+    if weight.dtype is torch.bfloat16 and x.dtype is torch.bfloat16:
+        return linear_nt(x, weight, out_dtype=torch.float32)
+    return linear_f32_nt(x, weight.float())
 
 
 def linear_f32_nt(x: torch.Tensor, weight: torch.Tensor):

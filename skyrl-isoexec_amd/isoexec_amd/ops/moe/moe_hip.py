@@ -12,7 +12,7 @@ from __future__ import annotations
 import torch
 
 from ... import _lib
-from ..mm.mm_hip import linear_f32_nt
+from ..mm.mm_hip import router_gemm
 
 
 def router_topk(logits: torch.Tensor, k: int, *, pre_softmax: bool = False, scaling_factor: float | None = None,
@@ -126,7 +126,7 @@ def moe_ffn_forward(x: torch.Tensor, router_weight: torch.Tensor, w1: torch.Tens
                     pre_softmax: bool = False, logit_bias: torch.Tensor | None = None,
                     scaling_factor: float | None = None, fp32_combine: bool = False, BM: int | None = None):
     """Router GEMM (fp32) -> top-k -> permutation -> grouped experts -> combine. ``x [T, H]`` bf16."""
-    logits = linear_f32_nt(x, router_weight.float())
+    logits = router_gemm(x, router_weight)
     if logits is None:
         raise RuntimeError("[isoexec-amd] router GEMM declined")
     if logit_bias is not None:

@@ -89,14 +89,14 @@ def test_moe_ffn_parity_and_batch_invariance(dprims):
     """Reduced config 3 (hidden 256, 16 experts, top-4, inter 128): the full chain against the
     oracle (device router logits fed to the oracle so the discrete choice is compared like for
     like), then every token alone == co-batched == co-batched under skewed routing, for every BM."""
-    from isoexec_amd.ops.mm.mm_hip import linear_f32_nt
+    from isoexec_amd.ops.mm.mm_hip import router_gemm
     from isoexec_amd.ops.moe.moe_hip import combine, experts_forward, moe_ffn_forward, permute, router_topk
 
     T, H, E, F, k = 300, 256, 16, 128, 4
     x, wr, w1, w2 = make_moe(T, H, E, F, seed=1)
     xd, wrd, w1d, w2d = (t.to(DEV) for t in (x, wr, w1, w2))
     for mode in (0, 1):
-        logits = linear_f32_nt(xd, wrd.float())
+        logits = router_gemm(xd, wrd)
         idx, prob, _, _ = router_topk(logits, k, pre_softmax=bool(mode))
         p = permute(idx, prob, E)
         eo = experts_forward(xd, w1d, w2d, p)
