@@ -51,24 +51,14 @@ __global__ __launch_bounds__(WM* WN * 64) void k_gemm_bf16_nt(const bf16_t* __re
   const int n_valid = (int)min((long)BN, (long)N - n0);
 
   // Tile-local buffer descriptors: rows past the matrix fall outside the range and read as 0.
-  const __amdgpu_buffer_rsrc_t x_rsrc = ix_make_rsrc(A + m0 * lda, (uint32_t)(((long)(m_valid - 1) * lda + K) * 2));
-  const __amdgpu_buffer_rsrc_t w_rsrc = ix_make_rsrc(W + n0 * ldw, (uint32_t)(((long)(n_valid - 1) * ldw + K) * 2));
-  const int kc = ix_fetch_kchunk();
-  uint32_t x_voff[Cfg::X_CH], w_voff[Cfg::W_CH];
-#pragma unroll
-  for (int j = 0; j < Cfg::X_CH; ++j) {
-    const int r = ix_fetch_row<Cfg>(j);
-    x_voff[j] = (r < m_valid) ? (uint32_t)(r * lda * 2 + kc * 16) : IX_OOB;
-  }
-#pragma unroll
-  for (int j = 0; j < Cfg::W_CH; ++j) {
-    const int r = ix_fetch_row<Cfg>(j);
-    w_voff[j] = (r < n_valid) ? (uint32_t)(r * ldw * 2 + kc * 16) : IX_OOB;
-  }
+  const ix_rsrc_t x_rsrc = ix_make_rsrc(A + m0 * lda, (uint32_t)(((long)(m_valid - 1) * lda + K) * 2));
+  const ix_rsrc_t w_rsrc = ix_make_rsrc(W + n0 * ldw, (uint32_t)(((long)(n_valid - 1) * ldw + K) * 2));
+  auto x_row = [&](int r) -> uint32_t { return (r < m_valid) ? (uint32_t)(r * lda * 2) : IX_OOB; };
+  auto w_row = [&](int r) -> uint32_t { return (r < n_valid) ? (uint32_t)(r * ldw * 2) : IX_OOB; };
 
   ix_f32x16 acc[Cfg::MI][Cfg::NI];
   ix_acc_zero<Cfg>(acc);
-  ix_gemm_mainloop<Cfg>(x_rsrc, x_voff, w_rsrc, w_voff, K, ix_lds, acc);
+  ix_gemm_mainloop<Cfg>(x_rsrc, x_row, w_rsrc, w_row, K, ix_lds, acc);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WN, wn = wave % WN;
@@ -158,6 +148,7 @@ static int ix_gemm_bf16_dispatch(const bf16_t* a, long lda, const bf16_t* w, lon
     case 1: return ix_gemm_bf16_launch<32, 256, 1, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
     case 2: return ix_gemm_bf16_launch<128, 128, 2, 2, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
     case 3: return ix_gemm_bf16_launch<256, 256, 2, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
+    case 4: return ix_gemm_bf16_launch<256, 256, 2, 2, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
     case 5: return ix_gemm_bf16_launch<128, 256, 2, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
     default: return IX_ERR_ARG;
   }
@@ -172,7 +163,7 @@ extern "C" int ix_gemm_bf16_nt(const void* A, long lda, const void* W, long ldw,
   // 16-byte row chunks: every row start and K itself must be a multiple of 8 elements.
   if ((K % 8) || (lda % 8) || (ldw % 8) || !ix_aligned(A, 16) || !ix_aligned(W, 16)) return IX_DECLINED;
   if (M > 0x7fffffffL || N > 0x7fffffffL || K > 0x7fffffffL) return IX_DECLINED;
-  if (lda * 2 * 256 >= 0x7fffffffL || ldw * 2 * 256 >= 0x7fffffffL) return IX_DECLINED;  // 32-bit tile offsets
+  if (lda * 2 * 256 >= 0x40000000L || ldw * 2 * 256 >= 0x40000000L) return IX_DECLINED;  // tile offsets < 1 GiB
   if (M == 0) return IX_OK;
   hipStream_t st = (hipStream_t)stream;
   const bf16_t *a = (const bf16_t*)A, *w = (const bf16_t*)W, *b = (const bf16_t*)bias;

@@ -16,9 +16,9 @@
 // "sequential over MMA k-steps" (ops/collectives/pik/csrc/fused_leaftree.cu:12-19).
 //
 // Data movement: operand tiles go HBM -> LDS directly (buffer_load ... lds, 16 bytes per lane, no
-// register staging), two LDS stages, one barrier per k-tile. Out-of-range rows and the K tail
-// are handled by the buffer descriptor's range check (they read as zero), so the loop has no
-// branches.
+// register staging) through a ring of LDS stages, one barrier per stage. Out-of-range rows and
+// the K tail are handled by the buffer descriptor's range check (they read as zero), so the loop
+// has no branches.
 #pragma once
 #include "ix_common.h"
 
@@ -27,11 +27,17 @@ typedef __attribute__((ext_vector_type(16))) float ix_f32x16;
 typedef __attribute__((address_space(3))) void ix_lds_void;
 
 #define IX_BK 64
-#define IX_OOB 0xFFFFFF00u  // a byte offset no buffer descriptor here admits
+#define IX_OOB 0x7FFFF000u  // a byte offset no buffer descriptor here admits (all are < 1 GiB)
 
-// LDS tile: [rows][64] bf16, row pitch 128 B; 16-byte chunk c of row r lives at slot c ^ (r & 7),
-// so the MFMA fragment reads (32 consecutive rows, one chunk) spread over all banks.
-__device__ __forceinline__ int ix_lds_off(int row, int chunk) { return row * 128 + ((chunk ^ (row & 7)) << 4); }
+// LDS tiles are [rows][k] bf16 with the 16-byte chunks of a row permuted by an XOR swizzle so that
+// an MFMA fragment read (32 consecutive rows, one chunk per lane group) spreads over the banks:
+//   full k-tile, row pitch 128 B: chunk c of row r at slot c ^ ix_swz8(r)
+//   half k-tile, row pitch  64 B: chunk c of row r at slot c ^ ix_swz4(r)
+// The two functions were picked by measuring ds_read_b128 throughput on gfx950 for every XOR of two
+// shifts of r: these reach ~188 B/clk/CU, where r&7 / no swizzle reach 118 / 32 (full) and 63 (half).
+__device__ __forceinline__ int ix_swz8(int r) { return (r >> 1) & 7; }
+__device__ __forceinline__ int ix_swz4(int r) { return (r >> 3) & 3; }
+__device__ __forceinline__ int ix_lds_off(int row, int chunk) { return row * 128 + ((chunk ^ ix_swz8(row)) << 4); }
 
 // Register i of lane l of a 32x32 accumulator holds result row (i/4)*8 + (l/32)*4 + (i%4)
 // (a weight row, i.e. an output column n) and result column l%32 (a token m).
@@ -46,57 +52,106 @@ struct IxGemmCfg {
   static constexpr int X_CH = BM * 8 / NT;  // 16-byte chunks fetched per thread per k-tile
   static constexpr int W_CH = BN * 8 / NT;
   static constexpr int STAGE_BYTES = (BM + BN) * 128;
-  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+  // Pipeline: a ring of four half-k-tile stages when the half-stage fetch divides evenly over the
+  // threads, else a ring of FULL_STAGES whole-k-tile stages (the 32-row decode tile).
+#ifdef IX_EXPERIMENT_FULL2
+  static constexpr bool HALF_RING = false;
+  static constexpr int FULL_STAGES = (BM + BN) * 128 * 3 <= 160 * 1024 ? 3 : 2;
+#else
+  static constexpr bool HALF_RING = ((BM * 4) % NT == 0) && ((BN * 4) % NT == 0);
+  static constexpr int FULL_STAGES = 3;
+#endif
+#ifndef IX_HALF_STAGES_MAX
+#define IX_HALF_STAGES_MAX 5
+#endif
+  // as many half-stages as fit in the 160 KiB of LDS, at most IX_HALF_STAGES_MAX, at least 4
+  static constexpr int HALF_STAGES =
+      (IX_HALF_STAGES_MAX * (STAGE_BYTES / 2) <= 160 * 1024) ? IX_HALF_STAGES_MAX : 4;
+  static constexpr int LDS_BYTES = HALF_RING ? HALF_STAGES * (STAGE_BYTES / 2) : FULL_STAGES * STAGE_BYTES;
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile must be MFMA multiples");
   static_assert((BM * 8) % NT == 0 && (BN * 8) % NT == 0, "fetch must divide evenly");
-  static_assert(NT % 64 == 0 && (NT / 8) % 8 == 0, "a thread's k-chunk must not depend on the fetch index");
+  static_assert(NT % 64 == 0, "whole waves");
 };
 
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t ix_make_rsrc(const void* base, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), (short)0, (int)bytes, 0x00020000);
+// Raw buffer descriptor (stride 0): base, size in bytes, dword 3 = 32-bit untyped data format.
+typedef __attribute__((ext_vector_type(4))) int ix_rsrc_t;
+__device__ __forceinline__ ix_rsrc_t ix_make_rsrc(const void* base, uint32_t bytes) {
+  const uint64_t b = reinterpret_cast<uint64_t>(base);
+  ix_rsrc_t r;
+  r.x = __builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+  r.y = __builtin_amdgcn_readfirstlane((int)(uint32_t)((b >> 32) & 0xffffu));
+  r.z = __builtin_amdgcn_readfirstlane((int)bytes);
+  r.w = 0x00020000;
+  return r;
 }
 
-// Thread t fetches LDS chunk q = t + j*NT of each operand tile: tile row q/8, slot q%8, which
-// holds k-chunk (q%8) ^ (row&7). These helpers give the row and the byte offset of that chunk
-// inside a row; the caller turns the row into a buffer offset (or IX_OOB for a missing row).
-template <typename Cfg>
-__device__ __forceinline__ int ix_fetch_row(int j) { return (threadIdx.x + j * Cfg::NT) >> 3; }
-__device__ __forceinline__ int ix_fetch_kchunk() { return (threadIdx.x & 7) ^ ((threadIdx.x >> 3) & 7); }
+// 16 bytes per lane, memory -> LDS without passing through registers: lane l's data lands at LDS
+// byte address lds_addr + 16*l (lds_addr wave-uniform, carried in M0). Written as inline assembly so
+// that the compiler does not count these loads: it would otherwise force "all loads done" before
+// every LDS read, and the ring of stages below relies on waiting only for the oldest group
+// (explicit s_waitcnt vmcnt(N); vector loads retire in order).
+__device__ __forceinline__ void ix_dma16(ix_rsrc_t rsrc, uint32_t lds_addr, uint32_t voff, int soff) {
+#ifdef IX_EXPERIMENT_NO_DMA
+  return;
+#endif
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t ix_lds_addr(const char* p) {
+  return (uint32_t)reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) char*)p);
+}
 
-// Main loop. x_voff[j] / w_voff[j]: byte offset (row start + this thread's k-chunk) of fetch j
-// into the activation / weight buffer, or IX_OOB. acc[mi][ni]: tokens mi*32.., outputs ni*32..
-template <typename Cfg, typename XOff, typename WOff, typename Acc>
-__device__ __forceinline__ void ix_gemm_mainloop(__amdgpu_buffer_rsrc_t x_rsrc, const XOff& x_voff,
-                                                 __amdgpu_buffer_rsrc_t w_rsrc, const WOff& w_voff, int K,
-                                                 char* lds, Acc& acc) {
-  constexpr int NT = Cfg::NT, BM = Cfg::BM;
+// s_waitcnt immediate for "at most N vector-memory operations outstanding" (expcnt, lgkmcnt unconstrained).
+#define IX_VMCNT(N) (((N) & 15) | (((N) >> 4) << 14) | 0x0F70)
+
+// ---- pipeline A: a ring of FULL_STAGES stages, one full k-tile (64) each --------------------------
+// Thread t fetches LDS chunk q = t + j*NT of each operand tile: tile row q/8, slot q%8, which
+// holds k-chunk (q%8) ^ ix_swz8(row). Every iteration issues the same number of loads (past the end they
+// fall outside the buffer range), so "tile kt has landed" is one constant wait.
+template <typename Cfg, typename XRow, typename WRow, typename Acc>
+__device__ __forceinline__ void ix_gemm_mainloop_full(ix_rsrc_t x_rsrc, const XRow& x_row,
+                                                      ix_rsrc_t w_rsrc, const WRow& w_row, int K,
+                                                      char* lds, Acc& acc) {
+  constexpr int NT = Cfg::NT, BM = Cfg::BM, S = Cfg::FULL_STAGES;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
-  const int kc = ix_fetch_kchunk();
   const int KT = (K + IX_BK - 1) / IX_BK;
-  // stage layout: [X tile: BM rows][W tile: BN rows]
-  const int wave_chunk_byte = (wave * 64) * 16;
+  const uint32_t lds_base = __builtin_amdgcn_readfirstlane(ix_lds_addr(lds) + (wave * 64) * 16);
+  const int K2 = K * 2;
 
-  // Only the last k-tile can be partial; its out-of-range chunks are sent out of the buffer's range.
-  uint32_t x_last[Cfg::X_CH], w_last[Cfg::W_CH];
-  {
-    const bool kin = ((KT - 1) * IX_BK + kc * 8) < K;  // K % 8 == 0: a chunk is entirely in or out
+  // fetch j of this thread: tile row (tid + j*NT)/8, slot tid%8, i.e. k-chunk slot ^ swz8(row)
+  uint32_t x_voff[Cfg::X_CH], w_voff[Cfg::W_CH];
+  int x_kb[Cfg::X_CH], w_kb[Cfg::W_CH];
 #pragma unroll
-    for (int j = 0; j < Cfg::X_CH; ++j) x_last[j] = kin ? x_voff[j] : IX_OOB;
-#pragma unroll
-    for (int j = 0; j < Cfg::W_CH; ++j) w_last[j] = kin ? w_voff[j] : IX_OOB;
+  for (int j = 0; j < Cfg::X_CH; ++j) {
+    const int r = (tid + j * NT) >> 3;
+    x_kb[j] = ((tid & 7) ^ ix_swz8(r)) * 16;
+    x_voff[j] = x_row(r) + x_kb[j];
   }
-  auto fetch = [&](int kt, int stage, const uint32_t* xv, const uint32_t* wv) {
+#pragma unroll
+  for (int j = 0; j < Cfg::W_CH; ++j) {
+    const int r = (tid + j * NT) >> 3;
+    w_kb[j] = ((tid & 7) ^ ix_swz8(r)) * 16;
+    w_voff[j] = w_row(r) + w_kb[j];
+  }
+
+  auto issue = [&](int kt) {
     const int soff = kt * IX_BK * 2;
-    char* sbase = lds + stage * Cfg::STAGE_BYTES + wave_chunk_byte;
+    const uint32_t sbase = lds_base + (kt % S) * Cfg::STAGE_BYTES;
+    // chunks at or past K (the tail of the last tile, and whole tiles past the end) go out of range
 #pragma unroll
-    for (int j = 0; j < Cfg::X_CH; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (ix_lds_void*)(sbase + j * NT * 16), 16, xv[j], soff, 0, 0);
+    for (int j = 0; j < Cfg::X_CH; ++j) {
+      const uint32_t dead = (uint32_t)((K2 - 1 - (soff + x_kb[j])) >> 31) & IX_OOB;
+      ix_dma16(x_rsrc, sbase + j * NT * 16, x_voff[j] | dead, soff);
+    }
 #pragma unroll
-    for (int j = 0; j < Cfg::W_CH; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (ix_lds_void*)(sbase + BM * 128 + j * NT * 16), 16, wv[j],
-                                               soff, 0, 0);
+    for (int j = 0; j < Cfg::W_CH; ++j) {
+      const uint32_t dead = (uint32_t)((K2 - 1 - (soff + w_kb[j])) >> 31) & IX_OOB;
+      ix_dma16(w_rsrc, sbase + BM * 128 + j * NT * 16, w_voff[j] | dead, soff);
+    }
   };
 
   const int frow = lane & 31, fg = lane >> 5;
@@ -106,19 +161,17 @@ __device__ __forceinline__ void ix_gemm_mainloop(__amdgpu_buffer_rsrc_t x_rsrc, 
 #pragma unroll
   for (int ni = 0; ni < Cfg::NI; ++ni) w_foff[ni] = BM * 128 + ix_lds_off(wn * Cfg::TN + ni * 32 + frow, fg * 4);
 
-  if (KT == 1) fetch(0, 0, x_last, w_last); else fetch(0, 0, x_voff, w_voff);
+#pragma unroll
+  for (int p = 0; p < S - 1; ++p) issue(p);
   for (int kt = 0; kt < KT; ++kt) {
-    const int stage = kt & 1;
-    // tile kt has landed (it is the only fetch in flight) and everyone is done with stage^1
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+    __builtin_amdgcn_s_waitcnt(IX_VMCNT((S - 2) * (Cfg::X_CH + Cfg::W_CH)));
     __syncthreads();
-    if (kt + 2 < KT) fetch(kt + 1, stage ^ 1, x_voff, w_voff);
-    else if (kt + 1 < KT) fetch(kt + 1, stage ^ 1, x_last, w_last);
-    const char* sb = lds + stage * Cfg::STAGE_BYTES;
+    issue(kt + S - 1);  // into the stage consumed in iteration kt-1
+    const char* sb = lds + (kt % S) * Cfg::STAGE_BYTES;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       ix_bf16x8 xf[Cfg::MI], wf[Cfg::NI];
-      // chunk fg*4+s sits at slot (fg*4+s) ^ (row&7): flipping bits 0-1 of the chunk index flips
+      // chunk fg*4+s sits at slot (fg*4+s) ^ swz8(row): flipping bits 0-1 of the chunk index flips
       // the same bits of the slot, i.e. byte offset ^ (s << 4)
 #pragma unroll
       for (int mi = 0; mi < Cfg::MI; ++mi)
@@ -133,6 +186,119 @@ __device__ __forceinline__ void ix_gemm_mainloop(__amdgpu_buffer_rsrc_t x_rsrc, 
           acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[ni], xf[mi], acc[mi][ni], 0, 0, 0);
     }
   }
+  __builtin_amdgcn_s_waitcnt(IX_VMCNT(0));  // drain the out-of-range tail fetches before LDS is reused
+}
+
+// ---- pipeline B: a ring of HALF_STAGES (4 or 5) LDS stages of half a k-tile each ------------------
+// Half h of k-tile kt holds the 16-byte k-chunks {2h, 2h+1, 4+2h, 5+2h}: exactly what MFMA steps
+// s = 2h and 2h+1 consume (lane group 0: chunk s, lane group 1: chunk 4+s), so the K order of pipeline
+// A is kept while a fetch is issued three half-tiles ahead of its use. Row pitch 64 B; local chunk lc
+// of row r sits at slot lc ^ ((r>>1)&3). Every iteration issues the same number of loads (past the end
+// they fall outside the buffer range), so "all but the newest two groups have landed" is one constant.
+template <typename Cfg, typename XRow, typename WRow, typename Acc>
+__device__ __forceinline__ void ix_gemm_mainloop_h4(ix_rsrc_t x_rsrc, const XRow& x_row,
+                                                    ix_rsrc_t w_rsrc, const WRow& w_row, int K,
+                                                    char* lds, Acc& acc) {
+  constexpr int NT = Cfg::NT, BM = Cfg::BM, BN = Cfg::BN;
+  constexpr int XH = BM * 4 / NT, WH = BN * 4 / NT;  // loads per thread per half-stage
+  constexpr int HS = (BM + BN) * 64;                 // bytes per half-stage
+  static_assert(Cfg::HALF_RING && (NT / 4) % 32 == 0, "half-stage fetch must divide, swizzle independent of j");
+  constexpr int NS = Cfg::HALF_STAGES;               // ring length; fetches run NS-1 half-tiles ahead
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+  const int lc = (tid & 3) ^ ix_swz4(tid >> 2);         // local chunk this thread fetches (same for every j)
+  const int cb = ((lc & 1) | ((lc >> 1) << 2)) * 16;    // its byte offset in a row for half 0
+  const int NH = 2 * ((K + IX_BK - 1) / IX_BK);
+  const uint32_t lds_base = __builtin_amdgcn_readfirstlane(ix_lds_addr(lds) + (wave * 64) * 16);
+  const int K2 = K * 2;
+
+  uint32_t x_voff[XH], w_voff[WH];
+#pragma unroll
+  for (int j = 0; j < XH; ++j) x_voff[j] = x_row((tid + j * NT) >> 2) + cb;
+#pragma unroll
+  for (int j = 0; j < WH; ++j) w_voff[j] = w_row((tid + j * NT) >> 2) + cb;
+
+  auto issue = [&](int i) {
+    const int soff = (i >> 1) * (IX_BK * 2) + (i & 1) * 32;
+    // chunks at or past K (the tail of the last tile, and whole half-tiles past the end) go out of range
+    const uint32_t dead = (uint32_t)((K2 - 1 - (soff + cb)) >> 31) & IX_OOB;
+    const uint32_t sbase = lds_base + (i % NS) * HS;
+#pragma unroll
+    for (int j = 0; j < XH; ++j) ix_dma16(x_rsrc, sbase + j * NT * 16, x_voff[j] | dead, soff);
+#pragma unroll
+    for (int j = 0; j < WH; ++j) ix_dma16(w_rsrc, sbase + BM * 64 + j * NT * 16, w_voff[j] | dead, soff);
+  };
+
+  const int frow = lane & 31, fg = lane >> 5;
+  int x_foff[Cfg::MI], w_foff[Cfg::NI];
+#pragma unroll
+  for (int mi = 0; mi < Cfg::MI; ++mi) {
+    const int r = wm * Cfg::TM + mi * 32 + frow;
+    x_foff[mi] = r * 64 + (((fg * 2) ^ ix_swz4(r)) << 4);
+  }
+#pragma unroll
+  for (int ni = 0; ni < Cfg::NI; ++ni) {
+    const int r = wn * Cfg::TN + ni * 32 + frow;
+    w_foff[ni] = BM * 64 + r * 64 + (((fg * 2) ^ ix_swz4(r)) << 4);
+  }
+
+  // Software pipeline: the fragments of a step are read from LDS while the previous step's MFMAs
+  // run, and the wait + barrier that publishes the next half-tile sits between the two steps of an
+  // iteration, so its latency hides behind the second step's MFMAs.
+  ix_bf16x8 xa[Cfg::MI], wa[Cfg::NI], xb[Cfg::MI], wb[Cfg::NI];
+  auto frags = [&](const char* sb, int ls, ix_bf16x8* xf, ix_bf16x8* wf) {
+#pragma unroll
+    for (int mi = 0; mi < Cfg::MI; ++mi) xf[mi] = *reinterpret_cast<const ix_bf16x8*>(sb + (x_foff[mi] ^ (ls << 4)));
+#pragma unroll
+    for (int ni = 0; ni < Cfg::NI; ++ni) wf[ni] = *reinterpret_cast<const ix_bf16x8*>(sb + (w_foff[ni] ^ (ls << 4)));
+  };
+  auto mfmas = [&](const ix_bf16x8* xf, const ix_bf16x8* wf) {
+#ifdef IX_EXPERIMENT_NO_MFMA
+    asm volatile("" ::"v"(xf[0]), "v"(wf[0]));
+    return;
+#endif
+#pragma unroll
+    for (int mi = 0; mi < Cfg::MI; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < Cfg::NI; ++ni)
+        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[ni], xf[mi], acc[mi][ni], 0, 0, 0);
+  };
+
+#pragma unroll
+  for (int p = 0; p < NS - 1; ++p) issue(p);
+  __builtin_amdgcn_s_waitcnt(IX_VMCNT((NS - 2) * (XH + WH)));  // half-tile 0 has landed
+  __syncthreads();
+  frags(lds, 0, xa, wa);
+  for (int i = 0; i < NH; ++i) {
+    const char* sb = lds + (i % NS) * HS;
+    // sched_barrier(0): keep the compiler's scheduler from sinking the LDS reads below the MFMAs
+    frags(sb, 1, xb, wb);
+    __builtin_amdgcn_sched_barrier(0);
+    mfmas(xa, wa);
+    __builtin_amdgcn_sched_barrier(0);
+    // half-tile i+1 has landed once at most the NS-3 newer groups are still in flight; after the
+    // barrier every wave is past iteration i-1, whose stage the next fetch overwrites
+    __builtin_amdgcn_s_waitcnt(IX_VMCNT((NS - 3) * (XH + WH)));
+    __syncthreads();
+    issue(i + NS - 1);
+    frags(lds + ((i + 1) % NS) * HS, 0, xa, wa);
+    __builtin_amdgcn_sched_barrier(0);
+    mfmas(xb, wb);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  __builtin_amdgcn_s_waitcnt(IX_VMCNT(0));  // drain the out-of-range tail fetches before LDS is reused
+}
+
+// x_row(r) / w_row(r): byte offset of tile row r inside the operand's buffer, or IX_OOB.
+template <typename Cfg, typename XRow, typename WRow, typename Acc>
+__device__ __forceinline__ void ix_gemm_mainloop(ix_rsrc_t x_rsrc, const XRow& x_row,
+                                                 ix_rsrc_t w_rsrc, const WRow& w_row, int K, char* lds,
+                                                 Acc& acc) {
+  if constexpr (Cfg::HALF_RING)
+    ix_gemm_mainloop_h4<Cfg>(x_rsrc, x_row, w_rsrc, w_row, K, lds, acc);
+  else
+    ix_gemm_mainloop_full<Cfg>(x_rsrc, x_row, w_rsrc, w_row, K, lds, acc);
 }
 
 template <typename Cfg, typename Acc>

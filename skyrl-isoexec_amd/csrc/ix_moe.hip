@@ -345,25 +345,19 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc1_glu(const bf16_t* __res
   // activations: gathered token rows of x; weights: the expert's [2F, Hd] fc1 matrix with the
   // tile's rows interleaved so that each wave holds a gate tile (ni = 0) and its up tile (ni = 1):
   // tile row r -> wave r/64, half (r/32)&1, column n0h + 32*(r/64) + r%32.
-  const __amdgpu_buffer_rsrc_t x_rsrc = ix_make_rsrc(x, (uint32_t)(((long)(T - 1) * ldx + Hd) * 2));
-  const __amdgpu_buffer_rsrc_t w_rsrc = ix_make_rsrc(W1 + (long)e * 2 * F * Hd, (uint32_t)((long)2 * F * Hd * 2));
-  const int kc = ix_fetch_kchunk();
-  uint32_t x_voff[Cfg::X_CH], w_voff[Cfg::W_CH];
-#pragma unroll
-  for (int j = 0; j < Cfg::X_CH; ++j) {
-    const int r = ix_fetch_row<Cfg>(j);
-    x_voff[j] = (r < nrows) ? (uint32_t)((long)sorted_token[row0 + r] * ldx * 2 + kc * 16) : IX_OOB;
-  }
-#pragma unroll
-  for (int j = 0; j < Cfg::W_CH; ++j) {
-    const int r = ix_fetch_row<Cfg>(j);
+  const ix_rsrc_t x_rsrc = ix_make_rsrc(x, (uint32_t)(((long)(T - 1) * ldx + Hd) * 2));
+  const ix_rsrc_t w_rsrc = ix_make_rsrc(W1 + (long)e * 2 * F * Hd, (uint32_t)((long)2 * F * Hd * 2));
+  auto x_row = [&](int r) -> uint32_t {
+    return (r < nrows) ? (uint32_t)((long)sorted_token[row0 + r] * ldx * 2) : IX_OOB;
+  };
+  auto w_row = [&](int r) -> uint32_t {
     const int col = n0h + (r >> 6) * 32 + (r & 31);
-    w_voff[j] = (col < F) ? (uint32_t)(((long)((r >> 5) & 1) * F + col) * Hd * 2 + kc * 16) : IX_OOB;
-  }
+    return (col < F) ? (uint32_t)(((long)((r >> 5) & 1) * F + col) * Hd * 2) : IX_OOB;
+  };
 
   ix_f32x16 acc[Cfg::MI][2];
   ix_acc_zero<Cfg>(acc);
-  ix_gemm_mainloop<Cfg>(x_rsrc, x_voff, w_rsrc, w_voff, Hd, ix_lds, acc);
+  ix_gemm_mainloop<Cfg>(x_rsrc, x_row, w_rsrc, w_row, Hd, ix_lds, acc);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WN, wn = wave % WN;
@@ -407,24 +401,14 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc2(const bf16_t* __restric
   const long n0 = (long)nt * BN;
   const int n_valid = (int)min((long)BN, (long)Hd - n0);
 
-  const __amdgpu_buffer_rsrc_t x_rsrc = ix_make_rsrc(inter + row0 * F, (uint32_t)((long)nrows * F * 2));
-  const __amdgpu_buffer_rsrc_t w_rsrc = ix_make_rsrc(W2 + ((long)e * Hd + n0) * F, (uint32_t)((long)n_valid * F * 2));
-  const int kc = ix_fetch_kchunk();
-  uint32_t x_voff[Cfg::X_CH], w_voff[Cfg::W_CH];
-#pragma unroll
-  for (int j = 0; j < Cfg::X_CH; ++j) {
-    const int r = ix_fetch_row<Cfg>(j);
-    x_voff[j] = (r < nrows) ? (uint32_t)(r * F * 2 + kc * 16) : IX_OOB;
-  }
-#pragma unroll
-  for (int j = 0; j < Cfg::W_CH; ++j) {
-    const int r = ix_fetch_row<Cfg>(j);
-    w_voff[j] = (r < n_valid) ? (uint32_t)(r * F * 2 + kc * 16) : IX_OOB;
-  }
+  const ix_rsrc_t x_rsrc = ix_make_rsrc(inter + row0 * F, (uint32_t)((long)nrows * F * 2));
+  const ix_rsrc_t w_rsrc = ix_make_rsrc(W2 + ((long)e * Hd + n0) * F, (uint32_t)((long)n_valid * F * 2));
+  auto x_row = [&](int r) -> uint32_t { return (r < nrows) ? (uint32_t)(r * F * 2) : IX_OOB; };
+  auto w_row = [&](int r) -> uint32_t { return (r < n_valid) ? (uint32_t)(r * F * 2) : IX_OOB; };
 
   ix_f32x16 acc[Cfg::MI][Cfg::NI];
   ix_acc_zero<Cfg>(acc);
-  ix_gemm_mainloop<Cfg>(x_rsrc, x_voff, w_rsrc, w_voff, F, ix_lds, acc);
+  ix_gemm_mainloop<Cfg>(x_rsrc, x_row, w_rsrc, w_row, F, ix_lds, acc);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WN, wn = wave % WN;
@@ -481,7 +465,7 @@ extern "C" int ix_moe_experts(const void* x, long ldx, const int* sorted_token, 
     return IX_ERR_ARG;
   if (T < 0 || rows < 0 || Hd <= 0 || F <= 0 || max_tiles < 0 || ldx < Hd) return IX_ERR_ARG;
   // 32-bit buffer offsets: the activation matrix, one expert's weights and one row tile must fit
-  if (T * ldx * 2 >= 0x7fffffffL || 2 * F * Hd * 2 >= 0x7fffffffL || 256 * F * 2 >= 0x7fffffffL) return IX_DECLINED;
+  if (T * ldx * 2 >= 0x40000000L || 2 * F * Hd * 2 >= 0x40000000L || 256 * F * 2 >= 0x40000000L) return IX_DECLINED;
   if ((Hd % 8) || (F % 8) || (ldx % 8) || !ix_aligned(x, 16) || !ix_aligned(W1, 16) || !ix_aligned(W2, 16) ||
       !ix_aligned(inter, 16) || !ix_aligned(expert_out, 8))
     return IX_DECLINED;
