@@ -24,6 +24,9 @@ for p in (ROOT, os.path.join(ROOT, "skyrl-isoexec_amd")):
 
 PEAK_MFMA_BF16_TFLOPS = 2500.0  # MI355X dense bf16
 PEAK_HBM_GBS = 8000.0
+# HBM-side bytes per launch of the dominant kernels, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by
+# what the same counters read for a 1 GiB copy (x2.0 / x1.0); see profiles/*.txt. Workload-specific.
+MEASURED_TRAFFIC_BYTES = {"dense_head_M4096_gemm": 12.71e9, "gdn_decode_B256": 1.1016e9}
 
 
 class KernelTimer:
@@ -106,8 +109,9 @@ def dense_head(args):
         "config": {"workload": "dense_head: RMSNorm(4096) + LM head [151936,4096] + log-softmax/gather",
                    "tokens_per_step": M, "hidden": K, "vocab": V, "gemm_tile": args.tile},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_MFMA_BF16_TFLOPS, "traffic": None,
-                     "kernel": "k_gemm_bf16_nt", "kernel_ms": gemm_ms},
+                     "frac": achieved / PEAK_MFMA_BF16_TFLOPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES["dense_head_M4096_gemm"] if M == 4096 else None,
+                     "kernel": "k_gemm_bf16_nt (+ 7 us row-max reduce)", "kernel_ms": gemm_ms},
         "kernels_ms": {"rmsnorm": t_norm.mean_ms(), "gemm": gemm_ms, "logprob": lp_ms},
         "logprob_hbm": {"bound": "hbm", "achieved": M * V * 2 / (lp_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
                         "unit": "GB/s", "frac": M * V * 2 / (lp_ms * 1e-3) / 1e9 / PEAK_HBM_GBS},
@@ -176,7 +180,9 @@ def gdn_decode(args):
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
             "config": {"workload": f"gdn_decode B={B} HV=32 K=V=128 (state R+W 4 MiB/seq/step)"},
             "roofline": {"bound": "hbm", "achieved": by / (ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": by / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None, "kernel": "k_gdn_scan",
+                         "frac": by / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                         "traffic": MEASURED_TRAFFIC_BYTES["gdn_decode_B256"] if B == 256 else None,
+                         "kernel": "k_gdn_scan",
                          "kernel_ms": ms}}
 
 
