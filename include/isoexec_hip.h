@@ -129,7 +129,9 @@ int ix_gemm_f32_nt(const void* A, int a_dtype, long lda, const void* W, long ldw
  * q/k/v/beta/o share io_dtype. state_pool fp32 [rows, HV, V, K]. cu_seqlens int32
  * [N+1]. state_indices int32: pool row for (sequence n, token t) at [n*stride + t]; column 0
  * loads, a positive entry at column t stores after token t, row index <= 0 at column 0 skips
- * the sequence. HV % H == 0 (GQA: head hv reads q/k head hv / (HV/H)). K in {32,64,128,256}.
+ * the sequence. stride 0 is the compact form: state_indices [N] holds one row per sequence, loaded
+ * before its first token and stored once after its last. HV % H == 0 (GQA: head hv reads q/k
+ * head hv / (HV/H)). K in {32,64,128,256}.
  * time_tile: tokens staged per LDS fill (<= 64, 0 = default); does not change results. */
 int ix_gdn_scan(const void* q, const void* k, const void* v, const float* g, const void* beta, void* o,
                 int io_dtype, long q_pitch, long k_pitch, long v_pitch, float* state_pool,

@@ -86,7 +86,9 @@ __global__ __launch_bounds__(256) void k_gdn_scan(const TIO* __restrict__ q, con
   const int t_begin = cu[n], t_end = cu[n + 1];
   const int len = t_end - t_begin;
   if (len <= 0) return;
-  const int row0 = sidx[n * sidx_stride];
+  // Stride 0: one row per sequence, loaded at the first token and stored once after the last.
+  const long sbase = sidx_stride == 0 ? (long)n : (long)n * sidx_stride;
+  const int row0 = sidx[sbase];
   if (row0 <= 0) {  // null lane: no state, outputs defined as zero
     for (int i = tid; i < len * R; i += 256) {
       const int tt = i / R, rr = i % R;
@@ -120,7 +122,7 @@ __global__ __launch_bounds__(256) void k_gdn_scan(const TIO* __restrict__ q, con
       const long src = (long)(t_begin + t0 + i) * HV + hv;
       egf[i] = ix_exp(g[src]);
       btf[i] = ix_ld(beta + src);
-      sif[i] = sidx[n * sidx_stride + t0 + i];
+      sif[i] = sidx_stride == 0 ? (t0 + i == len - 1 ? row0 : 0) : sidx[sbase + t0 + i];
     }
     __syncthreads();
     for (int tt = 0; tt < nt; ++tt) {

@@ -54,7 +54,8 @@ def gdn_recurrent_kernel(
 
     ``q, k``: ``[B, T, H, K]`` already L2-normalised (H may be GQA-compressed: ``HV % H == 0``);
     ``v``: ``[B, T, HV, V]``; ``g`` (fp32), ``beta``: ``[B, T, HV]``; ``ssm_state`` fp32 pool
-    ``[S, HV, V, K]``; ``state_indices`` ``[N]`` (one-token decode) or ``[N, Tmax]``; ``cu_seqlens``
+    ``[S, HV, V, K]``; ``state_indices`` ``[N]`` (one row per sequence, stored after its last token) or ``[N, Tmax]``
+    (column 0 loads, a positive entry at column t stores after token t); ``cu_seqlens``
     ``[N+1]`` int32 for a packed batch (then ``B == 1``), ``None`` for ``[B, T, ...]``.
     """
     _lib.require_device(q, k, v, g, beta, ssm_state, state_indices, cu_seqlens)
@@ -83,8 +84,9 @@ def gdn_recurrent_kernel(
     bf = _flatten_tokens(beta, 1).to(io).contiguous()
     idx = state_indices.to(torch.int32)
     if idx.ndim == 1:
+        # One row per sequence: loaded before its first token, stored once after its last.
         idx = idx.contiguous()
-        idx_stride = 1
+        idx_stride = 0
     else:
         if idx.stride(1) != 1:
             idx = idx.contiguous()
