@@ -323,7 +323,8 @@ __global__ __launch_bounds__(256) void k_gdn_conv(const bf16_t* __restrict__ x, 
                                                   const bf16_t* __restrict__ pool, const int* __restrict__ cu,
                                                   const int* __restrict__ rows_in, int N, long D, int W,
                                                   int silu, long total) {
-  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  // Two grid dimensions: one dimension may not exceed 2^32 threads, and a packed prefill does.
+  const long i = ((long)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
   if (i >= total) return;
   const int t = (int)(i / D);
   const int d = (int)(i % D);
@@ -373,9 +374,11 @@ extern "C" int ix_gdn_conv(const void* x, const void* weight, const void* bias, 
   hipStream_t st = (hipStream_t)stream;
   const long total = total_tokens * D;
   if (total > 0 && N > 0) {
-    const long grid = (total + 255) / 256;
-    if (grid > 0x7fffffffL) return IX_DECLINED;
-    hipLaunchKernelGGL(k_gdn_conv, dim3((unsigned)grid), dim3(256), 0, st, (const bf16_t*)x, (const bf16_t*)weight,
+    const long blocks = (total + 255) / 256;
+    const long gx = blocks < (1L << 22) ? blocks : (1L << 22);
+    const long gy = (blocks + gx - 1) / gx;
+    if (gy > 65535) return IX_DECLINED;
+    hipLaunchKernelGGL(k_gdn_conv, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st, (const bf16_t*)x, (const bf16_t*)weight,
                        (const bf16_t*)bias, (bf16_t*)y, (const bf16_t*)conv_pool, cu_seqlens, state_rows_in, (int)N,
                        D, (int)W, silu, total);
   }
