@@ -138,6 +138,25 @@ int ix_gdn_scan(const void* q, const void* k, const void* v, const float* g, con
                 const int* cu_seqlens, const int* state_indices, long state_indices_stride, long N, long H,
                 long HV, long K, long V, float scale, int time_tile, void* stream);
 
+/* attention.varlen (ops/attention/_register.py:15-47; varlen_backend.py; megatron_varlen_attn.py): causal
+ * grouped-query attention with ONE walk over the keys of each query (the reference's num_splits=1
+ * pin), so a query's bits do not depend on the launch it ran in. bf16 only, D = 128.
+ * q [Tq, HQ, D] with token pitch q_pitch; k, v [*, HKV, D] with token pitch kv_pitch (elements); o
+ * [Tq, HQ, D] contiguous. cu_q int32 [N+1] packs the queries. Sequence n's keys are the tokens
+ * kv_start[n] .. kv_start[n] + q_pos0[n] + len_q[n] - 1 of k/v; its first query sits at absolute
+ * position q_pos0[n] (NULL: 0 for every sequence; a negative entry marks a null lane whose outputs are
+ * zero). max_q_len >= the longest query run. HQ % HKV == 0 and HQ / HKV in {1,2,4,8,16,32}. */
+int ix_attn_varlen(const void* q, long q_pitch, const void* k, const void* v, long kv_pitch, void* o,
+                   const int* cu_q, const long* kv_start, const int* q_pos0, long N, long max_q_len, long HQ,
+                   long HKV, long D, float scale, void* stream);
+
+/* rope.rope (ops/rope/_register.py:17-77; rope_fused.py:66-108): rotate-half rotary embedding over the
+ * first R lanes of every head, in place, with the three-round bf16 multiply-add
+ * bf16(bf16(x*cos) + bf16(rot*sin)). x [tokens, heads, D] with token pitch x_pitch; cos/sin bf16
+ * [positions, R]; positions int32 [tokens]. */
+int ix_rope_inplace(void* x, long x_pitch, const void* cos_table, const void* sin_table, const int* positions,
+                    long tokens, long heads, long D, long R, void* stream);
+
 /* gdn_l2norm (gdn_ops.py:202-213): y = x * (1/sqrt(sum x^2 + eps)) over rows of K.
  * x [tokens, H, K] with token pitch x_pitch; y [tokens, H, K] contiguous. */
 int ix_gdn_l2norm(const void* x, long x_pitch, void* y, int io_dtype, long tokens, long H, long K, float eps,

@@ -1,0 +1,277 @@
+// Causal grouped-query attention over packed sequences with ONE walk of the keys per query, and
+// rotary position embedding.
+//
+// The canonical function, per (query token at absolute position p, query head h):
+//   keys 0..p of the query's own sequence are walked in blocks of 32, block b = keys [32b, 32b+32);
+//   per block:  s_j  = (q . k_j) * scale                 bf16 MFMA, fp32 accumulate, d in 8 steps of 16
+//               s_j  = -inf for j > p
+//               m'   = max(m, max_j s_j)
+//               a    = exp2((m - m') * log2e)            (ix_exp_fast)
+//               p_j  = exp2((s_j - m') * log2e)
+//               l    = l * a + (lo + hi)                 lo/hi: the two halves' sums, see ix_attn_block
+//               O    = O * a + sum_j bf16(p_j) * v_j     bf16 MFMA, fp32 accumulate, keys in 2 steps of 16
+//   out = bf16(O / l).
+// Nothing in that chain depends on which other queries share the launch: a workgroup holds the
+// queries of 32/GROUP * 4 consecutive tokens for the GROUP query heads of one key/value head, every
+// MFMA row or column belongs to one query, and a block that lies wholly beyond a query's position is
+// an exact no-op for it (a = 1, p_j = 0), so whether a wave computes or skips it gives the same bits.
+// A one-token decode step and a full-sequence pass therefore agree bit for bit.
+#include "ix_common.h"
+#include "../../include/isoexec_hip.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 ix_bf16x8;
+typedef __attribute__((ext_vector_type(16))) float ix_f32x16;
+
+#define IX_ATTN_D 128
+#define IX_ATTN_BN 32
+#define IX_ATTN_KP (IX_ATTN_D * 2 + 16)  // bytes per key row of the K tile
+#define IX_ATTN_VP (IX_ATTN_BN * 2 + 8)  // bytes per d row of the transposed V tile
+
+struct IxAttnStage {
+  uint4 k0, k1, v0, v1;
+};
+
+// Thread t stages 16 consecutive d of key t/8 (two 16-byte loads from each of K and V).
+__device__ __forceinline__ void ix_attn_fetch(IxAttnStage& st, const bf16_t* __restrict__ kbase,
+                                              const bf16_t* __restrict__ vbase, long kv_pitch, int kb, int key_limit) {
+  const int key = kb * IX_ATTN_BN + (int)(threadIdx.x >> 3);
+  const int dch = (threadIdx.x & 7) * 16;
+  if (key <= key_limit) {
+    const uint4* kp = reinterpret_cast<const uint4*>(kbase + (long)key * kv_pitch + dch);
+    const uint4* vp = reinterpret_cast<const uint4*>(vbase + (long)key * kv_pitch + dch);
+    st.k0 = kp[0]; st.k1 = kp[1]; st.v0 = vp[0]; st.v1 = vp[1];
+  } else {  // beyond the last key any query of this workgroup needs: zeros, never read from memory
+    st.k0 = st.k1 = st.v0 = st.v1 = make_uint4(0, 0, 0, 0);
+  }
+}
+
+__device__ __forceinline__ void ix_attn_commit(const IxAttnStage& st, char* ldsK, char* ldsV) {
+  const int key = threadIdx.x >> 3;
+  const int dch = (threadIdx.x & 7) * 16;
+  uint4* kd = reinterpret_cast<uint4*>(ldsK + key * IX_ATTN_KP + dch * 2);
+  kd[0] = st.k0; kd[1] = st.k1;
+  const uint32_t w[8] = {st.v0.x, st.v0.y, st.v0.z, st.v0.w, st.v1.x, st.v1.y, st.v1.z, st.v1.w};
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    *reinterpret_cast<bf16_t*>(ldsV + (dch + 2 * j) * IX_ATTN_VP + key * 2) = (bf16_t)(w[j] & 0xffffu);
+    *reinterpret_cast<bf16_t*>(ldsV + (dch + 2 * j + 1) * IX_ATTN_VP + key * 2) = (bf16_t)(w[j] >> 16);
+  }
+}
+
+// One block of 32 keys for the 32 queries of a wave. Lane (qc = lane % 32, hf = lane / 32) holds
+// query qc; of the block's keys it holds, in register i, key (i/4)*8 + hf*4 + i%4.
+__device__ __forceinline__ void ix_attn_block(const char* ldsK, const char* ldsV, const ix_bf16x8 (&qf)[8],
+                                              ix_f32x16 (&O)[4], float& m, float& l, int kb, int qpos, float scale) {
+  const int lane = threadIdx.x & 63;
+  const int qc = lane & 31, hf = lane >> 5;
+  ix_f32x16 sacc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) sacc[i] = 0.0f;
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    const ix_bf16x8 kf = *reinterpret_cast<const ix_bf16x8*>(ldsK + qc * IX_ATTN_KP + (16 * s + hf * 8) * 2);
+    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], sacc, 0, 0, 0);
+  }
+  float sv[16];
+  float bm = IX_NEG_INF;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int key = kb * IX_ATTN_BN + (i >> 2) * 8 + hf * 4 + (i & 3);
+    const float x = sacc[i] * scale;
+    sv[i] = key <= qpos ? x : IX_NEG_INF;
+    bm = fmaxf(bm, sv[i]);
+  }
+  bm = fmaxf(bm, __shfl_xor(bm, 32, IX_WAVE));
+  const float m_new = fmaxf(m, bm);
+  const float alpha = ix_exp_fast(m - m_new);
+  float p[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) p[i] = ix_exp_fast(sv[i] - m_new);
+  const float pa[8] = {p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]};
+  const float pb[8] = {p[8], p[9], p[10], p[11], p[12], p[13], p[14], p[15]};
+  const float mine = ix_tree8(pa) + ix_tree8(pb);
+  const float other = __shfl_xor(mine, 32, IX_WAVE);
+  const float tot = hf ? other + mine : mine + other;  // (half 0) + (half 1) on both lanes
+  l = l * alpha + tot;
+  m = m_new;
+  ix_bf16x8 pf[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    uint32_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = ix_pack_bf2(p[8 * s + 2 * j], p[8 * s + 2 * j + 1]);
+    pf[s] = *reinterpret_cast<const ix_bf16x8*>(w);
+  }
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) O[dt][i] = O[dt][i] * alpha;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const char* row = ldsV + (qc + 32 * dt) * IX_ATTN_VP;
+      uint2 lo = *reinterpret_cast<const uint2*>(row + (16 * s + hf * 4) * 2);
+      uint2 hi = *reinterpret_cast<const uint2*>(row + (16 * s + 8 + hf * 4) * 2);
+      const uint32_t w[4] = {lo.x, lo.y, hi.x, hi.y};
+      const ix_bf16x8 vf = *reinterpret_cast<const ix_bf16x8*>(w);
+      O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[s], O[dt], 0, 0, 0);
+    }
+  }
+}
+
+template <int GROUP>
+__global__ __launch_bounds__(256) void k_attn_varlen(const bf16_t* __restrict__ q, long q_pitch,
+                                                     const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
+                                                     long kv_pitch, bf16_t* __restrict__ o,
+                                                     const int* __restrict__ cu_q, const long* __restrict__ kv_start,
+                                                     const int* __restrict__ q_pos0, int HQ, float scale) {
+  constexpr int TOK_W = 32 / GROUP;   // tokens per wave
+  constexpr int TOK_WG = 4 * TOK_W;   // tokens per workgroup
+  __shared__ __attribute__((aligned(16))) char ldsK[IX_ATTN_BN * IX_ATTN_KP];
+  __shared__ __attribute__((aligned(16))) char ldsV[IX_ATTN_D * IX_ATTN_VP];
+  const int n = blockIdx.y, g = blockIdx.z;
+  const int qb = cu_q[n];
+  const int len = cu_q[n + 1] - qb;
+  const int t0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * TOK_WG;  // long tiles first
+  if (t0 >= len) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int qc = lane & 31, hf = lane >> 5;
+  const int rel = t0 + wave * TOK_W + qc / GROUP;
+  const int h = g * GROUP + qc % GROUP;
+  const bool live = rel < len;
+  const int p0 = q_pos0 ? q_pos0[n] : 0;
+  bf16_t* orow = o + ((long)(qb + rel) * HQ + h) * IX_ATTN_D;
+  if (p0 < 0) {  // null lane: defined output, nothing read
+    if (live) {
+      for (int dt = 0; dt < 4; ++dt)
+        for (int i = 0; i < 16; ++i) orow[32 * dt + (i >> 2) * 8 + hf * 4 + (i & 3)] = 0;
+    }
+    return;
+  }
+  // A padding column carries a zero query and no causal limit: finite scores, result discarded.
+  const int qpos = live ? p0 + rel : 0x7fffffff;
+  ix_bf16x8 qf[8];
+  {
+    const bf16_t* qrow = q + (long)(qb + (live ? rel : 0)) * q_pitch + (long)h * IX_ATTN_D;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      uint4 w = make_uint4(0, 0, 0, 0);
+      if (live) w = *reinterpret_cast<const uint4*>(qrow + 16 * s + hf * 8);
+      qf[s] = *reinterpret_cast<const ix_bf16x8*>(&w);
+    }
+  }
+  const int last_tok = min(len, t0 + TOK_WG) - 1;
+  const int key_limit = p0 + last_tok;                       // last key any query here may see
+  const int nblocks = key_limit / IX_ATTN_BN + 1;
+  const int wave_last = min(len - 1, t0 + wave * TOK_W + TOK_W - 1);
+  const int wave_blocks = wave_last >= t0 + wave * TOK_W ? (p0 + wave_last) / IX_ATTN_BN + 1 : 0;
+  const long kv0 = kv_start[n];
+  const bf16_t* kbase = k + kv0 * kv_pitch + (long)g * IX_ATTN_D;
+  const bf16_t* vbase = v + kv0 * kv_pitch + (long)g * IX_ATTN_D;
+
+  ix_f32x16 O[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
+  float m = IX_NEG_INF, l = 0.0f;
+
+  IxAttnStage st;
+  ix_attn_fetch(st, kbase, vbase, kv_pitch, 0, key_limit);
+  for (int kb = 0; kb < nblocks; ++kb) {
+    __syncthreads();  // every wave is done reading the previous block
+    ix_attn_commit(st, ldsK, ldsV);
+    __syncthreads();
+    if (kb + 1 < nblocks) ix_attn_fetch(st, kbase, vbase, kv_pitch, kb + 1, key_limit);
+    if (kb < wave_blocks) ix_attn_block(ldsK, ldsV, qf, O, m, l, kb, qpos, scale);
+  }
+  if (live) {
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) {
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const int d = 32 * dt + i4 * 8 + hf * 4;
+        uint2 w;
+        w.x = ix_pack_bf2(O[dt][4 * i4 + 0] / l, O[dt][4 * i4 + 1] / l);
+        w.y = ix_pack_bf2(O[dt][4 * i4 + 2] / l, O[dt][4 * i4 + 3] / l);
+        *reinterpret_cast<uint2*>(orow + d) = w;
+      }
+    }
+  }
+}
+
+extern "C" int ix_attn_varlen(const void* q, long q_pitch, const void* k, const void* v, long kv_pitch, void* o,
+                              const int* cu_q, const long* kv_start, const int* q_pos0, long N, long max_q_len,
+                              long HQ, long HKV, long D, float scale, void* stream) {
+  if (!q || !k || !v || !o || !cu_q || !kv_start) return IX_ERR_ARG;
+  if (N < 0 || max_q_len < 0 || HQ <= 0 || HKV <= 0 || HQ % HKV != 0) return IX_ERR_ARG;
+  if (D != IX_ATTN_D) return IX_DECLINED;
+  if (q_pitch % 8 != 0 || kv_pitch % 8 != 0 || !ix_aligned(q, 16) || !ix_aligned(k, 16) || !ix_aligned(v, 16) ||
+      !ix_aligned(o, 8))
+    return IX_DECLINED;
+  if (N == 0 || max_q_len == 0) return IX_OK;
+  if (N > 65535 || HKV > 65535) return IX_DECLINED;
+  const int group = (int)(HQ / HKV);
+  hipStream_t st = (hipStream_t)stream;
+#define IX_ATTN_LAUNCH(G)                                                                                       \
+  case G: {                                                                                                     \
+    const long tok_wg = 4 * (32 / G);                                                                           \
+    const long tiles = (max_q_len + tok_wg - 1) / tok_wg;                                                       \
+    if (tiles > 0x7fffffffL) return IX_DECLINED;                                                                \
+    hipLaunchKernelGGL(k_attn_varlen<G>, dim3((unsigned)tiles, (unsigned)N, (unsigned)HKV), dim3(256), 0, st,   \
+                       (const bf16_t*)q, q_pitch, (const bf16_t*)k, (const bf16_t*)v, kv_pitch, (bf16_t*)o,    \
+                       cu_q, kv_start, q_pos0, (int)HQ, scale);                                                 \
+    break;                                                                                                      \
+  }
+  switch (group) {
+    IX_ATTN_LAUNCH(1)
+    IX_ATTN_LAUNCH(2)
+    IX_ATTN_LAUNCH(4)
+    IX_ATTN_LAUNCH(8)
+    IX_ATTN_LAUNCH(16)
+    IX_ATTN_LAUNCH(32)
+    default:
+      return IX_DECLINED;
+  }
+#undef IX_ATTN_LAUNCH
+  return ix_launch_status();
+}
+
+// ---- rotary position embedding -------------------------------------------------------------------
+// x [tokens, heads, D] (token pitch x_pitch), rotated in place over its first R lanes:
+//   y[d]       = bf16( bf16(x[d]       * cos[d])       + bf16((-x[d + R/2]) * sin[d]) )        d <  R/2
+//   y[d + R/2] = bf16( bf16(x[d + R/2] * cos[d + R/2]) + bf16(  x[d]        * sin[d + R/2]) )
+// Three bf16 rounds per output, each product and the sum computed in fp32. cos/sin: [positions, R]
+// bf16 tables; pos[t] picks the row.
+__global__ __launch_bounds__(256) void k_rope(bf16_t* __restrict__ x, long x_pitch, const bf16_t* __restrict__ cs,
+                                              const bf16_t* __restrict__ sn, const int* __restrict__ pos, long total,
+                                              int heads, int D, int R) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int half = R >> 1;
+  const int d = (int)(i % half);
+  const long th = i / half;
+  const int hd = (int)(th % heads);
+  const long t = th / heads;
+  bf16_t* row = x + t * x_pitch + (long)hd * D;
+  const long tab = (long)pos[t] * R;
+  const float a = ix_bf2f(row[d]), b = ix_bf2f(row[d + half]);
+  const float c0 = ix_bf2f(cs[tab + d]), c1 = ix_bf2f(cs[tab + d + half]);
+  const float s0 = ix_bf2f(sn[tab + d]), s1 = ix_bf2f(sn[tab + d + half]);
+  const float lo = ix_rbf(a * c0) + ix_rbf((b * -1.0f) * s0);
+  const float hi = ix_rbf(b * c1) + ix_rbf(a * s1);
+  row[d] = ix_f2bf(lo);
+  row[d + half] = ix_f2bf(hi);
+}
+
+extern "C" int ix_rope_inplace(void* x, long x_pitch, const void* cos_table, const void* sin_table,
+                               const int* positions, long tokens, long heads, long D, long R, void* stream) {
+  if (!x || !cos_table || !sin_table || !positions || tokens < 0 || heads <= 0 || D <= 0) return IX_ERR_ARG;
+  if (R <= 0 || R % 2 != 0 || R > D) return IX_ERR_ARG;
+  const long total = tokens * heads * (R / 2);
+  if (total == 0) return IX_OK;
+  const long grid = (total + 255) / 256;
+  if (grid > (1L << 24)) return IX_DECLINED;
+  hipLaunchKernelGGL(k_rope, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, (bf16_t*)x, x_pitch,
+                     (const bf16_t*)cos_table, (const bf16_t*)sin_table, positions, total, (int)heads, (int)D, (int)R);
+  return ix_launch_status();
+}

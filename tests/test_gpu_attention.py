@@ -1,0 +1,200 @@
+"""GPU parity of the attention and rope kernels.
+
+Attention's two matrix products run on the matrix cores, whose internal summation order is not
+public, so the oracle comparison on random inputs carries a tolerance (stated below), exactly as for
+the dense GEMM. What is bit-exact: inputs whose partial sums are exact in any order (known answers),
+and every invariance -- a query's bits do not depend on the other queries, on how the sequence was cut
+into calls, or on where its keys live.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from _util import DevicePrims, bf16_to_np, cpu_gen, np_bits, np_to_bf16, same_bits
+from oracle import attention as o_attn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+D = 128
+
+
+@pytest.fixture(scope="module")
+def dprims():
+    return DevicePrims(DEV)
+
+
+def attn(q, k, v, lens, **kw):
+    from isoexec_amd.ops.attention.varlen_attn import varlen_attention
+
+    cu = torch.tensor(np.cumsum([0] + list(lens)), dtype=torch.int32, device=DEV)
+    return varlen_attention(q, k, v, cu, max(lens), **kw)
+
+
+def rand_qkv(T, HQ, HKV, seed):
+    g = cpu_gen(seed)
+    mk = lambda h: torch.randn(T, h, D, generator=g).to(torch.bfloat16)
+    return mk(HQ), mk(HKV), mk(HKV)
+
+
+@pytest.mark.parametrize("HQ,HKV", [(8, 1), (4, 4), (32, 4), (2, 1), (16, 1)])
+def test_known_answers_are_bit_exact(HQ, HKV, dprims):
+    """Scores are small integers with the maximum at key 0, values are small integers: every partial
+    sum is exact in any order, so kernel and oracle must agree on every bit. Pins the causal mask, the
+    head grouping, the key order of the value product and the denominator's summation order."""
+    lens = [1, 2, 31, 32, 33, 64]
+    T = sum(lens)
+    rng = np.random.default_rng(HQ * 10 + HKV)
+    group = HQ // HKV
+    q = np.zeros((T, HQ, D), np.float32)
+    k = np.zeros((T, HKV, D), np.float32)
+    for h in range(HQ):
+        q[:, h, (7 * h) % D] = 8.0  # head h reads lane 7h of its key head
+    v = rng.integers(-4, 5, size=(T, HKV, D)).astype(np.float32)
+    start = 0
+    for n in lens:
+        for g in range(HKV):
+            for h in range(g * group, (g + 1) * group):
+                k[start : start + n, g, (7 * h) % D] = -rng.integers(0, 5, size=n)
+                k[start, g, (7 * h) % D] = 0  # key 0 holds the maximum
+        start += n
+    got = attn(np_to_bf16(q, DEV), np_to_bf16(k, DEV), np_to_bf16(v, DEV), lens, scale=0.125)
+    start = 0
+    for n in lens:
+        sl = slice(start, start + n)
+        want = o_attn.attend_causal(q[sl], k[sl], v[sl], scale=0.125, prims=dprims)
+        assert np.array_equal(np_bits(bf16_to_np(got[sl])), np_bits(want)), n
+        start += n
+
+
+def test_random_inputs_within_tolerance_of_oracle_and_float64(dprims):
+    """Config-4 head layout (32 query heads, 4 key/value heads, d 128). Tolerance: 2^-7 of the
+    output scale against the oracle (one bf16 ulp where an fp32 sum lands near a rounding boundary),
+    2^-6 against float64 softmax attention."""
+    lens = [150, 37]
+    T = sum(lens)
+    q, k, v = rand_qkv(T, 32, 4, seed=1)
+    got = bf16_to_np(attn(q.to(DEV), k.to(DEV), v.to(DEV), lens))
+    start = 0
+    for n in lens:
+        sl = slice(start, start + n)
+        f = lambda t: bf16_to_np(t[sl])
+        want = o_attn.attend_causal(f(q), f(k), f(v), prims=dprims)
+        truth = o_attn.attend_fp64(f(q), f(k), f(v))
+        scale = np.abs(truth).max()
+        assert np.abs(got[sl] - want).max() <= 2.0 ** -7 * scale
+        assert (got[sl] != want).mean() < 0.05
+        assert np.abs(got[sl] - truth).max() <= 2.0 ** -6 * scale
+        start += n
+
+
+def test_a_querys_bits_do_not_depend_on_the_call_shape():
+    """One sequence of 300 tokens, config-4 heads: the packed full pass, the same sequence among
+    others, a chunked prefill, and prefill followed by one-token decode steps out of a KV cache."""
+    from isoexec_amd.ops.attention.varlen_attn import KVCache, varlen_attention
+
+    T, HQ, HKV = 300, 32, 4
+    q, k, v = (t.to(DEV) for t in rand_qkv(T, HQ, HKV, seed=2))
+    full = attn(q, k, v, [T])
+    # among other sequences, at another place in the pack
+    qo, ko, vo = (t.to(DEV) for t in rand_qkv(77, HQ, HKV, seed=3))
+    mixed = attn(torch.cat([qo, q, qo[:5]]), torch.cat([ko, k, ko[:5]]), torch.cat([vo, v, vo[:5]]), [77, T, 5])
+    assert same_bits(mixed[77 : 77 + T], full)
+    # strided inputs: q, k, v as slices of one projection buffer
+    buf = torch.cat([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], dim=1)
+    qs = buf[:, : HQ * D].unflatten(1, (HQ, D))
+    ks = buf[:, HQ * D : (HQ + HKV) * D].unflatten(1, (HKV, D))
+    vs = buf[:, (HQ + HKV) * D :].unflatten(1, (HKV, D))
+    assert same_bits(attn(qs, ks, vs, [T]), full)
+    # chunked prefill and decode against a cache whose rows are not where the packed keys were
+    cache = KVCache(rows=3, max_len=512, num_kv_heads=HKV, device=DEV)
+    row = 2
+    kf, vf = cache.flat()
+    kv_start = torch.tensor([row * cache.max_len], dtype=torch.int64, device=DEV)
+    done = 0
+    for n in (64, 1, 100, 35):  # chunks of a chunked prefill
+        idx = torch.arange(done, done + n, device=DEV) + row * cache.max_len
+        cache.write(idx, k[done : done + n], v[done : done + n])
+        cu = torch.tensor([0, n], dtype=torch.int32, device=DEV)
+        pos0 = torch.tensor([done], dtype=torch.int32, device=DEV)
+        o = varlen_attention(q[done : done + n], kf, vf, cu, n, kv_start=kv_start, q_pos0=pos0)
+        assert same_bits(o, full[done : done + n]), (done, n)
+        done += n
+    cu1 = torch.tensor([0, 1], dtype=torch.int32, device=DEV)
+    for t in range(done, T):  # one-token decode steps
+        cache.write(torch.tensor([row * cache.max_len + t], device=DEV), k[t : t + 1], v[t : t + 1])
+        o = varlen_attention(q[t : t + 1], kf, vf, cu1, 1, kv_start=kv_start, q_pos0=torch.tensor([t], dtype=torch.int32, device=DEV))
+        assert same_bits(o, full[t : t + 1]), t
+
+
+def test_batched_decode_with_null_lanes():
+    """A decode batch: three live sequences at different context lengths and two padded lanes."""
+    from isoexec_amd.ops.attention.varlen_attn import KVCache, varlen_attention
+
+    HQ, HKV = 32, 4
+    lens = [40, 129, 7]
+    cache = KVCache(rows=4, max_len=256, num_kv_heads=HKV, device=DEV)
+    kf, vf = cache.flat()
+    fulls, qs = [], []
+    for i, n in enumerate(lens):
+        q, k, v = (t.to(DEV) for t in rand_qkv(n, HQ, HKV, seed=10 + i))
+        cache.write(torch.arange(n, device=DEV) + (i + 1) * cache.max_len, k, v)
+        fulls.append(attn(q, k, v, [n]))
+        qs.append(q)
+    junk = torch.randn(1, HQ, D, device=DEV).to(torch.bfloat16)
+    qd = torch.cat([qs[0][-1:], junk, qs[1][-1:], qs[2][-1:], junk])
+    kv_start = torch.tensor([1, 0, 2, 3, 0], dtype=torch.int64, device=DEV) * cache.max_len
+    pos0 = torch.tensor([lens[0] - 1, -1, lens[1] - 1, lens[2] - 1, -1], dtype=torch.int32, device=DEV)
+    cu = torch.arange(6, dtype=torch.int32, device=DEV)
+    o = varlen_attention(qd, kf, vf, cu, 1, kv_start=kv_start, q_pos0=pos0)
+    assert same_bits(o[0:1], fulls[0][-1:]) and same_bits(o[2:3], fulls[1][-1:]) and same_bits(o[3:4], fulls[2][-1:])
+    assert not o[1].any() and not o[4].any()
+
+
+def test_argument_checks():
+    from isoexec_amd.ops.attention.varlen_attn import varlen_attention
+
+    q, k, v = (t.to(DEV) for t in rand_qkv(8, 4, 2, seed=5))
+    cu = torch.tensor([0, 8], dtype=torch.int32, device=DEV)
+    with pytest.raises(RuntimeError, match="bf16 only"):
+        varlen_attention(q.float(), k, v, cu, 8)
+    with pytest.raises(RuntimeError, match="declined"):
+        varlen_attention(q[..., :64].contiguous(), k[..., :64].contiguous(), v[..., :64].contiguous(), cu, 8)
+    with pytest.raises(RuntimeError, match="declined"):
+        varlen_attention(torch.cat([q, q[:, :2]], 1), k, v, cu, 8)  # 6 query heads over 2: group 3
+    with pytest.raises(RuntimeError, match="int32"):
+        varlen_attention(q, k, v, cu.long(), 8)
+    empty = varlen_attention(q[:0], k, v, torch.zeros(1, dtype=torch.int32, device=DEV), 0)
+    assert empty.shape == (0, 4, D)
+
+
+def test_rope_bit_exact_in_place_on_a_strided_slice():
+    from isoexec_amd.ops.rope.rope_hip import apply_rope_, rope_tables
+
+    T, HQ, HKV, R = 50, 6, 2, 64
+    g = cpu_gen(6)
+    buf = torch.randn(T, (HQ + 2 * HKV) * D, generator=g).to(torch.bfloat16)
+    buf[3, :D] = torch.tensor([0.0, -0.0] * (D // 2)).to(torch.bfloat16)  # signed zeros travel through
+    pos = torch.randint(0, 4000, (T,), generator=g, dtype=torch.int32)
+    cos_d, sin_d = rope_tables(4096, R, 1e6, device=DEV)
+    cos_o, sin_o = o_attn.rope_tables(4096, R, 1e6)
+    assert np.array_equal(np_bits(bf16_to_np(cos_d)), np_bits(cos_o)) and np.array_equal(np_bits(bf16_to_np(sin_d)), np_bits(sin_o))
+    dbuf = buf.to(DEV)
+    qv = dbuf[:, : HQ * D].unflatten(1, (HQ, D))
+    kv = dbuf[:, HQ * D : (HQ + HKV) * D].unflatten(1, (HKV, D))
+    apply_rope_(qv, cos_d, sin_d, pos.to(DEV))
+    apply_rope_(kv, cos_d, sin_d, pos.to(DEV))
+    host = bf16_to_np(buf)
+    want_q = o_attn.rope(host[:, : HQ * D].reshape(T, HQ, D), cos_o, sin_o, pos.numpy())
+    want_k = o_attn.rope(host[:, HQ * D : (HQ + HKV) * D].reshape(T, HKV, D), cos_o, sin_o, pos.numpy())
+    got = bf16_to_np(dbuf)
+    assert np.array_equal(np_bits(got[:, : HQ * D].reshape(T, HQ, D)), np_bits(want_q))
+    assert np.array_equal(np_bits(got[:, HQ * D : (HQ + HKV) * D].reshape(T, HKV, D)), np_bits(want_k))
+    assert np.array_equal(np_bits(got[:, (HQ + HKV) * D :]), np_bits(host[:, (HQ + HKV) * D :]))  # v untouched
+    # full rotary width, and a row's bits do not depend on the other rows
+    cos_f, sin_f = rope_tables(64, D, 1e4, device=DEV)
+    x = torch.randn(9, 3, D, generator=g).to(torch.bfloat16).to(DEV)
+    p = torch.arange(9, dtype=torch.int32, device=DEV)
+    whole = apply_rope_(x.clone(), cos_f, sin_f, p)
+    one = apply_rope_(x[4:5].clone(), cos_f, sin_f, p[4:5])
+    assert same_bits(one, whole[4:5]) and same_bits(whole[0], x[0])
