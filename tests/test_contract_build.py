@@ -288,11 +288,16 @@ def test_arch_tags():
 
 def test_shipped_registry_and_policy_agree():
     reg = build_registry()
-    assert registered_families() == ["mm", "norms", "logprobs", "gdn", "moe"]
+    assert registered_families() == ["mm", "attention", "rope", "norms", "logprobs", "gdn", "moe"]
     for op in reg.ops.values():
         for spec in op.impls.values():
             assert spec.supported_archs == GFX, (op.name, spec.impl_id)
     assert policy.policy_matches_registry_capabilities(qwen3_5.PATH_PROFILE, reg) == []
+    assert policy.policy_matches_registry_capabilities(qwen3_5.PROFILE, reg) == []
+    full = policy.derive_selections(qwen3_5.PROFILE)
+    assert full[("attention.varlen", "engine_decode")].pinned_constants == {"num_splits": 1}
+    assert ("rope.rope", "trainer_fwd") in full and frozenset(full) == reg.installed_keys() - {
+        (op, s) for op in ("gdn.l2norm", "gdn.gating") for s in ALL}
     sels = policy.derive_selections(qwen3_5.PATH_PROFILE)
     assert ("gdn.l2norm", "trainer_fwd") not in sels and ("gdn.state", "trainer_fwd") not in sels
     assert sels[("logprobs.log_softmax", "engine_decode")].pinned_constants == {"leaves": 8, "block": 4096, "accum": "kahan_fp32"}
@@ -318,6 +323,14 @@ def test_model_contract_builds_and_is_reproducible():
         qwen3_5.build(other_arch_reg, arch="gfx942", profile=qwen3_5.PATH_PROFILE)
     with pytest.raises(CB.PinValidationError, match="kernel='chunk'"):
         qwen3_5.build(reg, arch="gfx950", profile=qwen3_5.PATH_PROFILE.with_overrides(gdn_kernel="chunk"))
+    # The whole model adds the attention and rope entries: more logical ops, so a different meaning.
+    whole = qwen3_5.build(reg, arch="gfx950")
+    assert {("attention.varlen",), ("rope.rope",)} <= {e.region for e in whole.composition}
+    assert whole.identities.semantic != a.identities.semantic and K.validate(whole) == []
+    with pytest.raises(CB.PinValidationError, match="num_splits=2"):
+        CB.build_execution_contract(reg, {**policy.derive_selections(qwen3_5.PROFILE),
+                                          ("attention.varlen", "engine_decode"): policy.entry("hip_varlen_ns1", pinned={"num_splits": 2})},
+                                    arch="gfx950", model="m")
 
 
 def test_policy_exceptions_and_refusals():
@@ -441,7 +454,6 @@ def test_get_process_contract_builds_once_and_writes_the_artifact(monkeypatch, t
     import isoexec_amd.core.arch as arch_mod
     import isoexec_amd.models.qwen3_5 as q
 
-    monkeypatch.setattr(q, "PROFILE", q.PATH_PROFILE.with_overrides(name_patterns=q.PROFILE.name_patterns))
     path = tmp_path / "contract.json"
     monkeypatch.setenv("ISOEXEC_CONTRACT_PATH", str(path))
     assert process_contract.get_process_contract() is None
