@@ -1,0 +1,359 @@
+"""A hybrid GatedDeltaNet / attention / mixture-of-experts model served two ways over ONE set of ops.
+
+``TrainerModel`` scores whole packed sequences in one pass (the role of the reference's Megatron
+trainer forward); ``RolloutEngine`` prefills prompts and then decodes token by token out of state
+pools and a key/value cache (the role of its vLLM rollout forward, isoexec/runtimes/vllm/
+gptmodel_vllm.py). Both are thin drivers over ``_Blocks``, which holds every projection, norm and
+mixture call, so the two runtimes differ only in how tokens are cut into calls and where sequence
+state lives -- the things the kernels are invariant to. The logprob a rollout records for a sampled
+token therefore equals, bit for bit, the logprob the trainer later assigns to it.
+
+Layer layout (pre-norm residual stream, hidden H):
+    h -> norm -> mixer -> (+h, norm) -> mixture of experts -> (+h) -> next layer
+    mixer = GatedDeltaNet (in_proj -> causal conv -> l2norm/gate -> delta-rule scan -> gated norm ->
+            out_proj) on three layers of four, causal grouped-query attention with rotary embedding
+            (qkv_proj -> rope -> attention -> o_proj) on the fourth.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+from ..ops.attention.varlen_attn import KVCache, varlen_attention
+from ..ops.gdn.gdn_ops import conv_packed, gdn_native_core
+from ..ops.gdn.gdn_recurrent_state import RecurrentGDN
+from ..ops.logprobs.rowinv import leaves, sampled_forward
+from ..ops.mm.mm_hip import linear_nt
+from ..ops.moe.moe_hip import moe_ffn_forward
+from ..ops.norms.fused_outnorm import fused_add_rms_norm_gamma, fused_gated_out_norm, fused_rms_norm_gamma
+from ..ops.rope.rope_hip import apply_rope_, rope_tables
+
+
+@dataclass(frozen=True)
+class HybridConfig:
+    hidden: int = 2048
+    vocab: int = 151936
+    layers: int = 8
+    attention_every: int = 4  # layers 3, 7, ... (0-based) are attention; the rest GatedDeltaNet
+    # GatedDeltaNet
+    gdn_k_heads: int = 16
+    gdn_v_heads: int = 32
+    gdn_head_dim: int = 128
+    conv_width: int = 4
+    # attention
+    q_heads: int = 32
+    kv_heads: int = 4
+    head_dim: int = 128
+    rope_theta: float = 1.0e6
+    max_positions: int = 4096
+    # mixture of experts
+    experts: int = 128
+    topk: int = 8
+    expert_inter: int = 768
+    eps: float = 1.0e-6
+
+    def is_attention(self, layer: int) -> bool:
+        return (layer + 1) % self.attention_every == 0
+
+    @property
+    def gdn_qkv(self) -> int:
+        return 2 * self.gdn_k_heads * self.gdn_head_dim + self.gdn_v_heads * self.gdn_head_dim
+
+    @property
+    def gdn_z(self) -> int:
+        return self.gdn_v_heads * self.gdn_head_dim
+
+
+def _normal(shape, std, gen, device, dtype=torch.bfloat16):
+    return (torch.randn(shape, generator=gen, device=device) * std).to(dtype)
+
+
+@dataclass
+class HybridWeights:
+    """Random-initialised parameters (N(0, 0.02) projections, zero-centred norm gains)."""
+
+    embed: torch.Tensor
+    lm_head: torch.Tensor
+    final_norm: torch.Tensor
+    layers: list = field(default_factory=list)
+
+    @classmethod
+    def make(cls, cfg: HybridConfig, seed: int = 0, device="cuda") -> "HybridWeights":
+        g = torch.Generator(device=device)
+        g.manual_seed(seed)
+        H = cfg.hidden
+        w = cls(embed=_normal((cfg.vocab, H), 1.0, g, device), lm_head=_normal((cfg.vocab, H), 0.02, g, device),
+                final_norm=_normal((H,), 0.02, g, device))
+        for i in range(cfg.layers):
+            lw = {
+                "pre_norm": _normal((H,), 0.02, g, device),
+                "post_norm": _normal((H,), 0.02, g, device),
+                "router": _normal((cfg.experts, H), 0.02, g, device),
+                "w1": _normal((cfg.experts, 2 * cfg.expert_inter, H), 0.02, g, device),
+                "w2": _normal((cfg.experts, H, cfg.expert_inter), 0.02, g, device),
+            }
+            if cfg.is_attention(i):
+                lw["qkv_proj"] = _normal(((cfg.q_heads + 2 * cfg.kv_heads) * cfg.head_dim, H), 0.02, g, device)
+                lw["o_proj"] = _normal((H, cfg.q_heads * cfg.head_dim), 0.02, g, device)
+            else:
+                lw["in_proj"] = _normal((cfg.gdn_qkv + cfg.gdn_z + 2 * cfg.gdn_v_heads, H), 0.02, g, device)
+                lw["conv_weight"] = _normal((cfg.gdn_qkv, cfg.conv_width), 0.4, g, device)
+                lw["conv_bias"] = _normal((cfg.gdn_qkv,), 0.1, g, device)
+                lw["A_log"] = _normal((cfg.gdn_v_heads,), 0.3, g, device, torch.float32)
+                lw["dt_bias"] = _normal((cfg.gdn_v_heads,), 0.3, g, device, torch.float32)
+                lw["out_norm"] = _normal((cfg.gdn_head_dim,), 0.02, g, device)
+                lw["out_proj"] = _normal((H, cfg.gdn_z), 0.02, g, device)
+            w.layers.append(lw)
+        return w
+
+
+def _linear(x, w):
+    out = linear_nt(x, w)
+    if out is None:
+        raise RuntimeError(f"[isoexec-amd] GEMM declined for x {tuple(x.shape)} {x.dtype} w {tuple(w.shape)}")
+    return out
+
+
+class _Blocks:
+    """Every weight-bearing call of a layer, shared by both runtimes."""
+
+    def __init__(self, cfg: HybridConfig, weights: HybridWeights):
+        self.cfg, self.w = cfg, weights
+        dev = weights.embed.device
+        self.cos, self.sin = rope_tables(cfg.max_positions, cfg.head_dim, cfg.rope_theta, device=dev)
+
+    def embed(self, tokens: torch.Tensor) -> torch.Tensor:
+        return self.w.embed.index_select(0, tokens)
+
+    def gdn_in(self, layer: int, x: torch.Tensor):
+        """-> pre-conv ``qkv [T, D]`` (contiguous), and views ``z [T, HV, V]``, ``b``, ``a [T, HV]``."""
+        c = self.cfg
+        proj = _linear(x, self.w.layers[layer]["in_proj"])
+        qkv = proj[:, : c.gdn_qkv].contiguous()
+        z = proj[:, c.gdn_qkv : c.gdn_qkv + c.gdn_z].unflatten(1, (c.gdn_v_heads, c.gdn_head_dim))
+        b = proj[:, c.gdn_qkv + c.gdn_z : c.gdn_qkv + c.gdn_z + c.gdn_v_heads]
+        a = proj[:, c.gdn_qkv + c.gdn_z + c.gdn_v_heads :]
+        return qkv, z, b, a
+
+    def gdn_out(self, layer: int, o: torch.Tensor, z: torch.Tensor) -> torch.Tensor:
+        lw = self.w.layers[layer]
+        normed = fused_gated_out_norm(o, z, lw["out_norm"], self.cfg.eps)
+        return _linear(normed.view(o.shape[0], -1), lw["out_proj"])
+
+    def attn_qkv(self, layer: int, x: torch.Tensor, positions: torch.Tensor):
+        """-> views ``q [T, HQ, D]``, ``k, v [T, HKV, D]`` of one projection buffer, q and k rotated."""
+        c = self.cfg
+        proj = _linear(x, self.w.layers[layer]["qkv_proj"])
+        nq, nk = c.q_heads * c.head_dim, c.kv_heads * c.head_dim
+        q = proj[:, :nq].unflatten(1, (c.q_heads, c.head_dim))
+        k = proj[:, nq : nq + nk].unflatten(1, (c.kv_heads, c.head_dim))
+        v = proj[:, nq + nk :].unflatten(1, (c.kv_heads, c.head_dim))
+        apply_rope_(q, self.cos, self.sin, positions)
+        apply_rope_(k, self.cos, self.sin, positions)
+        return q, k, v
+
+    def attn_out(self, layer: int, o: torch.Tensor) -> torch.Tensor:
+        return _linear(o.view(o.shape[0], -1), self.w.layers[layer]["o_proj"])
+
+    def moe(self, layer: int, x: torch.Tensor) -> torch.Tensor:
+        lw = self.w.layers[layer]
+        return moe_ffn_forward(x, lw["router"], lw["w1"], lw["w2"], self.cfg.topk, pre_softmax=True)
+
+    def run_layers(self, h: torch.Tensor, mixer) -> torch.Tensor:
+        """The residual stream over all layers; ``mixer(layer, x)`` is the runtime's own part."""
+        c = self.cfg
+        x = fused_rms_norm_gamma(h, self.w.layers[0]["pre_norm"], c.eps)
+        for i in range(c.layers):
+            lw = self.w.layers[i]
+            x, h = fused_add_rms_norm_gamma(mixer(i, x), h, lw["post_norm"], c.eps)
+            delta = self.moe(i, x)
+            nxt = self.w.layers[i + 1]["pre_norm"] if i + 1 < c.layers else self.w.final_norm
+            x, h = fused_add_rms_norm_gamma(delta, h, nxt, c.eps)
+        return x  # final-normed hidden states
+
+    def logits(self, x: torch.Tensor, want_row_max: bool = False):
+        got = linear_nt(x, self.w.lm_head, want_row_max=want_row_max)
+        if got is None:
+            raise RuntimeError("[isoexec-amd] LM-head GEMM declined")
+        return got
+
+    def sampled_logprobs(self, x: torch.Tensor, targets: torch.Tensor) -> torch.Tensor:
+        logits, row_max = self.logits(x, want_row_max=True)
+        lp, _ = sampled_forward(logits, targets, leaves(), row_max=row_max)
+        return lp
+
+
+class TrainerModel:
+    """Full-sequence scoring over packed sequences."""
+
+    def __init__(self, cfg: HybridConfig, weights: HybridWeights):
+        self.cfg, self.blocks = cfg, _Blocks(cfg, weights)
+
+    @torch.no_grad()
+    def hidden_states(self, tokens: torch.Tensor, lens: list) -> torch.Tensor:
+        """``tokens`` int64 [sum(lens)] packed; returns the final-normed hidden states [sum(lens), H]."""
+        b, c = self.blocks, self.cfg
+        dev = tokens.device
+        offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        cu = torch.from_numpy(offs).to(dev)
+        positions = torch.from_numpy(np.concatenate([np.arange(n, dtype=np.int32) for n in lens])).to(dev)
+        max_len = int(max(lens))
+
+        def mixer(i, x):
+            lw = b.w.layers[i]
+            if c.is_attention(i):
+                q, k, v = b.attn_qkv(i, x, positions)
+                return b.attn_out(i, varlen_attention(q, k, v, cu, max_len))
+            qkv, z, bb, a = b.gdn_in(i, x)
+            y = conv_packed(qkv, lw["conv_weight"], lw["conv_bias"], cu_seqlens=cu)
+            kd = c.gdn_k_heads * c.gdn_head_dim
+            q = y[:, :kd].unflatten(1, (c.gdn_k_heads, c.gdn_head_dim))
+            k = y[:, kd : 2 * kd].unflatten(1, (c.gdn_k_heads, c.gdn_head_dim))
+            v = y[:, 2 * kd :].unflatten(1, (c.gdn_v_heads, c.gdn_head_dim))
+            o = gdn_native_core(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), a, bb, lw["A_log"], lw["dt_bias"], cu_seqlens=cu)
+            return b.gdn_out(i, o[0], z)
+
+        return b.run_layers(b.embed(tokens), mixer)
+
+    @torch.no_grad()
+    def response_logprobs(self, tokens: torch.Tensor, lens: list, prompt_lens: list) -> list:
+        """Logprob of every response token: for sequence n, tokens ``prompt_lens[n] .. lens[n]-1``,
+        each scored from the hidden state one position earlier. Returns a list of fp32 tensors."""
+        x = self.hidden_states(tokens, lens)
+        rows, targets, start = [], [], 0
+        for n, p in zip(lens, prompt_lens):
+            rows.append(torch.arange(start + p - 1, start + n - 1, device=tokens.device))
+            targets.append(tokens[start + p : start + n])
+            start += n
+        lp = self.blocks.sampled_logprobs(x.index_select(0, torch.cat(rows)), torch.cat(targets))
+        return list(lp.split([n - p for n, p in zip(lens, prompt_lens)]))
+
+
+class RolloutEngine:
+    """Prefill, then one token per step per sequence, out of per-layer state."""
+
+    def __init__(self, cfg: HybridConfig, weights: HybridWeights, max_num_seqs: int, max_len: int):
+        self.cfg, self.blocks = cfg, _Blocks(cfg, weights)
+        dev = weights.embed.device
+        self.max_len = max_len
+        self.gdn, self.kv = {}, {}
+        for i in range(cfg.layers):
+            lw = weights.layers[i]
+            if cfg.is_attention(i):
+                self.kv[i] = KVCache(max_num_seqs, max_len, cfg.kv_heads, cfg.head_dim, device=dev)
+            else:
+                self.gdn[i] = RecurrentGDN(
+                    capacity=max_num_seqs, conv_weight=lw["conv_weight"], conv_bias=lw["conv_bias"], A_log=lw["A_log"],
+                    dt_bias=lw["dt_bias"], num_k_heads=cfg.gdn_k_heads, head_k_dim=cfg.gdn_head_dim,
+                    num_v_heads=cfg.gdn_v_heads, head_v_dim=cfg.gdn_head_dim, device=dev, driver_managed=True)
+        # One row table names a request's place in the key/value caches; the GatedDeltaNet layers keep
+        # their own (identical) tables so each can be released or evicted with its pool.
+        self.kv_rows: dict[int, int] = {}
+        self.free_kv_rows = list(range(max_num_seqs, 0, -1))
+        self.context: dict[int, int] = {}
+
+    def _kv_row(self, slot: int) -> int:
+        if slot not in self.kv_rows:
+            if not self.free_kv_rows:
+                raise RuntimeError("[isoexec-amd] key/value cache exhausted: release finished requests first")
+            self.kv_rows[slot] = self.free_kv_rows.pop()
+        return self.kv_rows[slot]
+
+    def release(self, slot: int) -> None:
+        for layer in self.gdn.values():
+            layer.release_slot(slot)
+        row = self.kv_rows.pop(slot, None)
+        if row is not None:
+            self.free_kv_rows.append(row)
+        self.context.pop(slot, None)
+
+    @torch.no_grad()
+    def prefill(self, slots: list, tokens: torch.Tensor, lens: list) -> torch.Tensor:
+        """Prompts packed in ``tokens``; returns the final-normed hidden state of each prompt's LAST
+        token ``[N, H]`` (the row the first response token is sampled from)."""
+        b, c = self.blocks, self.cfg
+        dev = tokens.device
+        offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        cu = torch.from_numpy(offs).to(dev)
+        positions = torch.from_numpy(np.concatenate([np.arange(n, dtype=np.int32) for n in lens])).to(dev)
+        rows = [self._kv_row(s) for s in slots]
+        kv_index = torch.from_numpy(np.concatenate([r * self.max_len + np.arange(n, dtype=np.int64) for r, n in zip(rows, lens)])).to(dev)
+        kv_start = torch.tensor([r * self.max_len for r in rows], dtype=torch.int64, device=dev)
+        slots_t = torch.tensor(slots, dtype=torch.int64, device=dev)
+        max_len = int(max(lens))
+        qsl = [int(o) for o in offs]
+
+        def mixer(i, x):
+            if c.is_attention(i):
+                q, k, v = b.attn_qkv(i, x, positions)
+                self.kv[i].write(kv_index, k, v)
+                kf, vf = self.kv[i].flat()
+                return b.attn_out(i, varlen_attention(q, kf, vf, cu, max_len, kv_start=kv_start))
+            qkv, z, bb, a = b.gdn_in(i, x)
+            o = self.gdn[i].prefill(slots_t, slots, qkv, a, bb, qsl, prefill_query_start_loc=cu)
+            return b.gdn_out(i, o, z)
+
+        x = b.run_layers(b.embed(tokens), mixer)
+        for s, n in zip(slots, lens):
+            self.context[s] = n
+        return x.index_select(0, torch.from_numpy(offs[1:].astype(np.int64) - 1).to(dev))
+
+    @torch.no_grad()
+    def decode(self, slots: list, tokens: torch.Tensor) -> torch.Tensor:
+        """Feed one token per sequence; returns the final-normed hidden states ``[N, H]``."""
+        b, c = self.blocks, self.cfg
+        dev = tokens.device
+        n = len(slots)
+        ctx = np.array([self.context[s] for s in slots], dtype=np.int32)
+        if int(ctx.max()) >= self.max_len:
+            raise RuntimeError(f"[isoexec-amd] a sequence reached the cache length {self.max_len}")
+        rows = np.array([self.kv_rows[s] for s in slots], dtype=np.int64)
+        meta = torch.from_numpy(np.stack([ctx.astype(np.int64), rows * self.max_len, rows * self.max_len + ctx])).to(dev)
+        positions = meta[0].to(torch.int32)
+        kv_start, kv_index = meta[1], meta[2]
+        cu = torch.arange(n + 1, dtype=torch.int32, device=dev)
+        slots_t = torch.tensor(slots, dtype=torch.int64, device=dev)
+
+        def mixer(i, x):
+            if c.is_attention(i):
+                q, k, v = b.attn_qkv(i, x, positions)
+                self.kv[i].write(kv_index, k, v)
+                kf, vf = self.kv[i].flat()
+                return b.attn_out(i, varlen_attention(q, kf, vf, cu, 1, kv_start=kv_start, q_pos0=positions))
+            qkv, z, bb, a = b.gdn_in(i, x)
+            return b.gdn_out(i, self.gdn[i].decode(slots_t, qkv, a, bb), z)
+
+        x = b.run_layers(b.embed(tokens), mixer)
+        for s in slots:
+            self.context[s] += 1
+        return x
+
+    @torch.no_grad()
+    def generate(self, slots: list, prompts: torch.Tensor, prompt_lens: list, steps: int, *, seed: int = 0,
+                 full_row_logprobs=None):
+        """Sample ``steps`` tokens per sequence (Gumbel-max over the logits, seeded) and record each
+        sampled token's logprob as the engine reports it. ``full_row_logprobs(logits) -> [N, V] fp32``
+        is the engine's logprob producer (default: the row-invariant full-row entry). Returns
+        ``(tokens [N, steps] int64, logprobs [N, steps] fp32)``."""
+        from ..ops.logprobs.rowinv import full_forward
+
+        if full_row_logprobs is None:
+            full_row_logprobs = lambda logits: full_forward(logits, leaves())
+        dev = prompts.device
+        g = torch.Generator(device=dev)
+        g.manual_seed(seed)
+        x = self.prefill(slots, prompts, prompt_lens)
+        out_tok, out_lp = [], []
+        for step in range(steps):
+            logits = self.blocks.logits(x)
+            lp_rows = full_row_logprobs(logits)
+            u = torch.rand(logits.shape, generator=g, device=dev).clamp_(min=1e-20)
+            tok = (logits.float() - torch.log(-torch.log(u))).argmax(dim=-1)
+            out_tok.append(tok)
+            out_lp.append(lp_rows.gather(1, tok.unsqueeze(1)).squeeze(1))
+            if step + 1 < steps:
+                x = self.decode(slots, tok)
+        return torch.stack(out_tok, dim=1), torch.stack(out_lp, dim=1)
