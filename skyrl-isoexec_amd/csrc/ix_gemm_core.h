@@ -67,7 +67,16 @@ struct IxGemmCfg {
   // as many half-stages as fit in the 160 KiB of LDS, at most IX_HALF_STAGES_MAX, at least 4
   static constexpr int HALF_STAGES =
       (IX_HALF_STAGES_MAX * (STAGE_BYTES / 2) <= 160 * 1024) ? IX_HALF_STAGES_MAX : 4;
-  static constexpr int LDS_BYTES = HALF_RING ? HALF_STAGES * (STAGE_BYTES / 2) : FULL_STAGES * STAGE_BYTES;
+  // Square tiles may instead use a ring of whole-k-tile operand units (pipeline C).
+#ifndef IX_NO_UNIT_RING
+  static constexpr int UNITS = (160 * 1024) / (BM * 128) > 9 ? 9 : (160 * 1024) / (BM * 128);
+  static constexpr bool UNIT_RING = BM == BN && UNITS >= 5 && X_CH >= 1;
+#else
+  static constexpr int UNITS = 0;
+  static constexpr bool UNIT_RING = false;
+#endif
+  static constexpr int LDS_BYTES = UNIT_RING ? UNITS * BM * 128
+                                             : (HALF_RING ? HALF_STAGES * (STAGE_BYTES / 2) : FULL_STAGES * STAGE_BYTES);
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile must be MFMA multiples");
   static_assert((BM * 8) % NT == 0 && (BN * 8) % NT == 0, "fetch must divide evenly");
   static_assert(NT % 64 == 0, "whole waves");
@@ -290,12 +299,118 @@ __device__ __forceinline__ void ix_gemm_mainloop_h4(ix_rsrc_t x_rsrc, const XRow
   __builtin_amdgcn_s_waitcnt(IX_VMCNT(0));  // drain the out-of-range tail fetches before LDS is reused
 }
 
+// ---- pipeline C: a ring of whole-k-tile OPERAND units (square tiles only) --------------------------
+// Unit u = 2*kt holds the X rows of k-tile kt, unit 2*kt+1 its W rows; each is BM rows of 128 bytes, so
+// every fetch moves whole 128-byte lines. The ring holds NU units: the two being consumed and NU-2 in
+// flight. One barrier per k-tile: after it every wave is done with k-tile kt-1, whose two slots take the
+// next two units. The K order is that of pipeline A.
+template <typename Cfg, typename XRow, typename WRow, typename Acc>
+__device__ __forceinline__ void ix_gemm_mainloop_units(ix_rsrc_t x_rsrc, const XRow& x_row,
+                                                       ix_rsrc_t w_rsrc, const WRow& w_row, int K,
+                                                       char* lds, Acc& acc) {
+  constexpr int NT = Cfg::NT, CH = Cfg::X_CH, UNIT = Cfg::BM * 128, NU = Cfg::UNITS;
+  static_assert(Cfg::BM == Cfg::BN && NU >= 5, "operand ring needs square tiles and five units");
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+  const int KT = (K + IX_BK - 1) / IX_BK;
+  const uint32_t lds_base = __builtin_amdgcn_readfirstlane(ix_lds_addr(lds) + (wave * 64) * 16);
+  const int K2 = K * 2;
+
+  uint32_t x_voff[CH], w_voff[CH];
+  int kb[CH];
+#pragma unroll
+  for (int j = 0; j < CH; ++j) {
+    const int r = (tid + j * NT) >> 3;
+    kb[j] = ((tid & 7) ^ ix_swz8(r)) * 16;
+    x_voff[j] = x_row(r) + kb[j];
+    w_voff[j] = w_row(r) + kb[j];
+  }
+  // unit u -> slot u % NU, tracked incrementally
+  auto issue = [&](ix_rsrc_t rsrc, const uint32_t (&voff)[CH], int kt, int slot) {
+    const int soff = kt * IX_BK * 2;
+    const uint32_t sbase = lds_base + slot * UNIT;
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      const uint32_t dead = (uint32_t)((K2 - 1 - (soff + kb[j])) >> 31) & IX_OOB;
+      ix_dma16(rsrc, sbase + j * NT * 16, voff[j] | dead, soff);
+    }
+  };
+  const int frow = lane & 31, fg = lane >> 5;
+  int x_foff[Cfg::MI], w_foff[Cfg::NI];
+#pragma unroll
+  for (int mi = 0; mi < Cfg::MI; ++mi) x_foff[mi] = ix_lds_off(wm * Cfg::TM + mi * 32 + frow, fg * 4);
+#pragma unroll
+  for (int ni = 0; ni < Cfg::NI; ++ni) w_foff[ni] = ix_lds_off(wn * Cfg::TN + ni * 32 + frow, fg * 4);
+
+  ix_bf16x8 xa[Cfg::MI], wa[Cfg::NI], xb[Cfg::MI], wb[Cfg::NI];
+  auto frags = [&](const char* xs, const char* ws, int s, ix_bf16x8* xf, ix_bf16x8* wf) {
+#pragma unroll
+    for (int mi = 0; mi < Cfg::MI; ++mi) xf[mi] = *reinterpret_cast<const ix_bf16x8*>(xs + (x_foff[mi] ^ (s << 4)));
+#pragma unroll
+    for (int ni = 0; ni < Cfg::NI; ++ni) wf[ni] = *reinterpret_cast<const ix_bf16x8*>(ws + (w_foff[ni] ^ (s << 4)));
+  };
+  auto mfmas = [&](const ix_bf16x8* xf, const ix_bf16x8* wf) {
+#ifdef IX_EXPERIMENT_NO_MFMA
+    asm volatile("" ::"v"(xf[0]), "v"(wf[0]));
+    return;
+#endif
+#pragma unroll
+    for (int mi = 0; mi < Cfg::MI; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < Cfg::NI; ++ni)
+        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[ni], xf[mi], acc[mi][ni], 0, 0, 0);
+  };
+
+  // prologue: units 0 .. NU-3
+  int is = 0;  // slot of the next unit to issue
+#pragma unroll
+  for (int u = 0; u < NU - 2; ++u) {
+    if (u & 1) issue(w_rsrc, w_voff, u >> 1, is); else issue(x_rsrc, x_voff, u >> 1, is);
+    is = is + 1 == NU ? 0 : is + 1;
+  }
+  int cs = 0;            // slot of the X unit being consumed
+  int nu = NU - 2;       // index of the next unit to issue
+  for (int kt = 0; kt < KT; ++kt) {
+    __builtin_amdgcn_s_waitcnt(IX_VMCNT((NU - 4) * CH));  // units 2kt and 2kt+1 have landed
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      if (nu & 1) issue(w_rsrc, w_voff, nu >> 1, is); else issue(x_rsrc, x_voff, nu >> 1, is);
+      is = is + 1 == NU ? 0 : is + 1;
+      ++nu;
+    }
+    const char* xs = lds + cs * UNIT;
+    const int wsl = cs + 1 == NU ? 0 : cs + 1;
+    const char* ws = lds + wsl * UNIT;
+    cs = wsl + 1 == NU ? 0 : wsl + 1;
+    frags(xs, ws, 0, xa, wa);
+    frags(xs, ws, 1, xb, wb);
+    __builtin_amdgcn_sched_barrier(0);
+    mfmas(xa, wa);
+    __builtin_amdgcn_sched_barrier(0);
+    frags(xs, ws, 2, xa, wa);
+    __builtin_amdgcn_sched_barrier(0);
+    mfmas(xb, wb);
+    __builtin_amdgcn_sched_barrier(0);
+    frags(xs, ws, 3, xb, wb);
+    __builtin_amdgcn_sched_barrier(0);
+    mfmas(xa, wa);
+    __builtin_amdgcn_sched_barrier(0);
+    mfmas(xb, wb);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  __builtin_amdgcn_s_waitcnt(IX_VMCNT(0));
+}
+
 // x_row(r) / w_row(r): byte offset of tile row r inside the operand's buffer, or IX_OOB.
 template <typename Cfg, typename XRow, typename WRow, typename Acc>
 __device__ __forceinline__ void ix_gemm_mainloop(ix_rsrc_t x_rsrc, const XRow& x_row,
                                                  ix_rsrc_t w_rsrc, const WRow& w_row, int K, char* lds,
                                                  Acc& acc) {
-  if constexpr (Cfg::HALF_RING)
+  if constexpr (Cfg::UNIT_RING)
+    ix_gemm_mainloop_units<Cfg>(x_rsrc, x_row, w_rsrc, w_row, K, lds, acc);
+  else if constexpr (Cfg::HALF_RING)
     ix_gemm_mainloop_h4<Cfg>(x_rsrc, x_row, w_rsrc, w_row, K, lds, acc);
   else
     ix_gemm_mainloop_full<Cfg>(x_rsrc, x_row, w_rsrc, w_row, K, lds, acc);
