@@ -5,7 +5,7 @@ Default workload (``dense_head``, BASELINE.json configs[1]): M = 4096 hidden sta
 log-softmax + target gather. One step = one pass over the 4096 tokens; inputs are resident in HBM
 before the timed region. Prints ONE JSON line.
 
-Other workloads (``--workload gdn_decode | gdn_prefill | moe``) time configs[2] and configs[3] with
+Other workloads (``--workload gdn_decode | moe | hybrid``) time configs[2], configs[3] and configs[4] with
 the same contract; they are extra lines for profiling, not the headline.
 """
 
@@ -218,12 +218,82 @@ def moe(args):
                          "kernel": "whole FFN (router + grouped GEMMs + combine)", "kernel_ms": ms}}
 
 
+def hybrid(args):
+    """BASELINE.json configs[4]: the 8-layer hybrid model. One step = one trainer scoring pass over
+    ``--seqs`` sequences of prompt + response tokens; the rollout's prefill and decode are timed beside it."""
+    import torch
+
+    from isoexec_amd.runtimes.hybrid import HybridConfig, HybridWeights, RolloutEngine, TrainerModel
+
+    dev = "cuda:0"
+    cfg = HybridConfig()
+    n, prompt, resp = args.seqs, args.prompt, args.response
+    w = HybridWeights.make(cfg, seed=0, device=dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(1)
+    tokens = torch.randint(0, cfg.vocab, (n * (prompt + resp),), device=dev, generator=g)
+    lens, plens = [prompt + resp] * n, [prompt] * n
+    trainer = TrainerModel(cfg, w)
+    fn = lambda: trainer.response_logprobs(tokens, lens, plens)
+    for _ in range(args.warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        fn()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    # rollout: prefill once, then timed decode steps at batch n
+    engine = RolloutEngine(cfg, w, max_num_seqs=n, max_len=prompt + resp)
+    slots = list(range(n))
+    prompts = tokens.view(n, -1)[:, :prompt].reshape(-1)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    x = engine.prefill(slots, prompts, plens)
+    torch.cuda.synchronize()
+    t_prefill = time.perf_counter() - t0
+    dec_steps = min(resp - 1, 64)
+    nxt = tokens.view(n, -1)[:, prompt:prompt + dec_steps]
+    from isoexec_amd.ops.logprobs.rowinv import full_forward, leaves
+    for sidx in range(4):
+        x = engine.decode(slots, nxt[:, sidx].contiguous())
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for sidx in range(4, dec_steps):
+        x = engine.decode(slots, nxt[:, sidx].contiguous())
+        full_forward(engine.blocks.logits(x), leaves())
+    torch.cuda.synchronize()
+    t_dec = (time.perf_counter() - t0) / (dec_steps - 4)
+    total = n * (prompt + resp)
+    # dense-equivalent flops per token: projections + experts (top-8) + router, and the LM head on scored rows
+    per_tok = 0
+    for i in range(cfg.layers):
+        if cfg.is_attention(i):
+            per_tok += 2 * cfg.hidden * ((cfg.q_heads + 2 * cfg.kv_heads) * cfg.head_dim + cfg.q_heads * cfg.head_dim)
+        else:
+            per_tok += 2 * cfg.hidden * (cfg.gdn_qkv + cfg.gdn_z + 2 * cfg.gdn_v_heads + cfg.gdn_z)
+        per_tok += 75.5e6
+    fl = total * per_tok + n * resp * 2 * cfg.hidden * cfg.vocab
+    return {"metric": "trainer-fwd tokens/s at bitwise parity (hybrid model)", "value": total / dt, "unit": "tokens/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt * 1e3, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": f"hybrid: 8 layers (3 GDN : 1 attention) + MoE, vocab 151936; {n} x ({prompt} + {resp}) tokens"},
+            "roofline": {"bound": "mfma", "achieved": fl / dt / 1e12, "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s",
+                         "frac": fl / dt / 1e12 / PEAK_MFMA_BF16_TFLOPS, "traffic": None,
+                         "kernel": "whole trainer pass (GEMM flops only; scans, attention and norms not counted)"},
+            "rollout": {"prefill_tokens_per_s": n * prompt / t_prefill, "decode_ms_per_step": t_dec * 1e3,
+                        "decode_tokens_per_s": n / t_dec, "batch": n}}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="dense_head", choices=["dense_head", "gdn_decode", "moe"])
+    ap.add_argument("--workload", default="dense_head", choices=["dense_head", "gdn_decode", "moe", "hybrid"])
+    ap.add_argument("--seqs", type=int, default=64)
+    ap.add_argument("--prompt", type=int, default=2048)
+    ap.add_argument("--response", type=int, default=512)
     ap.add_argument("--tokens", type=int, default=None)
     ap.add_argument("--batch", type=int, default=256)
     ap.add_argument("--tile", type=int, default=0)
@@ -240,7 +310,7 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(3)
-    out = {"dense_head": dense_head, "gdn_decode": gdn_decode, "moe": moe}[args.workload](args)
+    out = {"dense_head": dense_head, "gdn_decode": gdn_decode, "moe": moe, "hybrid": hybrid}[args.workload](args)
     print(json.dumps(out))
 
 

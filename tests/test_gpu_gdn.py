@@ -225,6 +225,15 @@ def test_conv_bit_exact_prefill_decode_and_state(dprims):
         outs.append(gdn_causal_conv_batched(xt.view(1, 1, D), w.to(DEV), b.to(DEV), initial_state=state)[0])
         state = torch.cat([state[..., 1:], xt.view(1, D, 1)], dim=-1)
     assert same_bits(torch.cat(outs), y[:12])
+    # The vector path (W = 4, D a multiple of 8) and the scalar path compute the same function: a width
+    # the vector path does not take, and a channel count it cannot.
+    for (D2, W2) in ((100, 4), (64, 3), (8, 2)):
+        x2 = torch.randn(19, D2, generator=g).to(torch.bfloat16)
+        w2 = (0.5 * torch.randn(D2, W2, generator=g)).to(torch.bfloat16)
+        b2 = (0.1 * torch.randn(D2, generator=g)).to(torch.bfloat16)
+        want_y, want_s = o_gdn.causal_conv(bf16_to_np(x2), bf16_to_np(w2), bf16_to_np(b2), prims=dprims)
+        y2, s2 = gdn_causal_conv(x2.to(DEV), w2.to(DEV), b2.to(DEV), return_final_state=True)
+        assert same_bits(y2.cpu(), np_to_bf16(want_y)) and same_bits(s2.cpu(), np_to_bf16(want_s)), (D2, W2)
 
 
 def test_native_core_varlen_equals_decode_steps():
