@@ -73,17 +73,44 @@ __device__ __forceinline__ float ix_tree8_max(const float (&a)[8]) {
 // group aligned to L). Step s adds lane^s; fp add is commutative, so both partners hold the
 // same bits after each step and every lane of the group ends with the tree's root:
 //   level 1: p[2i]+p[2i+1], level 2: those pairs, ...
-template <int L>
-__device__ __forceinline__ float ix_lane_tree(float v) {
-#pragma unroll
-  for (int s = 1; s < L; s <<= 1) v = v + __shfl_xor(v, s, IX_WAVE);
-  return v;
+// The value held by lane (lane ^ S). Distances below 16 stay inside a row of 16 lanes and use the
+// data-parallel-primitive lane controls of the vector ALU (no trip through the LDS crossbar):
+//   1, 2: quad permutes; 8: rotate the row by 8; 4: rotate by 12 or by 4, chosen by bit 2 of the lane.
+// Larger distances go through the cross-lane permute.
+template <int S>
+__device__ __forceinline__ float ix_xor_lane(float v) {
+  const int x = __float_as_int(v);
+  if constexpr (S == 1) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, x, 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+  } else if constexpr (S == 2) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, x, 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+  } else if constexpr (S == 4) {
+    const int up = __builtin_amdgcn_update_dpp(0, x, 0x12C, 0xF, 0xF, true);          // row_ror:12 -> lane i reads i+4
+    const int dn = __builtin_amdgcn_update_dpp(0, x, 0x124, 0xF, 0xF, true);          // row_ror:4  -> lane i reads i-4
+    return __int_as_float((threadIdx.x & 4) ? dn : up);
+  } else if constexpr (S == 8) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, x, 0x128, 0xF, 0xF, true));  // row_ror:8
+  } else {
+    return __shfl_xor(v, S, IX_WAVE);
+  }
 }
-template <int L>
+template <int L, int S = 1>
+__device__ __forceinline__ float ix_lane_tree(float v) {
+  if constexpr (S < L) {
+    v = v + ix_xor_lane<S>(v);
+    return ix_lane_tree<L, S * 2>(v);
+  } else {
+    return v;
+  }
+}
+template <int L, int S = 1>
 __device__ __forceinline__ float ix_lane_max(float v) {
-#pragma unroll
-  for (int s = 1; s < L; s <<= 1) v = fmaxf(v, __shfl_xor(v, s, IX_WAVE));
-  return v;
+  if constexpr (S < L) {
+    v = fmaxf(v, ix_xor_lane<S>(v));
+    return ix_lane_max<L, S * 2>(v);
+  } else {
+    return v;
+  }
 }
 
 // ---- 8-element group loads ----------------------------------------------------------------

@@ -53,7 +53,10 @@ __device__ __forceinline__ float ix_gdn_step(float (&S)[8], const float (&kk)[8]
   return ix_lane_tree<KS>(ix_dot8(S, qs));
 }
 
-template <int KS, typename TIO>
+// RPL state rows per lane group: lane group r of the workgroup owns rows r, r + 256/KS, ... Each row is
+// computed exactly as with RPL = 1 (same lanes per row, same order); holding several rows per lane only
+// shares the k/q fetch and gives the scheduler independent chains to interleave.
+template <int KS, int RPL, typename TIO>
 __global__ __launch_bounds__(256) void k_gdn_scan(const TIO* __restrict__ q, const TIO* __restrict__ k,
                                                   const TIO* __restrict__ v, const float* __restrict__ g,
                                                   const TIO* __restrict__ beta, TIO* __restrict__ o,
@@ -62,7 +65,8 @@ __global__ __launch_bounds__(256) void k_gdn_scan(const TIO* __restrict__ q, con
                                                   long k_pitch, long v_pitch, int H, int HV, int V, float scale,
                                                   int TT) {
   constexpr int K = KS * 8;
-  constexpr int R = 256 / KS;  // state rows per workgroup
+  constexpr int RW = 256 / KS;   // state rows per pass over the lanes
+  constexpr int R = RW * RPL;    // state rows per workgroup
   extern __shared__ __align__(16) char ix_lds[];
   float* kf = reinterpret_cast<float*>(ix_lds);  // [TT][K]
   float* qf = kf + TT * K;                       // [TT][K], pre-scaled
@@ -81,7 +85,7 @@ __global__ __launch_bounds__(256) void k_gdn_scan(const TIO* __restrict__ q, con
   const int h = hv / (HV / H);
   const int tid = threadIdx.x;
   const int sub = tid % KS, r = tid / KS;
-  const int vrow = vb * R + r;
+  const int vrow = vb * R + r;  // row of pass 0; pass j adds j * RW
 
   const int t_begin = cu[n], t_end = cu[n + 1];
   const int len = t_end - t_begin;
@@ -97,22 +101,43 @@ __global__ __launch_bounds__(256) void k_gdn_scan(const TIO* __restrict__ q, con
     return;
   }
 
-  float S[8];
-  {
-    const float* sp = state + (((long)row0 * HV + hv) * V + vrow) * K + sub * 8;
+  // q and k rows can be fetched 8 elements at a time when every row start is 16/32-byte aligned
+  constexpr long AL = 16 * sizeof(TIO) / 2;
+  const bool vec_qk = (q_pitch % 8 == 0) && (k_pitch % 8 == 0) && ((uintptr_t)q % AL == 0) && ((uintptr_t)k % AL == 0);
+  float S[RPL][8];
+#pragma unroll
+  for (int j = 0; j < RPL; ++j) {
+    const float* sp = state + (((long)row0 * HV + hv) * V + vrow + j * RW) * K + sub * 8;
     const float4 a = *reinterpret_cast<const float4*>(sp);
     const float4 b = *reinterpret_cast<const float4*>(sp + 4);
-    S[0] = a.x; S[1] = a.y; S[2] = a.z; S[3] = a.w; S[4] = b.x; S[5] = b.y; S[6] = b.z; S[7] = b.w;
+    S[j][0] = a.x; S[j][1] = a.y; S[j][2] = a.z; S[j][3] = a.w;
+    S[j][4] = b.x; S[j][5] = b.y; S[j][6] = b.z; S[j][7] = b.w;
   }
 
   for (int t0 = 0; t0 < len; t0 += TT) {
     const int nt = min(TT, len - t0);
     __syncthreads();
-    for (int i = tid; i < nt * K; i += 256) {
-      const int tt = i / K, kk = i % K;
-      const long tok = t_begin + t0 + tt;
-      kf[i] = ix_ld(k + tok * k_pitch + h * K + kk);
-      qf[i] = ix_ld(q + tok * q_pitch + h * K + kk) * scale;
+    if (vec_qk) {  // 8 elements (16 bytes) per load
+      for (int i = tid; i < nt * (K / 8); i += 256) {
+        const int tt = i / (K / 8), kk = (i % (K / 8)) * 8;
+        const long tok = t_begin + t0 + tt;
+        float a[8], b[8];
+        ix_load8(k + tok * k_pitch + h * K + kk, 8, true, 0.0f, a);
+        ix_load8(q + tok * q_pitch + h * K + kk, 8, true, 0.0f, b);
+        float* kd = kf + tt * K + kk;
+        float* qd = qf + tt * K + kk;
+        *reinterpret_cast<float4*>(kd) = make_float4(a[0], a[1], a[2], a[3]);
+        *reinterpret_cast<float4*>(kd + 4) = make_float4(a[4], a[5], a[6], a[7]);
+        *reinterpret_cast<float4*>(qd) = make_float4(b[0] * scale, b[1] * scale, b[2] * scale, b[3] * scale);
+        *reinterpret_cast<float4*>(qd + 4) = make_float4(b[4] * scale, b[5] * scale, b[6] * scale, b[7] * scale);
+      }
+    } else {
+      for (int i = tid; i < nt * K; i += 256) {
+        const int tt = i / K, kk = i % K;
+        const long tok = t_begin + t0 + tt;
+        kf[i] = ix_ld(k + tok * k_pitch + h * K + kk);
+        qf[i] = ix_ld(q + tok * q_pitch + h * K + kk) * scale;
+      }
     }
     for (int i = tid; i < nt * R; i += 256) {
       const int tt = i / R, rr = i % R;
@@ -135,13 +160,22 @@ __global__ __launch_bounds__(256) void k_gdn_scan(const TIO* __restrict__ q, con
         const float4 d = *reinterpret_cast<const float4*>(qf + tt * K + sub * 8 + 4);
         qs[0] = c.x; qs[1] = c.y; qs[2] = c.z; qs[3] = c.w; qs[4] = d.x; qs[5] = d.y; qs[6] = d.z; qs[7] = d.w;
       }
-      const float ov = ix_gdn_step<KS>(S, kk, qs, vf[tt * R + r], egf[tt], btf[tt]);
-      if (sub == 0) of[tt * R + r] = ov;
+      const float eg = egf[tt], bt = btf[tt];
+      float ov[RPL];
+#pragma unroll
+      for (int j = 0; j < RPL; ++j) ov[j] = ix_gdn_step<KS>(S[j], kk, qs, vf[tt * R + j * RW + r], eg, bt);
+      if (sub == 0) {
+#pragma unroll
+        for (int j = 0; j < RPL; ++j) of[tt * R + j * RW + r] = ov[j];
+      }
       const int si = sif[tt];
       if (si > 0) {
-        float* sp = state + (((long)si * HV + hv) * V + vrow) * K + sub * 8;
-        *reinterpret_cast<float4*>(sp) = make_float4(S[0], S[1], S[2], S[3]);
-        *reinterpret_cast<float4*>(sp + 4) = make_float4(S[4], S[5], S[6], S[7]);
+#pragma unroll
+        for (int j = 0; j < RPL; ++j) {
+          float* sp = state + (((long)si * HV + hv) * V + vrow + j * RW) * K + sub * 8;
+          *reinterpret_cast<float4*>(sp) = make_float4(S[j][0], S[j][1], S[j][2], S[j][3]);
+          *reinterpret_cast<float4*>(sp + 4) = make_float4(S[j][4], S[j][5], S[j][6], S[j][7]);
+        }
       }
     }
     __syncthreads();
@@ -156,17 +190,17 @@ static size_t ix_gdn_lds_bytes(int K, int R, int TT) {
   return (size_t)TT * (2 * K + 2 * R + 3) * sizeof(float);
 }
 
-template <int KS, typename TIO>
-static int ix_gdn_scan_launch(const void* q, const void* k, const void* v, const float* g, const void* beta,
-                              void* o, float* state, const int* cu, const int* sidx, long sidx_stride,
-                              long q_pitch, long k_pitch, long v_pitch, long N, int H, int HV, int V, float scale,
-                              int TT, hipStream_t st) {
-  constexpr int R = 256 / KS;
+template <int KS, int RPL, typename TIO>
+static int ix_gdn_scan_launch_rpl(const void* q, const void* k, const void* v, const float* g, const void* beta,
+                                  void* o, float* state, const int* cu, const int* sidx, long sidx_stride,
+                                  long q_pitch, long k_pitch, long v_pitch, long N, int H, int HV, int V, float scale,
+                                  int TT, hipStream_t st) {
+  constexpr int R = (256 / KS) * RPL;
   if (V % R != 0) return IX_DECLINED;
   const long grid = N * HV * (V / R);
   if (grid > 0x7fffffffL) return IX_DECLINED;
   const size_t lds = ix_gdn_lds_bytes(KS * 8, R, TT);
-  auto kern = k_gdn_scan<KS, TIO>;
+  auto kern = k_gdn_scan<KS, RPL, TIO>;
   if (lds > 48 * 1024) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return IX_ERR_LAUNCH;
@@ -175,6 +209,32 @@ static int ix_gdn_scan_launch(const void* q, const void* k, const void* v, const
                      (const TIO*)beta, (TIO*)o, state, cu, sidx, sidx_stride, q_pitch, k_pitch, v_pitch, H, HV, V,
                      scale, TT);
   return ix_launch_status();
+}
+
+// Rows per lane group: a staging choice like the time tile (bits 8.. of time_tile force it). More rows per
+// workgroup share each k/q fetch and interleave independent chains, but leave fewer workgroups.
+template <int KS, typename TIO>
+static int ix_gdn_scan_launch(const void* q, const void* k, const void* v, const float* g, const void* beta,
+                              void* o, float* state, const int* cu, const int* sidx, long sidx_stride,
+                              long q_pitch, long k_pitch, long v_pitch, long N, int H, int HV, int V, float scale,
+                              int TT, int rpl, hipStream_t st) {
+  constexpr int RW = 256 / KS;
+  if (V % RW != 0) return IX_DECLINED;
+  const long groups = N * HV * (V / RW);  // workgroups at one row per lane group
+  if (rpl <= 0) rpl = (V % (RW * 4) == 0 && groups >= 4 * 2048) ? 4 : (V % (RW * 2) == 0 && groups >= 2 * 1024) ? 2 : 1;
+  while (rpl > 1 && V % (RW * rpl) != 0) rpl >>= 1;
+#define IX_RPL_CASE(R_)                                                                                          \
+  case R_:                                                                                                       \
+    return ix_gdn_scan_launch_rpl<KS, R_, TIO>(q, k, v, g, beta, o, state, cu, sidx, sidx_stride, q_pitch, k_pitch, \
+                                               v_pitch, N, H, HV, V, scale, TT, st);
+  switch (rpl) {
+    IX_RPL_CASE(1)
+    IX_RPL_CASE(2)
+    IX_RPL_CASE(4)
+    default:
+      return IX_ERR_ARG;
+  }
+#undef IX_RPL_CASE
 }
 
 extern "C" int ix_gdn_scan(const void* q, const void* k, const void* v, const float* g, const void* beta, void* o,
@@ -187,7 +247,11 @@ extern "C" int ix_gdn_scan(const void* q, const void* k, const void* v, const fl
   if (io_dtype != IX_DT_F32 && io_dtype != IX_DT_BF16) return IX_DECLINED;
   if (N == 0) return IX_OK;
   if (!ix_aligned(state_pool, 16)) return IX_DECLINED;
-  int TT = time_tile <= 0 ? 32 : time_tile;
+  const int rpl = time_tile > 0 ? (time_tile >> 8) : 0;
+  // default time tile: short tiles keep more workgroups resident when there are many, long tiles
+  // amortise the staging when there are few
+  int TT = time_tile <= 0 ? 0 : (time_tile & 0xff);
+  if (TT <= 0) TT = (N * HV * (V / 16) >= 4096) ? 16 : 64;
   if (TT > 64) TT = 64;
   hipStream_t st = (hipStream_t)stream;
 #define IX_SCAN_CASE(KSV)                                                                                         \
@@ -195,10 +259,10 @@ extern "C" int ix_gdn_scan(const void* q, const void* k, const void* v, const fl
     if (io_dtype == IX_DT_BF16)                                                                                   \
       return ix_gdn_scan_launch<KSV, bf16_t>(q, k, v, g, beta, o, state_pool, cu_seqlens, state_indices,         \
                                              state_indices_stride, q_pitch, k_pitch, v_pitch, N, (int)H,         \
-                                             (int)HV, (int)V, scale, TT, st);                                    \
+                                             (int)HV, (int)V, scale, TT, rpl, st);                               \
     return ix_gdn_scan_launch<KSV, float>(q, k, v, g, beta, o, state_pool, cu_seqlens, state_indices,            \
                                           state_indices_stride, q_pitch, k_pitch, v_pitch, N, (int)H, (int)HV,   \
-                                          (int)V, scale, TT, st);                                                \
+                                          (int)V, scale, TT, rpl, st);                                           \
   }
   IX_SCAN_CASE(4)
   IX_SCAN_CASE(8)

@@ -222,3 +222,10 @@ def test_compact_state_index_form_equals_the_full_map(dprims):
         pools.append(pool)
     assert same_bits(outs[0], outs[1]) and same_bits(pools[0], pools[1])
     assert same_bits(pools[0][3], start[3].to(DEV)) and not same_bits(pools[0][4], start[4].to(DEV))
+    # Rows held per lane group (1, 2, 4) and the time tile are staging choices: same bits.
+    for rpl in (1, 2, 4):
+        for tt in (16, 64):
+            pool = start.clone().to(DEV)
+            got = gdn_recurrent_kernel(bf(q), bf(k), bf(v), gate.to(DEV), bf(beta), ssm_state=pool, state_indices=rows,
+                                       cu_seqlens=cu, time_tile=tt | (rpl << 8))
+            assert same_bits(got, outs[0]) and same_bits(pool, pools[0]), (rpl, tt)
