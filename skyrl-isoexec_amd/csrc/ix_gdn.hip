@@ -150,7 +150,7 @@ __global__ __launch_bounds__(256) void k_gdn_scan(const TIO* __restrict__ q, con
       sif[i] = sidx_stride == 0 ? (t0 + i == len - 1 ? row0 : 0) : sidx[sbase + t0 + i];
     }
     __syncthreads();
-    for (int tt = 0; tt < nt; ++tt) {
+    auto token = [&](int tt) {
       float kk[8], qs[8];
       {
         const float4 a = *reinterpret_cast<const float4*>(kf + tt * K + sub * 8);
@@ -168,14 +168,25 @@ __global__ __launch_bounds__(256) void k_gdn_scan(const TIO* __restrict__ q, con
 #pragma unroll
         for (int j = 0; j < RPL; ++j) of[tt * R + j * RW + r] = ov[j];
       }
-      const int si = sif[tt];
-      if (si > 0) {
+    };
+    auto store_state = [&](int si) {
 #pragma unroll
-        for (int j = 0; j < RPL; ++j) {
-          float* sp = state + (((long)si * HV + hv) * V + vrow + j * RW) * K + sub * 8;
-          *reinterpret_cast<float4*>(sp) = make_float4(S[j][0], S[j][1], S[j][2], S[j][3]);
-          *reinterpret_cast<float4*>(sp + 4) = make_float4(S[j][4], S[j][5], S[j][6], S[j][7]);
-        }
+      for (int j = 0; j < RPL; ++j) {
+        float* sp = state + (((long)si * HV + hv) * V + vrow + j * RW) * K + sub * 8;
+        *reinterpret_cast<float4*>(sp) = make_float4(S[j][0], S[j][1], S[j][2], S[j][3]);
+        *reinterpret_cast<float4*>(sp + 4) = make_float4(S[j][4], S[j][5], S[j][6], S[j][7]);
+      }
+    };
+    if (sidx_stride == 0) {
+      // one store, after the sequence's last token: the token loop carries no per-token check
+#pragma unroll 4
+      for (int tt = 0; tt < nt; ++tt) token(tt);
+      if (t0 + nt == len) store_state(row0);
+    } else {
+      for (int tt = 0; tt < nt; ++tt) {
+        token(tt);
+        const int si = sif[tt];
+        if (si > 0) store_state(si);
       }
     }
     __syncthreads();
@@ -221,7 +232,7 @@ static int ix_gdn_scan_launch(const void* q, const void* k, const void* v, const
   constexpr int RW = 256 / KS;
   if (V % RW != 0) return IX_DECLINED;
   const long groups = N * HV * (V / RW);  // workgroups at one row per lane group
-  if (rpl <= 0) rpl = (V % (RW * 4) == 0 && groups >= 4 * 2048) ? 4 : (V % (RW * 2) == 0 && groups >= 2 * 1024) ? 2 : 1;
+  if (rpl <= 0) rpl = (V % (RW * 2) == 0 && groups >= 2 * 1024) ? 2 : 1;  // measured: 4 rows gain nothing over 2
   while (rpl > 1 && V % (RW * rpl) != 0) rpl >>= 1;
 #define IX_RPL_CASE(R_)                                                                                          \
   case R_:                                                                                                       \
