@@ -264,6 +264,18 @@ def hybrid(args):
         full_forward(engine.blocks.logits(x), leaves())
     torch.cuda.synchronize()
     t_dec = (time.perf_counter() - t0) / (dec_steps - 4)
+    # the same steps replayed from a captured graph
+    graph = engine.capture_decode(slots)
+    more = tokens.view(n, -1)[:, prompt + dec_steps:prompt + dec_steps + 40]
+    for sidx in range(4):
+        graph.step(more[:, sidx].contiguous())
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for sidx in range(4, 40):
+        x = graph.step(more[:, sidx].contiguous())
+        full_forward(engine.blocks.logits(x), leaves())
+    torch.cuda.synchronize()
+    t_graph = (time.perf_counter() - t0) / 36
     total = n * (prompt + resp)
     # dense-equivalent flops per token: projections + experts (top-8) + router, and the LM head on scored rows
     per_tok = 0
@@ -282,7 +294,8 @@ def hybrid(args):
                          "frac": fl / dt / 1e12 / PEAK_MFMA_BF16_TFLOPS, "traffic": None,
                          "kernel": "whole trainer pass (GEMM flops only; scans, attention and norms not counted)"},
             "rollout": {"prefill_tokens_per_s": n * prompt / t_prefill, "decode_ms_per_step": t_dec * 1e3,
-                        "decode_tokens_per_s": n / t_dec, "batch": n}}
+                        "decode_tokens_per_s": n / t_dec, "graph_decode_ms_per_step": t_graph * 1e3,
+                        "graph_decode_tokens_per_s": n / t_graph, "batch": n}}
 
 
 def main():

@@ -128,14 +128,19 @@ static int ix_gemm_bf16_launch(const bf16_t* A, long lda, const bf16_t* W, long 
   return ix_launch_status();
 }
 
-static int ix_gemm_tile_for(long M, int tile) {
+// Which tile shape runs (0 = choose). Few rows means the launch is a weight stream: what matters is enough
+// workgroups to pull it, so a narrow output (small N) takes the 64 x 32 tile. Never changes a bit.
+static int ix_gemm_tile_for(long M, long N, int tile) {
   if (tile != 0) return tile;
-  return (M <= 32) ? 1 : (M <= 128) ? 2 : 3;
+  if (M > 128) return 3;
+  if (M <= 32 && (N + 255) / 256 >= 192) return 1;
+  if (M > 32 && ((M + 127) / 128) * ((N + 127) / 128) >= 192) return 2;
+  return 6;
 }
 
 extern "C" long ix_gemm_bf16_n_tiles(long M, long N, int tile) {
-  const int t = ix_gemm_tile_for(M, tile);
-  const long bn = (t == 2) ? 128 : 256;
+  const int t = ix_gemm_tile_for(M, N, tile);
+  const long bn = (t == 2) ? 128 : (t == 6) ? 32 : 256;
   return N <= 0 ? 0 : (N + bn - 1) / bn;
 }
 
@@ -144,12 +149,13 @@ static int ix_gemm_bf16_dispatch(const bf16_t* a, long lda, const bf16_t* w, lon
                                  long ldc, long M, long N, long K, int tile, float* parts, long parts_ld,
                                  hipStream_t st) {
   // `tile` only picks which workgroup owns an element (0 = by M); the bits do not depend on it.
-  switch (ix_gemm_tile_for(M, tile)) {
+  switch (ix_gemm_tile_for(M, N, tile)) {
     case 1: return ix_gemm_bf16_launch<32, 256, 1, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
     case 2: return ix_gemm_bf16_launch<128, 128, 2, 2, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
     case 3: return ix_gemm_bf16_launch<256, 256, 2, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
     case 4: return ix_gemm_bf16_launch<256, 256, 2, 2, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
     case 5: return ix_gemm_bf16_launch<128, 256, 2, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
+    case 6: return ix_gemm_bf16_launch<64, 32, 2, 1, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
     default: return IX_ERR_ARG;
   }
 }

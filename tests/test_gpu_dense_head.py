@@ -91,7 +91,7 @@ def test_add_rmsnorm_bit_exact():
 
 
 # ---- dense GEMM ----------------------------------------------------------------------------------
-@pytest.mark.parametrize("tile", [1, 2, 3, 5])
+@pytest.mark.parametrize("tile", [1, 2, 3, 4, 5, 6])
 def test_gemm_small_integer_known_answer(tile):
     """Small-integer operands: every partial sum is exact in fp32, so any correct kernel returns
     exactly the integer matmul. Catches a wrong fragment layout, a dropped k-slice, a bad tail."""
@@ -134,7 +134,7 @@ def test_gemm_row_bits_independent_of_M_and_tile():
     a = torch.randn(513, K, generator=g).to(torch.bfloat16).to(DEV)
     w = (0.02 * torch.randn(N, K, generator=g)).to(torch.bfloat16).to(DEV)
     ref = linear_nt(a, w, tile=3)
-    for tile in (1, 2, 5):
+    for tile in (1, 2, 4, 5, 6):
         assert same_bits(linear_nt(a, w, tile=tile), ref)
     for M in (1, 7, 64):
         assert same_bits(linear_nt(a[:M].contiguous(), w), ref[:M])
@@ -155,7 +155,7 @@ def test_gemm_fp32_out_row_max_and_fused_head(dprims):
     wl = (0.05 * torch.randn(V, K, generator=g)).to(torch.bfloat16).to(DEV)
     t = torch.randint(0, V, (M,), generator=g).to(DEV)
     x = fused_rms_norm_gamma(h, wn, 1e-6)
-    for tile in (1, 2, 3, 5):
+    for tile in (1, 2, 3, 4, 5, 6):
         c16, rm = linear_nt(x, wl, tile=tile, want_row_max=True)
         c32, rm32 = linear_nt(x, wl, tile=tile, out_dtype=torch.float32, want_row_max=True)
         assert same_bits(c32.to(torch.bfloat16), c16)
