@@ -345,6 +345,9 @@ __device__ __forceinline__ void ix_gemm_mainloop_units(ix_rsrc_t x_rsrc, const X
 
   ix_bf16x8 xa[Cfg::MI], wa[Cfg::NI], xb[Cfg::MI], wb[Cfg::NI];
   auto frags = [&](const char* xs, const char* ws, int s, ix_bf16x8* xf, ix_bf16x8* wf) {
+#ifdef IX_EXPERIMENT_NO_FRAG
+    return;
+#endif
 #pragma unroll
     for (int mi = 0; mi < Cfg::MI; ++mi) xf[mi] = *reinterpret_cast<const ix_bf16x8*>(xs + (x_foff[mi] ^ (s << 4)));
 #pragma unroll
