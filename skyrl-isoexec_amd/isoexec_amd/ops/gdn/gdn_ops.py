@@ -38,6 +38,20 @@ def _flatten_tokens(t: torch.Tensor, tail: int) -> torch.Tensor:
     return t.reshape(b * n, *t.shape[2:])
 
 
+_CU_CACHE: dict = {}
+
+
+def _uniform_cu(batch: int, length: int, device) -> torch.Tensor:
+    """Token offsets of ``batch`` sequences of equal ``length``; cached, so a decode loop creates none."""
+    key = (batch, length, str(device))
+    cu = _CU_CACHE.get(key)
+    if cu is None:
+        if len(_CU_CACHE) > 64:
+            _CU_CACHE.clear()
+        cu = _CU_CACHE[key] = torch.arange(0, (batch + 1) * length, length, dtype=torch.int32, device=device)
+    return cu
+
+
 def gdn_recurrent_kernel(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -72,7 +86,7 @@ def gdn_recurrent_kernel(
         raise RuntimeError("[isoexec-amd] q/k/v must share a dtype")
     dev = q.device
     if cu_seqlens is None:
-        cu = torch.arange(0, (B + 1) * T, T, dtype=torch.int32, device=dev)
+        cu = _uniform_cu(B, T, dev)
         n_seq = B
     else:
         if B != 1:
