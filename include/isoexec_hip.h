@@ -171,10 +171,11 @@ int ix_gdn_gate(const void* a, const void* b, const float* A_log, const float* d
 
 /* gdn_causal_conv / gdn_causal_conv_batched (gdn_ops.py:74-170) over packed tokens, and the
  * engine's window-slide update (gdn_recurrent_state.py:686-707,814-825) when every sequence has
- * one token. x,y bf16 [tokens, D]; weight bf16 [D, W]; bias bf16 [D] or NULL; conv_pool bf16
+ * one token. x bf16 [tokens, D] with token pitch x_pitch (elements; a slice of a wider projection buffer needs
+ * no copy), y bf16 [tokens, D] contiguous; weight bf16 [D, W]; bias bf16 [D] or NULL; conv_pool bf16
  * [rows, D, W-1] oldest first. state_rows_in[n] <= 0 (or NULL) = no history; state_rows_out[n]
  * > 0 stores the last W-1 inputs to that row (may equal the input row). */
-int ix_gdn_conv(const void* x, const void* weight, const void* bias, void* y, void* conv_pool,
+int ix_gdn_conv(const void* x, long x_pitch, const void* weight, const void* bias, void* y, void* conv_pool,
                 const int* cu_seqlens, const int* state_rows_in, const int* state_rows_out, long N,
                 long total_tokens, long D, long W, int silu, void* stream);
 

@@ -385,15 +385,17 @@ __device__ __forceinline__ int ix_seq_of(const int* __restrict__ cu, int N, int 
   return lo;
 }
 
-__device__ __forceinline__ float ix_conv_xp(const bf16_t* __restrict__ x, const bf16_t* __restrict__ pool,
-                                            int srow, int t_begin, int rel, long D, int d, int W) {
+__device__ __forceinline__ float ix_conv_xp(const bf16_t* __restrict__ x, long x_pitch,
+                                            const bf16_t* __restrict__ pool, int srow, int t_begin, int rel, long D,
+                                            int d, int W) {
   // rel: position relative to the sequence start; negative -> history slot W-1+rel
-  if (rel >= 0) return ix_bf2f(x[(long)(t_begin + rel) * D + d]);
+  if (rel >= 0) return ix_bf2f(x[(long)(t_begin + rel) * x_pitch + d]);
   if (srow <= 0) return 0.0f;
   return ix_bf2f(pool[((long)srow * D + d) * (W - 1) + (W - 1 + rel)]);
 }
 
-__global__ __launch_bounds__(256) void k_gdn_conv(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+__global__ __launch_bounds__(256) void k_gdn_conv(const bf16_t* __restrict__ x, long x_pitch,
+                                                  const bf16_t* __restrict__ w,
                                                   const bf16_t* __restrict__ bias, bf16_t* __restrict__ y,
                                                   const bf16_t* __restrict__ pool, const int* __restrict__ cu,
                                                   const int* __restrict__ rows_in, int N, long D, int W,
@@ -409,7 +411,7 @@ __global__ __launch_bounds__(256) void k_gdn_conv(const bf16_t* __restrict__ x, 
   const int srow = rows_in ? rows_in[n] : 0;
   float acc = 0.0f;
   for (int j = 0; j < W; ++j) {
-    const float xv = ix_conv_xp(x, pool, srow, t_begin, rel - (W - 1) + j, D, d, W);
+    const float xv = ix_conv_xp(x, x_pitch, pool, srow, t_begin, rel - (W - 1) + j, D, d, W);
     const float p = ix_bf2f(w[(long)d * W + j]) * xv;
     acc = acc + p;
   }
@@ -418,50 +420,13 @@ __global__ __launch_bounds__(256) void k_gdn_conv(const bf16_t* __restrict__ x, 
   y[i] = ix_f2bf(acc);
 }
 
-// Eight consecutive channels of one token per thread: 16-byte loads and stores. Per channel the
-// arithmetic is that of k_gdn_conv, statement for statement, so the two kernels agree bit for bit.
+// Eight consecutive channels of four consecutive tokens per thread: 16-byte loads and stores, and inside a
+// sequence each input row is loaded once for the four windows that cover it. Per channel the arithmetic is that
+// of k_gdn_conv, statement for statement, so the two kernels agree bit for bit.
 template <int W>
-__global__ __launch_bounds__(256) void k_gdn_conv8(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                   const bf16_t* __restrict__ bias, bf16_t* __restrict__ y,
-                                                   const bf16_t* __restrict__ pool, const int* __restrict__ cu,
-                                                   const int* __restrict__ rows_in, int N, long D, int silu,
-                                                   long total8) {
-  const long i = ((long)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
-  if (i >= total8) return;
-  const long D8 = D >> 3;
-  const int t = (int)(i / D8);
-  const int d = (int)(i % D8) * 8;
-  const int n = ix_seq_of(cu, N, t);
-  const int t_begin = cu[n];
-  const int rel = t - t_begin;
-  const int srow = rows_in ? rows_in[n] : 0;
-  float xv[W][8];
-#pragma unroll
-  for (int j = 0; j < W; ++j) {
-    const int r = rel - (W - 1) + j;
-    if (r >= 0) {
-      const uint4 u = *reinterpret_cast<const uint4*>(x + (long)(t_begin + r) * D + d);
-      const uint32_t q[4] = {u.x, u.y, u.z, u.w};
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        xv[j][2 * c] = __uint_as_float(q[c] << 16);
-        xv[j][2 * c + 1] = __uint_as_float(q[c] & 0xffff0000u);
-      }
-    } else {
-#pragma unroll
-      for (int c = 0; c < 8; ++c)
-        xv[j][c] = srow > 0 ? ix_bf2f(pool[((long)srow * D + d + c) * (W - 1) + (W - 1 + r)]) : 0.0f;
-    }
-  }
-  // weights of 8 channels: 8*W consecutive bf16
-  float wv[8][W];
-  {
-    const bf16_t* wp = w + (long)d * W;
-#pragma unroll
-    for (int c = 0; c < 8; ++c)
-#pragma unroll
-      for (int j = 0; j < W; ++j) wv[c][j] = ix_bf2f(wp[c * W + j]);
-  }
+__device__ __forceinline__ void ix_conv8_finish(const float (&xv)[W][8], const float (&wv)[8][W],
+                                                const bf16_t* __restrict__ bias, int d, int silu,
+                                                bf16_t* __restrict__ yrow) {
   uint32_t out[4];
 #pragma unroll
   for (int c = 0; c < 8; c += 2) {
@@ -480,10 +445,81 @@ __global__ __launch_bounds__(256) void k_gdn_conv8(const bf16_t* __restrict__ x,
     }
     out[c >> 1] = ix_pack_bf2(r2[0], r2[1]);
   }
-  *reinterpret_cast<uint4*>(y + (long)t * D + d) = make_uint4(out[0], out[1], out[2], out[3]);
+  *reinterpret_cast<uint4*>(yrow) = make_uint4(out[0], out[1], out[2], out[3]);
 }
 
-__global__ __launch_bounds__(256) void k_gdn_conv_state(const bf16_t* __restrict__ x, bf16_t* __restrict__ pool,
+__device__ __forceinline__ void ix_unpack8(const uint4 u, float (&o)[8]) {
+  const uint32_t q[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    o[2 * c] = __uint_as_float(q[c] << 16);
+    o[2 * c + 1] = __uint_as_float(q[c] & 0xffff0000u);
+  }
+}
+
+template <int W, int TOK>
+__global__ __launch_bounds__(256) void k_gdn_conv8(const bf16_t* __restrict__ x, long x_pitch,
+                                                   const bf16_t* __restrict__ w, const bf16_t* __restrict__ bias,
+                                                   bf16_t* __restrict__ y, const bf16_t* __restrict__ pool,
+                                                   const int* __restrict__ cu, const int* __restrict__ rows_in,
+                                                   int N, long D, int silu, int T, long total) {
+  const long i = ((long)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
+  if (i >= total) return;
+  const long D8 = D >> 3;
+  const int t0 = (int)(i / D8) * TOK;
+  const int d = (int)(i % D8) * 8;
+  float wv[8][W];
+  {
+    const bf16_t* wp = w + (long)d * W;
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+#pragma unroll
+      for (int j = 0; j < W; ++j) wv[c][j] = ix_bf2f(wp[c * W + j]);
+  }
+  const int n0 = ix_seq_of(cu, N, t0);
+  const int b0 = cu[n0], e0 = cu[n0 + 1];
+  if (t0 - (W - 1) >= b0 && t0 + TOK <= e0) {
+    // all TOK windows lie inside one sequence: TOK + W - 1 rows serve TOK outputs
+    float xr[TOK + W - 1][8];
+#pragma unroll
+    for (int r = 0; r < TOK + W - 1; ++r)
+      ix_unpack8(*reinterpret_cast<const uint4*>(x + (long)(t0 - (W - 1) + r) * x_pitch + d), xr[r]);
+#pragma unroll
+    for (int q = 0; q < TOK; ++q) {
+      float xv[W][8];
+#pragma unroll
+      for (int j = 0; j < W; ++j)
+#pragma unroll
+        for (int c = 0; c < 8; ++c) xv[j][c] = xr[q + j][c];
+      ix_conv8_finish<W>(xv, wv, bias, d, silu, y + (long)(t0 + q) * D + d);
+    }
+    return;
+  }
+  for (int q = 0; q < TOK; ++q) {
+    const int t = t0 + q;
+    if (t >= T) break;
+    const int n = ix_seq_of(cu, N, t);
+    const int t_begin = cu[n];
+    const int rel = t - t_begin;
+    const int srow = rows_in ? rows_in[n] : 0;
+    float xv[W][8];
+#pragma unroll
+    for (int j = 0; j < W; ++j) {
+      const int r = rel - (W - 1) + j;
+      if (r >= 0) {
+        ix_unpack8(*reinterpret_cast<const uint4*>(x + (long)(t_begin + r) * x_pitch + d), xv[j]);
+      } else {
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+          xv[j][c] = srow > 0 ? ix_bf2f(pool[((long)srow * D + d + c) * (W - 1) + (W - 1 + r)]) : 0.0f;
+      }
+    }
+    ix_conv8_finish<W>(xv, wv, bias, d, silu, y + (long)t * D + d);
+  }
+}
+
+__global__ __launch_bounds__(256) void k_gdn_conv_state(const bf16_t* __restrict__ x, long x_pitch,
+                                                        bf16_t* __restrict__ pool,
                                                         const int* __restrict__ cu,
                                                         const int* __restrict__ rows_in,
                                                         const int* __restrict__ rows_out, int N, long D, int W) {
@@ -498,40 +534,43 @@ __global__ __launch_bounds__(256) void k_gdn_conv_state(const bf16_t* __restrict
   bf16_t tmp[8];
   for (int j = 0; j < W - 1; ++j) {
     // new history slot j holds the input at relative position len - (W-1) + j
-    const float xv = ix_conv_xp(x, pool, srow, t_begin, len - (W - 1) + j, D, d, W);
+    const float xv = ix_conv_xp(x, x_pitch, pool, srow, t_begin, len - (W - 1) + j, D, d, W);
     tmp[j] = ix_f2bf(xv);  // exact: the value is a bf16 already
   }
   for (int j = 0; j < W - 1; ++j) pool[((long)orow * D + d) * (W - 1) + j] = tmp[j];
 }
 
-extern "C" int ix_gdn_conv(const void* x, const void* weight, const void* bias, void* y, void* conv_pool,
-                           const int* cu_seqlens, const int* state_rows_in, const int* state_rows_out, long N,
-                           long total_tokens, long D, long W, int silu, void* stream) {
-  if (!x || !weight || !y || !cu_seqlens || N < 0 || total_tokens < 0 || D <= 0) return IX_ERR_ARG;
+extern "C" int ix_gdn_conv(const void* x, long x_pitch, const void* weight, const void* bias, void* y,
+                           void* conv_pool, const int* cu_seqlens, const int* state_rows_in,
+                           const int* state_rows_out, long N, long total_tokens, long D, long W, int silu,
+                           void* stream) {
+  if (!x || !weight || !y || !cu_seqlens || N < 0 || total_tokens < 0 || D <= 0 || x_pitch < D) return IX_ERR_ARG;
   if (W < 1 || W > 8) return IX_DECLINED;
   if ((state_rows_in || state_rows_out) && !conv_pool) return IX_ERR_ARG;
   if (total_tokens > 0x7fffffffL || N > 0x7fffffffL) return IX_DECLINED;
   hipStream_t st = (hipStream_t)stream;
   const long total = total_tokens * D;
   if (total > 0 && N > 0) {
-    const bool vec8 = (W == 4) && (D % 8 == 0) && ix_aligned(x, 16) && ix_aligned(y, 16);
-    const long blocks = ((vec8 ? total / 8 : total) + 255) / 256;
+    constexpr int TOK = 4;
+    const bool vec8 = (W == 4) && (D % 8 == 0) && (x_pitch % 8 == 0) && ix_aligned(x, 16) && ix_aligned(y, 16);
+    const long work = vec8 ? ((total_tokens + TOK - 1) / TOK) * (D / 8) : total;
+    const long blocks = (work + 255) / 256;
     const long gx = blocks < (1L << 22) ? blocks : (1L << 22);
     const long gy = (blocks + gx - 1) / gx;
     if (gy > 65535) return IX_DECLINED;
     if (vec8)
-      hipLaunchKernelGGL(k_gdn_conv8<4>, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st, (const bf16_t*)x,
-                         (const bf16_t*)weight, (const bf16_t*)bias, (bf16_t*)y, (const bf16_t*)conv_pool, cu_seqlens,
-                         state_rows_in, (int)N, D, silu, total / 8);
+      hipLaunchKernelGGL((k_gdn_conv8<4, TOK>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st, (const bf16_t*)x,
+                         x_pitch, (const bf16_t*)weight, (const bf16_t*)bias, (bf16_t*)y, (const bf16_t*)conv_pool,
+                         cu_seqlens, state_rows_in, (int)N, D, silu, (int)total_tokens, work);
     else
-    hipLaunchKernelGGL(k_gdn_conv, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st, (const bf16_t*)x, (const bf16_t*)weight,
-                       (const bf16_t*)bias, (bf16_t*)y, (const bf16_t*)conv_pool, cu_seqlens, state_rows_in, (int)N,
-                       D, (int)W, silu, total);
+      hipLaunchKernelGGL(k_gdn_conv, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st, (const bf16_t*)x, x_pitch,
+                         (const bf16_t*)weight, (const bf16_t*)bias, (bf16_t*)y, (const bf16_t*)conv_pool, cu_seqlens,
+                         state_rows_in, (int)N, D, (int)W, silu, total);
   }
   if (state_rows_out && N > 0 && W > 1) {
     const long grid = (N * D + 255) / 256;
     if (grid > 0x7fffffffL) return IX_DECLINED;
-    hipLaunchKernelGGL(k_gdn_conv_state, dim3((unsigned)grid), dim3(256), 0, st, (const bf16_t*)x,
+    hipLaunchKernelGGL(k_gdn_conv_state, dim3((unsigned)grid), dim3(256), 0, st, (const bf16_t*)x, x_pitch,
                        (bf16_t*)conv_pool, cu_seqlens, state_rows_in, state_rows_out, (int)N, D, (int)W);
   }
   return ix_launch_status();

@@ -163,14 +163,16 @@ def conv_packed(x, weight, bias, *, cu_seqlens, conv_state=None, rows_in=None, r
     W = weight.shape[-1]
     if weight.shape[0] != D:
         raise ValueError(f"weight {tuple(weight.shape)} incompatible with x dim {D}")
-    xc, wc = x.contiguous(), weight.contiguous()
-    y = torch.empty_like(xc)
+    # x may be a column slice of a wider buffer (row pitch > D); only its rows must be unit-stride
+    xc = x if x.stride(1) == 1 and x.stride(0) >= D else x.contiguous()
+    wc = weight.contiguous()
+    y = torch.empty(T, D, dtype=x.dtype, device=x.device)
     n_seq = cu_seqlens.numel() - 1
     rc = _lib.check(
-        _lib.lib().ix_gdn_conv(xc.data_ptr(), wc.data_ptr(), _lib.ptr(None if bias is None else bias.contiguous()),
-                               y.data_ptr(), _lib.ptr(conv_state), cu_seqlens.data_ptr(), _lib.ptr(rows_in),
-                               _lib.ptr(rows_out), n_seq, T, D, W, int(activation is not None),
-                               _lib.current_stream(x.device)), "ix_gdn_conv")
+        _lib.lib().ix_gdn_conv(xc.data_ptr(), xc.stride(0), wc.data_ptr(),
+                               _lib.ptr(None if bias is None else bias.contiguous()), y.data_ptr(), _lib.ptr(conv_state),
+                               cu_seqlens.data_ptr(), _lib.ptr(rows_in), _lib.ptr(rows_out), n_seq, T, D, W,
+                               int(activation is not None), _lib.current_stream(x.device)), "ix_gdn_conv")
     if rc != _lib.IX_OK:
         raise RuntimeError(f"[isoexec-amd] ix_gdn_conv declined W={W}")
     return y

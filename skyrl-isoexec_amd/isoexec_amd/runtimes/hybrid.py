@@ -129,10 +129,10 @@ class _Blocks:
         return self.w.embed.index_select(0, tokens)
 
     def gdn_in(self, layer: int, x: torch.Tensor):
-        """-> pre-conv ``qkv [T, D]`` (contiguous), and views ``z [T, HV, V]``, ``b``, ``a [T, HV]``."""
+        """-> views of one projection buffer: pre-conv ``qkv [T, D]``, ``z [T, HV, V]``, ``b``, ``a [T, HV]``."""
         c = self.cfg
         proj = _linear(x, self.w.layers[layer]["in_proj"])
-        qkv = proj[:, : c.gdn_qkv].contiguous()
+        qkv = proj[:, : c.gdn_qkv]
         z = proj[:, c.gdn_qkv : c.gdn_qkv + c.gdn_z].unflatten(1, (c.gdn_v_heads, c.gdn_head_dim))
         b = proj[:, c.gdn_qkv + c.gdn_z : c.gdn_qkv + c.gdn_z + c.gdn_v_heads]
         a = proj[:, c.gdn_qkv + c.gdn_z + c.gdn_v_heads :]
