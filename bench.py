@@ -218,6 +218,60 @@ def moe(args):
                          "kernel": "whole FFN (router + grouped GEMMs + combine)", "kernel_ms": ms}}
 
 
+def attention(args):
+    """Causal grouped-query attention, config 4 layout: ``--seqs`` sequences of prompt + response tokens packed
+    (prefill shape), then one decode step for the same sequences out of a key/value cache."""
+    import torch
+
+    from isoexec_amd.ops.attention.varlen_attn import KVCache, varlen_attention
+
+    dev = "cuda:0"
+    n, L, HQ, HKV, D = args.seqs, args.prompt + args.response, 32, 4, 128
+    q = torch.randn(n * L, HQ, D, device=dev).to(torch.bfloat16)
+    k = torch.randn(n * L, HKV, D, device=dev).to(torch.bfloat16)
+    v = torch.randn(n * L, HKV, D, device=dev).to(torch.bfloat16)
+    cu = torch.arange(0, (n + 1) * L, L, dtype=torch.int32, device=dev)
+    fn = lambda: varlen_attention(q, k, v, cu, L)
+    timer = KernelTimer()
+    for _ in range(args.warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        timer(fn)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    ms = timer.mean_ms()
+    fl = n * 4.0 * (L * (L + 1) / 2) * HQ * D  # QK^T and PV over the causal half
+    # decode: one query per sequence against L cached keys
+    cache = KVCache(n, L, HKV, D, device=dev)
+    cache.k[1:].copy_(k.view(n, L, HKV, D))
+    cache.v[1:].copy_(v.view(n, L, HKV, D))
+    kf, vf = cache.flat()
+    qd = q.view(n, L, HQ, D)[:, -1].contiguous()
+    cud = torch.arange(n + 1, dtype=torch.int32, device=dev)
+    kv_start = torch.arange(1, n + 1, dtype=torch.int64, device=dev) * L
+    pos0 = torch.full((n,), L - 1, dtype=torch.int32, device=dev)
+    dec = lambda: varlen_attention(qd, kf, vf, cud, 1, kv_start=kv_start, q_pos0=pos0)
+    tdec = KernelTimer()
+    for _ in range(3):
+        dec()
+    for _ in range(20):
+        tdec(dec)
+    torch.cuda.synchronize()
+    dms = tdec.mean_ms()
+    dbytes = n * L * HKV * D * 2 * 2
+    return {"metric": "attention prefill tokens/s", "value": n * L / dt, "unit": "tokens/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt * 1e3, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": f"attention: {n} x {L} tokens, 32 query / 4 kv heads, d 128, causal, one key walk"},
+            "roofline": {"bound": "mfma", "achieved": fl / (ms * 1e-3) / 1e12, "peak": PEAK_MFMA_BF16_TFLOPS,
+                         "unit": "TFLOP/s", "frac": fl / (ms * 1e-3) / 1e12 / PEAK_MFMA_BF16_TFLOPS, "traffic": None,
+                         "kernel": "k_attn_varlen<8>", "kernel_ms": ms},
+            "decode": {"bound": "hbm", "kernel_ms": dms, "achieved": dbytes / (dms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                       "unit": "GB/s", "frac": dbytes / (dms * 1e-3) / 1e9 / PEAK_HBM_GBS, "batch": n, "context": L}}
+
+
 def hybrid(args):
     """BASELINE.json configs[4]: the 8-layer hybrid model. One step = one trainer scoring pass over
     ``--seqs`` sequences of prompt + response tokens; the rollout's prefill and decode are timed beside it."""
@@ -303,7 +357,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="dense_head", choices=["dense_head", "gdn_decode", "moe", "hybrid"])
+    ap.add_argument("--workload", default="dense_head", choices=["dense_head", "gdn_decode", "moe", "hybrid", "attention"])
     ap.add_argument("--seqs", type=int, default=64)
     ap.add_argument("--prompt", type=int, default=2048)
     ap.add_argument("--response", type=int, default=512)
@@ -323,7 +377,7 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(3)
-    out = {"dense_head": dense_head, "gdn_decode": gdn_decode, "moe": moe, "hybrid": hybrid}[args.workload](args)
+    out = {"dense_head": dense_head, "gdn_decode": gdn_decode, "moe": moe, "hybrid": hybrid, "attention": attention}[args.workload](args)
     print(json.dumps(out))
 
 

@@ -27,41 +27,52 @@ typedef __attribute__((ext_vector_type(16))) float ix_f32x16;
 #define IX_ATTN_KP (IX_ATTN_D * 2 + 16)  // bytes per key row of the K tile
 #define IX_ATTN_VP (IX_ATTN_BN * 2 + 8)  // bytes per d row of the transposed V tile
 
+// A workgroup of NT threads stages a block of 32 keys x 128 d of K and of V: 512 16-byte chunks each, CPT per
+// thread. Chunk c = tid * CPT + j holds d (c % 16) * 8 .. +8 of key c / 16.
+template <int CPT>
 struct IxAttnStage {
-  uint4 k0, k1, v0, v1;
+  uint4 k[CPT], v[CPT];
 };
 
-// Thread t stages 16 consecutive d of key t/8 (two 16-byte loads from each of K and V).
-__device__ __forceinline__ void ix_attn_fetch(IxAttnStage& st, const bf16_t* __restrict__ kbase,
+template <int CPT>
+__device__ __forceinline__ void ix_attn_fetch(IxAttnStage<CPT>& st, const bf16_t* __restrict__ kbase,
                                               const bf16_t* __restrict__ vbase, long kv_pitch, int kb, int key_limit) {
-  const int key = kb * IX_ATTN_BN + (int)(threadIdx.x >> 3);
-  const int dch = (threadIdx.x & 7) * 16;
-  if (key <= key_limit) {
-    const uint4* kp = reinterpret_cast<const uint4*>(kbase + (long)key * kv_pitch + dch);
-    const uint4* vp = reinterpret_cast<const uint4*>(vbase + (long)key * kv_pitch + dch);
-    st.k0 = kp[0]; st.k1 = kp[1]; st.v0 = vp[0]; st.v1 = vp[1];
-  } else {  // beyond the last key any query of this workgroup needs: zeros, never read from memory
-    st.k0 = st.k1 = st.v0 = st.v1 = make_uint4(0, 0, 0, 0);
+#pragma unroll
+  for (int j = 0; j < CPT; ++j) {
+    const int c = threadIdx.x * CPT + j;
+    const int key = kb * IX_ATTN_BN + (c >> 4);
+    const int dch = (c & 15) * 8;
+    if (key <= key_limit) {
+      st.k[j] = *reinterpret_cast<const uint4*>(kbase + (long)key * kv_pitch + dch);
+      st.v[j] = *reinterpret_cast<const uint4*>(vbase + (long)key * kv_pitch + dch);
+    } else {  // beyond the last key any query of this workgroup needs: zeros, never read from memory
+      st.k[j] = st.v[j] = make_uint4(0, 0, 0, 0);
+    }
   }
 }
 
-__device__ __forceinline__ void ix_attn_commit(const IxAttnStage& st, char* ldsK, char* ldsV) {
-  const int key = threadIdx.x >> 3;
-  const int dch = (threadIdx.x & 7) * 16;
-  uint4* kd = reinterpret_cast<uint4*>(ldsK + key * IX_ATTN_KP + dch * 2);
-  kd[0] = st.k0; kd[1] = st.k1;
-  const uint32_t w[8] = {st.v0.x, st.v0.y, st.v0.z, st.v0.w, st.v1.x, st.v1.y, st.v1.z, st.v1.w};
+template <int CPT>
+__device__ __forceinline__ void ix_attn_commit(const IxAttnStage<CPT>& st, char* ldsK, char* ldsV) {
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    *reinterpret_cast<bf16_t*>(ldsV + (dch + 2 * j) * IX_ATTN_VP + key * 2) = (bf16_t)(w[j] & 0xffffu);
-    *reinterpret_cast<bf16_t*>(ldsV + (dch + 2 * j + 1) * IX_ATTN_VP + key * 2) = (bf16_t)(w[j] >> 16);
+  for (int j = 0; j < CPT; ++j) {
+    const int c = threadIdx.x * CPT + j;
+    const int key = c >> 4;
+    const int dch = (c & 15) * 8;
+    *reinterpret_cast<uint4*>(ldsK + key * IX_ATTN_KP + dch * 2) = st.k[j];
+    const uint32_t w[4] = {st.v[j].x, st.v[j].y, st.v[j].z, st.v[j].w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      *reinterpret_cast<bf16_t*>(ldsV + (dch + 2 * e) * IX_ATTN_VP + key * 2) = (bf16_t)(w[e] & 0xffffu);
+      *reinterpret_cast<bf16_t*>(ldsV + (dch + 2 * e + 1) * IX_ATTN_VP + key * 2) = (bf16_t)(w[e] >> 16);
+    }
   }
 }
 
 // One block of 32 keys for the 32 queries of a wave. Lane (qc = lane % 32, hf = lane / 32) holds
 // query qc; of the block's keys it holds, in register i, key (i/4)*8 + hf*4 + i%4.
 __device__ __forceinline__ void ix_attn_block(const char* ldsK, const char* ldsV, const ix_bf16x8 (&qf)[8],
-                                              ix_f32x16 (&O)[4], float& m, float& l, int kb, int qpos, float scale) {
+                                              ix_f32x16 (&O)[4], float& m, float& l, int kb, int qpos, int min_qpos,
+                                              float scale) {
   const int lane = threadIdx.x & 63;
   const int qc = lane & 31, hf = lane >> 5;
   ix_f32x16 sacc;
@@ -72,14 +83,24 @@ __device__ __forceinline__ void ix_attn_block(const char* ldsK, const char* ldsV
     const ix_bf16x8 kf = *reinterpret_cast<const ix_bf16x8*>(ldsK + qc * IX_ATTN_KP + (16 * s + hf * 8) * 2);
     sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], sacc, 0, 0, 0);
   }
+  // A block that ends at or before the wave's smallest position needs no mask (wave-uniform test).
+  const bool need_mask = kb * IX_ATTN_BN + IX_ATTN_BN - 1 > min_qpos;
   float sv[16];
   float bm = IX_NEG_INF;
+  if (need_mask) {
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int key = kb * IX_ATTN_BN + (i >> 2) * 8 + hf * 4 + (i & 3);
-    const float x = sacc[i] * scale;
-    sv[i] = key <= qpos ? x : IX_NEG_INF;
-    bm = fmaxf(bm, sv[i]);
+    for (int i = 0; i < 16; ++i) {
+      const int key = kb * IX_ATTN_BN + (i >> 2) * 8 + hf * 4 + (i & 3);
+      const float x = sacc[i] * scale;
+      sv[i] = key <= qpos ? x : IX_NEG_INF;
+      bm = fmaxf(bm, sv[i]);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      sv[i] = sacc[i] * scale;
+      bm = fmaxf(bm, sv[i]);
+    }
   }
   bm = fmaxf(bm, __shfl_xor(bm, 32, IX_WAVE));
   const float m_new = fmaxf(m, bm);
@@ -94,6 +115,8 @@ __device__ __forceinline__ void ix_attn_block(const char* ldsK, const char* ldsV
   const float tot = hf ? other + mine : mine + other;  // (half 0) + (half 1) on both lanes
   l = l * alpha + tot;
   m = m_new;
+  // x * 1.0f is x: when no query of the wave moved its maximum, the rescale is skipped for all of them.
+  const bool rescale = __any(alpha != 1.0f);
   ix_bf16x8 pf[2];
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
@@ -104,8 +127,10 @@ __device__ __forceinline__ void ix_attn_block(const char* ldsK, const char* ldsV
   }
 #pragma unroll
   for (int dt = 0; dt < 4; ++dt) {
+    if (rescale) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) O[dt][i] = O[dt][i] * alpha;
+      for (int i = 0; i < 16; ++i) O[dt][i] = O[dt][i] * alpha;
+    }
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
       const char* row = ldsV + (qc + 32 * dt) * IX_ATTN_VP;
@@ -118,16 +143,20 @@ __device__ __forceinline__ void ix_attn_block(const char* ldsK, const char* ldsV
   }
 }
 
-template <int GROUP>
-__global__ __launch_bounds__(256) void k_attn_varlen(const bf16_t* __restrict__ q, long q_pitch,
+// NW waves per workgroup (4 or 8): NW * 32 / GROUP consecutive tokens share each staged key block, so a larger
+// workgroup pulls fewer key/value bytes per query; which queries share a workgroup never reaches the arithmetic.
+template <int GROUP, int NW>
+__global__ __launch_bounds__(NW * 64) void k_attn_varlen(const bf16_t* __restrict__ q, long q_pitch,
                                                      const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
                                                      long kv_pitch, bf16_t* __restrict__ o,
                                                      const int* __restrict__ cu_q, const long* __restrict__ kv_start,
                                                      const int* __restrict__ q_pos0, int HQ, float scale) {
   constexpr int TOK_W = 32 / GROUP;   // tokens per wave
-  constexpr int TOK_WG = 4 * TOK_W;   // tokens per workgroup
-  __shared__ __attribute__((aligned(16))) char ldsK[IX_ATTN_BN * IX_ATTN_KP];
-  __shared__ __attribute__((aligned(16))) char ldsV[IX_ATTN_D * IX_ATTN_VP];
+  constexpr int TOK_WG = NW * TOK_W;  // tokens per workgroup
+  constexpr int CPT = 512 / (NW * 64);
+  // two LDS copies of the key/value block: block kb+1 is written while block kb is still being read
+  __shared__ __attribute__((aligned(16))) char ldsK[2][IX_ATTN_BN * IX_ATTN_KP];
+  __shared__ __attribute__((aligned(16))) char ldsV[2][IX_ATTN_D * IX_ATTN_VP];
   const int n = blockIdx.y, g = blockIdx.z;
   const int qb = cu_q[n];
   const int len = cu_q[n + 1] - qb;
@@ -164,6 +193,8 @@ __global__ __launch_bounds__(256) void k_attn_varlen(const bf16_t* __restrict__ 
   const int nblocks = key_limit / IX_ATTN_BN + 1;
   const int wave_last = min(len - 1, t0 + wave * TOK_W + TOK_W - 1);
   const int wave_blocks = wave_last >= t0 + wave * TOK_W ? (p0 + wave_last) / IX_ATTN_BN + 1 : 0;
+  // smallest position among the wave's live queries (its first token); padding columns have no limit
+  const int wave_min_qpos = p0 + t0 + wave * TOK_W;
   const long kv0 = kv_start[n];
   const bf16_t* kbase = k + kv0 * kv_pitch + (long)g * IX_ATTN_D;
   const bf16_t* vbase = v + kv0 * kv_pitch + (long)g * IX_ATTN_D;
@@ -175,14 +206,26 @@ __global__ __launch_bounds__(256) void k_attn_varlen(const bf16_t* __restrict__ 
     for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
   float m = IX_NEG_INF, l = 0.0f;
 
-  IxAttnStage st;
-  ix_attn_fetch(st, kbase, vbase, kv_pitch, 0, key_limit);
-  for (int kb = 0; kb < nblocks; ++kb) {
-    __syncthreads();  // every wave is done reading the previous block
-    ix_attn_commit(st, ldsK, ldsV);
+  // Two register stages: while block kb is multiplied, block kb+1 sits in LDS and blocks kb+2 and kb+3 are
+  // in flight from memory. One barrier per block.
+  IxAttnStage<CPT> sa, sb;
+  ix_attn_fetch(sa, kbase, vbase, kv_pitch, 0, key_limit);
+  if (nblocks > 1) ix_attn_fetch(sb, kbase, vbase, kv_pitch, 1, key_limit);
+  ix_attn_commit(sa, ldsK[0], ldsV[0]);
+  if (nblocks > 2) ix_attn_fetch(sa, kbase, vbase, kv_pitch, 2, key_limit);
+  __syncthreads();
+  for (int kb = 0; kb < nblocks; kb += 2) {
+    // even block: compute from copy 0; publish block kb+1 (stage b) into copy 1; refill stage b with kb+3
+    if (kb < wave_blocks) ix_attn_block(ldsK[0], ldsV[0], qf, O, m, l, kb, qpos, wave_min_qpos, scale);
+    if (kb + 1 < nblocks) ix_attn_commit(sb, ldsK[1], ldsV[1]);
+    if (kb + 3 < nblocks) ix_attn_fetch(sb, kbase, vbase, kv_pitch, kb + 3, key_limit);
     __syncthreads();
-    if (kb + 1 < nblocks) ix_attn_fetch(st, kbase, vbase, kv_pitch, kb + 1, key_limit);
-    if (kb < wave_blocks) ix_attn_block(ldsK, ldsV, qf, O, m, l, kb, qpos, scale);
+    if (kb + 1 >= nblocks) break;
+    // odd block: compute from copy 1; publish block kb+2 (stage a) into copy 0; refill stage a with kb+4
+    if (kb + 1 < wave_blocks) ix_attn_block(ldsK[1], ldsV[1], qf, O, m, l, kb + 1, qpos, wave_min_qpos, scale);
+    if (kb + 2 < nblocks) ix_attn_commit(sa, ldsK[0], ldsV[0]);
+    if (kb + 4 < nblocks) ix_attn_fetch(sa, kbase, vbase, kv_pitch, kb + 4, key_limit);
+    __syncthreads();
   }
   if (live) {
 #pragma unroll
@@ -212,16 +255,21 @@ extern "C" int ix_attn_varlen(const void* q, long q_pitch, const void* k, const 
   if (N > 65535 || HKV > 65535) return IX_DECLINED;
   const int group = (int)(HQ / HKV);
   hipStream_t st = (hipStream_t)stream;
-#define IX_ATTN_LAUNCH(G)                                                                                       \
-  case G: {                                                                                                     \
-    const long tok_wg = 4 * (32 / G);                                                                           \
+#define IX_ATTN_LAUNCH_NW(G, NWV)                                                                               \
+  {                                                                                                             \
+    const long tok_wg = NWV * (32 / G);                                                                         \
     const long tiles = (max_q_len + tok_wg - 1) / tok_wg;                                                       \
     if (tiles > 0x7fffffffL) return IX_DECLINED;                                                                \
-    hipLaunchKernelGGL(k_attn_varlen<G>, dim3((unsigned)tiles, (unsigned)N, (unsigned)HKV), dim3(256), 0, st,   \
-                       (const bf16_t*)q, q_pitch, (const bf16_t*)k, (const bf16_t*)v, kv_pitch, (bf16_t*)o,    \
-                       cu_q, kv_start, q_pos0, (int)HQ, scale);                                                 \
-    break;                                                                                                      \
+    hipLaunchKernelGGL((k_attn_varlen<G, NWV>), dim3((unsigned)tiles, (unsigned)N, (unsigned)HKV),              \
+                       dim3(NWV * 64), 0, st, (const bf16_t*)q, q_pitch, (const bf16_t*)k, (const bf16_t*)v,    \
+                       kv_pitch, (bf16_t*)o, cu_q, kv_start, q_pos0, (int)HQ, scale);                           \
   }
+#define IX_ATTN_LAUNCH(G)                                                                                       \
+  case G:                                                                                                       \
+    if (big) IX_ATTN_LAUNCH_NW(G, 8) else IX_ATTN_LAUNCH_NW(G, 4)                                               \
+    break;
+  // long query runs (prefill) use eight waves per workgroup, short ones (decode, small chunks) four
+  const bool big = max_q_len >= 8 * (32 / group);
   switch (group) {
     IX_ATTN_LAUNCH(1)
     IX_ATTN_LAUNCH(2)
@@ -232,6 +280,7 @@ extern "C" int ix_attn_varlen(const void* q, long q_pitch, const void* k, const 
     default:
       return IX_DECLINED;
   }
+#undef IX_ATTN_LAUNCH_NW
 #undef IX_ATTN_LAUNCH
   return ix_launch_status();
 }

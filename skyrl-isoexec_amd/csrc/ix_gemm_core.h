@@ -27,6 +27,10 @@ typedef __attribute__((ext_vector_type(16))) float ix_f32x16;
 typedef __attribute__((address_space(3))) void ix_lds_void;
 
 #define IX_BK 64
+// Differential-profiling switches, never defined by the Makefile: IX_EXPERIMENT_NO_DMA drops the memory -> LDS
+// fetches, IX_EXPERIMENT_NO_FRAG the LDS fragment reads, IX_EXPERIMENT_NO_MFMA the matrix instructions (results are
+// then meaningless; only the timing of what remains is of interest), IX_NO_UNIT_RING selects the half-tile ring for
+// square tiles.
 #define IX_OOB 0x7FFFF000u  // a byte offset no buffer descriptor here admits (all are < 1 GiB)
 
 // LDS tiles are [rows][k] bf16 with the 16-byte chunks of a row permuted by an XOR swizzle so that
@@ -54,16 +58,9 @@ struct IxGemmCfg {
   static constexpr int STAGE_BYTES = (BM + BN) * 128;
   // Pipeline: a ring of four half-k-tile stages when the half-stage fetch divides evenly over the
   // threads, else a ring of FULL_STAGES whole-k-tile stages (the 32-row decode tile).
-#ifdef IX_EXPERIMENT_FULL2
-  static constexpr bool HALF_RING = false;
-  static constexpr int FULL_STAGES = (BM + BN) * 128 * 3 <= 160 * 1024 ? 3 : 2;
-#else
   static constexpr bool HALF_RING = ((BM * 4) % NT == 0) && ((BN * 4) % NT == 0);
   static constexpr int FULL_STAGES = 3;
-#endif
-#ifndef IX_HALF_STAGES_MAX
 #define IX_HALF_STAGES_MAX 5
-#endif
   // as many half-stages as fit in the 160 KiB of LDS, at most IX_HALF_STAGES_MAX, at least 4
   static constexpr int HALF_STAGES =
       (IX_HALF_STAGES_MAX * (STAGE_BYTES / 2) <= 160 * 1024) ? IX_HALF_STAGES_MAX : 4;
