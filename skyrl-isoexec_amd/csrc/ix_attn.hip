@@ -25,47 +25,53 @@ typedef __attribute__((ext_vector_type(16))) float ix_f32x16;
 #define IX_ATTN_D 128
 #define IX_ATTN_BN 32
 #define IX_ATTN_KP (IX_ATTN_D * 2 + 16)  // bytes per key row of the K tile
-#define IX_ATTN_VP (IX_ATTN_BN * 2 + 8)  // bytes per d row of the transposed V tile
+// Bytes per key row of the V tile. 80 dwords: the four key rows that one transpose read of 32 lanes touches
+// (16 dwords each) then fall on four disjoint quarters of the 64 banks.
+#define IX_ATTN_VP (IX_ATTN_D * 2 + 64)
+
+typedef __attribute__((ext_vector_type(4))) short ix_s16x4;
 
 // A workgroup of NT threads stages a block of 32 keys x 128 d of K and of V: 512 16-byte chunks each, CPT per
-// thread. Chunk c = tid * CPT + j holds d (c % 16) * 8 .. +8 of key c / 16.
-template <int CPT>
+// thread. Chunk c = j * NT + tid holds d (c % 16) * 8 .. +8 of key c / 16; both tiles keep the key-major layout
+// of memory, so a chunk is one 16-byte store.
+// Named members, not arrays: the stages must live in registers whatever the unroller decides.
 struct IxAttnStage {
-  uint4 k[CPT], v[CPT];
+  uint4 k0, v0, k1, v1;
 };
 
-template <int CPT>
-__device__ __forceinline__ void ix_attn_fetch(IxAttnStage<CPT>& st, const bf16_t* __restrict__ kbase,
-                                              const bf16_t* __restrict__ vbase, long kv_pitch, int kb, int key_limit) {
-#pragma unroll
-  for (int j = 0; j < CPT; ++j) {
-    const int c = threadIdx.x * CPT + j;
-    const int key = kb * IX_ATTN_BN + (c >> 4);
-    const int dch = (c & 15) * 8;
-    if (key <= key_limit) {
-      st.k[j] = *reinterpret_cast<const uint4*>(kbase + (long)key * kv_pitch + dch);
-      st.v[j] = *reinterpret_cast<const uint4*>(vbase + (long)key * kv_pitch + dch);
-    } else {  // beyond the last key any query of this workgroup needs: zeros, never read from memory
-      st.k[j] = st.v[j] = make_uint4(0, 0, 0, 0);
-    }
+template <int NT>
+__device__ __forceinline__ void ix_attn_fetch1(uint4& kk, uint4& vv, int j, const bf16_t* __restrict__ kbase,
+                                               const bf16_t* __restrict__ vbase, long kv_pitch, int kb, int key_limit) {
+  const int c = j * NT + threadIdx.x;
+  const int key = kb * IX_ATTN_BN + (c >> 4);
+  const int dch = (c & 15) * 8;
+  kk = vv = make_uint4(0, 0, 0, 0);  // beyond the last key any query of this workgroup needs: zeros, nothing read
+  if (key <= key_limit) {
+    kk = *reinterpret_cast<const uint4*>(kbase + (long)key * kv_pitch + dch);
+    vv = *reinterpret_cast<const uint4*>(vbase + (long)key * kv_pitch + dch);
   }
 }
 
 template <int CPT>
-__device__ __forceinline__ void ix_attn_commit(const IxAttnStage<CPT>& st, char* ldsK, char* ldsV) {
-#pragma unroll
-  for (int j = 0; j < CPT; ++j) {
-    const int c = threadIdx.x * CPT + j;
-    const int key = c >> 4;
-    const int dch = (c & 15) * 8;
-    *reinterpret_cast<uint4*>(ldsK + key * IX_ATTN_KP + dch * 2) = st.k[j];
-    const uint32_t w[4] = {st.v[j].x, st.v[j].y, st.v[j].z, st.v[j].w};
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      *reinterpret_cast<bf16_t*>(ldsV + (dch + 2 * e) * IX_ATTN_VP + key * 2) = (bf16_t)(w[e] & 0xffffu);
-      *reinterpret_cast<bf16_t*>(ldsV + (dch + 2 * e + 1) * IX_ATTN_VP + key * 2) = (bf16_t)(w[e] >> 16);
-    }
-  }
+__device__ __forceinline__ void ix_attn_fetch(IxAttnStage& st, const bf16_t* __restrict__ kbase,
+                                              const bf16_t* __restrict__ vbase, long kv_pitch, int kb, int key_limit) {
+  ix_attn_fetch1<512 / CPT>(st.k0, st.v0, 0, kbase, vbase, kv_pitch, kb, key_limit);
+  if (CPT > 1) ix_attn_fetch1<512 / CPT>(st.k1, st.v1, 1, kbase, vbase, kv_pitch, kb, key_limit);
+}
+
+template <int NT>
+__device__ __forceinline__ void ix_attn_commit1(const uint4& kk, const uint4& vv, int j, char* ldsK, char* ldsV) {
+  const int c = j * NT + threadIdx.x;
+  const int key = c >> 4;
+  const int dch = (c & 15) * 8;
+  *reinterpret_cast<uint4*>(ldsK + key * IX_ATTN_KP + dch * 2) = kk;
+  *reinterpret_cast<uint4*>(ldsV + key * IX_ATTN_VP + dch * 2) = vv;
+}
+
+template <int CPT>
+__device__ __forceinline__ void ix_attn_commit(const IxAttnStage& st, char* ldsK, char* ldsV) {
+  ix_attn_commit1<512 / CPT>(st.k0, st.v0, 0, ldsK, ldsV);
+  if (CPT > 1) ix_attn_commit1<512 / CPT>(st.k1, st.v1, 1, ldsK, ldsV);
 }
 
 // One block of 32 keys for the 32 queries of a wave. Lane (qc = lane % 32, hf = lane / 32) holds
@@ -125,6 +131,8 @@ __device__ __forceinline__ void ix_attn_block(const char* ldsK, const char* ldsV
     for (int j = 0; j < 4; ++j) w[j] = ix_pack_bf2(p[8 * s + 2 * j], p[8 * s + 2 * j + 1]);
     pf[s] = *reinterpret_cast<const ix_bf16x8*>(w);
   }
+  // this lane's address inside the 4 key x 16 d patch its group of 16 lanes transposes
+  const char* vsrc = ldsV + (hf * 4 + ((lane & 15) >> 2)) * IX_ATTN_VP + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
 #pragma unroll
   for (int dt = 0; dt < 4; ++dt) {
     if (rescale) {
@@ -133,10 +141,15 @@ __device__ __forceinline__ void ix_attn_block(const char* ldsK, const char* ldsV
     }
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      const char* row = ldsV + (qc + 32 * dt) * IX_ATTN_VP;
-      uint2 lo = *reinterpret_cast<const uint2*>(row + (16 * s + hf * 4) * 2);
-      uint2 hi = *reinterpret_cast<const uint2*>(row + (16 * s + 8 + hf * 4) * 2);
-      const uint32_t w[4] = {lo.x, lo.y, hi.x, hi.y};
+      // The lane needs V[key][d = 32 dt + qc] for keys 16 s + hf * 4 + 0..3 and those 8 further on. A transpose
+      // read works in groups of 16 lanes: lane i of a group receives, as element e, element i % 4 of the 8 bytes
+      // that lane 4 e + i / 4 of the group addressed. With lane j addressing key j / 4, d 4 * (j % 4) .. +4 of the
+      // group's 4 key x 16 d patch, lane i ends up with keys 0..3 at d = i.
+      typedef __attribute__((address_space(3))) ix_s16x4 lds_s16x4;
+      const char* src = vsrc + (16 * s) * IX_ATTN_VP + 64 * dt;
+      const ix_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(src));
+      const ix_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(src + 8 * IX_ATTN_VP));
+      const ix_s16x4 w[2] = {lo, hi};
       const ix_bf16x8 vf = *reinterpret_cast<const ix_bf16x8*>(w);
       O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[s], O[dt], 0, 0, 0);
     }
@@ -156,7 +169,7 @@ __global__ __launch_bounds__(NW * 64) void k_attn_varlen(const bf16_t* __restric
   constexpr int CPT = 512 / (NW * 64);
   // two LDS copies of the key/value block: block kb+1 is written while block kb is still being read
   __shared__ __attribute__((aligned(16))) char ldsK[2][IX_ATTN_BN * IX_ATTN_KP];
-  __shared__ __attribute__((aligned(16))) char ldsV[2][IX_ATTN_D * IX_ATTN_VP];
+  __shared__ __attribute__((aligned(16))) char ldsV[2][IX_ATTN_BN * IX_ATTN_VP];
   const int n = blockIdx.y, g = blockIdx.z;
   const int qb = cu_q[n];
   const int len = cu_q[n + 1] - qb;
@@ -208,23 +221,23 @@ __global__ __launch_bounds__(NW * 64) void k_attn_varlen(const bf16_t* __restric
 
   // Two register stages: while block kb is multiplied, block kb+1 sits in LDS and blocks kb+2 and kb+3 are
   // in flight from memory. One barrier per block.
-  IxAttnStage<CPT> sa, sb;
-  ix_attn_fetch(sa, kbase, vbase, kv_pitch, 0, key_limit);
-  if (nblocks > 1) ix_attn_fetch(sb, kbase, vbase, kv_pitch, 1, key_limit);
-  ix_attn_commit(sa, ldsK[0], ldsV[0]);
-  if (nblocks > 2) ix_attn_fetch(sa, kbase, vbase, kv_pitch, 2, key_limit);
+  IxAttnStage sa, sb;
+  ix_attn_fetch<CPT>(sa, kbase, vbase, kv_pitch, 0, key_limit);
+  if (nblocks > 1) ix_attn_fetch<CPT>(sb, kbase, vbase, kv_pitch, 1, key_limit);
+  ix_attn_commit<CPT>(sa, ldsK[0], ldsV[0]);
+  if (nblocks > 2) ix_attn_fetch<CPT>(sa, kbase, vbase, kv_pitch, 2, key_limit);
   __syncthreads();
   for (int kb = 0; kb < nblocks; kb += 2) {
     // even block: compute from copy 0; publish block kb+1 (stage b) into copy 1; refill stage b with kb+3
     if (kb < wave_blocks) ix_attn_block(ldsK[0], ldsV[0], qf, O, m, l, kb, qpos, wave_min_qpos, scale);
-    if (kb + 1 < nblocks) ix_attn_commit(sb, ldsK[1], ldsV[1]);
-    if (kb + 3 < nblocks) ix_attn_fetch(sb, kbase, vbase, kv_pitch, kb + 3, key_limit);
+    if (kb + 1 < nblocks) ix_attn_commit<CPT>(sb, ldsK[1], ldsV[1]);
+    if (kb + 3 < nblocks) ix_attn_fetch<CPT>(sb, kbase, vbase, kv_pitch, kb + 3, key_limit);
     __syncthreads();
     if (kb + 1 >= nblocks) break;
     // odd block: compute from copy 1; publish block kb+2 (stage a) into copy 0; refill stage a with kb+4
     if (kb + 1 < wave_blocks) ix_attn_block(ldsK[1], ldsV[1], qf, O, m, l, kb + 1, qpos, wave_min_qpos, scale);
-    if (kb + 2 < nblocks) ix_attn_commit(sa, ldsK[0], ldsV[0]);
-    if (kb + 4 < nblocks) ix_attn_fetch(sa, kbase, vbase, kv_pitch, kb + 4, key_limit);
+    if (kb + 2 < nblocks) ix_attn_commit<CPT>(sa, ldsK[0], ldsV[0]);
+    if (kb + 4 < nblocks) ix_attn_fetch<CPT>(sa, kbase, vbase, kv_pitch, kb + 4, key_limit);
     __syncthreads();
   }
   if (live) {
