@@ -46,7 +46,8 @@ extern "C" {
 #define IX_PRIM_SOFTPLUS 5
 #define IX_PRIM_RSQRT_IEEE 6
 #define IX_PRIM_ROUND_BF16 7
-#define IX_PRIM_COUNT 8
+#define IX_PRIM_EXP2 8
+#define IX_PRIM_COUNT 9
 
 int ix_abi_version(void);
 const char* ix_arch_tag(void); /* "gfx950"; counterpart of core/arch.py:27-51 detect_arch() tags */

@@ -3,8 +3,9 @@
 Attention follows the reference's contract for this op -- causal grouped-query attention with a
 single walk of the keys, so a query's value is independent of the call it ran in
 (isoexec/ops/attention/_register.py:15-47, varlen_backend.py:1-10) -- in the block-wise online form
-the device kernel fixes: blocks of 32 keys, fp32 running max / denominator / accumulator, bf16
-probabilities into the value product. The two matrix products are computed here in float64 and
+the device kernel fixes: blocks of 32 keys, fp32 running max (of the unscaled scores) / denominator /
+accumulator, probabilities 2 ** fma(s, c, -m c) with c = scale * log2(e), bf16 probabilities into the
+value product, one reciprocal of the denominator at the end. The two matrix products are computed here in float64 and
 rounded once to fp32: the device's matrix instruction sums the same products in an order that is not
 part of its public contract, so oracle and kernel agree to the last few fp32 bits of a block, not bit
 for bit, except on inputs whose partial sums are exact in any order (the known-answer cases).
@@ -22,7 +23,7 @@ from __future__ import annotations
 
 import numpy as np
 
-from .prims import DEFAULT, Prims, pairwise_tree, round_bf16
+from .prims import DEFAULT, LOG2E, Prims, pairwise_tree, round_bf16
 
 F32 = np.float32
 BLOCK = 32
@@ -41,15 +42,18 @@ def attend_one(q, K, V, scale, prims: Prims = DEFAULT, block: int = BLOCK):
     l = F32(0.0)
     O = np.zeros(D, dtype=F32)
     q64 = q.astype(np.float64)
+    c = F32(F32(scale) * LOG2E)  # scale > 0: the running maximum is kept in unscaled units
     for b0 in range(0, L, block):
         kb, vb = K[b0 : b0 + block], V[b0 : b0 + block]
         n = kb.shape[0]
         s = (kb.astype(np.float64) @ q64).astype(F32)
-        s = (s * F32(scale)).astype(F32)
         m_new = max(m, s.max())
-        alpha = prims.exp_fast(np.array([m - m_new], dtype=F32))[0] if np.isfinite(m) else F32(0.0)
+        alpha = prims.exp2(np.array([F32(m - m_new) * c], dtype=F32))[0] if np.isfinite(m) else F32(0.0)
+        mc = F32(m_new * c)
         p = np.zeros(block, dtype=F32)
-        p[:n] = prims.exp_fast((s - m_new).astype(F32))
+        # fused multiply-add: the product is exact in float64, the difference is rounded once more there
+        # (a double rounding that moves the fp32 result by at most one ulp in rare cases)
+        p[:n] = prims.exp2((s.astype(np.float64) * np.float64(c) - np.float64(mc)).astype(F32))
         # Row sum: each half-wave adds its 16 keys as two 8-trees, then half 0 + half 1.
         idx = np.arange(block)
         halves = []
@@ -64,7 +68,7 @@ def attend_one(q, K, V, scale, prims: Prims = DEFAULT, block: int = BLOCK):
         pv = (round_bf16(p[:n]).astype(np.float64) @ vb.astype(np.float64)).astype(F32)
         O = ((O * alpha).astype(F32) + pv).astype(F32)
         m = F32(m_new)
-    return round_bf16((O / l).astype(F32))
+    return round_bf16((O * F32(F32(1.0) / l)).astype(F32))
 
 
 def attend_causal(q, k, v, scale=None, q_pos0: int = 0, prims: Prims = DEFAULT, block: int = BLOCK):

@@ -40,6 +40,11 @@ class Prims:
     def exp_fast(self, x):  # device: one multiply then v_exp_f32
         return np.exp2((x.astype(F32) * LOG2E).astype(F32)).astype(F32)
 
+    def exp2(self, x):  # device: bare v_exp_f32, results below the normal range flush to zero
+        with np.errstate(under="ignore"):
+            y = np.exp2(x.astype(F32)).astype(F32)
+        return np.where(np.abs(y) < np.finfo(F32).tiny, F32(0.0), y).astype(F32)
+
     def log1p(self, x):
         return np.log1p(x.astype(F32)).astype(F32)
 

@@ -3,14 +3,15 @@
 //
 // The canonical function, per (query token at absolute position p, query head h):
 //   keys 0..p of the query's own sequence are walked in blocks of 32, block b = keys [32b, 32b+32);
-//   per block:  s_j  = (q . k_j) * scale                 bf16 MFMA, fp32 accumulate, d in 8 steps of 16
+//   with c = scale * log2(e) (one fp32 product), per block:
+//               s_j  = q . k_j                           bf16 MFMA, fp32 accumulate, d in 8 steps of 16
 //               s_j  = -inf for j > p
-//               m'   = max(m, max_j s_j)
-//               a    = exp2((m - m') * log2e)            (ix_exp_fast)
-//               p_j  = exp2((s_j - m') * log2e)
+//               m'   = max(m, max_j s_j)                 running maximum of the UNSCALED scores (scale > 0)
+//               a    = exp2((m - m') * c)                exactly 1 when the maximum did not move
+//               p_j  = exp2(fma(s_j, c, -(m' * c)))      one fused multiply-add per score
 //               l    = l * a + (lo + hi)                 lo/hi: the two halves' sums, see ix_attn_block
 //               O    = O * a + sum_j bf16(p_j) * v_j     bf16 MFMA, fp32 accumulate, keys in 2 steps of 16
-//   out = bf16(O / l).
+//   out = bf16(O * (1 / l)), one IEEE reciprocal per query.
 // Nothing in that chain depends on which other queries share the launch: a workgroup holds the
 // queries of 32/GROUP * 4 consecutive tokens for the GROUP query heads of one key/value head, every
 // MFMA row or column belongs to one query, and a block that lies wholly beyond a query's position is
@@ -78,7 +79,7 @@ __device__ __forceinline__ void ix_attn_commit(const IxAttnStage& st, char* ldsK
 // query qc; of the block's keys it holds, in register i, key (i/4)*8 + hf*4 + i%4.
 __device__ __forceinline__ void ix_attn_block(const char* ldsK, const char* ldsV, const ix_bf16x8 (&qf)[8],
                                               ix_f32x16 (&O)[4], float& m, float& l, int kb, int qpos, int min_qpos,
-                                              float scale) {
+                                              float c) {
   const int lane = threadIdx.x & 63;
   const int qc = lane & 31, hf = lane >> 5;
   ix_f32x16 sacc;
@@ -91,29 +92,23 @@ __device__ __forceinline__ void ix_attn_block(const char* ldsK, const char* ldsV
   }
   // A block that ends at or before the wave's smallest position needs no mask (wave-uniform test).
   const bool need_mask = kb * IX_ATTN_BN + IX_ATTN_BN - 1 > min_qpos;
-  float sv[16];
-  float bm = IX_NEG_INF;
   if (need_mask) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int key = kb * IX_ATTN_BN + (i >> 2) * 8 + hf * 4 + (i & 3);
-      const float x = sacc[i] * scale;
-      sv[i] = key <= qpos ? x : IX_NEG_INF;
-      bm = fmaxf(bm, sv[i]);
-    }
-  } else {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      sv[i] = sacc[i] * scale;
-      bm = fmaxf(bm, sv[i]);
+      sacc[i] = key <= qpos ? sacc[i] : IX_NEG_INF;
     }
   }
+  float bm = sacc[0];
+#pragma unroll
+  for (int i = 1; i < 16; ++i) bm = fmaxf(bm, sacc[i]);
   bm = fmaxf(bm, __shfl_xor(bm, 32, IX_WAVE));
   const float m_new = fmaxf(m, bm);
-  const float alpha = ix_exp_fast(m - m_new);
+  const float alpha = ix_exp2((m - m_new) * c);
+  const float mc = -(m_new * c);
   float p[16];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) p[i] = ix_exp_fast(sv[i] - m_new);
+  for (int i = 0; i < 16; ++i) p[i] = ix_exp2(__builtin_fmaf(sacc[i], c, mc));
   const float pa[8] = {p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]};
   const float pb[8] = {p[8], p[9], p[10], p[11], p[12], p[13], p[14], p[15]};
   const float mine = ix_tree8(pa) + ix_tree8(pb);
@@ -128,7 +123,7 @@ __device__ __forceinline__ void ix_attn_block(const char* ldsK, const char* ldsV
   for (int s = 0; s < 2; ++s) {
     uint32_t w[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) w[j] = ix_pack_bf2(p[8 * s + 2 * j], p[8 * s + 2 * j + 1]);
+    for (int j = 0; j < 4; ++j) w[j] = ix_pack_bf2_hw(p[8 * s + 2 * j], p[8 * s + 2 * j + 1]);
     pf[s] = *reinterpret_cast<const ix_bf16x8*>(w);
   }
   // this lane's address inside the 4 key x 16 d patch its group of 16 lanes transposes
@@ -218,6 +213,7 @@ __global__ __launch_bounds__(NW * 64) void k_attn_varlen(const bf16_t* __restric
 #pragma unroll
     for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
   float m = IX_NEG_INF, l = 0.0f;
+  const float c = scale * IX_LOG2E;
 
   // Two register stages: while block kb is multiplied, block kb+1 sits in LDS and blocks kb+2 and kb+3 are
   // in flight from memory. One barrier per block.
@@ -229,26 +225,27 @@ __global__ __launch_bounds__(NW * 64) void k_attn_varlen(const bf16_t* __restric
   __syncthreads();
   for (int kb = 0; kb < nblocks; kb += 2) {
     // even block: compute from copy 0; publish block kb+1 (stage b) into copy 1; refill stage b with kb+3
-    if (kb < wave_blocks) ix_attn_block(ldsK[0], ldsV[0], qf, O, m, l, kb, qpos, wave_min_qpos, scale);
+    if (kb < wave_blocks) ix_attn_block(ldsK[0], ldsV[0], qf, O, m, l, kb, qpos, wave_min_qpos, c);
     if (kb + 1 < nblocks) ix_attn_commit<CPT>(sb, ldsK[1], ldsV[1]);
     if (kb + 3 < nblocks) ix_attn_fetch<CPT>(sb, kbase, vbase, kv_pitch, kb + 3, key_limit);
     __syncthreads();
     if (kb + 1 >= nblocks) break;
     // odd block: compute from copy 1; publish block kb+2 (stage a) into copy 0; refill stage a with kb+4
-    if (kb + 1 < wave_blocks) ix_attn_block(ldsK[1], ldsV[1], qf, O, m, l, kb + 1, qpos, wave_min_qpos, scale);
+    if (kb + 1 < wave_blocks) ix_attn_block(ldsK[1], ldsV[1], qf, O, m, l, kb + 1, qpos, wave_min_qpos, c);
     if (kb + 2 < nblocks) ix_attn_commit<CPT>(sa, ldsK[0], ldsV[0]);
     if (kb + 4 < nblocks) ix_attn_fetch<CPT>(sa, kbase, vbase, kv_pitch, kb + 4, key_limit);
     __syncthreads();
   }
   if (live) {
+    const float inv = 1.0f / l;
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt) {
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         const int d = 32 * dt + i4 * 8 + hf * 4;
         uint2 w;
-        w.x = ix_pack_bf2(O[dt][4 * i4 + 0] / l, O[dt][4 * i4 + 1] / l);
-        w.y = ix_pack_bf2(O[dt][4 * i4 + 2] / l, O[dt][4 * i4 + 3] / l);
+        w.x = ix_pack_bf2_hw(O[dt][4 * i4 + 0] * inv, O[dt][4 * i4 + 1] * inv);
+        w.y = ix_pack_bf2_hw(O[dt][4 * i4 + 2] * inv, O[dt][4 * i4 + 3] * inv);
         *reinterpret_cast<uint2*>(orow + d) = w;
       }
     }
@@ -260,6 +257,7 @@ extern "C" int ix_attn_varlen(const void* q, long q_pitch, const void* k, const 
                               long HQ, long HKV, long D, float scale, void* stream) {
   if (!q || !k || !v || !o || !cu_q || !kv_start) return IX_ERR_ARG;
   if (N < 0 || max_q_len < 0 || HQ <= 0 || HKV <= 0 || HQ % HKV != 0) return IX_ERR_ARG;
+  if (!(scale > 0.0f) || scale > 3.0e38f) return IX_ERR_ARG;  // the running maximum is kept unscaled
   if (D != IX_ATTN_D) return IX_DECLINED;
   if (q_pitch % 8 != 0 || kv_pitch % 8 != 0 || !ix_aligned(q, 16) || !ix_aligned(k, 16) || !ix_aligned(v, 16) ||
       !ix_aligned(o, 8))

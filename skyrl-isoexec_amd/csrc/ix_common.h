@@ -42,6 +42,16 @@ __device__ __forceinline__ uint32_t ix_pack_bf2(float lo, float hi) {
   return (uint32_t)ix_f2bf(lo) | ((uint32_t)ix_f2bf(hi) << 16);
 }
 
+// The same rounding by the hardware pack-convert (identical to ix_f2bf on every non-NaN bit pattern; a NaN
+// keeps its payload instead of becoming 0x7fc0). For values that cannot be NaN unless the inputs were.
+typedef __attribute__((ext_vector_type(2))) __bf16 ix_hw_bf16x2;
+typedef __attribute__((ext_vector_type(2))) float ix_hw_f32x2;
+__device__ __forceinline__ uint32_t ix_pack_bf2_hw(float lo, float hi) {
+  const ix_hw_f32x2 v = {lo, hi};
+  const ix_hw_bf16x2 r = __builtin_convertvector(v, ix_hw_bf16x2);
+  return *reinterpret_cast<const uint32_t*>(&r);
+}
+
 // ---- the transcendental primitives -------------------------------------------------------
 // One definition each; every kernel of an op family calls these and nothing else, so prefill
 // and decode, M=1 and M=4096, see the same function. ix_prim_unary (ix_prims.hip) exports
@@ -51,6 +61,8 @@ __device__ __forceinline__ float ix_log(float x) { return logf(x); }        // o
 __device__ __forceinline__ float ix_log1p(float x) { return log1pf(x); }    // ocml
 // Fast exp for the vocabulary sum: one multiply and one v_exp_f32. Argument is always <= 0.
 __device__ __forceinline__ float ix_exp_fast(float x) { return __builtin_amdgcn_exp2f(x * IX_LOG2E); }
+// The bare hardware 2^x (about 1 ulp; results below the normal range flush to zero).
+__device__ __forceinline__ float ix_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 // IEEE divide and square root (correctly rounded; hipcc's default for fp32), so 1/sqrt is
 // reproducible on any IEEE host.
 __device__ __forceinline__ float ix_rsqrt_ieee(float x) { return 1.0f / sqrtf(x); }

@@ -20,6 +20,7 @@ __global__ __launch_bounds__(256) void k_prim_unary(int op, const float* __restr
     case IX_PRIM_SOFTPLUS: r = ix_softplus(v); break;
     case IX_PRIM_RSQRT_IEEE: r = ix_rsqrt_ieee(v); break;
     case IX_PRIM_ROUND_BF16: r = ix_rbf(v); break;
+    case IX_PRIM_EXP2: r = ix_exp2(v); break;
     default: r = v; break;
   }
   y[i] = r;

@@ -28,6 +28,7 @@ PRIM = {
     "softplus": 5,
     "rsqrt_ieee": 6,
     "round_bf16": 7,
+    "exp2": 8,
 }
 
 P = c_void_p

@@ -57,6 +57,9 @@ class DevicePrims(Prims):
     def exp_fast(self, x):
         return self._run("exp_fast", x)
 
+    def exp2(self, x):
+        return self._run("exp2", x)
+
     def sigmoid(self, x):
         return self._run("sigmoid", x)
 
