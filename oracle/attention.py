@@ -3,8 +3,8 @@
 Attention follows the reference's contract for this op -- causal grouped-query attention with a
 single walk of the keys, so a query's value is independent of the call it ran in
 (isoexec/ops/attention/_register.py:15-47, varlen_backend.py:1-10) -- in the block-wise online form
-the device kernel fixes: blocks of 32 keys, fp32 running max (of the unscaled scores) / denominator /
-accumulator, probabilities 2 ** fma(s, c, -m c) with c = scale * log2(e), bf16 probabilities into the
+the device kernel fixes: blocks of 32 keys, an fp32 reference point (a running maximum of the unscaled
+scores that moves only when exceeded by more than 2^8), fp32 denominator and accumulator, probabilities 2 ** fma(s, c, -m c) with c = scale * log2(e), bf16 probabilities into the
 value product, one reciprocal of the denominator at the end. The two matrix products are computed here in float64 and
 rounded once to fp32: the device's matrix instruction sums the same products in an order that is not
 part of its public contract, so oracle and kernel agree to the last few fp32 bits of a block, not bit
@@ -27,6 +27,7 @@ from .prims import DEFAULT, LOG2E, Prims, pairwise_tree, round_bf16
 
 F32 = np.float32
 BLOCK = 32
+LAZY = F32(8.0)
 
 
 def _half_of(key_in_block: np.ndarray) -> np.ndarray:
@@ -47,7 +48,10 @@ def attend_one(q, K, V, scale, prims: Prims = DEFAULT, block: int = BLOCK):
         kb, vb = K[b0 : b0 + block], V[b0 : b0 + block]
         n = kb.shape[0]
         s = (kb.astype(np.float64) @ q64).astype(F32)
-        m_new = max(m, s.max())
+        bm = F32(s.max())
+        # the reference point moves only when the block maximum exceeds it by more than 2^8 (in the exponent)
+        with np.errstate(invalid="ignore"):
+            m_new = bm if F32(F32(bm - m) * c) > LAZY else m
         alpha = prims.exp2(np.array([F32(m - m_new) * c], dtype=F32))[0] if np.isfinite(m) else F32(0.0)
         mc = F32(m_new * c)
         p = np.zeros(block, dtype=F32)

@@ -6,93 +6,132 @@
 //   with c = scale * log2(e) (one fp32 product), per block:
 //               s_j  = q . k_j                           bf16 MFMA, fp32 accumulate, d in 8 steps of 16
 //               s_j  = -inf for j > p
-//               m'   = max(m, max_j s_j)                 running maximum of the UNSCALED scores (scale > 0)
-//               a    = exp2((m - m') * c)                exactly 1 when the maximum did not move
-//               p_j  = exp2(fma(s_j, c, -(m' * c)))      one fused multiply-add per score
+//               b    = max_j s_j                         the block's maximum, UNSCALED (scale > 0)
+//               m'   = b if (b - m) * c > 8 else m       the reference point moves only when the maximum has
+//                                                        grown by more than 2^8; m starts at -inf
+//               a    = exp2((m - m') * c)                exactly 1 when the reference did not move
+//               p_j  = exp2(fma(s_j, c, -(m' * c)))      one fused multiply-add per score; p_j <= 2^8 (1 + eps)
 //               l    = l * a + (lo + hi)                 lo/hi: the two halves' sums, see ix_attn_block
 //               O    = O * a + sum_j bf16(p_j) * v_j     bf16 MFMA, fp32 accumulate, keys in 2 steps of 16
 //   out = bf16(O * (1 / l)), one IEEE reciprocal per query.
 // Nothing in that chain depends on which other queries share the launch: a workgroup holds the
 // queries of 32/GROUP * 4 consecutive tokens for the GROUP query heads of one key/value head, every
 // MFMA row or column belongs to one query, and a block that lies wholly beyond a query's position is
-// an exact no-op for it (a = 1, p_j = 0), so whether a wave computes or skips it gives the same bits.
+// an exact no-op for it (b = -inf, a = 1, p_j = 0), so whether a wave computes or skips it gives the same bits.
 // A one-token decode step and a full-sequence pass therefore agree bit for bit.
-#include "ix_common.h"
+#include "ix_gemm_core.h"
 #include "../../include/isoexec_hip.h"
-
-typedef __attribute__((ext_vector_type(8))) __bf16 ix_bf16x8;
-typedef __attribute__((ext_vector_type(16))) float ix_f32x16;
 
 #define IX_ATTN_D 128
 #define IX_ATTN_BN 32
-#define IX_ATTN_KP (IX_ATTN_D * 2 + 16)  // bytes per key row of the K tile
-// Bytes per key row of the V tile. 80 dwords: the four key rows that one transpose read of 32 lanes touches
-// (16 dwords each) then fall on four disjoint quarters of the 64 banks.
-#define IX_ATTN_VP (IX_ATTN_D * 2 + 64)
+#define IX_ATTN_ROW (IX_ATTN_D * 2)                 // bytes per key row of a tile
+#define IX_ATTN_TILE (IX_ATTN_BN * IX_ATTN_ROW)     // one K or V tile of a block: 8 KiB
+#define IX_ATTN_STAGE (2 * IX_ATTN_TILE)            // K tile, then V tile
+#ifndef IX_ATTN_STAGES_BIG
+#define IX_ATTN_STAGES_BIG 4    // ring depth of the eight-wave kernel
+#endif
+#ifndef IX_ATTN_STAGES_SMALL
+#define IX_ATTN_STAGES_SMALL 4  // ring depth of the four-wave kernel
+#endif
 
 typedef __attribute__((ext_vector_type(4))) short ix_s16x4;
+typedef __attribute__((address_space(3))) ix_s16x4 ix_lds_s16x4;
 
-// A workgroup of NT threads stages a block of 32 keys x 128 d of K and of V: 512 16-byte chunks each, CPT per
-// thread. Chunk c = j * NT + tid holds d (c % 16) * 8 .. +8 of key c / 16; both tiles keep the key-major layout
-// of memory, so a chunk is one 16-byte store.
-// Named members, not arrays: the stages must live in registers whatever the unroller decides.
-struct IxAttnStage {
-  uint4 k0, v0, k1, v1;
+// Key/value blocks go memory -> LDS directly (16 bytes per lane, no registers) into a ring of S stages. Both
+// tiles keep memory's key-major layout, 256 bytes per key, with the 16-byte chunks of a row permuted:
+//   K: chunk c of key r sits at slot c ^ (r & 15)         a fragment read takes one chunk of 32 consecutive keys
+//   V: chunk c of key r sits at slot c ^ ((r & 3) << 2)   a transpose read takes 4 chunks of 4 consecutive keys
+// so that either read spreads over all LDS banks. A lane's LDS destination is fixed by its position in the
+// wave (destination = base + 16 * lane), so the permutation is applied to the memory address it fetches.
+template <int NT>
+struct IxAttnFetch {
+  static constexpr int CPT = 512 / NT;  // chunks per thread per tile
+  uint32_t voff_k[CPT], voff_v[CPT];    // byte offsets inside a block: key row * pitch + chunk * 16
+  uint32_t lds0;                        // LDS address of this wave's first destination in stage 0
+  __device__ __forceinline__ void init(const char* lds, uint32_t pitch_bytes) {
+    const int wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+      const int q = j * NT + threadIdx.x;
+      const int row = q >> 4, slot = q & 15;
+      voff_k[j] = (uint32_t)row * pitch_bytes + (uint32_t)((slot ^ (row & 15)) << 4);
+      voff_v[j] = (uint32_t)row * pitch_bytes + (uint32_t)((slot ^ ((row & 3) << 2)) << 4);
+    }
+    lds0 = __builtin_amdgcn_readfirstlane(ix_lds_addr(lds) + wave * 1024);
+  }
+  // Block kb of the sequence into ring stage `stage`. Keys beyond key_limit lie outside the buffer range and
+  // arrive as zeros; a block wholly beyond it is all zeros and touches no memory.
+  __device__ __forceinline__ void issue(const bf16_t* kbase, const bf16_t* vbase, long kv_pitch, int kb, int stage,
+                                        int key_limit) const {
+    const int rows = min(IX_ATTN_BN, key_limit + 1 - kb * IX_ATTN_BN);
+    const uint32_t bytes = rows > 0 ? (uint32_t)(rows - 1) * (uint32_t)(kv_pitch * 2) + IX_ATTN_ROW : 0u;
+    const long first = rows > 0 ? (long)kb * IX_ATTN_BN * kv_pitch : 0;
+    const ix_rsrc_t rk = ix_make_rsrc(kbase + first, bytes);
+    const ix_rsrc_t rv = ix_make_rsrc(vbase + first, bytes);
+    const uint32_t dst = __builtin_amdgcn_readfirstlane(lds0 + stage * IX_ATTN_STAGE);
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+      ix_dma16(rk, dst + j * NT * 16, voff_k[j], 0);
+      ix_dma16(rv, dst + IX_ATTN_TILE + j * NT * 16, voff_v[j], 0);
+    }
+  }
 };
 
-template <int NT>
-__device__ __forceinline__ void ix_attn_fetch1(uint4& kk, uint4& vv, int j, const bf16_t* __restrict__ kbase,
-                                               const bf16_t* __restrict__ vbase, long kv_pitch, int kb, int key_limit) {
-  const int c = j * NT + threadIdx.x;
-  const int key = kb * IX_ATTN_BN + (c >> 4);
-  const int dch = (c & 15) * 8;
-  kk = vv = make_uint4(0, 0, 0, 0);  // beyond the last key any query of this workgroup needs: zeros, nothing read
-  if (key <= key_limit) {
-    kk = *reinterpret_cast<const uint4*>(kbase + (long)key * kv_pitch + dch);
-    vv = *reinterpret_cast<const uint4*>(vbase + (long)key * kv_pitch + dch);
+// Lane (qc = lane % 32, hf = lane / 32) holds query qc. Of a block's 32 scores it holds, in register i, the
+// one of key (i/4)*8 + hf*4 + i%4.
+struct IxAttnLane {
+  uint32_t k_addr;  // LDS byte offset in a K tile of key row qc, chunk hf (step s: XOR with s << 5)
+  uint32_t v_addr;  // LDS byte offset in a V tile of this lane's 8 bytes of the first transpose patch
+  __device__ __forceinline__ void init() {
+    const int lane = threadIdx.x & 63;
+    const int qc = lane & 31, hf = lane >> 5;
+    k_addr = qc * IX_ATTN_ROW + ((hf ^ (qc & 15)) << 4);
+    // A transpose read works in groups of 16 lanes: lane i of a group receives, as element e, element i % 4 of
+    // the 8 bytes that lane 4 e + i / 4 addressed. With lane j addressing key j / 4, d 4 (j % 4) .. +4 of the
+    // group's 4 key x 16 d patch, lane i ends up with keys 0..3 at d = i. The group (lane / 16) % 2 takes the
+    // d half, hf the key quad.
+    const int rl = (lane >> 2) & 3;                             // key within the quad
+    const int cl = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);   // 16-byte chunk within the 64 bytes of a d tile
+    v_addr = (hf * 4 + rl) * IX_ATTN_ROW + (((rl << 2) | cl) << 4) + 8 * (lane & 1);
   }
-}
+};
 
-template <int CPT>
-__device__ __forceinline__ void ix_attn_fetch(IxAttnStage& st, const bf16_t* __restrict__ kbase,
-                                              const bf16_t* __restrict__ vbase, long kv_pitch, int kb, int key_limit) {
-  ix_attn_fetch1<512 / CPT>(st.k0, st.v0, 0, kbase, vbase, kv_pitch, kb, key_limit);
-  if (CPT > 1) ix_attn_fetch1<512 / CPT>(st.k1, st.v1, 1, kbase, vbase, kv_pitch, kb, key_limit);
-}
-
-template <int NT>
-__device__ __forceinline__ void ix_attn_commit1(const uint4& kk, const uint4& vv, int j, char* ldsK, char* ldsV) {
-  const int c = j * NT + threadIdx.x;
-  const int key = c >> 4;
-  const int dch = (c & 15) * 8;
-  *reinterpret_cast<uint4*>(ldsK + key * IX_ATTN_KP + dch * 2) = kk;
-  *reinterpret_cast<uint4*>(ldsV + key * IX_ATTN_VP + dch * 2) = vv;
-}
-
-template <int CPT>
-__device__ __forceinline__ void ix_attn_commit(const IxAttnStage& st, char* ldsK, char* ldsV) {
-  ix_attn_commit1<512 / CPT>(st.k0, st.v0, 0, ldsK, ldsV);
-  if (CPT > 1) ix_attn_commit1<512 / CPT>(st.k1, st.v1, 1, ldsK, ldsV);
-}
-
-// One block of 32 keys for the 32 queries of a wave. Lane (qc = lane % 32, hf = lane / 32) holds
-// query qc; of the block's keys it holds, in register i, key (i/4)*8 + hf*4 + i%4.
-__device__ __forceinline__ void ix_attn_block(const char* ldsK, const char* ldsV, const ix_bf16x8 (&qf)[8],
-                                              ix_f32x16 (&O)[4], float& m, float& l, int kb, int qpos, int min_qpos,
-                                              float c) {
-  const int lane = threadIdx.x & 63;
-  const int qc = lane & 31, hf = lane >> 5;
-  ix_f32x16 sacc;
+// S^T = K Q^T for one block: 8 steps of 16 along d.
+__device__ __forceinline__ void ix_attn_scores(const char* tileK, const IxAttnLane& ln, const ix_bf16x8 (&qf)[8],
+                                               ix_f32x16& sacc) {
 #pragma unroll
   for (int i = 0; i < 16; ++i) sacc[i] = 0.0f;
 #pragma unroll
   for (int s = 0; s < 8; ++s) {
-    const ix_bf16x8 kf = *reinterpret_cast<const ix_bf16x8*>(ldsK + qc * IX_ATTN_KP + (16 * s + hf * 8) * 2);
+    const ix_bf16x8 kf = *reinterpret_cast<const ix_bf16x8*>(tileK + (ln.k_addr ^ (s << 5)));
     sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], sacc, 0, 0, 0);
   }
-  // A block that ends at or before the wave's smallest position needs no mask (wave-uniform test).
-  const bool need_mask = kb * IX_ATTN_BN + IX_ATTN_BN - 1 > min_qpos;
-  if (need_mask) {
+}
+
+// The V^T fragments of one block: vf[dt][s] holds, for d = 32 dt + qc, keys 16 s + hf * 4 + 0..3 and those 8
+// further on -- the same key slots the probabilities of this lane sit in.
+__device__ __forceinline__ void ix_attn_values(const char* tileV, const IxAttnLane& ln, ix_bf16x8 (&vf)[4][2]) {
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt) {
+    const char* src = tileV + (ln.v_addr ^ (dt << 6));
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const ix_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((ix_lds_s16x4*)(src + (16 * s) * IX_ATTN_ROW));
+      const ix_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((ix_lds_s16x4*)(src + (16 * s + 8) * IX_ATTN_ROW));
+      const ix_s16x4 w[2] = {lo, hi};
+      vf[dt][s] = *reinterpret_cast<const ix_bf16x8*>(w);
+    }
+  }
+}
+
+// Online-softmax update of one block from its raw scores, then O^T += V^T P^T. MASK: the block reaches beyond
+// the position of some query of the wave.
+#define IX_ATTN_LAZY 8.0f
+template <bool MASK>
+__device__ __forceinline__ void ix_attn_update(ix_f32x16& sacc, const ix_bf16x8 (&vf)[4][2], ix_f32x16 (&O)[4],
+                                               float& m, float& l, int kb, int qpos, float c) {
+  const int hf = (threadIdx.x & 63) >> 5;
+  if (MASK) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int key = kb * IX_ATTN_BN + (i >> 2) * 8 + hf * 4 + (i & 3);
@@ -103,7 +142,7 @@ __device__ __forceinline__ void ix_attn_block(const char* ldsK, const char* ldsV
 #pragma unroll
   for (int i = 1; i < 16; ++i) bm = fmaxf(bm, sacc[i]);
   bm = fmaxf(bm, __shfl_xor(bm, 32, IX_WAVE));
-  const float m_new = fmaxf(m, bm);
+  const float m_new = (bm - m) * c > IX_ATTN_LAZY ? bm : m;
   const float alpha = ix_exp2((m - m_new) * c);
   const float mc = -(m_new * c);
   float p[16];
@@ -116,8 +155,6 @@ __device__ __forceinline__ void ix_attn_block(const char* ldsK, const char* ldsV
   const float tot = hf ? other + mine : mine + other;  // (half 0) + (half 1) on both lanes
   l = l * alpha + tot;
   m = m_new;
-  // x * 1.0f is x: when no query of the wave moved its maximum, the rescale is skipped for all of them.
-  const bool rescale = __any(alpha != 1.0f);
   ix_bf16x8 pf[2];
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
@@ -126,34 +163,39 @@ __device__ __forceinline__ void ix_attn_block(const char* ldsK, const char* ldsV
     for (int j = 0; j < 4; ++j) w[j] = ix_pack_bf2_hw(p[8 * s + 2 * j], p[8 * s + 2 * j + 1]);
     pf[s] = *reinterpret_cast<const ix_bf16x8*>(w);
   }
-  // this lane's address inside the 4 key x 16 d patch its group of 16 lanes transposes
-  const char* vsrc = ldsV + (hf * 4 + ((lane & 15) >> 2)) * IX_ATTN_VP + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  // x * 1.0f is x: when no query of the wave moved its reference, the rescale is skipped for all of them.
+  if (__any(alpha != 1.0f)) {
 #pragma unroll
-  for (int dt = 0; dt < 4; ++dt) {
-    if (rescale) {
+    for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) O[dt][i] = O[dt][i] * alpha;
-    }
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      // The lane needs V[key][d = 32 dt + qc] for keys 16 s + hf * 4 + 0..3 and those 8 further on. A transpose
-      // read works in groups of 16 lanes: lane i of a group receives, as element e, element i % 4 of the 8 bytes
-      // that lane 4 e + i / 4 of the group addressed. With lane j addressing key j / 4, d 4 * (j % 4) .. +4 of the
-      // group's 4 key x 16 d patch, lane i ends up with keys 0..3 at d = i.
-      typedef __attribute__((address_space(3))) ix_s16x4 lds_s16x4;
-      const char* src = vsrc + (16 * s) * IX_ATTN_VP + 64 * dt;
-      const ix_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(src));
-      const ix_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(src + 8 * IX_ATTN_VP));
-      const ix_s16x4 w[2] = {lo, hi};
-      const ix_bf16x8 vf = *reinterpret_cast<const ix_bf16x8*>(w);
-      O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[s], O[dt], 0, 0, 0);
-    }
   }
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][s], pf[s], O[dt], 0, 0, 0);
+}
+
+// One step of the skewed loop: block kb's values and update, with the scores of block kb + 1 (from the next
+// ring stage) issued in between so that the matrix pipeline works while the softmax arithmetic runs. Past the
+// wave's last block those scores are computed from whatever the stage holds and never used.
+template <bool MASK>
+__device__ __forceinline__ void ix_attn_step(const char* stage, const char* stage_next, const IxAttnLane& ln,
+                                             const ix_bf16x8 (&qf)[8], ix_f32x16& sacc, ix_f32x16 (&O)[4], float& m,
+                                             float& l, int kb, int qpos, float c) {
+  ix_bf16x8 vf[4][2];
+  ix_attn_values(stage + IX_ATTN_TILE, ln, vf);
+  ix_f32x16 snext;
+  ix_attn_scores(stage_next, ln, qf, snext);
+  ix_attn_update<MASK>(sacc, vf, O, m, l, kb, qpos, c);
+  sacc = snext;
 }
 
 // NW waves per workgroup (4 or 8): NW * 32 / GROUP consecutive tokens share each staged key block, so a larger
 // workgroup pulls fewer key/value bytes per query; which queries share a workgroup never reaches the arithmetic.
-template <int GROUP, int NW>
+// Inside a wave the loop is skewed by one block: while block kb goes through its softmax, the scores of block
+// kb + 1 are already in the matrix pipeline.
+template <int GROUP, int NW, int S>
 __global__ __launch_bounds__(NW * 64) void k_attn_varlen(const bf16_t* __restrict__ q, long q_pitch,
                                                      const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
                                                      long kv_pitch, bf16_t* __restrict__ o,
@@ -161,10 +203,10 @@ __global__ __launch_bounds__(NW * 64) void k_attn_varlen(const bf16_t* __restric
                                                      const int* __restrict__ q_pos0, int HQ, float scale) {
   constexpr int TOK_W = 32 / GROUP;   // tokens per wave
   constexpr int TOK_WG = NW * TOK_W;  // tokens per workgroup
-  constexpr int CPT = 512 / (NW * 64);
-  // two LDS copies of the key/value block: block kb+1 is written while block kb is still being read
-  __shared__ __attribute__((aligned(16))) char ldsK[2][IX_ATTN_BN * IX_ATTN_KP];
-  __shared__ __attribute__((aligned(16))) char ldsV[2][IX_ATTN_BN * IX_ATTN_VP];
+  constexpr int NT = NW * 64;
+  constexpr int CPT = 512 / NT;
+  static_assert(S >= 3, "the ring holds the block being read, the next one and at least one in flight");
+  extern __shared__ __align__(16) char ix_attn_lds[];
   const int n = blockIdx.y, g = blockIdx.z;
   const int qb = cu_q[n];
   const int len = cu_q[n + 1] - qb;
@@ -201,8 +243,9 @@ __global__ __launch_bounds__(NW * 64) void k_attn_varlen(const bf16_t* __restric
   const int nblocks = key_limit / IX_ATTN_BN + 1;
   const int wave_last = min(len - 1, t0 + wave * TOK_W + TOK_W - 1);
   const int wave_blocks = wave_last >= t0 + wave * TOK_W ? (p0 + wave_last) / IX_ATTN_BN + 1 : 0;
-  // smallest position among the wave's live queries (its first token); padding columns have no limit
-  const int wave_min_qpos = p0 + t0 + wave * TOK_W;
+  // A block that ends at or before the smallest position among the wave's live queries (its first token; padding
+  // columns have no limit) needs no mask: blocks below first_masked.
+  const int first_masked = (p0 + t0 + wave * TOK_W + 1) / IX_ATTN_BN;
   const long kv0 = kv_start[n];
   const bf16_t* kbase = k + kv0 * kv_pitch + (long)g * IX_ATTN_D;
   const bf16_t* vbase = v + kv0 * kv_pitch + (long)g * IX_ATTN_D;
@@ -215,27 +258,40 @@ __global__ __launch_bounds__(NW * 64) void k_attn_varlen(const bf16_t* __restric
   float m = IX_NEG_INF, l = 0.0f;
   const float c = scale * IX_LOG2E;
 
-  // Two register stages: while block kb is multiplied, block kb+1 sits in LDS and blocks kb+2 and kb+3 are
-  // in flight from memory. One barrier per block.
-  IxAttnStage sa, sb;
-  ix_attn_fetch<CPT>(sa, kbase, vbase, kv_pitch, 0, key_limit);
-  if (nblocks > 1) ix_attn_fetch<CPT>(sb, kbase, vbase, kv_pitch, 1, key_limit);
-  ix_attn_commit<CPT>(sa, ldsK[0], ldsV[0]);
-  if (nblocks > 2) ix_attn_fetch<CPT>(sa, kbase, vbase, kv_pitch, 2, key_limit);
+  IxAttnFetch<NT> fetch;
+  fetch.init(ix_attn_lds, (uint32_t)(kv_pitch * 2));
+  IxAttnLane ln;
+  ln.init();
+  // The q loads above are the only vector-memory operations the compiler counts; they have been consumed
+  // (converted into qf) before the first wait below is trusted to speak of the ring alone.
+  __builtin_amdgcn_s_waitcnt(IX_VMCNT(0));
+#pragma unroll
+  for (int b = 0; b < S - 1; ++b) fetch.issue(kbase, vbase, kv_pitch, b, b, key_limit);
+  __builtin_amdgcn_s_waitcnt(IX_VMCNT((S - 2) * 2 * CPT));  // block 0 has landed
   __syncthreads();
-  for (int kb = 0; kb < nblocks; kb += 2) {
-    // even block: compute from copy 0; publish block kb+1 (stage b) into copy 1; refill stage b with kb+3
-    if (kb < wave_blocks) ix_attn_block(ldsK[0], ldsV[0], qf, O, m, l, kb, qpos, wave_min_qpos, c);
-    if (kb + 1 < nblocks) ix_attn_commit<CPT>(sb, ldsK[1], ldsV[1]);
-    if (kb + 3 < nblocks) ix_attn_fetch<CPT>(sb, kbase, vbase, kv_pitch, kb + 3, key_limit);
+  ix_f32x16 sacc;
+  if (wave_blocks > 0) ix_attn_scores(ix_attn_lds, ln, qf, sacc);
+  int st = 0;  // ring stage of block kb
+  for (int kb = 0; kb < nblocks; ++kb) {
+    // Blocks 0 .. kb+S-2 have been issued; all but the newest S-3 of them, so blocks up to kb+1, have landed for
+    // this thread after the wait and for every thread after the barrier. The barrier also says that every wave
+    // is done with block kb-1, whose stage the next fetch overwrites.
+    __builtin_amdgcn_s_waitcnt(IX_VMCNT((S - 3) * 2 * CPT));
     __syncthreads();
-    if (kb + 1 >= nblocks) break;
-    // odd block: compute from copy 1; publish block kb+2 (stage a) into copy 0; refill stage a with kb+4
-    if (kb + 1 < wave_blocks) ix_attn_block(ldsK[1], ldsV[1], qf, O, m, l, kb + 1, qpos, wave_min_qpos, c);
-    if (kb + 2 < nblocks) ix_attn_commit<CPT>(sa, ldsK[0], ldsV[0]);
-    if (kb + 4 < nblocks) ix_attn_fetch<CPT>(sa, kbase, vbase, kv_pitch, kb + 4, key_limit);
-    __syncthreads();
+    const int st_free = st == 0 ? S - 1 : st - 1;
+    const int st_next = st == S - 1 ? 0 : st + 1;
+    fetch.issue(kbase, vbase, kv_pitch, kb + S - 1, st_free, key_limit);
+    if (kb < wave_blocks) {
+      const char* cur = ix_attn_lds + st * IX_ATTN_STAGE;
+      const char* nxt = ix_attn_lds + st_next * IX_ATTN_STAGE;
+      if (kb < first_masked)
+        ix_attn_step<false>(cur, nxt, ln, qf, sacc, O, m, l, kb, qpos, c);
+      else
+        ix_attn_step<true>(cur, nxt, ln, qf, sacc, O, m, l, kb, qpos, c);
+    }
+    st = st_next;
   }
+  __builtin_amdgcn_s_waitcnt(IX_VMCNT(0));  // nothing may still be on its way into LDS when the wave ends
   if (live) {
     const float inv = 1.0f / l;
 #pragma unroll
@@ -252,6 +308,27 @@ __global__ __launch_bounds__(NW * 64) void k_attn_varlen(const bf16_t* __restric
   }
 }
 
+template <int GROUP, int NW, int S>
+static int ix_attn_launch(const void* q, long q_pitch, const void* k, const void* v, long kv_pitch, void* o,
+                          const int* cu_q, const long* kv_start, const int* q_pos0, long N, long max_q_len, long HQ,
+                          long HKV, float scale, hipStream_t st) {
+  constexpr int LDS = S * IX_ATTN_STAGE;
+  auto kern = k_attn_varlen<GROUP, NW, S>;
+  static bool attr_set = false;  // per instantiation
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS) != hipSuccess)
+      return IX_ERR_LAUNCH;
+    attr_set = true;
+  }
+  const long tok_wg = NW * (32 / GROUP);
+  const long tiles = (max_q_len + tok_wg - 1) / tok_wg;
+  if (tiles > 0x7fffffffL) return IX_DECLINED;
+  hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)N, (unsigned)HKV), dim3(NW * 64), LDS, st,
+                     (const bf16_t*)q, q_pitch, (const bf16_t*)k, (const bf16_t*)v, kv_pitch, (bf16_t*)o, cu_q,
+                     kv_start, q_pos0, (int)HQ, scale);
+  return ix_launch_status();
+}
+
 extern "C" int ix_attn_varlen(const void* q, long q_pitch, const void* k, const void* v, long kv_pitch, void* o,
                               const int* cu_q, const long* kv_start, const int* q_pos0, long N, long max_q_len,
                               long HQ, long HKV, long D, float scale, void* stream) {
@@ -264,23 +341,17 @@ extern "C" int ix_attn_varlen(const void* q, long q_pitch, const void* k, const 
     return IX_DECLINED;
   if (N == 0 || max_q_len == 0) return IX_OK;
   if (N > 65535 || HKV > 65535) return IX_DECLINED;
+  if (kv_pitch >= (1L << 26)) return IX_DECLINED;  // a block's byte range must fit the 32-bit buffer size
   const int group = (int)(HQ / HKV);
   hipStream_t st = (hipStream_t)stream;
-#define IX_ATTN_LAUNCH_NW(G, NWV)                                                                               \
-  {                                                                                                             \
-    const long tok_wg = NWV * (32 / G);                                                                         \
-    const long tiles = (max_q_len + tok_wg - 1) / tok_wg;                                                       \
-    if (tiles > 0x7fffffffL) return IX_DECLINED;                                                                \
-    hipLaunchKernelGGL((k_attn_varlen<G, NWV>), dim3((unsigned)tiles, (unsigned)N, (unsigned)HKV),              \
-                       dim3(NWV * 64), 0, st, (const bf16_t*)q, q_pitch, (const bf16_t*)k, (const bf16_t*)v,    \
-                       kv_pitch, (bf16_t*)o, cu_q, kv_start, q_pos0, (int)HQ, scale);                           \
-  }
-#define IX_ATTN_LAUNCH(G)                                                                                       \
-  case G:                                                                                                       \
-    if (big) IX_ATTN_LAUNCH_NW(G, 8) else IX_ATTN_LAUNCH_NW(G, 4)                                               \
-    break;
   // long query runs (prefill) use eight waves per workgroup, short ones (decode, small chunks) four
   const bool big = max_q_len >= 8 * (32 / group);
+#define IX_ATTN_LAUNCH(G)                                                                                          \
+  case G:                                                                                                          \
+    return big ? ix_attn_launch<G, 8, IX_ATTN_STAGES_BIG>(q, q_pitch, k, v, kv_pitch, o, cu_q, kv_start, q_pos0, N, \
+                                                          max_q_len, HQ, HKV, scale, st)                           \
+               : ix_attn_launch<G, 4, IX_ATTN_STAGES_SMALL>(q, q_pitch, k, v, kv_pitch, o, cu_q, kv_start, q_pos0, \
+                                                            N, max_q_len, HQ, HKV, scale, st);
   switch (group) {
     IX_ATTN_LAUNCH(1)
     IX_ATTN_LAUNCH(2)
@@ -291,9 +362,7 @@ extern "C" int ix_attn_varlen(const void* q, long q_pitch, const void* k, const 
     default:
       return IX_DECLINED;
   }
-#undef IX_ATTN_LAUNCH_NW
 #undef IX_ATTN_LAUNCH
-  return ix_launch_status();
 }
 
 // ---- rotary position embedding -------------------------------------------------------------------
