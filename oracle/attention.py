@@ -40,7 +40,7 @@ def attend_one(q, K, V, scale, prims: Prims = DEFAULT, block: int = BLOCK):
     Returns ``o [D]`` as fp32 holding bf16 values."""
     L, D = K.shape
     m = F32(-np.inf)
-    l = F32(0.0)
+    l = [F32(0.0), F32(0.0)]  # one share of the denominator per half-wave
     O = np.zeros(D, dtype=F32)
     q64 = q.astype(np.float64)
     c = F32(F32(scale) * LOG2E)  # scale > 0: the running maximum is kept in unscaled units
@@ -67,12 +67,11 @@ def attend_one(q, K, V, scale, prims: Prims = DEFAULT, block: int = BLOCK):
             for c0 in range(8, len(mine), 8):
                 acc = F32(acc + F32(pairwise_tree(mine[c0 : c0 + 8][None, :])[0]))
             halves.append(acc)
-        tot = F32(halves[0] + halves[1])
-        l = F32(F32(l * alpha) + tot)
+        l = [F32(F32(l[hf] * alpha) + halves[hf]) for hf in (0, 1)]
         pv = (round_bf16(p[:n]).astype(np.float64) @ vb.astype(np.float64)).astype(F32)
         O = ((O * alpha).astype(F32) + pv).astype(F32)
         m = F32(m_new)
-    return round_bf16((O * F32(F32(1.0) / l)).astype(F32))
+    return round_bf16((O * F32(F32(1.0) / F32(l[0] + l[1]))).astype(F32))
 
 
 def attend_causal(q, k, v, scale=None, q_pos0: int = 0, prims: Prims = DEFAULT, block: int = BLOCK):

@@ -11,9 +11,9 @@
 //                                                        grown by more than 2^8; m starts at -inf
 //               a    = exp2((m - m') * c)                exactly 1 when the reference did not move
 //               p_j  = exp2(fma(s_j, c, -(m' * c)))      one fused multiply-add per score; p_j <= 2^8 (1 + eps)
-//               l    = l * a + (lo + hi)                 lo/hi: the two halves' sums, see ix_attn_block
+//               l_h  = l_h * a + sum of p_j over the 16 keys of half h (h = (j / 4) % 2), as two 8-trees
 //               O    = O * a + sum_j bf16(p_j) * v_j     bf16 MFMA, fp32 accumulate, keys in 2 steps of 16
-//   out = bf16(O * (1 / l)), one IEEE reciprocal per query.
+//   out = bf16(O * (1 / (l_0 + l_1))), one IEEE reciprocal per query.
 // Nothing in that chain depends on which other queries share the launch: a workgroup holds the
 // queries of 32/GROUP * 4 consecutive tokens for the GROUP query heads of one key/value head, every
 // MFMA row or column belongs to one query, and a block that lies wholly beyond a query's position is
@@ -96,16 +96,18 @@ struct IxAttnLane {
   }
 };
 
+// The K fragments of one block: kf[s] holds d 16 s + hf * 8 .. +8 of key qc.
+__device__ __forceinline__ void ix_attn_keys(const char* tileK, const IxAttnLane& ln, ix_bf16x8 (&kf)[8]) {
+#pragma unroll
+  for (int s = 0; s < 8; ++s) kf[s] = *reinterpret_cast<const ix_bf16x8*>(tileK + (ln.k_addr ^ (s << 5)));
+}
+
 // S^T = K Q^T for one block: 8 steps of 16 along d.
-__device__ __forceinline__ void ix_attn_scores(const char* tileK, const IxAttnLane& ln, const ix_bf16x8 (&qf)[8],
-                                               ix_f32x16& sacc) {
+__device__ __forceinline__ void ix_attn_scores(const ix_bf16x8 (&kf)[8], const ix_bf16x8 (&qf)[8], ix_f32x16& sacc) {
 #pragma unroll
   for (int i = 0; i < 16; ++i) sacc[i] = 0.0f;
 #pragma unroll
-  for (int s = 0; s < 8; ++s) {
-    const ix_bf16x8 kf = *reinterpret_cast<const ix_bf16x8*>(tileK + (ln.k_addr ^ (s << 5)));
-    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], sacc, 0, 0, 0);
-  }
+  for (int s = 0; s < 8; ++s) sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s], qf[s], sacc, 0, 0, 0);
 }
 
 // The V^T fragments of one block: vf[dt][s] holds, for d = 32 dt + qc, keys 16 s + hf * 4 + 0..3 and those 8
@@ -124,13 +126,29 @@ __device__ __forceinline__ void ix_attn_values(const char* tileV, const IxAttnLa
   }
 }
 
-// Online-softmax update of one block from its raw scores, then O^T += V^T P^T. MASK: the block reaches beyond
-// the position of some query of the wave.
+// max(x of this lane, x of the lane 32 away) without a trip through LDS.
+__device__ __forceinline__ float ix_attn_max_halves(float x) {
+  const uint32_t u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+// One step of the skewed loop. The softmax arithmetic of block kb needs only registers (its scores were
+// computed a step earlier), so it runs while the fragments of V (block kb) and of K (block kb + 1, from the
+// next ring stage) travel from LDS; then O^T += V^T P^T and the scores of block kb + 1. Past the wave's last
+// block those scores are computed from whatever the stage holds and never used.
+// MASK: the block reaches beyond the position of some query of the wave.
+// l is this HALF's share of the denominator: the 16 key slots the lane holds; the halves meet at the end.
 #define IX_ATTN_LAZY 8.0f
 template <bool MASK>
-__device__ __forceinline__ void ix_attn_update(ix_f32x16& sacc, const ix_bf16x8 (&vf)[4][2], ix_f32x16 (&O)[4],
-                                               float& m, float& l, int kb, int qpos, float c) {
+__device__ __forceinline__ void ix_attn_step(const char* stage, const char* stage_next, const IxAttnLane& ln,
+                                             const ix_bf16x8 (&qf)[8], ix_f32x16& sacc, ix_f32x16 (&O)[4], float& m,
+                                             float& l, int kb, int qpos, float c) {
   const int hf = (threadIdx.x & 63) >> 5;
+  ix_bf16x8 vf[4][2];
+  ix_attn_values(stage + IX_ATTN_TILE, ln, vf);
+  ix_bf16x8 kf[8];
+  ix_attn_keys(stage_next, ln, kf);
   if (MASK) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
@@ -141,7 +159,7 @@ __device__ __forceinline__ void ix_attn_update(ix_f32x16& sacc, const ix_bf16x8 
   float bm = sacc[0];
 #pragma unroll
   for (int i = 1; i < 16; ++i) bm = fmaxf(bm, sacc[i]);
-  bm = fmaxf(bm, __shfl_xor(bm, 32, IX_WAVE));
+  bm = ix_attn_max_halves(bm);
   const float m_new = (bm - m) * c > IX_ATTN_LAZY ? bm : m;
   const float alpha = ix_exp2((m - m_new) * c);
   const float mc = -(m_new * c);
@@ -150,10 +168,7 @@ __device__ __forceinline__ void ix_attn_update(ix_f32x16& sacc, const ix_bf16x8 
   for (int i = 0; i < 16; ++i) p[i] = ix_exp2(__builtin_fmaf(sacc[i], c, mc));
   const float pa[8] = {p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]};
   const float pb[8] = {p[8], p[9], p[10], p[11], p[12], p[13], p[14], p[15]};
-  const float mine = ix_tree8(pa) + ix_tree8(pb);
-  const float other = __shfl_xor(mine, 32, IX_WAVE);
-  const float tot = hf ? other + mine : mine + other;  // (half 0) + (half 1) on both lanes
-  l = l * alpha + tot;
+  l = l * alpha + (ix_tree8(pa) + ix_tree8(pb));
   m = m_new;
   ix_bf16x8 pf[2];
 #pragma unroll
@@ -174,21 +189,7 @@ __device__ __forceinline__ void ix_attn_update(ix_f32x16& sacc, const ix_bf16x8 
   for (int s = 0; s < 2; ++s)
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt) O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][s], pf[s], O[dt], 0, 0, 0);
-}
-
-// One step of the skewed loop: block kb's values and update, with the scores of block kb + 1 (from the next
-// ring stage) issued in between so that the matrix pipeline works while the softmax arithmetic runs. Past the
-// wave's last block those scores are computed from whatever the stage holds and never used.
-template <bool MASK>
-__device__ __forceinline__ void ix_attn_step(const char* stage, const char* stage_next, const IxAttnLane& ln,
-                                             const ix_bf16x8 (&qf)[8], ix_f32x16& sacc, ix_f32x16 (&O)[4], float& m,
-                                             float& l, int kb, int qpos, float c) {
-  ix_bf16x8 vf[4][2];
-  ix_attn_values(stage + IX_ATTN_TILE, ln, vf);
-  ix_f32x16 snext;
-  ix_attn_scores(stage_next, ln, qf, snext);
-  ix_attn_update<MASK>(sacc, vf, O, m, l, kb, qpos, c);
-  sacc = snext;
+  ix_attn_scores(kf, qf, sacc);
 }
 
 // NW waves per workgroup (4 or 8): NW * 32 / GROUP consecutive tokens share each staged key block, so a larger
@@ -270,7 +271,11 @@ __global__ __launch_bounds__(NW * 64) void k_attn_varlen(const bf16_t* __restric
   __builtin_amdgcn_s_waitcnt(IX_VMCNT((S - 2) * 2 * CPT));  // block 0 has landed
   __syncthreads();
   ix_f32x16 sacc;
-  if (wave_blocks > 0) ix_attn_scores(ix_attn_lds, ln, qf, sacc);
+  if (wave_blocks > 0) {
+    ix_bf16x8 kf[8];
+    ix_attn_keys(ix_attn_lds, ln, kf);
+    ix_attn_scores(kf, qf, sacc);
+  }
   int st = 0;  // ring stage of block kb
   for (int kb = 0; kb < nblocks; ++kb) {
     // Blocks 0 .. kb+S-2 have been issued; all but the newest S-3 of them, so blocks up to kb+1, have landed for
@@ -292,6 +297,9 @@ __global__ __launch_bounds__(NW * 64) void k_attn_varlen(const bf16_t* __restric
     st = st_next;
   }
   __builtin_amdgcn_s_waitcnt(IX_VMCNT(0));  // nothing may still be on its way into LDS when the wave ends
+  // the denominator: (half 0's share) + (half 1's share), in that order on both lanes
+  const float l_other = __shfl_xor(l, 32, IX_WAVE);
+  l = hf ? l_other + l : l + l_other;
   if (live) {
     const float inv = 1.0f / l;
 #pragma unroll

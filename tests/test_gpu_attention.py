@@ -67,6 +67,52 @@ def test_known_answers_are_bit_exact(HQ, HKV, dprims):
         start += n
 
 
+def test_growing_maximum_known_answers_are_bit_exact(dprims):
+    """scale = float32(ln 2) makes the exponent factor exactly 1, so integer scores give probabilities
+    that are exact powers of two; with values in {-1, 0, 1} every partial sum stays exact in any order.
+    The scores grow along the keys so that the reference point is moved (a rise of 10 and of 9), is
+    left alone (a rise of 6, and of exactly 8, the boundary), and probabilities above 1 (up to 2^8)
+    enter the value product and the denominator."""
+    HQ, HKV = 8, 1
+    lens = [130, 45]
+    T = sum(lens)
+    rng = np.random.default_rng(77)
+    q = np.zeros((T, HQ, D), np.float32)
+    k = np.zeros((T, HKV, D), np.float32)
+    v = rng.integers(-1, 2, size=(T, HKV, D)).astype(np.float32)
+    for h in range(HQ):
+        q[:, h, 7 * h] = 1.0
+    start = 0
+    for n in lens:
+        for h in range(HQ):
+            s = np.zeros(n)
+            j = np.arange(n)
+            blk1 = (j > 40) & (j < 64)
+            s[blk1] = rng.integers(4, 11, size=blk1.sum())
+            s[40:41] = 10  # rise of 10 over the reference 0: moved
+            blk2 = (j >= 64) & (j < 96)
+            s[blk2] = rng.integers(6, 11, size=blk2.sum())
+            if n > 70:
+                s[70] = 16  # rise of 6: not moved, probability 2^6
+            blk3 = (j >= 96) & (j < 128)
+            s[blk3] = rng.integers(10, 14, size=blk3.sum())
+            if n > 120:
+                s[[100, 120]] = 18  # rise of exactly 8: not moved, probability 2^8
+            if n > 128:
+                s[128:] = 19  # rise of 9: moved
+            k[start : start + n, 0, 7 * h] = s
+        start += n
+    scale = float(np.float32(np.log(2.0)))
+    assert np.float32(scale) * np.float32(1.44269504088896340736) == np.float32(1.0)
+    got = attn(np_to_bf16(q, DEV), np_to_bf16(k, DEV), np_to_bf16(v, DEV), lens, scale=scale)
+    start = 0
+    for n in lens:
+        sl = slice(start, start + n)
+        want = o_attn.attend_causal(q[sl], k[sl], v[sl], scale=scale, prims=dprims)
+        assert np.array_equal(np_bits(bf16_to_np(got[sl])), np_bits(want)), n
+        start += n
+
+
 def test_random_inputs_within_tolerance_of_oracle_and_float64(dprims):
     """Config-4 head layout (32 query heads, 4 key/value heads, d 128). Tolerance: 2^-7 of the
     output scale against the oracle (one bf16 ulp where an fp32 sum lands near a rounding boundary),
