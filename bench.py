@@ -26,7 +26,7 @@ PEAK_MFMA_BF16_TFLOPS = 2500.0  # MI355X dense bf16
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch of the dominant kernels, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by
 # what the same counters read for a 1 GiB copy (x2.0 / x1.0); see profiles/*.txt. Workload-specific.
-MEASURED_TRAFFIC_BYTES = {"dense_head_M4096_gemm": 14.39e9, "gdn_decode_B256": 1.1016e9}
+MEASURED_TRAFFIC_BYTES = {"dense_head_M4096_gemm": 9.08e9, "gdn_decode_B256": 1.1016e9}
 
 
 class KernelTimer:

@@ -9,13 +9,30 @@
 // and each XCD has its own L2: all M-tiles of one weight tile go to one XCD so a weight tile
 // is fetched from HBM by exactly one L2, while the (small) activation matrix is shared
 // through the memory-side cache.
+#ifndef IX_GEMM_GM
+#define IX_GEMM_GM 8  // M-tiles of a group
+#endif
+#ifndef IX_GEMM_GN
+#define IX_GEMM_GN 4  // weight tiles (per XCD) of a group
+#endif
 __device__ __forceinline__ bool ix_tile_of_block(long bid, int nb_m, int nb_n, int* tm, int* tn) {
   const int xcd = (int)(bid & 7);
   const long idx = bid >> 3;
-  const long nloc = idx / nb_m;
-  *tm = (int)(idx - nloc * nb_m);
-  *tn = (int)(nloc * 8 + xcd);
-  return *tn < nb_n;
+  // Inside an XCD the tiles run in groups of GM M-tiles x GN weight tiles -- about what its 32 CUs hold at a
+  // time -- so that a group pulls GM activation tiles and GN weight tiles through the L2 for GM * GN tiles.
+  const int nloc_total = (nb_n + 7) / 8;  // weight-tile columns of this XCD (the last may be absent)
+  const long per_ngroup = (long)IX_GEMM_GN * nb_m;
+  const long ng = idx / per_ngroup;
+  const long rem = idx - ng * per_ngroup;
+  const int gn = min(IX_GEMM_GN, nloc_total - (int)ng * IX_GEMM_GN);  // width of this (possibly last) group
+  const long per_mgroup = (long)IX_GEMM_GM * gn;
+  const long mg = rem / per_mgroup;
+  const long r2 = rem - mg * per_mgroup;
+  const int gm = min(IX_GEMM_GM, nb_m - (int)mg * IX_GEMM_GM);
+  const int nl = (int)(r2 / gm), ml = (int)(r2 - (long)nl * gm);
+  *tm = (int)mg * IX_GEMM_GM + ml;
+  *tn = ((int)ng * IX_GEMM_GN + nl) * 8 + xcd;
+  return *tn < nb_n && *tm < nb_m && nl < gn;
 }
 
 __device__ __forceinline__ void ix_store4(bf16_t* p, int valid, bool vec, const float (&v)[4]) {
@@ -45,6 +62,9 @@ __global__ __launch_bounds__(WM* WN * 64) void k_gemm_bf16_nt(const bf16_t* __re
   extern __shared__ __align__(16) char ix_lds[];
   int tm, tn;
   if (!ix_tile_of_block(blockIdx.x, nb_m, nb_n, &tm, &tn)) return;
+#ifdef IX_EXPERIMENT_SAME_TILE
+  tm = 0; tn = tn & 7;
+#endif
   const long m0 = (long)tm * BM;
   const long n0 = (long)tn * BN;
   const int m_valid = (int)min((long)BM, (long)M - m0);

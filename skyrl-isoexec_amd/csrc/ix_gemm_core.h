@@ -297,8 +297,9 @@ __device__ __forceinline__ void ix_gemm_mainloop_h4(ix_rsrc_t x_rsrc, const XRow
 }
 
 // ---- pipeline C: a ring of whole-k-tile OPERAND units (square tiles only) --------------------------
-// Unit u = 2*kt holds the X rows of k-tile kt, unit 2*kt+1 its W rows; each is BM rows of 128 bytes, so
-// every fetch moves whole 128-byte lines. The ring holds NU units: the two being consumed and NU-2 in
+// Unit u = 2*kt holds the W rows of k-tile kt, unit 2*kt+1 its X rows; each is BM rows of 128 bytes, so
+// every fetch moves whole 128-byte lines. A W unit is therefore issued two k-tiles before its use and an X unit
+// one and a half: the weights are the operand that comes from HBM, the activations are shared and cached. The ring holds NU units: the two being consumed and NU-2 in
 // flight. One barrier per k-tile: after it every wave is done with k-tile kt-1, whose two slots take the
 // next two units. The K order is that of pipeline A.
 template <typename Cfg, typename XRow, typename WRow, typename Acc>
@@ -366,25 +367,30 @@ __device__ __forceinline__ void ix_gemm_mainloop_units(ix_rsrc_t x_rsrc, const X
   int is = 0;  // slot of the next unit to issue
 #pragma unroll
   for (int u = 0; u < NU - 2; ++u) {
-    if (u & 1) issue(w_rsrc, w_voff, u >> 1, is); else issue(x_rsrc, x_voff, u >> 1, is);
+    if (u & 1) issue(x_rsrc, x_voff, u >> 1, is); else issue(w_rsrc, w_voff, u >> 1, is);
     is = is + 1 == NU ? 0 : is + 1;
   }
-  int cs = 0;            // slot of the X unit being consumed
+  int cs = 0;            // slot of the W unit being consumed
   int nu = NU - 2;       // index of the next unit to issue
   for (int kt = 0; kt < KT; ++kt) {
     __builtin_amdgcn_s_waitcnt(IX_VMCNT((NU - 4) * CH));  // units 2kt and 2kt+1 have landed
     __syncthreads();
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
-      if (nu & 1) issue(w_rsrc, w_voff, nu >> 1, is); else issue(x_rsrc, x_voff, nu >> 1, is);
+      if (nu & 1) issue(x_rsrc, x_voff, nu >> 1, is); else issue(w_rsrc, w_voff, nu >> 1, is);
       is = is + 1 == NU ? 0 : is + 1;
       ++nu;
     }
-    const char* xs = lds + cs * UNIT;
-    const int wsl = cs + 1 == NU ? 0 : cs + 1;
-    const char* ws = lds + wsl * UNIT;
-    cs = wsl + 1 == NU ? 0 : wsl + 1;
+    const char* ws = lds + cs * UNIT;
+    const int xsl = cs + 1 == NU ? 0 : cs + 1;
+    const char* xs = lds + xsl * UNIT;
+    cs = xsl + 1 == NU ? 0 : xsl + 1;
+    // The last quarter of k-tile kt-1 (fragments read before the barrier) is multiplied while the first
+    // fragments of k-tile kt travel from LDS: the matrix pipeline has work on both sides of the barrier.
     frags(xs, ws, 0, xa, wa);
+    __builtin_amdgcn_sched_barrier(0);
+    if (kt > 0) mfmas(xb, wb);
+    __builtin_amdgcn_sched_barrier(0);
     frags(xs, ws, 1, xb, wb);
     __builtin_amdgcn_sched_barrier(0);
     mfmas(xa, wa);
@@ -397,9 +403,8 @@ __device__ __forceinline__ void ix_gemm_mainloop_units(ix_rsrc_t x_rsrc, const X
     __builtin_amdgcn_sched_barrier(0);
     mfmas(xa, wa);
     __builtin_amdgcn_sched_barrier(0);
-    mfmas(xb, wb);
-    __builtin_amdgcn_sched_barrier(0);
   }
+  mfmas(xb, wb);
   __builtin_amdgcn_s_waitcnt(IX_VMCNT(0));
 }
 
