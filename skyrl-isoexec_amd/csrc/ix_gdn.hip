@@ -422,7 +422,7 @@ __global__ __launch_bounds__(256) void k_gdn_conv(const bf16_t* __restrict__ x, 
 
 // Eight consecutive channels of four consecutive tokens per thread: 16-byte loads and stores, and inside a
 // sequence each input row is loaded once for the four windows that cover it. Per channel the arithmetic is that
-// of k_gdn_conv, statement for statement, so the two kernels agree bit for bit.
+// of k_gdn_conv, statement for statement, so the two kernels agree bit for bit (a NaN keeps its payload here).
 template <int W>
 __device__ __forceinline__ void ix_conv8_finish(const float (&xv)[W][8], const float (&wv)[8][W],
                                                 const bf16_t* __restrict__ bias, int d, int silu,
@@ -443,7 +443,7 @@ __device__ __forceinline__ void ix_conv8_finish(const float (&xv)[W][8], const f
       if (silu) acc = acc * ix_sigmoid(acc);
       r2[e] = acc;
     }
-    out[c >> 1] = ix_pack_bf2(r2[0], r2[1]);
+    out[c >> 1] = ix_pack_bf2_hw(r2[0], r2[1]);
   }
   *reinterpret_cast<uint4*>(yrow) = make_uint4(out[0], out[1], out[2], out[3]);
 }

@@ -39,8 +39,9 @@ def test_prim_transcendentals_close_to_libm(dprims):
         got = dprims._run(name, arg)
         ref = getattr(host, name)(arg.astype(np.float32))
         rel = np.abs(got - ref) / np.maximum(np.abs(ref), 1e-30)
-        # exp_fast rounds its argument product once: relative error <= |x| * 2^-24 * ln2 + 1 ulp
-        tol = 6e-6 if name == "exp_fast" else 4e-7
+        # exp_fast, and the sigmoid built on the hardware 2^x, round their argument product once:
+        # relative error <= |x| * 2^-24 * ln2 + a few ulp
+        tol = 6e-6 if name in ("exp_fast", "sigmoid", "silu_div") else 4e-7
         assert rel.max() <= tol, (name, rel.max())
 
 
