@@ -5,34 +5,37 @@
 #include "ix_gemm_core.h"
 #include "../../include/isoexec_hip.h"
 
-// Workgroup -> tile map. Hardware hands consecutive workgroup ids to the 8 XCDs round-robin,
-// and each XCD has its own L2: all M-tiles of one weight tile go to one XCD so a weight tile
-// is fetched from HBM by exactly one L2, while the (small) activation matrix is shared
-// through the memory-side cache.
+// Workgroup -> tile map. Hardware hands consecutive workgroup ids to the 8 XCDs round-robin, and each XCD has
+// its own L2. The tiles are put in one order -- groups of GM M-tiles x GN weight tiles, about what an XCD's 32
+// CUs hold at a time, so that a group pulls GM activation tiles and GN weight tiles through the L2 for GM * GN
+// tiles; groups run down the M-tiles of GN weight-tile columns before moving to the next columns -- and that
+// order is cut into 8 equal runs, one per XCD: every XCD gets the same number of tiles whatever the shape, and
+// a weight tile is fetched by one L2 (two where a run ends inside its column group).
 #ifndef IX_GEMM_GM
 #define IX_GEMM_GM 8  // M-tiles of a group
 #endif
 #ifndef IX_GEMM_GN
-#define IX_GEMM_GN 4  // weight tiles (per XCD) of a group
+#define IX_GEMM_GN 4  // weight tiles of a group
 #endif
 __device__ __forceinline__ bool ix_tile_of_block(long bid, int nb_m, int nb_n, int* tm, int* tn) {
   const int xcd = (int)(bid & 7);
   const long idx = bid >> 3;
-  // Inside an XCD the tiles run in groups of GM M-tiles x GN weight tiles -- about what its 32 CUs hold at a
-  // time -- so that a group pulls GM activation tiles and GN weight tiles through the L2 for GM * GN tiles.
-  const int nloc_total = (nb_n + 7) / 8;  // weight-tile columns of this XCD (the last may be absent)
+  const long tiles = (long)nb_m * nb_n;
+  const long lo = tiles * xcd / 8, hi = tiles * (xcd + 1) / 8;  // this XCD's run of the tile order
+  const long l = lo + idx;
+  if (l >= hi) return false;
   const long per_ngroup = (long)IX_GEMM_GN * nb_m;
-  const long ng = idx / per_ngroup;
-  const long rem = idx - ng * per_ngroup;
-  const int gn = min(IX_GEMM_GN, nloc_total - (int)ng * IX_GEMM_GN);  // width of this (possibly last) group
+  const long ng = l / per_ngroup;
+  const long rem = l - ng * per_ngroup;
+  const int gn = min(IX_GEMM_GN, nb_n - (int)ng * IX_GEMM_GN);  // width of this (possibly last) column group
   const long per_mgroup = (long)IX_GEMM_GM * gn;
   const long mg = rem / per_mgroup;
   const long r2 = rem - mg * per_mgroup;
   const int gm = min(IX_GEMM_GM, nb_m - (int)mg * IX_GEMM_GM);
   const int nl = (int)(r2 / gm), ml = (int)(r2 - (long)nl * gm);
   *tm = (int)mg * IX_GEMM_GM + ml;
-  *tn = ((int)ng * IX_GEMM_GN + nl) * 8 + xcd;
-  return *tn < nb_n && *tm < nb_m && nl < gn;
+  *tn = (int)ng * IX_GEMM_GN + nl;
+  return true;
 }
 
 __device__ __forceinline__ void ix_store4(bf16_t* p, int valid, bool vec, const float (&v)[4]) {
@@ -131,7 +134,7 @@ static int ix_gemm_bf16_launch(const bf16_t* A, long lda, const bf16_t* W, long 
                                long ldc, long M, long N, long K, float* parts, long parts_ld, hipStream_t st) {
   using Cfg = IxGemmCfg<BM, BN, WM, WN>;
   const long nb_m = (M + BM - 1) / BM, nb_n = (N + BN - 1) / BN;
-  const long grid = 8 * nb_m * ((nb_n + 7) / 8);
+  const long grid = 8 * ((nb_m * nb_n + 7) / 8);  // 8 XCD runs of the tile order, the longest one sets the count
   if (grid > 0x7fffffffL) return IX_DECLINED;
   if (parts && parts_ld < nb_n) return IX_ERR_ARG;
   auto kern = k_gemm_bf16_nt<BM, BN, WM, WN, TC>;
@@ -152,6 +155,7 @@ static int ix_gemm_bf16_launch(const bf16_t* A, long lda, const bf16_t* W, long 
 // workgroups to pull it, so a narrow output (small N) takes the 64 x 32 tile. Never changes a bit.
 static int ix_gemm_tile_for(long M, long N, int tile) {
   if (tile != 0) return tile;
+  if (M > 128 && N <= 128) return 2;  // one 128-wide column of tiles (the router's gating product)
   if (M > 128) return 3;
   if (M <= 32 && (N + 255) / 256 >= 192) return 1;
   if (M > 32 && ((M + 127) / 128) * ((N + 127) / 128) >= 192) return 2;

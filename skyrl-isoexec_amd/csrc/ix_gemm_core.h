@@ -59,7 +59,11 @@ struct IxGemmCfg {
   // Pipeline: a ring of four half-k-tile stages when the half-stage fetch divides evenly over the
   // threads, else a ring of FULL_STAGES whole-k-tile stages (the 32-row decode tile).
   static constexpr bool HALF_RING = ((BM * 4) % NT == 0) && ((BN * 4) % NT == 0);
-  static constexpr int FULL_STAGES = 3;
+#ifndef IX_FULL_STAGES_MAX
+#define IX_FULL_STAGES_MAX 4
+#endif
+  // as many whole stages as fit in the 160 KiB of LDS, at most IX_FULL_STAGES_MAX, at least 3
+  static constexpr int FULL_STAGES = (IX_FULL_STAGES_MAX * STAGE_BYTES <= 160 * 1024) ? IX_FULL_STAGES_MAX : 3;
 #define IX_HALF_STAGES_MAX 5
   // as many half-stages as fit in the 160 KiB of LDS, at most IX_HALF_STAGES_MAX, at least 4
   static constexpr int HALF_STAGES =
