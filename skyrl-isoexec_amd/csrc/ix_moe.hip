@@ -325,6 +325,22 @@ extern "C" int ix_moe_permute(const int* topk_idx, const float* topk_prob, long 
 // ---------------------------------------------------------------------------------------------
 // Grouped GEMMs over the block map. A workgroup past the device-side tile count exits at once,
 // so the host never reads the routing back.
+//
+// Workgroup -> tile: hardware hands consecutive workgroup ids to the 8 XCDs round-robin and each XCD has its own
+// L2, so the tile order (row tile major, column tile minor: an expert's tiles are adjacent) is cut into 8 equal
+// runs, one per XCD. The ~32 tiles an XCD works on at a time then belong to one or two experts: an expert's
+// weights and a row tile's activations go through one L2 once, instead of through all eight.
+__device__ __forceinline__ bool ix_moe_tile_of_block(unsigned bid, int n_row_tiles, int nb_n, int* mt, int* nt) {
+  const int xcd = (int)(bid & 7);
+  const long idx = bid >> 3;
+  const long tiles = (long)n_row_tiles * nb_n;
+  const long lo = tiles * xcd / 8, hi = tiles * (xcd + 1) / 8;
+  const long l = lo + idx;
+  if (l >= hi) return false;
+  *mt = (int)(l / nb_n);
+  *nt = (int)(l - (long)*mt * nb_n);
+  return true;
+}
 template <int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc1_glu(const bf16_t* __restrict__ x, long ldx, int T,
                                                              const int* __restrict__ sorted_token,
@@ -335,8 +351,8 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc1_glu(const bf16_t* __res
   using Cfg = IxGemmCfg<BM, BN, WM, WN>;
   static_assert(Cfg::NI == 2, "a wave must hold one gate tile and its up tile");
   extern __shared__ __align__(16) char ix_lds[];
-  const int mt = blockIdx.x / nb_n, nt = blockIdx.x % nb_n;
-  if (mt >= meta[0]) return;
+  int mt, nt;
+  if (!ix_moe_tile_of_block(blockIdx.x, meta[0], nb_n, &mt, &nt)) return;
   const int e = meta[1 + mt];
   const long row0 = meta[1 + max_tiles + mt];
   const int nrows = meta[1 + 2 * max_tiles + mt];
@@ -393,8 +409,8 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc2(const bf16_t* __restric
                                                          bf16_t* __restrict__ out, int Hd, int F, int nb_n) {
   using Cfg = IxGemmCfg<BM, BN, WM, WN>;
   extern __shared__ __align__(16) char ix_lds[];
-  const int mt = blockIdx.x / nb_n, nt = blockIdx.x % nb_n;
-  if (mt >= meta[0]) return;
+  int mt, nt;
+  if (!ix_moe_tile_of_block(blockIdx.x, meta[0], nb_n, &mt, &nt)) return;
   const int e = meta[1 + mt];
   const long row0 = meta[1 + max_tiles + mt];
   const int nrows = meta[1 + 2 * max_tiles + mt];
@@ -451,9 +467,10 @@ static int ix_moe_experts_launch(const bf16_t* x, long ldx, int T, const int* so
   const long nb1 = (F + BN / 2 - 1) / (BN / 2);
   const long nb2 = (Hd + BN - 1) / BN;
   if (max_tiles * nb1 > 0x7fffffffL || max_tiles * nb2 > 0x7fffffffL) return IX_DECLINED;
-  hipLaunchKernelGGL(k1, dim3((unsigned)(max_tiles * nb1)), dim3(Cfg::NT), Cfg::LDS_BYTES, st, x, ldx, T,
+  // 8 XCD runs of the tile order; the longest run sets the count
+  hipLaunchKernelGGL(k1, dim3((unsigned)(8 * ((max_tiles * nb1 + 7) / 8))), dim3(Cfg::NT), Cfg::LDS_BYTES, st, x, ldx, T,
                      sorted_token, permuted_prob, W1, meta, (int)max_tiles, inter, Hd, F, (int)nb1);
-  hipLaunchKernelGGL(k2, dim3((unsigned)(max_tiles * nb2)), dim3(Cfg::NT), Cfg::LDS_BYTES, st, inter, W2, meta,
+  hipLaunchKernelGGL(k2, dim3((unsigned)(8 * ((max_tiles * nb2 + 7) / 8))), dim3(Cfg::NT), Cfg::LDS_BYTES, st, inter, W2, meta,
                      (int)max_tiles, out, Hd, F, (int)nb2);
   return ix_launch_status();
 }
