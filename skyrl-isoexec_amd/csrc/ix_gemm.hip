@@ -86,12 +86,38 @@ __global__ __launch_bounds__(WM* WN * 64) void k_gemm_bf16_nt(const bf16_t* __re
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WN, wn = wave % WN;
   float rmax[Cfg::MI];
+  // A whole bf16 tile with 16-byte aligned rows takes the wide stores (same values, same places).
+  const bool wide = sizeof(TC) == 2 && m_valid == BM && n_valid == BN && (ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(C) % 16 == 0);
 #pragma unroll
   for (int mi = 0; mi < Cfg::MI; ++mi) {
     rmax[mi] = IX_NEG_INF;
     const long m = m0 + wm * Cfg::TM + mi * 32 + (lane & 31);
 #pragma unroll
     for (int ni = 0; ni < Cfg::NI; ++ni) {
+      if (wide) {
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+          uint2 pk[2];
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const int q = 2 * p + h;
+            const long n = n0 + wn * Cfg::TN + ni * 32 + ix_acc_row(q * 4, lane);
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              v[e] = acc[mi][ni][q * 4 + e];
+              if (bias) v[e] = v[e] + ix_bf2f(bias[n + e]);
+              rmax[mi] = fmaxf(rmax[mi], v[e]);
+            }
+            pk[h].x = ix_pack_bf2(v[0], v[1]);
+            pk[h].y = ix_pack_bf2(v[2], v[3]);
+          }
+          const uint4 w = ix_join_halves(pk[0], pk[1]);
+          const long n = n0 + wn * Cfg::TN + ni * 32 + 16 * p + (lane >> 5) * 8;
+          *reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(C) + m * ldc + n) = w;
+        }
+        continue;
+      }
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const long n = n0 + wn * Cfg::TN + ni * 32 + ix_acc_row(q * 4, lane);

@@ -435,6 +435,16 @@ __device__ __forceinline__ void ix_acc_zero(Acc& acc) {
       for (int i = 0; i < 16; ++i) acc[mi][ni][i] = 0.0f;
 }
 
+// A 32x32 accumulator holds, for the token of this lane, output columns (i/4)*8 + hf*4 + i%4. For the column
+// blocks q = 2p and 2p+1 the two half-waves swap one packed pair each, after which the lower half holds columns
+// 16p .. 16p+7 and the upper half 16p+8 .. 16p+15 of the token: one 16-byte store per lane instead of two
+// 8-byte ones. lo/hi: this lane's packed columns of block 2p / 2p+1.
+__device__ __forceinline__ uint4 ix_join_halves(uint2 lo, uint2 hi) {
+  const auto x = __builtin_amdgcn_permlane32_swap(lo.x, hi.x, false, false);
+  const auto y = __builtin_amdgcn_permlane32_swap(lo.y, hi.y, false, false);
+  return make_uint4(x[0], y[0], x[1], y[1]);
+}
+
 // Store 4 consecutive output columns of one token (8 bytes when aligned and in range).
 __device__ __forceinline__ void ix_store4_bf16(bf16_t* __restrict__ p, int valid, bool vec, float a, float b,
                                                float c, float d) {

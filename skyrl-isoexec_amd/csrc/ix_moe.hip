@@ -377,12 +377,41 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc1_glu(const bf16_t* __res
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WN, wn = wave % WN;
+  // the wave's 32 columns all exist and rows are 16-byte aligned: two half-waves join their column blocks into
+  // 16-byte stores (same values, same places)
+  const bool wide = n0h + wn * 32 + 32 <= F && (reinterpret_cast<uintptr_t>(inter) % 16 == 0);
 #pragma unroll
   for (int mi = 0; mi < Cfg::MI; ++mi) {
     const int r = wm * Cfg::TM + mi * 32 + (lane & 31);
-    if (r >= nrows) continue;
-    const long m = row0 + r;
-    const float prob = permuted_prob[m];
+    const bool live = r < nrows;  // the same for the two lanes that share a row
+    const long m = row0 + (live ? r : 0);
+    const float prob = live ? permuted_prob[m] : 0.0f;
+    if (wide) {
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+        uint2 pk[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int q = 2 * p + h;
+          float v[4];
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const float gate = ix_rbf(acc[mi][0][q * 4 + c]);
+            const float up = ix_rbf(acc[mi][1][q * 4 + c]);
+            const float s = ix_rbf(ix_silu_div(gate));
+            const float h2 = ix_rbf(s * up);
+            v[c] = h2 * prob;
+          }
+          pk[h].x = ix_pack_bf2(v[0], v[1]);
+          pk[h].y = ix_pack_bf2(v[2], v[3]);
+        }
+        const uint4 w = ix_join_halves(pk[0], pk[1]);
+        const int col = n0h + wn * 32 + 16 * p + (lane >> 5) * 8;
+        if (live) *reinterpret_cast<uint4*>(inter + m * F + col) = w;
+      }
+      continue;
+    }
+    if (!live) continue;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int col = n0h + wn * 32 + ix_acc_row(q * 4, lane);
@@ -428,13 +457,31 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc2(const bf16_t* __restric
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WN, wn = wave % WN;
+  const bool wide = n_valid == BN && (Hd % 8 == 0) && (reinterpret_cast<uintptr_t>(out) % 16 == 0);
 #pragma unroll
   for (int mi = 0; mi < Cfg::MI; ++mi) {
     const int r = wm * Cfg::TM + mi * 32 + (lane & 31);
-    if (r >= nrows) continue;
+    const bool live = r < nrows;  // the same for the two lanes that share a row
     const long m = row0 + r;
 #pragma unroll
     for (int ni = 0; ni < Cfg::NI; ++ni) {
+      if (wide) {
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+          uint2 pk[2];
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const int q = 2 * p + h;
+            pk[h].x = ix_pack_bf2(acc[mi][ni][q * 4], acc[mi][ni][q * 4 + 1]);
+            pk[h].y = ix_pack_bf2(acc[mi][ni][q * 4 + 2], acc[mi][ni][q * 4 + 3]);
+          }
+          const uint4 w = ix_join_halves(pk[0], pk[1]);
+          const long n = n0 + wn * Cfg::TN + ni * 32 + 16 * p + (lane >> 5) * 8;
+          if (live) *reinterpret_cast<uint4*>(out + m * Hd + n) = w;
+        }
+        continue;
+      }
+      if (!live) continue;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const long n = n0 + wn * Cfg::TN + ni * 32 + ix_acc_row(q * 4, lane);
