@@ -110,11 +110,11 @@ int ix_add_rmsnorm_gamma(const void* x, const void* residual, const void* weight
  * accumulator itself (the router's fp32 gating product when its fp32 weight is bf16-exact).
  * lda/ldw/ldc are row pitches in elements. bias (bf16 [N]) may be NULL. tile: 0 auto.
  * row_max_parts: NULL, or fp32 [M, parts_ld] receiving per column tile the max of the stored
- * values, parts_ld >= ix_gemm_bf16_n_tiles(M, N, tile). */
+ * values, parts_ld >= ix_gemm_bf16_n_tiles(M, N, K, tile). */
 int ix_gemm_bf16_nt(const void* A, long lda, const void* W, long ldw, const void* bias, void* C, int c_dtype,
                     long ldc, long M, long N, long K, int tile, float* row_max_parts, long parts_ld,
                     void* stream);
-long ix_gemm_bf16_n_tiles(long M, long N, int tile);
+long ix_gemm_bf16_n_tiles(long M, long N, long K, int tile);
 
 /* Router gating GEMM (moe/_register.py:59-66): C fp32 [M,N] = A[M,K] . W[N,K]^T with W fp32 and
  * A fp32 or bf16 (a_dtype), fp32 accumulate in a fixed K order. */
@@ -147,7 +147,9 @@ int ix_gdn_scan(const void* q, const void* k, const void* v, const float* g, con
  * [Tq, HQ, D] contiguous. cu_q int32 [N+1] packs the queries. Sequence n's keys are the tokens
  * kv_start[n] .. kv_start[n] + q_pos0[n] + len_q[n] - 1 of k/v; its first query sits at absolute
  * position q_pos0[n] (NULL: 0 for every sequence; a negative entry marks a null lane whose outputs are
- * zero). max_q_len >= the longest query run. HQ % HKV == 0 and HQ / HKV in {1,2,4,8,16,32}. */
+ * zero). max_q_len >= the longest query run. HQ % HKV == 0 and HQ / HKV in {1,2,4,8,16,32}.
+ * scale must be positive and finite (the running reference point is kept on the unscaled scores);
+ * kv_pitch < 2^26. Returns IX_ERR_ARG / IX_DECLINED otherwise. */
 int ix_attn_varlen(const void* q, long q_pitch, const void* k, const void* v, long kv_pitch, void* o,
                    const int* cu_q, const long* kv_start, const int* q_pos0, long N, long max_q_len, long HQ,
                    long HKV, long D, float scale, void* stream);

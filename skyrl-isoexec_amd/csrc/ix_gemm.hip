@@ -177,19 +177,42 @@ static int ix_gemm_bf16_launch(const bf16_t* A, long lda, const bf16_t* W, long 
   return ix_launch_status();
 }
 
-// Which tile shape runs (0 = choose). Few rows means the launch is a weight stream: what matters is enough
-// workgroups to pull it, so a narrow output (small N) takes the 64 x 32 tile. Never changes a bit.
-static int ix_gemm_tile_for(long M, long N, int tile) {
+// Which tile shape runs (0 = choose). Never changes a bit. The choice minimises a small cost model fitted to
+// measurements on MI355X: a launch runs in ceil(tiles / 256) waves of workgroups (one per CU), a workgroup costs
+// about 6 us plus K/64 k-tiles at a per-shape rate, and no shape streams the operands faster than ~5 TB/s. Big
+// square tiles win when there are enough of them to fill the chip several times over; a product with few rows or
+// few columns takes smaller tiles so that every CU has one.
+static int ix_gemm_tile_for(long M, long N, long K, int tile) {
   if (tile != 0) return tile;
   if (M > 128 && N <= 128) return 2;  // one 128-wide column of tiles (the router's gating product)
-  if (M > 128) return 3;
-  if (M <= 32 && (N + 255) / 256 >= 192) return 1;
-  if (M > 32 && ((M + 127) / 128) * ((N + 127) / 128) >= 192) return 2;
-  return 6;
+  struct Shape { int id, bm, bn; double us_per_ktile; };
+  // preference order on ties: larger tiles first
+  static const Shape shapes[] = {{3, 256, 256, 1.5}, {5, 128, 256, 0.75}, {2, 128, 128, 0.5},
+                                 {1, 32, 256, 0.4},  {6, 64, 32, 0.16}};
+  const double kt = (double)((K + 63) / 64);
+  const double stream_us = (double)(N + M) * (double)K * 2.0 / 5.0e6;  // both operands once at 5 TB/s
+  int best = 3;
+  double best_cost = 1e300, big_cost = 0.0;
+  for (const Shape& sh : shapes) {
+    const double tiles = (double)((M + sh.bm - 1) / sh.bm) * (double)((N + sh.bn - 1) / sh.bn);
+    const double waves = (double)(long)((tiles + 255.0) / 256.0);
+    double cost = waves * (6.0 + kt * sh.us_per_ktile);
+    if (cost < stream_us) cost = stream_us;
+    if (sh.id == 3) big_cost = cost;
+    if (cost < best_cost * 0.97) {  // a later (smaller) shape must win by a margin
+      best_cost = cost;
+      best = sh.id;
+    }
+  }
+  // With more than half a big tile of rows, the big tile keeps its place unless another shape is clearly ahead:
+  // at scale the smaller shapes pull more bytes through L2 than the per-k-tile rates above say.
+  if (M > 128 && big_cost <= 1.25 * best_cost) return 3;
+  return best;
 }
 
-extern "C" long ix_gemm_bf16_n_tiles(long M, long N, int tile) {
-  const int t = ix_gemm_tile_for(M, N, tile);
+// Row-max parts per row of C: one per column tile of the shape that runs.
+extern "C" long ix_gemm_bf16_n_tiles(long M, long N, long K, int tile) {
+  const int t = ix_gemm_tile_for(M, N, K, tile);
   const long bn = (t == 2) ? 128 : (t == 6) ? 32 : 256;
   return N <= 0 ? 0 : (N + bn - 1) / bn;
 }
@@ -199,7 +222,7 @@ static int ix_gemm_bf16_dispatch(const bf16_t* a, long lda, const bf16_t* w, lon
                                  long ldc, long M, long N, long K, int tile, float* parts, long parts_ld,
                                  hipStream_t st) {
   // `tile` only picks which workgroup owns an element (0 = by M); the bits do not depend on it.
-  switch (ix_gemm_tile_for(M, N, tile)) {
+  switch (ix_gemm_tile_for(M, N, K, tile)) {
     case 1: return ix_gemm_bf16_launch<32, 256, 1, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
     case 2: return ix_gemm_bf16_launch<128, 128, 2, 2, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
     case 3: return ix_gemm_bf16_launch<256, 256, 2, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);

@@ -54,7 +54,7 @@ SIGNATURES = {
         c_int,
         [P, c_long, P, c_long, P, P, c_int, c_long, c_long, c_long, c_long, c_int, P, c_long, P],
     ),
-    "ix_gemm_bf16_n_tiles": (c_long, [c_long, c_long, c_int]),
+    "ix_gemm_bf16_n_tiles": (c_long, [c_long, c_long, c_long, c_int]),
     "ix_gemm_f32_nt": (c_int, [P, c_int, c_long, P, c_long, P, c_long, c_long, c_long, c_long, P]),
     "ix_gdn_scan": (
         c_int,

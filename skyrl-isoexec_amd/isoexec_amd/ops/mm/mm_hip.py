@@ -43,7 +43,7 @@ def linear_nt(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None =
     parts = None
     n_parts = 0
     if want_row_max:
-        n_parts = int(L.ix_gemm_bf16_n_tiles(m, n, tile))
+        n_parts = int(L.ix_gemm_bf16_n_tiles(m, n, k, tile))
         parts = torch.empty(m, n_parts, dtype=torch.float32, device=x.device)
     stream = _lib.current_stream(x.device)
     rc = _lib.check(

@@ -210,6 +210,9 @@ def test_argument_checks():
         varlen_attention(torch.cat([q, q[:, :2]], 1), k, v, cu, 8)  # 6 query heads over 2: group 3
     with pytest.raises(RuntimeError, match="int32"):
         varlen_attention(q, k, v, cu.long(), 8)
+    for bad in (0.0, -0.125, float("inf"), float("nan")):  # the reference point lives on the unscaled scores
+        with pytest.raises(RuntimeError):
+            varlen_attention(q, k, v, cu, 8, scale=bad)
     empty = varlen_attention(q[:0], k, v, torch.zeros(1, dtype=torch.int32, device=DEV), 0)
     assert empty.shape == (0, 4, D)
 
