@@ -294,7 +294,7 @@ extern "C" size_t ix_moe_permute_scratch_ints(long T, long E) {
 
 extern "C" int ix_moe_pick_bm(long T, long k, long E) {
   const long avg = (T * k) / (E > 0 ? E : 1);
-  return avg >= 192 ? 256 : (avg >= 48 ? 128 : 32);
+  return avg >= 96 ? 256 : (avg >= 48 ? 128 : 32);
 }
 
 extern "C" int ix_moe_permute(const int* topk_idx, const float* topk_prob, long T, long E, long k, long BM,
