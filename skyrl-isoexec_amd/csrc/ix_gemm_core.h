@@ -29,7 +29,8 @@ typedef __attribute__((address_space(3))) void ix_lds_void;
 #define IX_BK 64
 // Differential-profiling switches, never defined by the Makefile: IX_EXPERIMENT_NO_DMA drops the memory -> LDS
 // fetches, IX_EXPERIMENT_NO_FRAG the LDS fragment reads, IX_EXPERIMENT_NO_MFMA the matrix instructions (results are
-// then meaningless; only the timing of what remains is of interest), IX_NO_UNIT_RING selects the half-tile ring for
+// then meaningless; only the timing of what remains is of interest), IX_EXPERIMENT_SAME_TILE (dense kernel) points
+// every workgroup at the same few tiles so that all fetches hit L2, IX_NO_UNIT_RING selects the half-tile ring for
 // square tiles.
 #define IX_OOB 0x7FFFF000u  // a byte offset no buffer descriptor here admits (all are < 1 GiB)
 
