@@ -201,17 +201,28 @@ __global__ __launch_bounds__(NW * 64) void k_attn_varlen(const bf16_t* __restric
                                                      const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
                                                      long kv_pitch, bf16_t* __restrict__ o,
                                                      const int* __restrict__ cu_q, const long* __restrict__ kv_start,
-                                                     const int* __restrict__ q_pos0, int HQ, float scale) {
+                                                     const int* __restrict__ q_pos0, int HQ, float scale,
+                                                     int n_seq, int n_kvh, int tiles) {
   constexpr int TOK_W = 32 / GROUP;   // tokens per wave
   constexpr int TOK_WG = NW * TOK_W;  // tokens per workgroup
   constexpr int NT = NW * 64;
   constexpr int CPT = 512 / NT;
   static_assert(S >= 3, "the ring holds the block being read, the next one and at least one in flight");
   extern __shared__ __align__(16) char ix_attn_lds[];
-  const int n = blockIdx.y, g = blockIdx.z;
+  // Workgroup -> (query tile, sequence, key/value head). Hardware deals consecutive workgroup ids to the 8 XCDs
+  // round-robin and each XCD has its own L2, so all query tiles of one (sequence, head) pair go to one XCD: its
+  // keys and values are fetched from memory by one L2 and then shared by the pair's tiles.
+  // The grid is 8 * ceil(pairs / 8) * tiles workgroups: XCD x takes the pairs x, x + 8, ...
+  const int pairs = n_seq * n_kvh;
+  const int xcd = (int)(blockIdx.x & 7);
+  const int idx = (int)(blockIdx.x >> 3);
+  const int slot = idx / tiles, tile = idx - slot * tiles;
+  const int pair = slot * 8 + xcd;
+  if (pair >= pairs) return;
+  const int n = pair % n_seq, g = pair / n_seq;
   const int qb = cu_q[n];
   const int len = cu_q[n + 1] - qb;
-  const int t0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * TOK_WG;  // long tiles first
+  const int t0 = (tiles - 1 - tile) * TOK_WG;  // long tiles first
   if (t0 >= len) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int qc = lane & 31, hf = lane >> 5;
@@ -331,9 +342,11 @@ static int ix_attn_launch(const void* q, long q_pitch, const void* k, const void
   const long tok_wg = NW * (32 / GROUP);
   const long tiles = (max_q_len + tok_wg - 1) / tok_wg;
   if (tiles > 0x7fffffffL) return IX_DECLINED;
-  hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)N, (unsigned)HKV), dim3(NW * 64), LDS, st,
-                     (const bf16_t*)q, q_pitch, (const bf16_t*)k, (const bf16_t*)v, kv_pitch, (bf16_t*)o, cu_q,
-                     kv_start, q_pos0, (int)HQ, scale);
+  const long grid = 8 * ((N * HKV + 7) / 8) * tiles;
+  if (grid > 0x7fffffffL) return IX_DECLINED;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), LDS, st, (const bf16_t*)q, q_pitch,
+                     (const bf16_t*)k, (const bf16_t*)v, kv_pitch, (bf16_t*)o, cu_q, kv_start, q_pos0, (int)HQ, scale,
+                     (int)N, (int)HKV, (int)tiles);
   return ix_launch_status();
 }
 
