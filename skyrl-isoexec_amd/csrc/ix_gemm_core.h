@@ -29,7 +29,8 @@ typedef __attribute__((address_space(3))) void ix_lds_void;
 #define IX_BK 64
 // Differential-profiling switches, never defined by the Makefile: IX_EXPERIMENT_NO_DMA drops the memory -> LDS
 // fetches, IX_EXPERIMENT_NO_FRAG the LDS fragment reads, IX_EXPERIMENT_NO_MFMA the matrix instructions (results are
-// then meaningless; only the timing of what remains is of interest), IX_EXPERIMENT_SAME_TILE (dense kernel) points
+// then meaningless; only the timing of what remains is of interest), IX_EXPERIMENT_NO_VMWAIT the wait for the
+// fetched units before each barrier (unit ring), IX_EXPERIMENT_SAME_TILE (dense kernel) points
 // every workgroup at the same few tiles so that all fetches hit L2, IX_NO_UNIT_RING selects the half-tile ring for
 // square tiles.
 #define IX_OOB 0x7FFFF000u  // a byte offset no buffer descriptor here admits (all are < 1 GiB)
@@ -378,7 +379,9 @@ __device__ __forceinline__ void ix_gemm_mainloop_units(ix_rsrc_t x_rsrc, const X
   int cs = 0;            // slot of the W unit being consumed
   int nu = NU - 2;       // index of the next unit to issue
   for (int kt = 0; kt < KT; ++kt) {
+#ifndef IX_EXPERIMENT_NO_VMWAIT
     __builtin_amdgcn_s_waitcnt(IX_VMCNT((NU - 4) * CH));  // units 2kt and 2kt+1 have landed
+#endif
     __syncthreads();
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
