@@ -17,24 +17,28 @@
 #ifndef IX_GEMM_GN
 #define IX_GEMM_GN 4  // weight tiles of a group
 #endif
-__device__ __forceinline__ bool ix_tile_of_block(long bid, int nb_m, int nb_n, int* tm, int* tn) {
-  const int xcd = (int)(bid & 7);
-  const long idx = bid >> 3;
-  const long tiles = (long)nb_m * nb_n;
-  const long lo = tiles * xcd / 8, hi = tiles * (xcd + 1) / 8;  // this XCD's run of the tile order
-  const long l = lo + idx;
+__device__ __forceinline__ bool ix_tile_of_block(unsigned bid, int nb_m, int nb_n, int* tm, int* tn) {
+  // 32-bit arithmetic throughout (the launch refuses more than 2^31 tiles): a 64-bit division costs a workgroup
+  // about a microsecond before its first fetch.
+  const unsigned xcd = bid & 7u;
+  const unsigned idx = bid >> 3;
+  const unsigned tiles = (unsigned)nb_m * (unsigned)nb_n;
+  // this XCD's run of the tile order: [tiles * xcd / 8, tiles * (xcd + 1) / 8)
+  const unsigned q = tiles >> 3, r = tiles & 7u;
+  const unsigned lo = q * xcd + ((r * xcd) >> 3), hi = q * (xcd + 1) + ((r * (xcd + 1)) >> 3);
+  const unsigned l = lo + idx;
   if (l >= hi) return false;
-  const long per_ngroup = (long)IX_GEMM_GN * nb_m;
-  const long ng = l / per_ngroup;
-  const long rem = l - ng * per_ngroup;
+  const unsigned per_ngroup = (unsigned)IX_GEMM_GN * (unsigned)nb_m;
+  const unsigned ng = l / per_ngroup;
+  const unsigned rem = l - ng * per_ngroup;
   const int gn = min(IX_GEMM_GN, nb_n - (int)ng * IX_GEMM_GN);  // width of this (possibly last) column group
-  const long per_mgroup = (long)IX_GEMM_GM * gn;
-  const long mg = rem / per_mgroup;
-  const long r2 = rem - mg * per_mgroup;
+  const unsigned per_mgroup = (unsigned)IX_GEMM_GM * (unsigned)gn;
+  const unsigned mg = rem / per_mgroup;
+  const unsigned r2 = rem - mg * per_mgroup;
   const int gm = min(IX_GEMM_GM, nb_m - (int)mg * IX_GEMM_GM);
-  const int nl = (int)(r2 / gm), ml = (int)(r2 - (long)nl * gm);
-  *tm = (int)mg * IX_GEMM_GM + ml;
-  *tn = (int)ng * IX_GEMM_GN + nl;
+  const unsigned nl = r2 / (unsigned)gm, ml = r2 - nl * (unsigned)gm;
+  *tm = (int)mg * IX_GEMM_GM + (int)ml;
+  *tn = (int)ng * IX_GEMM_GN + (int)nl;
   return true;
 }
 

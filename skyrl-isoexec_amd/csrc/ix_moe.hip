@@ -331,16 +331,18 @@ extern "C" int ix_moe_permute(const int* topk_idx, const float* topk_prob, long 
 // runs, one per XCD. The ~32 tiles an XCD works on at a time then belong to one or two experts: an expert's
 // weights and a row tile's activations go through one L2 once, instead of through all eight.
 __device__ __forceinline__ bool ix_moe_tile_of_block(unsigned bid, int n_row_tiles, int nb_n, int* mt, int* nt) {
-  const int xcd = (int)(bid & 7);
-  const long idx = bid >> 3;
-  const long tiles = (long)n_row_tiles * nb_n;
-  const long lo = tiles * xcd / 8, hi = tiles * (xcd + 1) / 8;
-  const long l = lo + idx;
+  const unsigned xcd = bid & 7u;
+  const unsigned idx = bid >> 3;
+  const unsigned tiles = (unsigned)n_row_tiles * (unsigned)nb_n;  // < 2^31: the launch checks the bound
+  const unsigned q = tiles >> 3, r = tiles & 7u;
+  const unsigned lo = q * xcd + ((r * xcd) >> 3), hi = q * (xcd + 1) + ((r * (xcd + 1)) >> 3);
+  const unsigned l = lo + idx;
   if (l >= hi) return false;
-  *mt = (int)(l / nb_n);
-  *nt = (int)(l - (long)*mt * nb_n);
+  *mt = (int)(l / (unsigned)nb_n);
+  *nt = (int)(l - (unsigned)*mt * (unsigned)nb_n);
   return true;
 }
+
 template <int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc1_glu(const bf16_t* __restrict__ x, long ldx, int T,
                                                              const int* __restrict__ sorted_token,
