@@ -27,11 +27,8 @@
 #define IX_ATTN_ROW (IX_ATTN_D * 2)                 // bytes per key row of a tile
 #define IX_ATTN_TILE (IX_ATTN_BN * IX_ATTN_ROW)     // one K or V tile of a block: 8 KiB
 #define IX_ATTN_STAGE (2 * IX_ATTN_TILE)            // K tile, then V tile
-#ifndef IX_ATTN_STAGES_BIG
-#define IX_ATTN_STAGES_BIG 4    // ring depth of the eight-wave kernel
-#endif
-#ifndef IX_ATTN_STAGES_SMALL
-#define IX_ATTN_STAGES_SMALL 4  // ring depth of the four-wave kernel
+#ifndef IX_ATTN_STAGES
+#define IX_ATTN_STAGES 4  // ring depth: 64 KiB of LDS per workgroup
 #endif
 
 typedef __attribute__((ext_vector_type(4))) short ix_s16x4;
@@ -192,12 +189,12 @@ __device__ __forceinline__ void ix_attn_step(const char* stage, const char* stag
   ix_attn_scores(kf, qf, sacc);
 }
 
-// NW waves per workgroup (4 or 8): NW * 32 / GROUP consecutive tokens share each staged key block, so a larger
-// workgroup pulls fewer key/value bytes per query; which queries share a workgroup never reaches the arithmetic.
+// NW waves per workgroup: NW * 32 / GROUP consecutive tokens share each staged key block; which queries share a
+// workgroup never reaches the arithmetic. Two workgroups per CU (register limit below).
 // Inside a wave the loop is skewed by one block: while block kb goes through its softmax, the scores of block
 // kb + 1 are already in the matrix pipeline.
 template <int GROUP, int NW, int S>
-__global__ __launch_bounds__(NW * 64) void k_attn_varlen(const bf16_t* __restrict__ q, long q_pitch,
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_attn_varlen(const bf16_t* __restrict__ q, long q_pitch,
                                                      const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
                                                      long kv_pitch, bf16_t* __restrict__ o,
                                                      const int* __restrict__ cu_q, const long* __restrict__ kv_start,
@@ -365,14 +362,14 @@ extern "C" int ix_attn_varlen(const void* q, long q_pitch, const void* k, const 
   if (kv_pitch >= (1L << 26)) return IX_DECLINED;  // a block's byte range must fit the 32-bit buffer size
   const int group = (int)(HQ / HKV);
   hipStream_t st = (hipStream_t)stream;
-  // long query runs (prefill) use eight waves per workgroup, short ones (decode, small chunks) four
-  const bool big = max_q_len >= 8 * (32 / group);
+  // Four waves per workgroup and at most 256 registers per wave: two workgroups share a CU, each behind its own
+  // barrier, so one's matrix work meets the other's softmax arithmetic (measured: an eight-wave workgroup, whose
+  // two waves per SIMD stand behind the same barrier, is 4 % slower on long prefills although it stages half as
+  // many key/value bytes per query; and a decode step runs 20-40 % faster with two workgroups per CU).
 #define IX_ATTN_LAUNCH(G)                                                                                          \
   case G:                                                                                                          \
-    return big ? ix_attn_launch<G, 8, IX_ATTN_STAGES_BIG>(q, q_pitch, k, v, kv_pitch, o, cu_q, kv_start, q_pos0, N, \
-                                                          max_q_len, HQ, HKV, scale, st)                           \
-               : ix_attn_launch<G, 4, IX_ATTN_STAGES_SMALL>(q, q_pitch, k, v, kv_pitch, o, cu_q, kv_start, q_pos0, \
-                                                            N, max_q_len, HQ, HKV, scale, st);
+    return ix_attn_launch<G, 4, IX_ATTN_STAGES>(q, q_pitch, k, v, kv_pitch, o, cu_q, kv_start, q_pos0, N, max_q_len, \
+                                                HQ, HKV, scale, st);
   switch (group) {
     IX_ATTN_LAUNCH(1)
     IX_ATTN_LAUNCH(2)
