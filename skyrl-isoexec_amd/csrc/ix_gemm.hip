@@ -182,26 +182,28 @@ static int ix_gemm_bf16_launch(const bf16_t* A, long lda, const bf16_t* W, long 
 }
 
 // Which tile shape runs (0 = choose). Never changes a bit. The choice minimises a small cost model fitted to
-// measurements on MI355X: a launch runs in ceil(tiles / 256) waves of workgroups (one per CU), a workgroup costs
+// measurements on MI355X: a launch runs in ceil(tiles / slots) waves of workgroups (one or two per CU), a workgroup costs
 // about 6 us plus K/64 k-tiles at a per-shape rate, and no shape streams the operands faster than ~5 TB/s. Big
 // square tiles win when there are enough of them to fill the chip several times over; a product with few rows or
 // few columns takes smaller tiles so that every CU has one.
 static int ix_gemm_tile_for(long M, long N, long K, int tile) {
   if (tile != 0) return tile;
   if (M > 128 && N <= 128) return 2;  // one 128-wide column of tiles (the router's gating product)
-  struct Shape { int id, bm, bn; double us_per_ktile; };
+  // slots: workgroups resident on the chip at once; us_per_ktile: with the CU to itself / shared with a second one
+  struct Shape { int id, bm, bn; double slots, us_per_ktile, us_per_ktile_shared; };
   // preference order on ties: larger tiles first
-  static const Shape shapes[] = {{3, 256, 256, 1.5}, {5, 128, 256, 0.75}, {2, 128, 128, 0.5},
-                                 {1, 32, 256, 0.4},  {6, 64, 32, 0.16}};
+  static const Shape shapes[] = {{3, 256, 256, 256.0, 1.5, 1.5},  {5, 128, 256, 256.0, 0.75, 0.75},
+                                 {2, 128, 128, 512.0, 0.6, 1.0},  {1, 32, 256, 256.0, 0.4, 0.4},
+                                 {6, 64, 32, 256.0, 0.16, 0.16}};
   const double kt = (double)((K + 63) / 64);
   const double stream_us = (double)(N + M) * (double)K * 2.0 / 5.0e6;  // both operands once at 5 TB/s
   int best = 3;
   double best_cost = 1e300, big_cost = 0.0;
   for (const Shape& sh : shapes) {
     const double tiles = (double)((M + sh.bm - 1) / sh.bm) * (double)((N + sh.bn - 1) / sh.bn);
-    const double waves = (double)(long)((tiles + 255.0) / 256.0);
-    double cost = waves * (6.0 + kt * sh.us_per_ktile);
-    if (cost < stream_us) cost = stream_us;
+    const double waves = (double)(long)((tiles + sh.slots - 1.0) / sh.slots);
+    double cost = waves * (6.0 + kt * (tiles > 256.0 ? sh.us_per_ktile_shared : sh.us_per_ktile));
+    if (cost < stream_us) cost = sh.id == 2 ? 0.9 * stream_us : stream_us;  // two workgroups per CU stream best
     if (sh.id == 3) big_cost = cost;
     if (cost < best_cost * 0.97) {  // a later (smaller) shape must win by a margin
       best_cost = cost;

@@ -72,7 +72,13 @@ struct IxGemmCfg {
       (IX_HALF_STAGES_MAX * (STAGE_BYTES / 2) <= 160 * 1024) ? IX_HALF_STAGES_MAX : 4;
   // Square tiles may instead use a ring of whole-k-tile operand units (pipeline C).
 #ifndef IX_NO_UNIT_RING
-  static constexpr int UNITS = (160 * 1024) / (BM * 128) > 9 ? 9 : (160 * 1024) / (BM * 128);
+  // Five units (the two being consumed, three in flight) for every square tile: the 256-row tile fills the LDS
+  // with them, and the 128-row tile's 80 KiB let two workgroups share a CU, each behind its own barrier (measured:
+  // +27 % over nine units and one workgroup per CU).
+#ifndef IX_UNITS_MAX
+#define IX_UNITS_MAX 5
+#endif
+  static constexpr int UNITS = (160 * 1024) / (BM * 128) > IX_UNITS_MAX ? IX_UNITS_MAX : (160 * 1024) / (BM * 128);
   static constexpr bool UNIT_RING = BM == BN && UNITS >= 5 && X_CH >= 1;
 #else
   static constexpr int UNITS = 0;
