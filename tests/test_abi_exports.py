@@ -37,6 +37,21 @@ def test_host_only_entry_points():
     assert h.ix_logprob_workspace_bytes(4, 151937, 8) == 0
 
 
+def test_gemm_tile_choice_is_a_host_decision_with_sane_answers():
+    """ix_gemm_bf16_n_tiles reports the row-max parts of the tile shape that would run: forced shapes give
+    ceil(N / width); the automatic choice takes the big square tile for a large product, a 128-wide tile for the
+    router's 128-column product, and a narrow tile when there are few rows and few columns."""
+    h = _lib.lib()
+    widths = {1: 256, 2: 128, 3: 256, 4: 256, 5: 256, 6: 32}
+    for tile, bn in widths.items():
+        for n in (1, 32, 128, 129, 2048, 151936):
+            assert h.ix_gemm_bf16_n_tiles(4096, n, 4096, tile) == -(-n // bn), (tile, n)
+    assert h.ix_gemm_bf16_n_tiles(4096, 151936, 4096, 0) == -(-151936 // 256)     # LM head: 256-wide tiles
+    assert h.ix_gemm_bf16_n_tiles(163840, 128, 2048, 0) == 1                       # gating product: one 128-wide column
+    assert h.ix_gemm_bf16_n_tiles(64, 2048, 2048, 0) == 2048 // 32                 # decode projection: 64 x 32 tiles
+    assert h.ix_gemm_bf16_n_tiles(0, 0, 4096, 0) == 0
+
+
 def test_product_path_has_no_cpu_fallback():
     import pytest
     import torch
