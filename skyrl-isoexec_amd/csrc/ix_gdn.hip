@@ -197,6 +197,164 @@ __global__ __launch_bounds__(256) void k_gdn_scan(const TIO* __restrict__ q, con
   }
 }
 
+// ---- the same scan with a state row held by a PAIR of lanes (K = 128) ---------------------------------------
+// Lane l and lane l + 32 of a wave own one state row: the lower one k = 0..63, the upper one k = 64..127, 64
+// state floats each. The row's arithmetic is that of k_gdn_scan statement for statement -- per 8-element slice the
+// same two multiply-add chains and their join (ix_dot8), the adjacent-pairwise tree over the 16 slice sums, here
+// three levels inside the lane (ix_tree8) and the last one across the two halves -- so the two kernels agree bit
+// for bit, and which one runs is a staging choice like the time tile. What changes is the cost: 15 of the 16 tree
+// adds per dot product no longer cross lanes, and a wave instruction serves 32 rows with 64 elements each instead
+// of 4 rows x RPL with 8: about 9.4 instead of 11.3 vector instructions per row and token.
+// Compact state form only (one pool row per sequence, stored after the last token).
+__device__ __forceinline__ float ix_add_halves(float v) {
+  const uint32_t u = __float_as_uint(v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);  // (own half) + (other half) or the reverse: same bits
+}
+
+template <typename TIO>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3)))
+void k_gdn_scan_pairs(const TIO* __restrict__ q, const TIO* __restrict__ k, const TIO* __restrict__ v,
+                      const float* __restrict__ g, const TIO* __restrict__ beta, TIO* __restrict__ o,
+                      float* __restrict__ state, const int* __restrict__ cu, const int* __restrict__ sidx,
+                      long q_pitch, long k_pitch, long v_pitch, int H, int HV, int V, float scale, int TT) {
+  constexpr int K = 128;
+  constexpr int R = 128;  // state rows per workgroup: 4 waves x 32 rows
+  extern __shared__ __align__(16) char ix_lds[];
+  float* kf = reinterpret_cast<float*>(ix_lds);  // [TT][K]
+  float* qf = kf + TT * K;                       // [TT][K], pre-scaled
+  float* vf = qf + TT * K;                       // [TT][R]
+  float* of = vf + TT * R;                       // [TT][R]
+  float* egf = of + TT * R;                      // [TT]
+  float* btf = egf + TT;                         // [TT]
+
+  const int VB = V / R;
+  long bid = blockIdx.x;
+  const int vb = (int)(bid % VB);
+  bid /= VB;
+  const int hv = (int)(bid % HV);
+  const int n = (int)(bid / HV);
+  const int h = hv / (HV / H);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int hf = lane >> 5;
+  const int r = wave * 32 + (lane & 31);
+  const int vrow = vb * R + r;
+
+  const int t_begin = cu[n], t_end = cu[n + 1];
+  const int len = t_end - t_begin;
+  if (len <= 0) return;
+  const int row0 = sidx[n];
+  if (row0 <= 0) {  // null lane: no state, outputs defined as zero
+    for (int i = tid; i < len * R; i += 256) {
+      const int tt = i / R, rr = i % R;
+      ix_st(o + ((long)(t_begin + tt) * HV + hv) * V + vb * R + rr, 0.0f);
+    }
+    return;
+  }
+  constexpr long AL = 16 * sizeof(TIO) / 2;
+  const bool vec_qk = (q_pitch % 8 == 0) && (k_pitch % 8 == 0) && ((uintptr_t)q % AL == 0) && ((uintptr_t)k % AL == 0);
+  float S[64];
+  float* srow = state + (((long)row0 * HV + hv) * V + vrow) * K + 64 * hf;
+#pragma unroll
+  for (int c = 0; c < 16; ++c) {
+    const float4 a = *reinterpret_cast<const float4*>(srow + 4 * c);
+    S[4 * c] = a.x; S[4 * c + 1] = a.y; S[4 * c + 2] = a.z; S[4 * c + 3] = a.w;
+  }
+
+  for (int t0 = 0; t0 < len; t0 += TT) {
+    const int nt = min(TT, len - t0);
+    __syncthreads();
+    if (vec_qk) {  // 8 elements (16 bytes) per load
+      for (int i = tid; i < nt * (K / 8); i += 256) {
+        const int tt = i / (K / 8), kk = (i % (K / 8)) * 8;
+        const long tok = t_begin + t0 + tt;
+        float a[8], b[8];
+        ix_load8(k + tok * k_pitch + h * K + kk, 8, true, 0.0f, a);
+        ix_load8(q + tok * q_pitch + h * K + kk, 8, true, 0.0f, b);
+        float* kd = kf + tt * K + kk;
+        float* qd = qf + tt * K + kk;
+        *reinterpret_cast<float4*>(kd) = make_float4(a[0], a[1], a[2], a[3]);
+        *reinterpret_cast<float4*>(kd + 4) = make_float4(a[4], a[5], a[6], a[7]);
+        *reinterpret_cast<float4*>(qd) = make_float4(b[0] * scale, b[1] * scale, b[2] * scale, b[3] * scale);
+        *reinterpret_cast<float4*>(qd + 4) = make_float4(b[4] * scale, b[5] * scale, b[6] * scale, b[7] * scale);
+      }
+    } else {
+      for (int i = tid; i < nt * K; i += 256) {
+        const int tt = i / K, kk = i % K;
+        const long tok = t_begin + t0 + tt;
+        kf[i] = ix_ld(k + tok * k_pitch + h * K + kk);
+        qf[i] = ix_ld(q + tok * q_pitch + h * K + kk) * scale;
+      }
+    }
+    for (int i = tid; i < nt * R; i += 256) {
+      const int tt = i / R, rr = i % R;
+      vf[i] = ix_ld(v + (long)(t_begin + t0 + tt) * v_pitch + (long)hv * V + vb * R + rr);
+    }
+    for (int i = tid; i < nt; i += 256) {
+      const long src = (long)(t_begin + t0 + i) * HV + hv;
+      egf[i] = ix_exp(g[src]);
+      btf[i] = ix_ld(beta + src);
+    }
+    __syncthreads();
+#pragma unroll 2
+    for (int tt = 0; tt < nt; ++tt) {
+      const float eg = egf[tt], bt = btf[tt], vv = vf[tt * R + r];
+      float x[64];  // this half's 64 elements of k, later of q
+      const float* kp = kf + tt * K + 64 * hf;
+#pragma unroll
+      for (int c = 0; c < 16; ++c) {
+        const float4 a = *reinterpret_cast<const float4*>(kp + 4 * c);
+        x[4 * c] = a.x; x[4 * c + 1] = a.y; x[4 * c + 2] = a.z; x[4 * c + 3] = a.w;
+      }
+      float part[8];
+#pragma unroll
+      for (int sl = 0; sl < 8; ++sl) {
+        float ss[8], xs[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          S[8 * sl + i] = S[8 * sl + i] * eg;
+          ss[i] = S[8 * sl + i];
+          xs[i] = x[8 * sl + i];
+        }
+        part[sl] = ix_dot8(ss, xs);
+      }
+      const float kv = ix_add_halves(ix_tree8(part));
+      const float d = (vv - kv) * bt;
+#pragma unroll
+      for (int i = 0; i < 64; ++i) S[i] = __builtin_fmaf(d, x[i], S[i]);
+      const float* qp = qf + tt * K + 64 * hf;
+#pragma unroll
+      for (int c = 0; c < 16; ++c) {
+        const float4 a = *reinterpret_cast<const float4*>(qp + 4 * c);
+        x[4 * c] = a.x; x[4 * c + 1] = a.y; x[4 * c + 2] = a.z; x[4 * c + 3] = a.w;
+      }
+#pragma unroll
+      for (int sl = 0; sl < 8; ++sl) {
+        float ss[8], xs[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          ss[i] = S[8 * sl + i];
+          xs[i] = x[8 * sl + i];
+        }
+        part[sl] = ix_dot8(ss, xs);
+      }
+      const float ov = ix_add_halves(ix_tree8(part));
+      if (hf == 0) of[tt * R + r] = ov;
+    }
+    if (t0 + nt == len) {
+#pragma unroll
+      for (int c = 0; c < 16; ++c)
+        *reinterpret_cast<float4*>(srow + 4 * c) = make_float4(S[4 * c], S[4 * c + 1], S[4 * c + 2], S[4 * c + 3]);
+    }
+    __syncthreads();
+    for (int i = tid; i < nt * R; i += 256) {
+      const int tt = i / R, rr = i % R;
+      ix_st(o + ((long)(t_begin + t0 + tt) * HV + hv) * V + vb * R + rr, of[i]);
+    }
+  }
+}
+
 static size_t ix_gdn_lds_bytes(int K, int R, int TT) {
   return (size_t)TT * (2 * K + 2 * R + 3) * sizeof(float);
 }
@@ -265,6 +423,25 @@ extern "C" int ix_gdn_scan(const void* q, const void* k, const void* v, const fl
   if (TT <= 0) TT = (N * HV * (V / 16) >= 4096) ? 16 : 64;
   if (TT > 64) TT = 64;
   hipStream_t st = (hipStream_t)stream;
+  // The lane-pair layout: compact state form, K = 128, whole groups of 128 rows, and enough workgroups to fill the
+  // chip (or forced by rows-per-lane-group code 16 in bits 8.. of time_tile). Same bits as the kernels below.
+  if (state_indices_stride == 0 && K == 128 && V % 128 == 0 &&
+      (rpl == 16 || (rpl == 0 && N * HV * (V / 128) >= 512))) {
+    const long grid = N * HV * (V / 128);
+    if (grid > 0x7fffffffL) return IX_DECLINED;
+    const int tt = time_tile > 0 && (time_tile & 0xff) > 0 ? TT : 16;
+    const size_t lds = ix_gdn_lds_bytes(128, 128, tt);
+    if (io_dtype == IX_DT_BF16)
+      hipLaunchKernelGGL((k_gdn_scan_pairs<bf16_t>), dim3((unsigned)grid), dim3(256), lds, st, (const bf16_t*)q,
+                         (const bf16_t*)k, (const bf16_t*)v, g, (const bf16_t*)beta, (bf16_t*)o, state_pool,
+                         cu_seqlens, state_indices, q_pitch, k_pitch, v_pitch, (int)H, (int)HV, (int)V, scale, tt);
+    else
+      hipLaunchKernelGGL((k_gdn_scan_pairs<float>), dim3((unsigned)grid), dim3(256), lds, st, (const float*)q,
+                         (const float*)k, (const float*)v, g, (const float*)beta, (float*)o, state_pool, cu_seqlens,
+                         state_indices, q_pitch, k_pitch, v_pitch, (int)H, (int)HV, (int)V, scale, tt);
+    return ix_launch_status();
+  }
+  if (rpl == 16) return IX_DECLINED;  // the lane-pair layout was asked for and does not apply
 #define IX_SCAN_CASE(KSV)                                                                                         \
   if (K == KSV * 8) {                                                                                             \
     if (io_dtype == IX_DT_BF16)                                                                                   \

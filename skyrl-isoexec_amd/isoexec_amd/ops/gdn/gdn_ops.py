@@ -220,17 +220,14 @@ def gdn_causal_conv_batched(x, weight, bias=None, *, initial_state=None, activat
 
 
 def _recurrent_scratch_state(q, v, cu_seqlens):
-    """A throwaway pool + index map for a stateless forward (gdn_ops.py:444-464): row 0 unused,
-    sequence n at row n+1, only column 0 of the map set."""
-    if cu_seqlens is not None:
-        N = cu_seqlens.numel() - 1
-        Tmax = q.shape[1]
-    else:
-        N, Tmax = q.shape[0], q.shape[1]
+    """A throwaway zero pool + row indices for a stateless forward (gdn_ops.py:444-464): row 0 unused,
+    sequence n at row n+1. One row per sequence (the compact form): the final state lands in the throwaway
+    pool instead of nowhere, which costs one 2 MB store per sequence and lets the scan run its branch-free
+    token loop; the outputs do not depend on where, or whether, the state is stored."""
+    N = cu_seqlens.numel() - 1 if cu_seqlens is not None else q.shape[0]
     HV, V, K = v.shape[-2], v.shape[-1], q.shape[-1]
     ssm_state = torch.zeros(N + 1, HV, V, K, dtype=torch.float32, device=q.device)
-    idx = torch.zeros(N, max(Tmax, 1), dtype=torch.int32, device=q.device)
-    idx[:, 0] = torch.arange(1, N + 1, dtype=torch.int32, device=q.device)
+    idx = torch.arange(1, N + 1, dtype=torch.int32, device=q.device)
     return ssm_state, idx
 
 

@@ -229,3 +229,33 @@ def test_compact_state_index_form_equals_the_full_map(dprims):
             got = gdn_recurrent_kernel(bf(q), bf(k), bf(v), gate.to(DEV), bf(beta), ssm_state=pool, state_indices=rows,
                                        cu_seqlens=cu, time_tile=tt | (rpl << 8))
             assert same_bits(got, outs[0]) and same_bits(pool, pools[0]), (rpl, tt)
+
+
+def test_lane_pair_layout_gives_the_same_bits():
+    """K = 128: a state row may be held by a pair of lanes (64 elements each, code 16 in bits 8.. of time_tile)
+    instead of 16 lanes with 8 each. Same slices, same chains, same tree -- outputs and final states must be
+    bit-equal to the 16-lane layout for every time tile, ragged lengths and a null lane included."""
+    from isoexec_amd.ops.gdn.gdn_ops import gdn_recurrent_kernel
+
+    Hh, Kk, HVv, Vv = 2, 128, 4, 128
+    g = cpu_gen(11)
+    lens = [5, 1, 64, 33, 130]
+    T = sum(lens)
+    bf = lambda t: t.to(torch.bfloat16).to(DEV)
+    q = torch.nn.functional.normalize(torch.randn(1, T, Hh, Kk, generator=g), dim=-1)
+    k = torch.nn.functional.normalize(torch.randn(1, T, Hh, Kk, generator=g), dim=-1)
+    v = torch.randn(1, T, HVv, Vv, generator=g)
+    gate = -torch.nn.functional.softplus(torch.randn(1, T, HVv, generator=g))
+    beta = torch.sigmoid(torch.randn(1, T, HVv, generator=g))
+    cu = torch.tensor(np.cumsum([0] + lens), dtype=torch.int32, device=DEV)
+    rows = torch.tensor([2, 0, 4, 1, 5], dtype=torch.int32, device=DEV)  # the second sequence is a null lane
+    start = torch.randn(6, HVv, Vv, Kk, generator=g)
+    ref_pool = start.clone().to(DEV)
+    ref = gdn_recurrent_kernel(bf(q), bf(k), bf(v), gate.to(DEV), bf(beta), ssm_state=ref_pool, state_indices=rows,
+                               cu_seqlens=cu, time_tile=16 | (1 << 8))
+    for tt in (8, 16, 64):
+        pool = start.clone().to(DEV)
+        got = gdn_recurrent_kernel(bf(q), bf(k), bf(v), gate.to(DEV), bf(beta), ssm_state=pool, state_indices=rows,
+                                   cu_seqlens=cu, time_tile=tt | (16 << 8))
+        assert same_bits(got, ref) and same_bits(pool, ref_pool), tt
+    assert same_bits(ref_pool[3], start[3].to(DEV)) and not same_bits(ref_pool[5], start[5].to(DEV))
