@@ -601,9 +601,8 @@ __global__ __launch_bounds__(256) void k_gdn_conv(const bf16_t* __restrict__ x, 
 // sequence each input row is loaded once for the four windows that cover it. Per channel the arithmetic is that
 // of k_gdn_conv, statement for statement, so the two kernels agree bit for bit (a NaN keeps its payload here).
 template <int W>
-__device__ __forceinline__ void ix_conv8_finish(const float (&xv)[W][8], const float (&wv)[8][W],
-                                                const bf16_t* __restrict__ bias, int d, int silu,
-                                                bf16_t* __restrict__ yrow) {
+__device__ __forceinline__ void ix_conv8_finish(const float (&xv)[W][8], const float (&wv)[8][W], bool has_bias,
+                                                const float (&bv)[8], int silu, bf16_t* __restrict__ yrow) {
   uint32_t out[4];
 #pragma unroll
   for (int c = 0; c < 8; c += 2) {
@@ -616,7 +615,7 @@ __device__ __forceinline__ void ix_conv8_finish(const float (&xv)[W][8], const f
         const float p = wv[c + e][j] * xv[j][c + e];
         acc = acc + p;
       }
-      if (bias) acc = acc + ix_bf2f(bias[d + c + e]);
+      if (has_bias) acc = acc + bv[c + e];
       if (silu) acc = acc * ix_sigmoid(acc);
       r2[e] = acc;
     }
@@ -645,30 +644,45 @@ __global__ __launch_bounds__(256) void k_gdn_conv8(const bf16_t* __restrict__ x,
   const long D8 = D >> 3;
   const int t0 = (int)(i / D8) * TOK;
   const int d = (int)(i % D8) * 8;
-  float wv[8][W];
+  float wv[8][W], bv[8];
   {
-    const bf16_t* wp = w + (long)d * W;
+    // 8 channels x W taps are 8 W consecutive elements (the host checked the alignment): W 16-byte loads
+    static_assert(W == 4, "the unpacking below assumes four taps");
+    const uint4* wp = reinterpret_cast<const uint4*>(w + (long)d * W);
 #pragma unroll
-    for (int c = 0; c < 8; ++c)
+    for (int c2 = 0; c2 < 4; ++c2) {
+      float t8[8];
+      ix_unpack8(wp[c2], t8);
 #pragma unroll
-      for (int j = 0; j < W; ++j) wv[c][j] = ix_bf2f(wp[c * W + j]);
+      for (int j = 0; j < 4; ++j) {
+        wv[2 * c2][j] = t8[j];
+        wv[2 * c2 + 1][j] = t8[4 + j];
+      }
+    }
+    // the channels' biases once per thread, not once per output
+    if (bias) {
+      ix_unpack8(*reinterpret_cast<const uint4*>(bias + d), bv);
+    } else {
+#pragma unroll
+      for (int c = 0; c < 8; ++c) bv[c] = 0.0f;
+    }
   }
+  const bool has_bias = bias != nullptr;
   const int n0 = ix_seq_of(cu, N, t0);
   const int b0 = cu[n0], e0 = cu[n0 + 1];
   if (t0 - (W - 1) >= b0 && t0 + TOK <= e0) {
     // all TOK windows lie inside one sequence: TOK + W - 1 rows serve TOK outputs
-    float xr[TOK + W - 1][8];
+    // the rows stay packed (4 registers each) until a window needs them
+    uint4 xr[TOK + W - 1];
 #pragma unroll
     for (int r = 0; r < TOK + W - 1; ++r)
-      ix_unpack8(*reinterpret_cast<const uint4*>(x + (long)(t0 - (W - 1) + r) * x_pitch + d), xr[r]);
+      xr[r] = *reinterpret_cast<const uint4*>(x + (long)(t0 - (W - 1) + r) * x_pitch + d);
 #pragma unroll
     for (int q = 0; q < TOK; ++q) {
       float xv[W][8];
 #pragma unroll
-      for (int j = 0; j < W; ++j)
-#pragma unroll
-        for (int c = 0; c < 8; ++c) xv[j][c] = xr[q + j][c];
-      ix_conv8_finish<W>(xv, wv, bias, d, silu, y + (long)(t0 + q) * D + d);
+      for (int j = 0; j < W; ++j) ix_unpack8(xr[q + j], xv[j]);
+      ix_conv8_finish<W>(xv, wv, has_bias, bv, silu, y + (long)(t0 + q) * D + d);
     }
     return;
   }
@@ -691,7 +705,7 @@ __global__ __launch_bounds__(256) void k_gdn_conv8(const bf16_t* __restrict__ x,
           xv[j][c] = srow > 0 ? ix_bf2f(pool[((long)srow * D + d + c) * (W - 1) + (W - 1 + r)]) : 0.0f;
       }
     }
-    ix_conv8_finish<W>(xv, wv, bias, d, silu, y + (long)t * D + d);
+    ix_conv8_finish<W>(xv, wv, has_bias, bv, silu, y + (long)t * D + d);
   }
 }
 
@@ -728,17 +742,28 @@ extern "C" int ix_gdn_conv(const void* x, long x_pitch, const void* weight, cons
   hipStream_t st = (hipStream_t)stream;
   const long total = total_tokens * D;
   if (total > 0 && N > 0) {
-    constexpr int TOK = 4;
-    const bool vec8 = (W == 4) && (D % 8 == 0) && (x_pitch % 8 == 0) && ix_aligned(x, 16) && ix_aligned(y, 16);
+    const bool vec8 = (W == 4) && (D % 8 == 0) && (x_pitch % 8 == 0) && ix_aligned(x, 16) && ix_aligned(y, 16) &&
+                      ix_aligned(weight, 16) && (!bias || ix_aligned(bias, 16));
+    // Outputs per thread: long sequences amortise the W - 1 rows of history over 16 outputs; short ones (a decode
+    // step has one token per sequence) keep one output per thread so the launch stays wide. Every output is
+    // computed by the same expression whichever is chosen.
+    const long avg_len = total_tokens / N;
+    const int TOK = !vec8 ? 1 : avg_len >= 64 ? 16 : avg_len >= 8 ? 4 : 1;
     const long work = vec8 ? ((total_tokens + TOK - 1) / TOK) * (D / 8) : total;
     const long blocks = (work + 255) / 256;
     const long gx = blocks < (1L << 22) ? blocks : (1L << 22);
     const long gy = (blocks + gx - 1) / gx;
     if (gy > 65535) return IX_DECLINED;
-    if (vec8)
-      hipLaunchKernelGGL((k_gdn_conv8<4, TOK>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st, (const bf16_t*)x,
-                         x_pitch, (const bf16_t*)weight, (const bf16_t*)bias, (bf16_t*)y, (const bf16_t*)conv_pool,
-                         cu_seqlens, state_rows_in, (int)N, D, silu, (int)total_tokens, work);
+#define IX_CONV8(TOK_)                                                                                              \
+  hipLaunchKernelGGL((k_gdn_conv8<4, TOK_>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st, (const bf16_t*)x,  \
+                     x_pitch, (const bf16_t*)weight, (const bf16_t*)bias, (bf16_t*)y, (const bf16_t*)conv_pool,     \
+                     cu_seqlens, state_rows_in, (int)N, D, silu, (int)total_tokens, work)
+    if (vec8) {
+      if (TOK == 16) IX_CONV8(16);
+      else if (TOK == 4) IX_CONV8(4);
+      else IX_CONV8(1);
+    }
+#undef IX_CONV8
     else
       hipLaunchKernelGGL(k_gdn_conv, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st, (const bf16_t*)x, x_pitch,
                          (const bf16_t*)weight, (const bf16_t*)bias, (bf16_t*)y, (const bf16_t*)conv_pool, cu_seqlens,
