@@ -26,7 +26,8 @@ PEAK_MFMA_BF16_TFLOPS = 2500.0  # MI355X dense bf16
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch of the dominant kernels, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by
 # what the same counters read for a 1 GiB copy (x2.0 / x1.0); see profiles/*.txt. Workload-specific.
-MEASURED_TRAFFIC_BYTES = {"dense_head_M4096_gemm": 9.08e9, "gdn_decode_B256": 1.1016e9}
+MEASURED_TRAFFIC_BYTES = {"dense_head_M4096_gemm": 9.08e9, "gdn_decode_B256": 1.1016e9,
+                          "moe_T16384_grouped_gemms": 3.80e9}
 
 
 class KernelTimer:
@@ -227,7 +228,8 @@ def moe(args):
             "config": {"workload": f"moe T={T} hidden 2048, 128 experts top-8, inter 768"},
             "roofline": {"bound": "mfma", "achieved": exp_fl / (exp_ms * 1e-3) / 1e12, "peak": PEAK_MFMA_BF16_TFLOPS,
                          "unit": "TFLOP/s", "frac": exp_fl / (exp_ms * 1e-3) / 1e12 / PEAK_MFMA_BF16_TFLOPS,
-                         "traffic": None, "kernel": "k_moe_fc1_glu + k_moe_fc2 (grouped GEMMs)", "kernel_ms": exp_ms},
+                         "traffic": MEASURED_TRAFFIC_BYTES["moe_T16384_grouped_gemms"] if T == 16384 else None,
+                         "kernel": "k_moe_fc1_glu + k_moe_fc2 (grouped GEMMs)", "kernel_ms": exp_ms},
             "whole_ffn": {"kernel_ms": ms, "achieved": fl / (ms * 1e-3) / 1e12, "unit": "TFLOP/s",
                           "frac": fl / (ms * 1e-3) / 1e12 / PEAK_MFMA_BF16_TFLOPS,
                           "kernels": "router product + router + permutation + grouped GEMMs + combine"}}
