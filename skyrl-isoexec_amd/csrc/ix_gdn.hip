@@ -424,9 +424,11 @@ extern "C" int ix_gdn_scan(const void* q, const void* k, const void* v, const fl
   if (TT > 64) TT = 64;
   hipStream_t st = (hipStream_t)stream;
   // The lane-pair layout: compact state form, K = 128, whole groups of 128 rows, and enough workgroups to fill the
-  // chip (or forced by rows-per-lane-group code 16 in bits 8.. of time_tile). Same bits as the kernels below.
+  // chip (or forced by rows-per-lane-group code 16 in bits 8.. of time_tile). Same bits as the kernels below. A
+  // time tile of 1 says one token per sequence (a decode step): that is a pure stream of the state, which the
+  // 16-lane layout does with more waves in flight.
   if (state_indices_stride == 0 && K == 128 && V % 128 == 0 &&
-      (rpl == 16 || (rpl == 0 && N * HV * (V / 128) >= 512))) {
+      (rpl == 16 || (rpl == 0 && (time_tile & 0xff) != 1 && N * HV * (V / 128) >= 512))) {
     const long grid = N * HV * (V / 128);
     if (grid > 0x7fffffffL) return IX_DECLINED;
     const int tt = time_tile > 0 && (time_tile & 0xff) > 0 ? TT : 16;
