@@ -157,6 +157,16 @@ __device__ __forceinline__ void ix_load8(const float* __restrict__ p, long valid
   }
 }
 
+// Eight bf16 held in a 16-byte register group, widened.
+__device__ __forceinline__ void ix_unpack8(const uint4 u, float (&o)[8]) {
+  const uint32_t q[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    o[2 * c] = __uint_as_float(q[c] << 16);
+    o[2 * c + 1] = __uint_as_float(q[c] & 0xffff0000u);
+  }
+}
+
 __device__ __forceinline__ void ix_store8_bf16(bf16_t* __restrict__ p, long valid, bool vec, const float (&v)[8]) {
   if (vec && valid >= 8) {
     uint4 u;

@@ -626,14 +626,6 @@ __device__ __forceinline__ void ix_conv8_finish(const float (&xv)[W][8], const f
   *reinterpret_cast<uint4*>(yrow) = make_uint4(out[0], out[1], out[2], out[3]);
 }
 
-__device__ __forceinline__ void ix_unpack8(const uint4 u, float (&o)[8]) {
-  const uint32_t q[4] = {u.x, u.y, u.z, u.w};
-#pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    o[2 * c] = __uint_as_float(q[c] << 16);
-    o[2 * c + 1] = __uint_as_float(q[c] & 0xffff0000u);
-  }
-}
 
 template <int W, int TOK>
 __global__ __launch_bounds__(256) void k_gdn_conv8(const bf16_t* __restrict__ x, long x_pitch,

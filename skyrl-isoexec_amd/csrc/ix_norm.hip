@@ -92,6 +92,81 @@ __global__ __launch_bounds__(256) void k_rmsnorm(const bf16_t* __restrict__ x, c
   }
 }
 
+// The same chain for a row that fits the registers of its lanes: N = LPR * 8 * NG columns, 16-byte aligned. Every
+// operand is fetched once, all loads are issued before the first use, and the sums run in the order of ix_row_sumsq
+// (chunks ascending per slot, ix_tree8, lane tree), so the results are those of k_rmsnorm.
+template <int LPR, int MODE, int NG>
+__global__ __launch_bounds__(256) void k_rmsnorm_reg(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                     bf16_t* __restrict__ out, long M, float eps, int zero_centered,
+                                                     const bf16_t* __restrict__ aux, long aux_stride_t, int HV,
+                                                     bf16_t* __restrict__ h_out) {
+  constexpr int RPB = 256 / LPR, N = LPR * 8 * NG;
+  const int tid = threadIdx.x;
+  const int sub = tid % LPR;
+  const long row = (long)blockIdx.x * RPB + tid / LPR;
+  const bool live = row < M;
+  const long rrow = live ? row : (M - 1);
+  const bf16_t* xr = x + rrow * N + sub * 8;
+  uint4 xp[NG], ap[NG], wp[NG];
+#pragma unroll
+  for (int c = 0; c < NG; ++c) xp[c] = *reinterpret_cast<const uint4*>(xr + c * LPR * 8);
+  if (MODE == 2) {
+    const bf16_t* rr = aux + rrow * N + sub * 8;
+#pragma unroll
+    for (int c = 0; c < NG; ++c) ap[c] = *reinterpret_cast<const uint4*>(rr + c * LPR * 8);
+  }
+  if (MODE == 1) {
+    const long t = rrow / HV, hh = rrow % HV;
+    const bf16_t* gr = aux + t * aux_stride_t + hh * N + sub * 8;
+#pragma unroll
+    for (int c = 0; c < NG; ++c) ap[c] = *reinterpret_cast<const uint4*>(gr + c * LPR * 8);
+  }
+#pragma unroll
+  for (int c = 0; c < NG; ++c) wp[c] = *reinterpret_cast<const uint4*>(w + sub * 8 + c * LPR * 8);
+
+  float xv[NG][8];
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int c = 0; c < NG; ++c) {
+    ix_unpack8(xp[c], xv[c]);
+    if (MODE == 2) {
+      float r[8];
+      ix_unpack8(ap[c], r);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) xv[c][i] = ix_rbf(xv[c][i] + r[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float sq = xv[c][i] * xv[c][i];
+      acc[i] = acc[i] + sq;
+    }
+  }
+  const float s = ix_lane_tree<LPR>(ix_tree8(acc));
+  const float ms = s / (float)N;
+  const float rstd = ix_rsqrt_ieee(ms + eps);
+  if (!live) return;
+  bf16_t* orow = out + row * N + sub * 8;
+#pragma unroll
+  for (int c = 0; c < NG; ++c) {
+    float wv[8], o[8];
+    ix_unpack8(wp[c], wv);
+    if (MODE == 2) ix_store8_bf16(h_out + row * N + sub * 8 + c * LPR * 8, 8, true, xv[c]);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float nb = ix_rbf(xv[c][i] * rstd);
+      const float gam = zero_centered ? ix_rbf(1.0f + wv[i]) : wv[i];
+      o[i] = ix_rbf(nb * gam);
+    }
+    if (MODE == 1) {
+      float g[8];
+      ix_unpack8(ap[c], g);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) o[i] = o[i] * ix_silu_div(g[i]);
+    }
+    ix_store8_bf16(orow + c * LPR * 8, 8, true, o);
+  }
+}
+
 static int ix_lpr_for(int N) {
   int groups = (N + 7) / 8, l = 1;
   while (l < groups && l < 64) l <<= 1;
@@ -109,6 +184,19 @@ static int ix_norm_launch(const bf16_t* x, const bf16_t* w, bf16_t* out, long M,
   const long rpb = 256 / lpr;
   const long grid = (M + rpb - 1) / rpb;
   if (grid > 0x7fffffffL) return IX_DECLINED;
+  // rows that fit their lanes' registers (N = lpr * 8 * {1, 2, 4, 8}), all operands 16-byte aligned
+  if (vec && (MODE != 1 || aux_stride_t % 8 == 0) && N % (lpr * 8) == 0) {
+    const int ng = N / (lpr * 8);
+#define IX_NORM_REG(L, G)                                                                                        \
+  if (lpr == L && ng == G) {                                                                                     \
+    hipLaunchKernelGGL((k_rmsnorm_reg<L, MODE, G>), dim3((unsigned)grid), dim3(256), 0, st, x, w, out, M, eps,   \
+                       zc, aux, aux_stride_t, HV, h_out);                                                        \
+    return ix_launch_status();                                                                                   \
+  }
+    IX_NORM_REG(8, 1) IX_NORM_REG(16, 1) IX_NORM_REG(32, 1) IX_NORM_REG(64, 1)
+    IX_NORM_REG(64, 2) IX_NORM_REG(64, 4) IX_NORM_REG(64, 8)
+#undef IX_NORM_REG
+  }
 #define IX_NORM_CASE(L)                                                                                          \
   case L:                                                                                                        \
     hipLaunchKernelGGL((k_rmsnorm<L, MODE>), dim3((unsigned)grid), dim3(256), 0, st, x, w, out, M, N, eps, zc,   \

@@ -46,7 +46,7 @@ def test_prim_transcendentals_close_to_libm(dprims):
 
 
 # ---- RMSNorm family --------------------------------------------------------------------------------
-@pytest.mark.parametrize("N", [128, 2048, 4096, 100, 24])
+@pytest.mark.parametrize("N", [128, 1024, 2048, 4096, 8192, 100, 24])
 @pytest.mark.parametrize("zc", [True, False])
 def test_rmsnorm_bit_exact_and_row_invariant(N, zc):
     from isoexec_amd.ops.norms.fused_outnorm import fused_rms_norm_gamma
