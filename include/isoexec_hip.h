@@ -168,9 +168,18 @@ int ix_gdn_l2norm(const void* x, long x_pitch, void* y, int io_dtype, long token
 
 /* gdn_gate_and_beta (gdn_ops.py:1197-1210) in the fp32 form of the fused core (gdn/_register.py:33-55):
  * g = -exp(A_log[hv]) * softplus(a + dt_bias[hv]) fp32; beta = sigmoid(b) in io_dtype.
- * a, b [tokens, HV]; A_log, dt_bias fp32 [HV]. */
-int ix_gdn_gate(const void* a, const void* b, const float* A_log, const float* dt_bias, float* g, void* beta,
-                int io_dtype, long tokens, long HV, void* stream);
+ * a, b [tokens, HV] with token pitches a_pitch, b_pitch (elements; column slices of a wider projection are read in
+ * place); g, beta [tokens, HV] contiguous; A_log, dt_bias fp32 [HV]. */
+int ix_gdn_gate(const void* a, long a_pitch, const void* b, long b_pitch, const float* A_log, const float* dt_bias,
+                float* g, void* beta, int io_dtype, long tokens, long HV, void* stream);
+
+/* cpr_resolve_rows (gdn_cpr_rows.py:29-80; eager chain gdn_recurrent_state.py:271-284): engine slot ids of a
+ * decode batch -> state-pool rows, one launch, host-free. slots int32 or int64 [n] (slots_i64). With slot2row
+ * (int64 [map_n]): row = slot2row[clamp(slot, 0, map_n - 1)]; with slot2row NULL: row = slot if 0 <= slot < blocks
+ * else 0. rows64 (may be NULL) and rows32 receive the rows. last_used + clock (both or neither): clock[0] += 1 and
+ * last_used[row] = clock[0] for every row of the batch (the decode step's use stamp). */
+int ix_gdn_resolve_rows(const void* slots, int slots_i64, long n, const int64_t* slot2row, long map_n, long blocks,
+                        int64_t* rows64, int* rows32, int64_t* last_used, int64_t* clock, void* stream);
 
 /* gdn_causal_conv / gdn_causal_conv_batched (gdn_ops.py:74-170) over packed tokens, and the
  * engine's window-slide update (gdn_recurrent_state.py:686-707,814-825) when every sequence has

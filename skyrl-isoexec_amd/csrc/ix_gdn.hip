@@ -490,17 +490,19 @@ __global__ __launch_bounds__(256) void k_gdn_l2norm(const TIO* __restrict__ x, T
 }
 
 template <typename TIO>
-__global__ __launch_bounds__(256) void k_gdn_gate(const TIO* __restrict__ a, const TIO* __restrict__ b,
+__global__ __launch_bounds__(256) void k_gdn_gate(const TIO* __restrict__ a, long a_pitch,
+                                                  const TIO* __restrict__ b, long b_pitch,
                                                   const float* __restrict__ A_log,
                                                   const float* __restrict__ dt_bias, float* __restrict__ g,
                                                   TIO* __restrict__ beta, long n, int HV) {
   const long i = (long)blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
-  const int hv = (int)(i % HV);
-  const float sp = ix_softplus(ix_ld(a + i) + dt_bias[hv]);
+  const long t = i / HV;
+  const int hv = (int)(i - t * HV);
+  const float sp = ix_softplus(ix_ld(a + t * a_pitch + hv) + dt_bias[hv]);
   const float neg_ea = -ix_exp(A_log[hv]);
   g[i] = neg_ea * sp;
-  ix_st(beta + i, ix_sigmoid(ix_ld(b + i)));
+  ix_st(beta + i, ix_sigmoid(ix_ld(b + t * b_pitch + hv)));
 }
 
 extern "C" int ix_gdn_l2norm(const void* x, long x_pitch, void* y, int io_dtype, long tokens, long H, long K,
@@ -530,9 +532,11 @@ extern "C" int ix_gdn_l2norm(const void* x, long x_pitch, void* y, int io_dtype,
   return IX_DECLINED;
 }
 
-extern "C" int ix_gdn_gate(const void* a, const void* b, const float* A_log, const float* dt_bias, float* g,
-                           void* beta, int io_dtype, long tokens, long HV, void* stream) {
-  if (!a || !b || !A_log || !dt_bias || !g || !beta || tokens < 0 || HV <= 0) return IX_ERR_ARG;
+extern "C" int ix_gdn_gate(const void* a, long a_pitch, const void* b, long b_pitch, const float* A_log,
+                           const float* dt_bias, float* g, void* beta, int io_dtype, long tokens, long HV,
+                           void* stream) {
+  if (!a || !b || !A_log || !dt_bias || !g || !beta || tokens < 0 || HV <= 0 || a_pitch < HV || b_pitch < HV)
+    return IX_ERR_ARG;
   if (io_dtype != IX_DT_F32 && io_dtype != IX_DT_BF16) return IX_DECLINED;
   const long n = tokens * HV;
   if (n == 0) return IX_OK;
@@ -540,11 +544,58 @@ extern "C" int ix_gdn_gate(const void* a, const void* b, const float* A_log, con
   if (grid > 0x7fffffffL) return IX_DECLINED;
   hipStream_t st = (hipStream_t)stream;
   if (io_dtype == IX_DT_BF16)
-    hipLaunchKernelGGL((k_gdn_gate<bf16_t>), dim3((unsigned)grid), dim3(256), 0, st, (const bf16_t*)a,
-                       (const bf16_t*)b, A_log, dt_bias, g, (bf16_t*)beta, n, (int)HV);
+    hipLaunchKernelGGL((k_gdn_gate<bf16_t>), dim3((unsigned)grid), dim3(256), 0, st, (const bf16_t*)a, a_pitch,
+                       (const bf16_t*)b, b_pitch, A_log, dt_bias, g, (bf16_t*)beta, n, (int)HV);
   else
-    hipLaunchKernelGGL((k_gdn_gate<float>), dim3((unsigned)grid), dim3(256), 0, st, (const float*)a,
-                       (const float*)b, A_log, dt_bias, g, (float*)beta, n, (int)HV);
+    hipLaunchKernelGGL((k_gdn_gate<float>), dim3((unsigned)grid), dim3(256), 0, st, (const float*)a, a_pitch,
+                       (const float*)b, b_pitch, A_log, dt_bias, g, (float*)beta, n, (int)HV);
+  return ix_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Slot ids -> state-pool rows for a decode batch in one launch (gdn_cpr_rows.py:29-46, the fused form of
+// gdn_recurrent_state.py:271-284): with a map, row = slot2row[clamp(slot, 0, map_n - 1)]; without one (the
+// engine's block ids are the rows), row = slot if 0 <= slot < blocks else 0. Optionally the same launch stamps the
+// rows' last-use clock (gdn_recurrent_state.py decode: clock += 1; last_used[rows] = clock). One workgroup, so
+// every lane reads the clock before lane 0 advances it.
+template <typename TS>
+__global__ __launch_bounds__(256) void k_gdn_resolve_rows(const TS* __restrict__ slots, long n,
+                                                          const int64_t* __restrict__ slot2row, long map_n,
+                                                          long blocks, int64_t* __restrict__ rows64,
+                                                          int* __restrict__ rows32, int64_t* __restrict__ last_used,
+                                                          int64_t* __restrict__ clock) {
+  const int64_t stamp = clock ? clock[0] + 1 : 0;
+  for (long i = threadIdx.x; i < n; i += 256) {
+    int64_t sl = (int64_t)slots[i];
+    int64_t r;
+    if (slot2row) {
+      sl = sl < 0 ? 0 : (sl > map_n - 1 ? map_n - 1 : sl);
+      r = slot2row[sl];
+    } else {
+      r = (sl >= 0 && sl < blocks) ? sl : 0;
+    }
+    if (rows64) rows64[i] = r;
+    rows32[i] = (int)r;
+    if (last_used) last_used[r] = stamp;
+  }
+  __syncthreads();
+  if (clock && threadIdx.x == 0) clock[0] = stamp;
+}
+
+extern "C" int ix_gdn_resolve_rows(const void* slots, int slots_i64, long n, const int64_t* slot2row, long map_n,
+                                   long blocks, int64_t* rows64, int* rows32, int64_t* last_used, int64_t* clock,
+                                   void* stream) {
+  if (n < 0 || (n > 0 && (!slots || !rows32))) return IX_ERR_ARG;
+  if (slot2row ? map_n <= 0 : blocks <= 0) return IX_ERR_ARG;
+  if ((last_used == nullptr) != (clock == nullptr)) return IX_ERR_ARG;
+  if (n == 0 && !clock) return IX_OK;
+  hipStream_t st = (hipStream_t)stream;
+  if (slots_i64)
+    hipLaunchKernelGGL(k_gdn_resolve_rows<int64_t>, dim3(1), dim3(256), 0, st, (const int64_t*)slots, n, slot2row,
+                       map_n, blocks, rows64, rows32, last_used, clock);
+  else
+    hipLaunchKernelGGL(k_gdn_resolve_rows<int>, dim3(1), dim3(256), 0, st, (const int*)slots, n, slot2row, map_n,
+                       blocks, rows64, rows32, last_used, clock);
   return ix_launch_status();
 }
 

@@ -141,13 +141,22 @@ def gdn_gate_and_beta(a: torch.Tensor, b: torch.Tensor, A_log: torch.Tensor, dt_
     """``g = -exp(A_log) * softplus(a + dt_bias)`` in fp32; ``beta = sigmoid(b)``. Elementwise."""
     _lib.require_device(a, b, A_log, dt_bias)
     HV = a.shape[-1]
-    ac, bc = a.contiguous(), b.contiguous()
+
+    def rows_of(t):
+        # [tokens, HV] with unit-stride rows is read in place at its token pitch (a column slice of a projection)
+        if t.ndim == 2 and t.stride(1) == 1 and t.stride(0) >= HV:
+            return t, t.stride(0)
+        return t.contiguous(), HV
+
+    (ac, ap), (bc, bp) = rows_of(a), rows_of(b)
     g = torch.empty(a.shape, dtype=torch.float32, device=a.device)
-    beta = torch.empty_like(bc)
+    beta = torch.empty(b.shape, dtype=b.dtype, device=b.device)
+    A32 = A_log if A_log.dtype is torch.float32 and A_log.is_contiguous() else A_log.float().contiguous()
+    dt32 = dt_bias if dt_bias.dtype is torch.float32 and dt_bias.is_contiguous() else dt_bias.float().contiguous()
     _lib.check(
-        _lib.lib().ix_gdn_gate(ac.data_ptr(), bc.data_ptr(), A_log.float().contiguous().data_ptr(),
-                               dt_bias.float().contiguous().data_ptr(), g.data_ptr(), beta.data_ptr(),
-                               _lib.dtype_code(a.dtype), ac.numel() // HV, HV, _lib.current_stream(a.device)),
+        _lib.lib().ix_gdn_gate(ac.data_ptr(), ap, bc.data_ptr(), bp, A32.data_ptr(), dt32.data_ptr(), g.data_ptr(),
+                               beta.data_ptr(), _lib.dtype_code(a.dtype), a.numel() // HV, HV,
+                               _lib.current_stream(a.device)),
         "ix_gdn_gate")
     return g, beta
 

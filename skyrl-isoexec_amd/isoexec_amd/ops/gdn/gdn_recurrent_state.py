@@ -389,8 +389,35 @@ class RecurrentGDN:
         return self.slot2row[s.clamp(0, self.slot2row.numel() - 1)]
 
     def _rows_pair(self, slots: torch.Tensor):
+        """``(rows int64, rows int32)``: one launch when the fused resolver serves the arguments
+        (gdn_recurrent_state.py:286-299), else the eager chain."""
+        if not self._native:
+            from .gdn_cpr_rows import cpr_resolve_rows, fused_rows_enabled
+
+            if fused_rows_enabled() and slots.is_cuda:
+                pair = cpr_resolve_rows(slots, self.slot2row)
+                if pair is not None:
+                    return pair
         rows = self._rows(slots)
         return rows, rows.to(torch.int32)
+
+    def _decode_rows(self, slots: torch.Tensor) -> torch.Tensor:
+        """int32 rows of a decode batch, with the rows' use stamp advanced (private pool only). One launch when
+        the fused resolver serves the arguments."""
+        from .gdn_cpr_rows import fused_rows_enabled, resolve_and_stamp
+
+        if fused_rows_enabled() and slots.is_cuda:
+            if self._native:
+                rows32 = resolve_and_stamp(slots, blocks=self.ssm_state.shape[0])
+            else:
+                rows32 = resolve_and_stamp(slots, slot2row=self.slot2row, last_used=self.last_used, clock=self._clock)
+            if rows32 is not None:
+                return rows32
+        rows, rows32 = self._rows_pair(slots)
+        if not self._native:
+            self._clock += 1
+            self.last_used[rows] = self._clock
+        return rows32
 
     def _split_qkv_raw(self, y: torch.Tensor):
         """Post-conv ``[T, D]`` -> views ``q, k [T, H, K]`` and ``v [T, HV, V]`` (token pitch D, no copy)."""
@@ -405,6 +432,11 @@ class RecurrentGDN:
         """As ``_split_qkv_raw`` with q and k L2-normalised. Heads stay GQA-compressed: the scan maps
         value head hv to key head ``hv // (HV / H)`` itself."""
         q, k, v = self._split_qkv_raw(y)
+        if y.ndim == 2 and y.stride(1) == 1:
+            # q and k are adjacent column blocks of y: one launch normalises the 2H rows of each token
+            H = self.num_k_heads
+            qk = gdn_l2norm(y[:, : 2 * H * self.head_k_dim].unflatten(1, (2 * H, self.head_k_dim)))
+            return qk[:, :H], qk[:, H:], v
         return gdn_l2norm(q), gdn_l2norm(k), v
 
     def _gate_and_beta(self, a: torch.Tensor, b: torch.Tensor):
@@ -489,7 +521,7 @@ class RecurrentGDN:
         ``o [N, HV, V]``. Host-free and shape-static. A padded lane resolves to row 0: it reads a zero
         convolution history, writes no state and returns zeros."""
         N = x.shape[0]
-        rows, rows32 = self._rows_pair(slots)
+        rows32 = self._decode_rows(slots)
         cu = self._decode_cu.get(N)
         if cu is None:
             cu = self._decode_cu[N] = torch.arange(N + 1, dtype=torch.int32, device=x.device)
@@ -500,7 +532,4 @@ class RecurrentGDN:
         g, beta = self._gate_and_beta(a, b)
         o = gdn_recurrent_kernel(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), g.unsqueeze(0), beta.unsqueeze(0),
                                  ssm_state=self.ssm_state, state_indices=rows32, cu_seqlens=cu, time_tile=1)
-        if not self._native:
-            self._clock += 1
-            self.last_used[rows] = self._clock
         return o[0]

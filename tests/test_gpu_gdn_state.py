@@ -259,3 +259,40 @@ def test_lane_pair_layout_gives_the_same_bits():
                                    cu_seqlens=cu, time_tile=tt | (16 << 8))
         assert same_bits(got, ref) and same_bits(pool, ref_pool), tt
     assert same_bits(ref_pool[3], start[3].to(DEV)) and not same_bits(ref_pool[5], start[5].to(DEV))
+
+
+def test_fused_row_resolver_equals_the_eager_chain():
+    """Slot ids -> rows in one launch (reference gdn_cpr_rows.py) against the index expression it replaces
+    (gdn_recurrent_state.py:271-284): clamped lookups for a private pool, identity with out-of-range ids on
+    row 0 for the engine's own blocks, both id widths, and the use stamp of the decode step."""
+    from isoexec_amd.ops.gdn.gdn_cpr_rows import cpr_resolve_rows, resolve_and_stamp
+
+    g = cpu_gen(77)
+    map_n, rows_n = 50, 9
+    slot2row = torch.randint(0, rows_n, (map_n,), generator=g, dtype=torch.int64).to(DEV)
+    ids = torch.tensor([3, 49, 50, 1000, -1, -7, 0, 3, 17], dtype=torch.int64)
+    for dt in (torch.int64, torch.int32):
+        slots = ids.to(dt).to(DEV)
+        want = slot2row[slots.long().clamp(0, map_n - 1)]
+        r64, r32 = cpr_resolve_rows(slots, slot2row)
+        assert r64.dtype is torch.int64 and r32.dtype is torch.int32
+        assert torch.equal(r64, want) and torch.equal(r32.long(), want)
+        # the engine's block ids are the rows: ids outside [0, blocks) read the null row
+        nat = resolve_and_stamp(slots, blocks=40)
+        s = slots.long()
+        assert torch.equal(nat.long(), torch.where(s < 40, s, torch.zeros_like(s)).clamp(min=0))
+    # the use stamp: clock += 1, last_used[rows] = clock, twice in a row, duplicates included
+    last_used = torch.zeros(rows_n, dtype=torch.int64, device=DEV)
+    clock = torch.full((), 41, dtype=torch.int64, device=DEV)
+    want_used = last_used.clone()
+    for step, sl in enumerate((ids[:4], ids[4:])):
+        slots = sl.to(DEV)
+        rows = slot2row[slots.clamp(0, map_n - 1)]
+        want_used[rows] = 42 + step
+        got = resolve_and_stamp(slots, slot2row=slot2row, last_used=last_used, clock=clock)
+        assert torch.equal(got.long(), rows)
+        assert int(clock) == 42 + step and torch.equal(last_used, want_used)
+    # shapes the resolver does not serve hand the caller back to the eager chain
+    assert cpr_resolve_rows(ids.view(3, 3).to(DEV), slot2row) is None
+    assert cpr_resolve_rows(ids.to(DEV), slot2row.int()) is None
+    assert cpr_resolve_rows(torch.empty(0, dtype=torch.int64, device=DEV), slot2row)[0].numel() == 0
