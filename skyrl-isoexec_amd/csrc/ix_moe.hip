@@ -281,6 +281,86 @@ __global__ __launch_bounds__(256) void k_moe_scatter(const int* __restrict__ top
   }
 }
 
+// The three steps above in one launch for a batch of at most one token tile (a decode step): the membership masks
+// stay in LDS, the expert offsets come from a workgroup-wide scan (two experts per lane), and every output is the
+// integer the general path writes.
+__global__ __launch_bounds__(256) void k_moe_permute_one_tile(const int* __restrict__ topk_idx,
+                                                              const float* __restrict__ topk_prob, int T, int E,
+                                                              int k, int BM, int max_tiles, int* __restrict__ counts,
+                                                              int* __restrict__ offsets,
+                                                              int* __restrict__ sorted_token,
+                                                              float* __restrict__ permuted_prob,
+                                                              int* __restrict__ combine_rows, int* __restrict__ meta) {
+  __shared__ int s_idx[IX_MOE_TILE_T * IX_MOE_KMAX];
+  __shared__ uint32_t s_mask[IX_MOE_EMAX * 8];
+  __shared__ int s_off[IX_MOE_EMAX + 1];
+  __shared__ int s_rows[256], s_tiles[256];
+  ix_moe_build_masks(topk_idx, 0, T, E, k, s_mask, s_idx);
+  const int tid = threadIdx.x;
+  // lane owns experts 2 tid and 2 tid + 1
+  int c[2], tl[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int e = 2 * tid + h;
+    c[h] = 0;
+    if (e < E) {
+#pragma unroll
+      for (int w = 0; w < 8; ++w) c[h] += __popc(s_mask[e * 8 + w]);
+    }
+    tl[h] = (c[h] + BM - 1) / BM;
+  }
+  s_rows[tid] = c[0] + c[1];
+  s_tiles[tid] = tl[0] + tl[1];
+  __syncthreads();
+  for (int d = 1; d < 256; d <<= 1) {  // inclusive scan over the 256 lane sums
+    const int a = tid >= d ? s_rows[tid - d] : 0;
+    const int b = tid >= d ? s_tiles[tid - d] : 0;
+    __syncthreads();
+    s_rows[tid] += a;
+    s_tiles[tid] += b;
+    __syncthreads();
+  }
+  int row0 = s_rows[tid] - (c[0] + c[1]);   // rows before expert 2 tid
+  int tile0 = s_tiles[tid] - (tl[0] + tl[1]);
+  int* tile_expert = meta + 1;
+  int* tile_row0 = tile_expert + max_tiles;
+  int* tile_nrows = tile_row0 + max_tiles;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int e = 2 * tid + h;
+    if (e < E) {
+      s_off[e] = row0;
+      counts[e] = c[h];
+      offsets[e] = row0;
+      int nt = tile0;
+      for (int r0 = 0; r0 < c[h] && nt < max_tiles; r0 += BM, ++nt) {
+        tile_expert[nt] = e;
+        tile_row0[nt] = row0 + r0;
+        tile_nrows[nt] = min(BM, c[h] - r0);
+      }
+    }
+    row0 += c[h];
+    tile0 += tl[h];
+  }
+  if (tid == 255) {
+    offsets[E] = s_rows[255];
+    meta[0] = min(s_tiles[255], max_tiles);
+  }
+  __syncthreads();
+  if (tid >= T) return;
+  for (int j = 0; j < k; ++j) {
+    const int e = s_idx[tid * k + j];
+    int local = __popc(s_mask[e * 8 + (tid >> 5)] & ((1u << (tid & 31)) - 1u));
+    for (int w = 0; w < (tid >> 5); ++w) local += __popc(s_mask[e * 8 + w]);
+    int rank = 0;
+    for (int j2 = 0; j2 < k; ++j2) rank += (s_idx[tid * k + j2] < e);
+    const int pos = s_off[e] + local;
+    sorted_token[pos] = tid;
+    permuted_prob[pos] = topk_prob[(long)tid * k + j];
+    combine_rows[(long)tid * k + rank] = pos;
+  }
+}
+
 extern "C" long ix_moe_max_tiles(long T, long k, long E, long BM) {
   if (T < 0 || k <= 0 || E <= 0 || BM <= 0) return 0;
   return (T * k + BM - 1) / BM + E;
@@ -309,6 +389,11 @@ extern "C" int ix_moe_permute(const int* topk_idx, const float* topk_prob, long 
   if (T * k > 0x7fffffffL) return IX_DECLINED;
   hipStream_t st = (hipStream_t)stream;
   const long ntiles = (T + IX_MOE_TILE_T - 1) / IX_MOE_TILE_T;
+  if (ntiles == 1) {
+    hipLaunchKernelGGL(k_moe_permute_one_tile, dim3(1), dim3(256), 0, st, topk_idx, topk_prob, (int)T, (int)E, (int)k,
+                       (int)BM, (int)max_tiles, counts, offsets, sorted_token, permuted_prob, combine_rows, tile_meta);
+    return ix_launch_status();
+  }
   int* tile_counts = scratch;
   int* tile_base = scratch + ntiles * E;
   if (ntiles > 0)

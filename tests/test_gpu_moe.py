@@ -60,7 +60,7 @@ def test_router_bit_exact_ties_and_nan(mode, E, k, dprims):
     assert torch.equal(i1, idx[5:6]) and same_bits(p1, prob[5:6])
 
 
-@pytest.mark.parametrize("T,E,k", [(1, 128, 8), (33, 128, 8), (700, 16, 4), (513, 128, 8)])
+@pytest.mark.parametrize("T,E,k", [(1, 128, 8), (33, 128, 8), (256, 128, 8), (200, 37, 2), (64, 512, 16), (257, 37, 2), (700, 16, 4), (513, 128, 8)])
 def test_permutation_exact(T, E, k):
     from isoexec_amd.ops.moe.moe_hip import permute, router_topk
 
