@@ -31,6 +31,15 @@ __device__ __forceinline__ bool ix_beats(float av, int ai, float bv, int bi, int
   return (av > bv) || (av == bv && ai < bi);
 }
 
+// One step of the wave-wide "best candidate" exchange at lane distance S (selection by ix_beats is associative
+// and commutative, so the exchange network does not matter; distances below 16 use the row-local lane controls).
+template <int S>
+__device__ __forceinline__ void ix_best_step(float& bv, int& bi, int sentinel) {
+  const float ov = ix_xor_lane<S>(bv);
+  const int oi = __float_as_int(ix_xor_lane<S>(__int_as_float(bi)));
+  if (ix_beats(ov, oi, bv, bi, sentinel)) { bv = ov; bi = oi; }
+}
+
 __device__ __forceinline__ float ix_tree_k(float (&t)[IX_MOE_KMAX], int k) {
 #pragma unroll
   for (int s = 1; s < IX_MOE_KMAX; s <<= 1) {
@@ -43,6 +52,8 @@ __device__ __forceinline__ float ix_tree_k(float (&t)[IX_MOE_KMAX], int k) {
   return t[0];
 }
 
+// EC = experts held per lane (E <= 64 EC): the instantiation only sets how many slots a lane carries.
+template <int EC>
 __global__ __launch_bounds__(256) void k_moe_router(const float* __restrict__ logits, long ld, int T, int E, int k,
                                                     int mode, float scaling, int* __restrict__ topk_idx,
                                                     float* __restrict__ topk_prob, float* __restrict__ dense_probs,
@@ -50,10 +61,10 @@ __global__ __launch_bounds__(256) void k_moe_router(const float* __restrict__ lo
   const int lane = threadIdx.x & 63;
   const long t = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return;
-  float s[IX_MOE_EC];
-  bool live[IX_MOE_EC];
+  float s[EC];
+  bool live[EC];
 #pragma unroll
-  for (int c = 0; c < IX_MOE_EC; ++c) {
+  for (int c = 0; c < EC; ++c) {
     const int e = lane + 64 * c;
     live[c] = e < E;
     float v = live[c] ? logits[t * ld + e] : IX_NEG_INF;
@@ -63,17 +74,17 @@ __global__ __launch_bounds__(256) void k_moe_router(const float* __restrict__ lo
   if (mode == 1) {
     float m = IX_NEG_INF;
 #pragma unroll
-    for (int c = 0; c < IX_MOE_EC; ++c) m = fmaxf(m, s[c]);
+    for (int c = 0; c < EC; ++c) m = fmaxf(m, s[c]);
     m = ix_lane_max<64>(m);
     float z = 0.0f;
 #pragma unroll
-    for (int c = 0; c < IX_MOE_EC; ++c) {
+    for (int c = 0; c < EC; ++c) {
       s[c] = live[c] ? ix_exp(s[c] - m) : 0.0f;
       z = z + s[c];
     }
     z = ix_lane_tree<64>(z);
 #pragma unroll
-    for (int c = 0; c < IX_MOE_EC; ++c) s[c] = s[c] / z;
+    for (int c = 0; c < EC; ++c) s[c] = s[c] / z;
   }
   float vals[IX_MOE_KMAX];
   int idxs[IX_MOE_KMAX];
@@ -85,21 +96,21 @@ __global__ __launch_bounds__(256) void k_moe_router(const float* __restrict__ lo
       float bv = 0.0f;
       int bi = E;
 #pragma unroll
-      for (int c = 0; c < IX_MOE_EC; ++c) {
+      for (int c = 0; c < EC; ++c) {
         const int e = lane + 64 * c;
         if (live[c] && ix_beats(s[c], e, bv, bi, E)) { bv = s[c]; bi = e; }
       }
-#pragma unroll
-      for (int st = 1; st < 64; st <<= 1) {
-        const float ov = __shfl_xor(bv, st, IX_WAVE);
-        const int oi = __shfl_xor(bi, st, IX_WAVE);
-        if (ix_beats(ov, oi, bv, bi, E)) { bv = ov; bi = oi; }
-      }
+      ix_best_step<1>(bv, bi, E);
+      ix_best_step<2>(bv, bi, E);
+      ix_best_step<4>(bv, bi, E);
+      ix_best_step<8>(bv, bi, E);
+      ix_best_step<16>(bv, bi, E);
+      ix_best_step<32>(bv, bi, E);
       bi = min(bi, E - 1);
       vals[j] = bv;
       idxs[j] = bi;
 #pragma unroll
-      for (int c = 0; c < IX_MOE_EC; ++c)
+      for (int c = 0; c < EC; ++c)
         if (lane + 64 * c == bi) live[c] = false;
     }
   }
@@ -127,7 +138,7 @@ __global__ __launch_bounds__(256) void k_moe_router(const float* __restrict__ lo
   }
   if (dense_probs || dense_map) {
 #pragma unroll
-    for (int c = 0; c < IX_MOE_EC; ++c) {
+    for (int c = 0; c < EC; ++c) {
       const int e = lane + 64 * c;
       if (e < E) {
         float dp = 0.0f;
@@ -152,8 +163,13 @@ extern "C" int ix_moe_router_topk(const float* logits, long ld, long T, long E, 
   if (T == 0) return IX_OK;
   const long grid = (T + 3) / 4;
   if (grid > 0x7fffffffL) return IX_DECLINED;
-  hipLaunchKernelGGL(k_moe_router, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, logits, ld, (int)T,
-                     (int)E, (int)k, mode, scaling, topk_idx, topk_prob, dense_probs, dense_map);
+#define IX_ROUTER(EC_)                                                                                            \
+  hipLaunchKernelGGL(k_moe_router<EC_>, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, logits, ld,      \
+                     (int)T, (int)E, (int)k, mode, scaling, topk_idx, topk_prob, dense_probs, dense_map)
+  if (E <= 128) IX_ROUTER(2);
+  else if (E <= 256) IX_ROUTER(4);
+  else IX_ROUTER(IX_MOE_EC);
+#undef IX_ROUTER
   return ix_launch_status();
 }
 
