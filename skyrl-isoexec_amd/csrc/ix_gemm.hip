@@ -58,14 +58,14 @@ __device__ __forceinline__ void ix_store4(float* p, int valid, bool vec, const f
 // TC = bf16_t: C is the bf16 round of the fp32 accumulator; TC = float: the accumulator itself.
 // row_max_parts (optional): [M, parts_ld] fp32, entry (m, tn) = max over the tile's columns of the
 // values stored to C (exact, order-free), so a consumer can skip its own max pass over C.
-template <int BM, int BN, int WM, int WN, typename TC>
-__global__ __launch_bounds__(WM* WN * 64) void k_gemm_bf16_nt(const bf16_t* __restrict__ A, long lda,
+template <int BM, int BN, int WM, int WN, typename TC, int PW = 0>
+__global__ __launch_bounds__((WM * WN + PW) * 64) void k_gemm_bf16_nt(const bf16_t* __restrict__ A, long lda,
                                                               const bf16_t* __restrict__ W, long ldw,
                                                               const bf16_t* __restrict__ bias,
                                                               TC* __restrict__ C, long ldc, int M, int N, int K,
                                                               int nb_m, int nb_n, int vec_store,
                                                               float* __restrict__ row_max_parts, long parts_ld) {
-  using Cfg = IxGemmCfg<BM, BN, WM, WN>;
+  using Cfg = IxGemmCfg<BM, BN, WM, WN, PW>;
   extern __shared__ __align__(16) char ix_lds[];
   int tm, tn;
   if (!ix_tile_of_block(blockIdx.x, nb_m, nb_n, &tm, &tn)) return;
@@ -89,12 +89,14 @@ __global__ __launch_bounds__(WM* WN * 64) void k_gemm_bf16_nt(const bf16_t* __re
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WN, wn = wave % WN;
+  const bool computes = PW == 0 || wave < WM * WN;  // fetching waves hold no results
   float rmax[Cfg::MI];
   // A whole bf16 tile with 16-byte aligned rows takes the wide stores (same values, same places).
   const bool wide = sizeof(TC) == 2 && m_valid == BM && n_valid == BN && (ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(C) % 16 == 0);
 #pragma unroll
   for (int mi = 0; mi < Cfg::MI; ++mi) {
     rmax[mi] = IX_NEG_INF;
+    if (!computes) continue;
     const long m = m0 + wm * Cfg::TM + mi * 32 + (lane & 31);
 #pragma unroll
     for (int ni = 0; ni < Cfg::NI; ++ni) {
@@ -147,10 +149,10 @@ __global__ __launch_bounds__(WM* WN * 64) void k_gemm_bf16_nt(const bf16_t* __re
       float v = fmaxf(rmax[mi], __shfl_xor(rmax[mi], 32, IX_WAVE));
       // rounding is monotonic: the max of the rounded values is the rounded max
       if (sizeof(TC) == 2) v = ix_rbf(v);
-      if (lane < 32) s_max[wn * BM + wm * Cfg::TM + mi * 32 + lane] = v;
+      if (computes && lane < 32) s_max[wn * BM + wm * Cfg::TM + mi * 32 + lane] = v;
     }
     __syncthreads();
-    for (int r = threadIdx.x; r < m_valid; r += Cfg::NT) {
+    for (int r = threadIdx.x; r < m_valid; r += Cfg::NTT) {
       float v = s_max[r];
 #pragma unroll
       for (int w = 1; w < WN; ++w) v = fmaxf(v, s_max[w * BM + r]);
@@ -159,15 +161,15 @@ __global__ __launch_bounds__(WM* WN * 64) void k_gemm_bf16_nt(const bf16_t* __re
   }
 }
 
-template <int BM, int BN, int WM, int WN, typename TC>
+template <int BM, int BN, int WM, int WN, typename TC, int PW = 0>
 static int ix_gemm_bf16_launch(const bf16_t* A, long lda, const bf16_t* W, long ldw, const bf16_t* bias, TC* C,
                                long ldc, long M, long N, long K, float* parts, long parts_ld, hipStream_t st) {
-  using Cfg = IxGemmCfg<BM, BN, WM, WN>;
+  using Cfg = IxGemmCfg<BM, BN, WM, WN, PW>;
   const long nb_m = (M + BM - 1) / BM, nb_n = (N + BN - 1) / BN;
   const long grid = 8 * ((nb_m * nb_n + 7) / 8);  // 8 XCD runs of the tile order, the longest one sets the count
   if (grid > 0x7fffffffL) return IX_DECLINED;
   if (parts && parts_ld < nb_n) return IX_ERR_ARG;
-  auto kern = k_gemm_bf16_nt<BM, BN, WM, WN, TC>;
+  auto kern = k_gemm_bf16_nt<BM, BN, WM, WN, TC, PW>;
   static bool attr_set = false;  // per instantiation
   if (!attr_set) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES) !=
@@ -176,7 +178,7 @@ static int ix_gemm_bf16_launch(const bf16_t* A, long lda, const bf16_t* W, long 
     attr_set = true;
   }
   const int vec = (ldc % 4 == 0) && ix_aligned(C, 4 * sizeof(TC));
-  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(Cfg::NT), Cfg::LDS_BYTES, st, A, lda, W, ldw, bias, C, ldc,
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(Cfg::NTT), Cfg::LDS_BYTES, st, A, lda, W, ldw, bias, C, ldc,
                      (int)M, (int)N, (int)K, (int)nb_m, (int)nb_n, vec, parts, parts_ld);
   return ix_launch_status();
 }
@@ -229,12 +231,12 @@ static int ix_gemm_bf16_dispatch(const bf16_t* a, long lda, const bf16_t* w, lon
                                  hipStream_t st) {
   // `tile` only picks which workgroup owns an element (0 = by M); the bits do not depend on it.
   switch (ix_gemm_tile_for(M, N, K, tile)) {
-    case 1: return ix_gemm_bf16_launch<32, 256, 1, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
+    case 1: return ix_gemm_bf16_launch<32, 256, 1, 4, TC, 4>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
     case 2: return ix_gemm_bf16_launch<128, 128, 2, 2, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
     case 3: return ix_gemm_bf16_launch<256, 256, 2, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
     case 4: return ix_gemm_bf16_launch<256, 256, 2, 2, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
     case 5: return ix_gemm_bf16_launch<128, 256, 2, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
-    case 6: return ix_gemm_bf16_launch<64, 32, 2, 1, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
+    case 6: return ix_gemm_bf16_launch<64, 32, 2, 1, TC, 2>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
     default: return IX_ERR_ARG;
   }
 }

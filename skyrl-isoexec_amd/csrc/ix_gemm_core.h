@@ -49,10 +49,12 @@ __device__ __forceinline__ int ix_lds_off(int row, int chunk) { return row * 128
 // (a weight row, i.e. an output column n) and result column l%32 (a token m).
 __device__ __forceinline__ int ix_acc_row(int i, int lane) { return ((i >> 2) << 3) + ((lane >> 5) << 2) + (i & 3); }
 
-template <int BM_, int BN_, int WM_, int WN_>
+// PW_ > 0: PW_ extra waves that only fetch (pipeline D below); NT counts the computing threads, NTT all of them.
+template <int BM_, int BN_, int WM_, int WN_, int PW_ = 0>
 struct IxGemmCfg {
-  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
+  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, PW = PW_;
   static constexpr int NT = WM * WN * 64;
+  static constexpr int NTT = NT + PW * 64;
   static constexpr int TM = BM / WM, TN = BN / WN;
   static constexpr int MI = TM / 32, NI = TN / 32;
   static constexpr int X_CH = BM * 8 / NT;  // 16-byte chunks fetched per thread per k-tile
@@ -84,8 +86,12 @@ struct IxGemmCfg {
   static constexpr int UNITS = 0;
   static constexpr bool UNIT_RING = false;
 #endif
-  static constexpr int LDS_BYTES = UNIT_RING ? UNITS * BM * 128
-                                             : (HALF_RING ? HALF_STAGES * (STAGE_BYTES / 2) : FULL_STAGES * STAGE_BYTES);
+  // Pipeline D (fetching waves): as many whole stages as fit in 144 KiB, at most 8.
+  static constexpr int SPLIT_STAGES = (144 * 1024) / STAGE_BYTES > 8 ? 8 : (144 * 1024) / STAGE_BYTES;
+  static constexpr int LDS_BYTES =
+      PW > 0 ? SPLIT_STAGES * STAGE_BYTES
+             : (UNIT_RING ? UNITS * BM * 128
+                          : (HALF_RING ? HALF_STAGES * (STAGE_BYTES / 2) : FULL_STAGES * STAGE_BYTES));
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile must be MFMA multiples");
   static_assert((BM * 8) % NT == 0 && (BN * 8) % NT == 0, "fetch must divide evenly");
   static_assert(NT % 64 == 0, "whole waves");
@@ -422,12 +428,109 @@ __device__ __forceinline__ void ix_gemm_mainloop_units(ix_rsrc_t x_rsrc, const X
   __builtin_amdgcn_s_waitcnt(IX_VMCNT(0));
 }
 
+// ---- pipeline D: fetching waves and computing waves (small tiles) -----------------------------------------------
+// A tile with one or two MFMAs per wave and step is bound by instruction issue (a lone wave issues one instruction
+// every four cycles, and a k-tile costs it the fetch instructions, the ring bookkeeping, the LDS reads and the
+// MFMAs one after another). Here PW waves issue the fetches and wait for them, the WM*WN others only read
+// fragments and multiply; they meet at one barrier per k-tile, which both publishes k-tile kt and frees the stage
+// of k-tile kt-1 (its fragments were consumed by MFMAs before the barrier). A ring of SPLIT_STAGES whole k-tiles,
+// laid out as in pipeline A; the K order is that of pipeline A.
+template <typename Cfg, typename XRow, typename WRow, typename Acc>
+__device__ __forceinline__ void ix_gemm_mainloop_split(ix_rsrc_t x_rsrc, const XRow& x_row,
+                                                       ix_rsrc_t w_rsrc, const WRow& w_row, int K,
+                                                       char* lds, Acc& acc) {
+  constexpr int NP = Cfg::PW * 64, BM = Cfg::BM, S = Cfg::SPLIT_STAGES;
+  constexpr int XC = BM * 8 / NP, WC = Cfg::BN * 8 / NP;  // 16-byte chunks per fetching thread and k-tile
+  static_assert(S >= 3 && (BM * 8) % NP == 0 && (Cfg::BN * 8) % NP == 0, "fetch must divide over the fetching waves");
+  static_assert((S - 2) * (XC + WC) <= 63, "the wait counter holds 63 outstanding loads");
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int KT = (K + IX_BK - 1) / IX_BK;
+  if (wave >= Cfg::WM * Cfg::WN) {
+    // ---- fetching waves
+    const int pt = threadIdx.x - Cfg::NT;  // 0 .. NP-1
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane(ix_lds_addr(lds) + ((pt >> 6) * 64) * 16);
+    const int K2 = K * 2;
+    uint32_t x_voff[XC], w_voff[WC];
+    int x_kb[XC], w_kb[WC];
+#pragma unroll
+    for (int j = 0; j < XC; ++j) {
+      const int r = (pt + j * NP) >> 3;
+      x_kb[j] = ((pt & 7) ^ ix_swz8(r)) * 16;
+      x_voff[j] = x_row(r) + x_kb[j];
+    }
+#pragma unroll
+    for (int j = 0; j < WC; ++j) {
+      const int r = (pt + j * NP) >> 3;
+      w_kb[j] = ((pt & 7) ^ ix_swz8(r)) * 16;
+      w_voff[j] = w_row(r) + w_kb[j];
+    }
+    auto issue = [&](int kt, int slot) {
+      const int soff = kt * IX_BK * 2;
+      const uint32_t sbase = lds_base + slot * Cfg::STAGE_BYTES;
+#pragma unroll
+      for (int j = 0; j < XC; ++j) {
+        const uint32_t dead = (uint32_t)((K2 - 1 - (soff + x_kb[j])) >> 31) & IX_OOB;
+        ix_dma16(x_rsrc, sbase + j * NP * 16, x_voff[j] | dead, soff);
+      }
+#pragma unroll
+      for (int j = 0; j < WC; ++j) {
+        const uint32_t dead = (uint32_t)((K2 - 1 - (soff + w_kb[j])) >> 31) & IX_OOB;
+        ix_dma16(w_rsrc, sbase + BM * 128 + j * NP * 16, w_voff[j] | dead, soff);
+      }
+    };
+#pragma unroll
+    for (int p = 0; p < S - 1; ++p) issue(p, p);
+    int is = S - 1;
+    for (int kt = 0; kt < KT; ++kt) {
+      __builtin_amdgcn_s_waitcnt(IX_VMCNT((S - 2) * (XC + WC)));  // k-tile kt has landed
+      __syncthreads();
+      issue(kt + S - 1, is);  // into the stage of k-tile kt-1
+      is = is + 1 == S ? 0 : is + 1;
+    }
+    __builtin_amdgcn_s_waitcnt(IX_VMCNT(0));  // drain the out-of-range tail fetches before LDS is reused
+    return;
+  }
+  // ---- computing waves
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+  const int frow = lane & 31, fg = lane >> 5;
+  int x_foff[Cfg::MI], w_foff[Cfg::NI];
+#pragma unroll
+  for (int mi = 0; mi < Cfg::MI; ++mi) x_foff[mi] = ix_lds_off(wm * Cfg::TM + mi * 32 + frow, fg * 4);
+#pragma unroll
+  for (int ni = 0; ni < Cfg::NI; ++ni) w_foff[ni] = BM * 128 + ix_lds_off(wn * Cfg::TN + ni * 32 + frow, fg * 4);
+  int cs = 0;
+  for (int kt = 0; kt < KT; ++kt) {
+    __syncthreads();
+    const char* sb = lds + cs * Cfg::STAGE_BYTES;
+    cs = cs + 1 == S ? 0 : cs + 1;
+    ix_bf16x8 xf[4][Cfg::MI], wf[4][Cfg::NI];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+#pragma unroll
+      for (int mi = 0; mi < Cfg::MI; ++mi)
+        xf[s][mi] = *reinterpret_cast<const ix_bf16x8*>(sb + (x_foff[mi] ^ (s << 4)));
+#pragma unroll
+      for (int ni = 0; ni < Cfg::NI; ++ni)
+        wf[s][ni] = *reinterpret_cast<const ix_bf16x8*>(sb + (w_foff[ni] ^ (s << 4)));
+    }
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+      for (int mi = 0; mi < Cfg::MI; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < Cfg::NI; ++ni)
+          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[s][ni], xf[s][mi], acc[mi][ni], 0, 0, 0);
+  }
+}
+
 // x_row(r) / w_row(r): byte offset of tile row r inside the operand's buffer, or IX_OOB.
 template <typename Cfg, typename XRow, typename WRow, typename Acc>
 __device__ __forceinline__ void ix_gemm_mainloop(ix_rsrc_t x_rsrc, const XRow& x_row,
                                                  ix_rsrc_t w_rsrc, const WRow& w_row, int K, char* lds,
                                                  Acc& acc) {
-  if constexpr (Cfg::UNIT_RING)
+  if constexpr (Cfg::PW > 0)
+    ix_gemm_mainloop_split<Cfg>(x_rsrc, x_row, w_rsrc, w_row, K, lds, acc);
+  else if constexpr (Cfg::UNIT_RING)
     ix_gemm_mainloop_units<Cfg>(x_rsrc, x_row, w_rsrc, w_row, K, lds, acc);
   else if constexpr (Cfg::HALF_RING)
     ix_gemm_mainloop_h4<Cfg>(x_rsrc, x_row, w_rsrc, w_row, K, lds, acc);
