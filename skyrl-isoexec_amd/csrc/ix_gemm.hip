@@ -195,8 +195,8 @@ static int ix_gemm_tile_for(long M, long N, long K, int tile) {
   struct Shape { int id, bm, bn; double slots, us_per_ktile, us_per_ktile_shared; };
   // preference order on ties: larger tiles first
   static const Shape shapes[] = {{3, 256, 256, 256.0, 1.5, 1.5},  {5, 128, 256, 256.0, 0.75, 0.75},
-                                 {2, 128, 128, 512.0, 0.6, 1.0},  {1, 32, 256, 256.0, 0.4, 0.4},
-                                 {6, 64, 32, 256.0, 0.16, 0.16}};
+                                 {2, 128, 128, 512.0, 0.6, 1.0},  {1, 32, 256, 256.0, 0.55, 0.55},
+                                 {6, 64, 32, 512.0, 0.16, 0.16}};
   const double kt = (double)((K + 63) / 64);
   const double stream_us = (double)(N + M) * (double)K * 2.0 / 5.0e6;  // both operands once at 5 TB/s
   int best = 3;

@@ -86,8 +86,13 @@ struct IxGemmCfg {
   static constexpr int UNITS = 0;
   static constexpr bool UNIT_RING = false;
 #endif
-  // Pipeline D (fetching waves): as many whole stages as fit in 144 KiB, at most 8.
-  static constexpr int SPLIT_STAGES = (144 * 1024) / STAGE_BYTES > 8 ? 8 : (144 * 1024) / STAGE_BYTES;
+  // Pipeline D (fetching waves): as many whole stages as fit in 144 KiB; a small tile stops at
+  // IX_SPLIT_STAGES_SMALL so that two workgroups share a CU.
+#ifndef IX_SPLIT_STAGES_SMALL
+#define IX_SPLIT_STAGES_SMALL 6
+#endif
+  static constexpr int SPLIT_STAGES =
+      (144 * 1024) / STAGE_BYTES > IX_SPLIT_STAGES_SMALL ? IX_SPLIT_STAGES_SMALL : (144 * 1024) / STAGE_BYTES;
   static constexpr int LDS_BYTES =
       PW > 0 ? SPLIT_STAGES * STAGE_BYTES
              : (UNIT_RING ? UNITS * BM * 128

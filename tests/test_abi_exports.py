@@ -49,6 +49,8 @@ def test_gemm_tile_choice_is_a_host_decision_with_sane_answers():
     assert h.ix_gemm_bf16_n_tiles(4096, 151936, 4096, 0) == -(-151936 // 256)     # LM head: 256-wide tiles
     assert h.ix_gemm_bf16_n_tiles(163840, 128, 2048, 0) == 1                       # gating product: one 128-wide column
     assert h.ix_gemm_bf16_n_tiles(64, 2048, 2048, 0) == 2048 // 32                 # decode projection: 64 x 32 tiles
+    assert h.ix_gemm_bf16_n_tiles(64, 12352, 2048, 0) == 12352 // 32               # wide decode projection: the same
+    assert h.ix_gemm_bf16_n_tiles(256, 12352, 2048, 0) in (-(-12352 // 128), -(-12352 // 256))  # 256 rows: wider tiles
     assert h.ix_gemm_bf16_n_tiles(0, 0, 4096, 0) == 0
 
 
