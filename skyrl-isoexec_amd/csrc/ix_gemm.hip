@@ -85,6 +85,16 @@ __global__ __launch_bounds__((WM * WN + PW) * 64) void k_gemm_bf16_nt(const bf16
 
   ix_f32x16 acc[Cfg::MI][Cfg::NI];
   ix_acc_zero<Cfg>(acc);
+#ifdef IX_EXPERIMENT_RANDOM_LDS
+  {  // fill the whole LDS allocation with pseudo-random bf16 of magnitude ~1 (timing experiments without the fetch)
+    uint32_t h = (threadIdx.x + 1) * 2654435761u + blockIdx.x * 40503u;
+    for (int i = threadIdx.x; i < Cfg::LDS_BYTES / 4; i += Cfg::NTT) {
+      h ^= h << 13; h ^= h >> 17; h ^= h << 5;
+      reinterpret_cast<uint32_t*>(ix_lds)[i] = (h & 0x807f807fu) | 0x3f003f00u;
+    }
+    __syncthreads();
+  }
+#endif
   ix_gemm_mainloop<Cfg>(x_rsrc, x_row, w_rsrc, w_row, K, ix_lds, acc);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;

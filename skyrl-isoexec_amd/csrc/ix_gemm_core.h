@@ -31,8 +31,9 @@ typedef __attribute__((address_space(3))) void ix_lds_void;
 // fetches, IX_EXPERIMENT_NO_FRAG the LDS fragment reads, IX_EXPERIMENT_NO_MFMA the matrix instructions (results are
 // then meaningless; only the timing of what remains is of interest), IX_EXPERIMENT_NO_VMWAIT the wait for the
 // fetched units before each barrier (unit ring), IX_EXPERIMENT_SAME_TILE (dense kernel) points
-// every workgroup at the same few tiles so that all fetches hit L2, IX_NO_UNIT_RING selects the half-tile ring for
-// square tiles.
+// every workgroup at the same few tiles so that all fetches hit L2, IX_EXPERIMENT_RANDOM_LDS (dense kernel) fills the
+// LDS with random bf16 before the loop (for timing the loop without the fetch on realistic operand values),
+// IX_NO_UNIT_RING selects the half-tile ring for square tiles.
 #define IX_OOB 0x7FFFF000u  // a byte offset no buffer descriptor here admits (all are < 1 GiB)
 
 // LDS tiles are [rows][k] bf16 with the 16-byte chunks of a row permuted by an XOR swizzle so that
