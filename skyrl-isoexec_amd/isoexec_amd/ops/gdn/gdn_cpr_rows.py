@@ -13,6 +13,11 @@ from ... import _lib
 
 _ENV = "SKYRL_ISOEXEC_GDN_CPR_FUSED_ROWS"
 
+# served / declined call counts and the last decline's reason (gdn_cpr_rows.py:18-21)
+_served = 0
+_declined = 0
+_decline_reason = ""
+
 
 def fused_rows_enabled() -> bool:
     """Default on; the environment variable is a kill switch (gdn_cpr_rows.py:24-26)."""
@@ -24,6 +29,8 @@ def _resolve(slots, slot2row, blocks, last_used, clock, want64):
     dev = slots.device
     rows64 = torch.empty(n, dtype=torch.int64, device=dev) if want64 else None
     rows32 = torch.empty(n, dtype=torch.int32, device=dev)
+    global _served
+    _served += 1
     _lib.check(
         _lib.lib().ix_gdn_resolve_rows(slots.data_ptr(), int(slots.dtype is torch.int64), n, _lib.ptr(slot2row),
                                        0 if slot2row is None else slot2row.numel(), int(blocks),
@@ -33,17 +40,23 @@ def _resolve(slots, slot2row, blocks, last_used, clock, want64):
 
 
 def _servable(slots, slot2row) -> bool:
-    if slots.dim() != 1 or slots.dtype not in (torch.int32, torch.int64) or not slots.is_contiguous():
-        return False
-    if slot2row is not None and (slot2row.dim() != 1 or slot2row.dtype is not torch.int64 or not slot2row.is_contiguous()):
-        return False
-    return True
+    global _declined, _decline_reason
+    ok = slots.dim() == 1 and slots.dtype in (torch.int32, torch.int64) and slots.is_contiguous()
+    if ok and slot2row is not None:
+        ok = slot2row.dim() == 1 and slot2row.dtype is torch.int64 and slot2row.is_contiguous()
+    if not ok:
+        _declined += 1
+        _decline_reason = (
+            f"slots.dim={slots.dim()} slots.dtype={slots.dtype} "
+            + ("" if slot2row is None else f"map.dim={slot2row.dim()} map.dtype={slot2row.dtype} ")
+            + "(expected 1-D slots, 1-D int64 map)")
+    return ok
 
 
 def cpr_resolve_rows(slots: torch.Tensor, slot2row: torch.Tensor):
     """``(rows_int64, rows_int32)`` for a decode batch's engine slot ids; ``None`` to request the eager chain
     (gdn_cpr_rows.py:49-80)."""
-    if not _servable(slots, slot2row) or slot2row is None:
+    if slot2row is None or not _servable(slots, slot2row):
         return None
     _lib.require_device(slots, slot2row)
     return _resolve(slots, slot2row, 0, None, None, True)

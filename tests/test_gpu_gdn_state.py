@@ -281,6 +281,16 @@ def test_fused_row_resolver_equals_the_eager_chain():
         nat = resolve_and_stamp(slots, blocks=40)
         s = slots.long()
         assert torch.equal(nat.long(), torch.where(s < 40, s, torch.zeros_like(s)).clamp(min=0))
+    # every slot vector a replayed decode step can present, through the pool's own seam
+    from test_gdn_rows_host import make_pool, rows_eager, slot_vectors
+
+    rg = make_pool()
+    rg.slot2row = rg.slot2row.to(DEV)
+    for sv in slot_vectors(rg.slot2row.numel()):
+        rows, rows32 = rg._rows_pair(sv.to(DEV))
+        want = rows_eager(rg.slot2row, sv.to(DEV))
+        assert rows.dtype is torch.int64 and rows32.dtype is torch.int32
+        assert torch.equal(rows, want) and torch.equal(rows32.long(), want)
     # the use stamp: clock += 1, last_used[rows] = clock, twice in a row, duplicates included
     last_used = torch.zeros(rows_n, dtype=torch.int64, device=DEV)
     clock = torch.full((), 41, dtype=torch.int64, device=DEV)
