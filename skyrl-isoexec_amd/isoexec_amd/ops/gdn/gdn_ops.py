@@ -252,10 +252,59 @@ def gdn_recurrent(q, k, v, g, beta, *, initial_state=None, output_final_state=Fa
     return o, None
 
 
+def gdn_kernel_mode() -> str:
+    """The delta-rule kernel this process runs (gdn_ops.py:19-36); parsed in ``core/gdn_kernel_env``."""
+    from ...core.gdn_kernel_env import gdn_kernel_mode as _mode
+
+    return _mode()
+
+
+def recurrent_mode() -> bool:
+    return gdn_kernel_mode() == "recurrent"
+
+
+def cpr_mode() -> bool:
+    return gdn_kernel_mode() == "cpr"
+
+
+def fla_chunk_size() -> int:
+    """The chunk length of the boundary form (the reference reads vLLM's FLA_CHUNK_SIZE, 64; gdn_ops.py:216-219)."""
+    return 64
+
+
+def gdn_cpr(q, k, v, g, beta, *, initial_state=None, output_final_state=False, cu_seqlens=None):
+    """Stateless boundary-form forward: ``(o, None)`` (gdn_ops.py:1063-1116). A padded ``[B, T, ...]`` batch is
+    flattened to B packed sequences."""
+    if initial_state is not None or output_final_state:
+        raise NotImplementedError(
+            "isoexec GDN: gdn_cpr is the stateless (training/prefill-from-zero) entry point.")
+    from .gdn_cpr import gdn_cpr_fwd
+
+    B, T = q.shape[0], q.shape[1]
+    with torch.no_grad():
+        if cu_seqlens is None:
+            flat = lambda t: t.reshape(1, B * T, *t.shape[2:])
+            cu = torch.arange(0, (B + 1) * T, T, dtype=torch.int32, device=q.device)
+            o = gdn_cpr_fwd(flat(q), flat(k), flat(v), flat(g), flat(beta), cu_seqlens=cu, chunk_size=fla_chunk_size())
+            return o.reshape(B, T, *o.shape[2:]), None
+        return gdn_cpr_fwd(q, k, v, g, beta, cu_seqlens=cu_seqlens, chunk_size=fla_chunk_size()), None
+
+
 def gdn_core(q, k, v, g, beta, *, initial_state=None, output_final_state=False, cu_seqlens=None):
-    """The trainer's door (gdn_ops.py:1118-1194). One kernel mode exists here: recurrent."""
-    return gdn_recurrent(q, k, v, g, beta, initial_state=initial_state, output_final_state=output_final_state,
-                         cu_seqlens=cu_seqlens)
+    """The trainer's door (gdn_ops.py:1118-1194): :func:`gdn_recurrent` or :func:`gdn_cpr` per
+    :func:`gdn_kernel_mode` (``SKYRL_ISOEXEC_GDN_TRAINER_KERNEL`` overrides it for this door only). The
+    chunk-parallel kernel of the vocabulary is not served here: its bits depend on the chunk length, which the
+    recurrent and boundary forms do not have to pay for."""
+    from ...core.gdn_kernel_env import gdn_trainer_kernel_override
+
+    mode = gdn_trainer_kernel_override() or gdn_kernel_mode()
+    kw = dict(initial_state=initial_state, output_final_state=output_final_state, cu_seqlens=cu_seqlens)
+    if mode == "cpr":
+        return gdn_cpr(q, k, v, g, beta, **kw)
+    if mode == "recurrent":
+        return gdn_recurrent(q, k, v, g, beta, **kw)
+    raise NotImplementedError(
+        f"[isoexec-amd] delta-rule kernel {mode!r} is not served on gfx950; use 'recurrent' (default) or 'cpr'")
 
 
 def gdn_native_core_kernel(q, k, v, a, b, A_log, dt_bias, *, ssm_state, state_indices, cu_seqlens):
