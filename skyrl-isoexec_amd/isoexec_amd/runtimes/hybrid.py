@@ -151,8 +151,8 @@ class _Blocks:
         q = proj[:, :nq].unflatten(1, (c.q_heads, c.head_dim))
         k = proj[:, nq : nq + nk].unflatten(1, (c.kv_heads, c.head_dim))
         v = proj[:, nq + nk :].unflatten(1, (c.kv_heads, c.head_dim))
-        apply_rope_(q, self.cos, self.sin, positions)
-        apply_rope_(k, self.cos, self.sin, positions)
+        # q and k are adjacent column blocks with one head size: one launch rotates the q and kv heads of a token
+        apply_rope_(proj[:, : nq + nk].unflatten(1, (c.q_heads + c.kv_heads, c.head_dim)), self.cos, self.sin, positions)
         return q, k, v
 
     def attn_out(self, layer: int, o: torch.Tensor) -> torch.Tensor:
