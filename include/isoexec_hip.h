@@ -126,7 +126,7 @@ int ix_gemm_f32_nt(const void* A, int a_dtype, long lda, const void* W, long ldw
 /* gdn_recurrent_kernel (gdn_ops.py:400-441): the delta-rule scan over packed tokens, state pool
  * advanced in place. q,k [tokens, H, K] and v [tokens, HV, V] with token pitches q_pitch,
  * k_pitch, v_pitch (elements; heads contiguous inside a token, so slices of one projection
- * buffer need no copy); o [tokens, HV, V] contiguous; g fp32 [tokens, HV]; beta [tokens, HV];
+ * buffer need no copy); o [tokens, HV, V] contiguous, or NULL for a state-only pass; g fp32 [tokens, HV]; beta [tokens, HV];
  * q/k/v/beta/o share io_dtype. state_pool fp32 [rows, HV, V, K]. cu_seqlens int32
  * [N+1]. state_indices int32: pool row for (sequence n, token t) at [n*stride + t]; column 0
  * loads, a positive entry at column t stores after token t, row index <= 0 at column 0 skips
@@ -180,6 +180,21 @@ int ix_gdn_gate(const void* a, long a_pitch, const void* b, long b_pitch, const 
  * last_used[row] = clock[0] for every row of the batch (the decode step's use stamp). */
 int ix_gdn_resolve_rows(const void* slots, int slots_i64, long n, const int64_t* slot2row, long map_n, long blocks,
                         int64_t* rows64, int* rows32, int64_t* last_used, int64_t* clock, void* stream);
+
+/* cpr_buffer_scatter (gdn_cpr_scatter.py:24-76; eager form in CprGDN.decode, gdn_cpr_state.py): lane n of a decode
+ * step appends its prepared k [H*K] (token pitch k_pitch), v [HV*V] (v_pitch), g fp32 [HV], beta [HV] to the
+ * open-chunk buffers k_buf [rows, C, H, K], v_buf [rows, C, HV, V], g_buf fp32 [rows, C, HV], b_buf [rows, C, HV] at
+ * (row = rows[n], column = pos[row] % C), then pos[row] += 1 for row > 0 and due[row] = row if the new position is
+ * a multiple of C else 0. pos int64 [rows]; due int32 [rows]; a live row appears at most once among rows[0..N). */
+int ix_gdn_cpr_scatter(const void* k, long k_pitch, const void* v, long v_pitch, const float* g, const void* beta,
+                       const int* rows, int64_t* pos, void* k_buf, void* v_buf, float* g_buf, void* b_buf, int* due,
+                       int io_dtype, long N, long H, long K, long HV, long V, long C, void* stream);
+
+/* The hand-off that ends CprGDN._resync (gdn_cpr_state.py:644-646): for every row with due[row] > 0,
+ * running_state[row] = widen(round_to(snapshot_dtype, entry_state[row])); then due[] is cleared. Both pools fp32
+ * [rows, elems], elems % 4 == 0. */
+int ix_gdn_cpr_handoff(const float* entry_state, float* running_state, int* due, long rows, long elems,
+                       int snapshot_dtype, void* stream);
 
 /* gdn_causal_conv / gdn_causal_conv_batched (gdn_ops.py:74-170) over packed tokens, and the
  * engine's window-slide update (gdn_recurrent_state.py:686-707,814-825) when every sequence has

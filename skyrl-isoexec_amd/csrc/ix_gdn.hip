@@ -94,6 +94,7 @@ __global__ __launch_bounds__(256) void k_gdn_scan(const TIO* __restrict__ q, con
   const long sbase = sidx_stride == 0 ? (long)n : (long)n * sidx_stride;
   const int row0 = sidx[sbase];
   if (row0 <= 0) {  // null lane: no state, outputs defined as zero
+    if (!o) return;
     for (int i = tid; i < len * R; i += 256) {
       const int tt = i / R, rr = i % R;
       ix_st(o + ((long)(t_begin + tt) * HV + hv) * V + vb * R + rr, 0.0f);
@@ -190,9 +191,11 @@ __global__ __launch_bounds__(256) void k_gdn_scan(const TIO* __restrict__ q, con
       }
     }
     __syncthreads();
-    for (int i = tid; i < nt * R; i += 256) {
-      const int tt = i / R, rr = i % R;
-      ix_st(o + ((long)(t_begin + t0 + tt) * HV + hv) * V + vb * R + rr, of[i]);
+    if (o) {
+      for (int i = tid; i < nt * R; i += 256) {
+        const int tt = i / R, rr = i % R;
+        ix_st(o + ((long)(t_begin + t0 + tt) * HV + hv) * V + vb * R + rr, of[i]);
+      }
     }
   }
 }
@@ -246,6 +249,7 @@ void k_gdn_scan_pairs(const TIO* __restrict__ q, const TIO* __restrict__ k, cons
   if (len <= 0) return;
   const int row0 = sidx[n];
   if (row0 <= 0) {  // null lane: no state, outputs defined as zero
+    if (!o) return;
     for (int i = tid; i < len * R; i += 256) {
       const int tt = i / R, rr = i % R;
       ix_st(o + ((long)(t_begin + tt) * HV + hv) * V + vb * R + rr, 0.0f);
@@ -348,9 +352,11 @@ void k_gdn_scan_pairs(const TIO* __restrict__ q, const TIO* __restrict__ k, cons
         *reinterpret_cast<float4*>(srow + 4 * c) = make_float4(S[4 * c], S[4 * c + 1], S[4 * c + 2], S[4 * c + 3]);
     }
     __syncthreads();
-    for (int i = tid; i < nt * R; i += 256) {
-      const int tt = i / R, rr = i % R;
-      ix_st(o + ((long)(t_begin + t0 + tt) * HV + hv) * V + vb * R + rr, of[i]);
+    if (o) {
+      for (int i = tid; i < nt * R; i += 256) {
+        const int tt = i / R, rr = i % R;
+        ix_st(o + ((long)(t_begin + t0 + tt) * HV + hv) * V + vb * R + rr, of[i]);
+      }
     }
   }
 }
@@ -410,7 +416,7 @@ extern "C" int ix_gdn_scan(const void* q, const void* k, const void* v, const fl
                            int io_dtype, long q_pitch, long k_pitch, long v_pitch, float* state_pool,
                            const int* cu_seqlens, const int* state_indices, long state_indices_stride, long N,
                            long H, long HV, long K, long V, float scale, int time_tile, void* stream) {
-  if (!q || !k || !v || !g || !beta || !o || !state_pool || !cu_seqlens || !state_indices) return IX_ERR_ARG;
+  if (!q || !k || !v || !g || !beta || !state_pool || !cu_seqlens || !state_indices) return IX_ERR_ARG;
   if (N < 0 || H <= 0 || HV <= 0 || K <= 0 || V <= 0 || HV % H != 0 || state_indices_stride < 0) return IX_ERR_ARG;
   if (q_pitch < H * K || k_pitch < H * K || v_pitch < HV * V) return IX_ERR_ARG;
   if (io_dtype != IX_DT_F32 && io_dtype != IX_DT_BF16) return IX_DECLINED;
@@ -549,6 +555,94 @@ extern "C" int ix_gdn_gate(const void* a, long a_pitch, const void* b, long b_pi
   else
     hipLaunchKernelGGL((k_gdn_gate<float>), dim3((unsigned)grid), dim3(256), 0, st, (const float*)a, a_pitch,
                        (const float*)b, b_pitch, A_log, dt_bias, g, (float*)beta, n, (int)HV);
+  return ix_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Open-chunk bookkeeping of the boundary (cpr) engine state (gdn_cpr_scatter.py:24-76; eager form
+// gdn_cpr_state.py decode): lane n appends this step's prepared k, v, g, beta to the open-chunk buffers of its
+// pool row at column pos[row] % C, then pos[row] += 1 (not for row 0, which absorbs padded lanes), and marks the
+// row due for a boundary pass when its position has reached a multiple of C. One workgroup per lane; a live row
+// appears at most once per step.
+template <typename TIO>
+__global__ __launch_bounds__(256) void k_gdn_cpr_scatter(const TIO* __restrict__ k, long k_pitch,
+                                                         const TIO* __restrict__ v, long v_pitch,
+                                                         const float* __restrict__ g, const TIO* __restrict__ beta,
+                                                         const int* __restrict__ rows, int64_t* __restrict__ pos,
+                                                         TIO* __restrict__ k_buf, TIO* __restrict__ v_buf,
+                                                         float* __restrict__ g_buf, TIO* __restrict__ b_buf,
+                                                         int* __restrict__ due, int HK, int HVV, int HV, int C) {
+  const int n = blockIdx.x;
+  const int row = rows[n];
+  const int64_t p = pos[row];
+  const int col = (int)(p % C);
+  __syncthreads();  // every lane has read the position before lane 0 advances it
+  const long slot = (long)row * C + col;
+  for (int i = threadIdx.x; i < HK; i += 256) k_buf[slot * HK + i] = k[(long)n * k_pitch + i];
+  for (int i = threadIdx.x; i < HVV; i += 256) v_buf[slot * HVV + i] = v[(long)n * v_pitch + i];
+  for (int i = threadIdx.x; i < HV; i += 256) {
+    g_buf[slot * HV + i] = g[(long)n * HV + i];
+    b_buf[slot * HV + i] = beta[(long)n * HV + i];
+  }
+  if (threadIdx.x == 0 && row > 0) {
+    pos[row] = p + 1;
+    due[row] = ((p + 1) % C == 0) ? row : 0;
+  }
+}
+
+extern "C" int ix_gdn_cpr_scatter(const void* k, long k_pitch, const void* v, long v_pitch, const float* g,
+                                  const void* beta, const int* rows, int64_t* pos, void* k_buf, void* v_buf,
+                                  float* g_buf, void* b_buf, int* due, int io_dtype, long N, long H, long K, long HV,
+                                  long V, long C, void* stream) {
+  if (!k || !v || !g || !beta || !rows || !pos || !k_buf || !v_buf || !g_buf || !b_buf || !due) return IX_ERR_ARG;
+  if (N < 0 || H <= 0 || K <= 0 || HV <= 0 || V <= 0 || C <= 0 || k_pitch < H * K || v_pitch < HV * V)
+    return IX_ERR_ARG;
+  if (io_dtype != IX_DT_F32 && io_dtype != IX_DT_BF16) return IX_DECLINED;
+  if (N == 0) return IX_OK;
+  if (N > 0x7fffffffL) return IX_DECLINED;
+  hipStream_t st = (hipStream_t)stream;
+  if (io_dtype == IX_DT_BF16)
+    hipLaunchKernelGGL(k_gdn_cpr_scatter<bf16_t>, dim3((unsigned)N), dim3(256), 0, st, (const bf16_t*)k, k_pitch,
+                       (const bf16_t*)v, v_pitch, g, (const bf16_t*)beta, rows, pos, (bf16_t*)k_buf, (bf16_t*)v_buf,
+                       g_buf, (bf16_t*)b_buf, due, (int)(H * K), (int)(HV * V), (int)HV, (int)C);
+  else
+    hipLaunchKernelGGL(k_gdn_cpr_scatter<float>, dim3((unsigned)N), dim3(256), 0, st, (const float*)k, k_pitch,
+                       (const float*)v, v_pitch, g, (const float*)beta, rows, pos, (float*)k_buf, (float*)v_buf, g_buf,
+                       (float*)b_buf, due, (int)(H * K), (int)(HV * V), (int)HV, (int)C);
+  return ix_launch_status();
+}
+
+// The hand-off after a boundary pass (gdn_cpr_state.py:602-646): for every pool row marked due, the running state
+// becomes the snapshot of the fp32 chain (rounded to the wire dtype and widened back), and the mark is cleared.
+__global__ __launch_bounds__(256) void k_gdn_cpr_handoff(const float* __restrict__ entry, float* __restrict__ running,
+                                                         int* __restrict__ due, long elems, int snap_bf16) {
+  const int row = blockIdx.y;
+  if (due[row] <= 0) return;
+  const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i < elems) {
+    float4 x = *reinterpret_cast<const float4*>(entry + (long)row * elems + i);
+    if (snap_bf16) { x.x = ix_rbf(x.x); x.y = ix_rbf(x.y); x.z = ix_rbf(x.z); x.w = ix_rbf(x.w); }
+    *reinterpret_cast<float4*>(running + (long)row * elems + i) = x;
+  }
+}
+__global__ __launch_bounds__(256) void k_gdn_cpr_clear_due(int* __restrict__ due, int rows) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < rows) due[i] = 0;
+}
+
+extern "C" int ix_gdn_cpr_handoff(const float* entry_state, float* running_state, int* due, long rows, long elems,
+                                  int snapshot_dtype, void* stream) {
+  if (!entry_state || !running_state || !due || rows < 0 || elems <= 0) return IX_ERR_ARG;
+  if (snapshot_dtype != IX_DT_F32 && snapshot_dtype != IX_DT_BF16) return IX_DECLINED;
+  if ((elems % 4) || !ix_aligned(entry_state, 16) || !ix_aligned(running_state, 16)) return IX_DECLINED;
+  if (rows == 0) return IX_OK;
+  const long gx = (elems / 4 + 255) / 256;
+  if (rows > 65535 || gx > 0x7fffffffL) return IX_DECLINED;
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(k_gdn_cpr_handoff, dim3((unsigned)gx, (unsigned)rows), dim3(256), 0, st, entry_state,
+                     running_state, due, elems, snapshot_dtype == IX_DT_BF16);
+  // the marks are cleared by a second launch: every workgroup of the first reads its row's mark
+  hipLaunchKernelGGL(k_gdn_cpr_clear_due, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, due, (int)rows);
   return ix_launch_status();
 }
 

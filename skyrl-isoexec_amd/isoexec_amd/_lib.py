@@ -62,6 +62,8 @@ SIGNATURES = {
          c_long, c_float, c_int, P],
     ),
     "ix_gdn_l2norm": (c_int, [P, c_long, P, c_int, c_long, c_long, c_long, c_float, P]),
+    "ix_gdn_cpr_scatter": (c_int, [P, c_long, P, c_long, P, P, P, P, P, P, P, P, P, c_int, c_long, c_long, c_long, c_long, c_long, c_long, P]),
+    "ix_gdn_cpr_handoff": (c_int, [P, P, P, c_long, c_long, c_int, P]),
     "ix_gdn_resolve_rows": (c_int, [P, c_int, c_long, P, c_long, c_long, P, P, P, P, P]),
     "ix_gdn_gate": (c_int, [P, c_long, P, c_long, P, P, P, P, c_int, c_long, c_long, P]),
     "ix_gdn_conv": (c_int, [P, c_long, P, P, P, P, P, P, P, c_long, c_long, c_long, c_long, c_int, P]),

@@ -16,8 +16,10 @@ def register(reg) -> None:
                 supported_archs=GFX950,
                 rounding=RoundingSchedule(
                     machine_assertable={
-                        "kernel": OneOf("recurrent"),
+                        "kernel": OneOf("recurrent", "cpr"),
                         "state_dtype": "fp32",
+                        "cpr": "entry chain fp32 per chunk boundary; running state = chain rounded to the wire dtype "
+                               "at each boundary; chunk 64",
                         "recurrence": "token-level: S*=exp(g); v-=S.k; v*=beta; S+=k (x) v; o=S.q",
                         "dot": "8 state floats per lane as two fma chains (even, odd k), then lane tree",
                         "fma": "explicit only",

@@ -123,11 +123,12 @@ def sequence_metadata(cu_seqlens: torch.Tensor, chunk_size: int, device):
 
 
 def chunk_boundary_states(q, k, v, g, beta, cu_seqlens, chunk_size: int, initial_state=None,
-                          output_final_state: bool = False, lens=None, cu_fla=None):
+                          output_final_state: bool = False, lens=None, cu_fla=None, keep_fp32: bool = False):
     """``(h, final_state, chunk_indices)`` (gdn_cpr.py:104-179): ``h [1, M, HV, V, K]`` in the wire dtype is the
     snapshot of the state ENTERING each chunk, chunks in packed order; ``final_state [N, HV, V, K]`` fp32 is the
     unrounded chain at each sequence's end (or None). ``initial_state`` ``[N, HV, V, K]`` fp32 or None.
-    ``q`` may be None (the boundary states do not depend on it)."""
+    ``q`` may be None (the boundary states do not depend on it). ``keep_fp32`` returns ``h`` as the unrounded fp32
+    chain instead of the snapshot (for a caller that keeps the chain and snapshots it itself)."""
     if chunk_size < 2:
         raise ValueError("chunk_size must be at least 2")
     if k.ndim != 4 or k.shape[0] != 1:
@@ -168,10 +169,9 @@ def chunk_boundary_states(q, k, v, g, beta, cu_seqlens, chunk_size: int, initial
         else:
             idx[n, length - 1] = final0 + n
             final_rows.append(final0 + n)
-    qq = k if q is None else q
-    if M > 0:
-        gdn_recurrent_kernel(qq, k, v, g, beta, ssm_state=pool, state_indices=torch.from_numpy(idx).to(dev),
-                             cu_seqlens=cu_seqlens if cu_fla is None else cu_fla)
+    if M > 0:  # a state-only pass: q plays no part, nothing but the pool is written
+        gdn_recurrent_kernel(k, k, v, g, beta, ssm_state=pool, state_indices=torch.from_numpy(idx).to(dev),
+                             cu_seqlens=cu_seqlens if cu_fla is None else cu_fla, want_output=False)
     # the snapshot: entering states in packed chunk order, cast to the wire dtype
     h32 = torch.empty(M, HV, V, K, dtype=torch.float32, device=dev)
     rows_t = torch.tensor([r if r > 0 else 0 for r in bound_rows], dtype=torch.long, device=dev)
@@ -184,7 +184,7 @@ def chunk_boundary_states(q, k, v, g, beta, cu_seqlens, chunk_size: int, initial
         else:
             seqs = torch.tensor([-bound_rows[i] - 1 for i in first], dtype=torch.long, device=dev)
             h32[first_t] = initial_state.to(torch.float32)[seqs]
-    h = h32.to(k.dtype).unsqueeze(0)
+    h = (h32 if keep_fp32 else h32.to(k.dtype)).unsqueeze(0)
     final_state = None
     if output_final_state:
         final_state = pool[torch.tensor(final_rows, dtype=torch.long, device=dev)].clone() if N else pool[:0].clone()

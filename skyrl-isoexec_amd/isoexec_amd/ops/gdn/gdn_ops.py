@@ -63,8 +63,10 @@ def gdn_recurrent_kernel(
     state_indices: torch.Tensor,
     cu_seqlens: torch.Tensor | None = None,
     time_tile: int = 0,
+    want_output: bool = True,
 ) -> torch.Tensor:
-    """The delta-rule scan. Advances ``ssm_state`` IN PLACE. Returns ``o`` shaped like ``v``.
+    """The delta-rule scan. Advances ``ssm_state`` IN PLACE. Returns ``o`` shaped like ``v`` (``None`` for a
+    state-only pass, ``want_output=False``: nothing but the state pool is written).
 
     ``q, k``: ``[B, T, H, K]`` already L2-normalised (H may be GQA-compressed: ``HV % H == 0``);
     ``v``: ``[B, T, HV, V]``; ``g`` (fp32), ``beta``: ``[B, T, HV]``; ``ssm_state`` fp32 pool
@@ -107,17 +109,19 @@ def gdn_recurrent_kernel(
         idx_stride = idx.stride(0)
     if idx.shape[0] != n_seq:
         raise RuntimeError(f"[isoexec-amd] state_indices has {idx.shape[0]} rows for {n_seq} sequences")
-    o = torch.empty(qf.shape[0], HV, V, dtype=io, device=dev)
+    o = torch.empty(qf.shape[0], HV, V, dtype=io, device=dev) if want_output else None
     if time_tile == 0 and cu_seqlens is None and T == 1:
         time_tile = 1
     rc = _lib.check(
         _lib.lib().ix_gdn_scan(
-            qf.data_ptr(), kf.data_ptr(), vf.data_ptr(), gf.data_ptr(), bf.data_ptr(), o.data_ptr(),
+            qf.data_ptr(), kf.data_ptr(), vf.data_ptr(), gf.data_ptr(), bf.data_ptr(), _lib.ptr(o),
             _lib.dtype_code(io), _token_pitch(qf), _token_pitch(kf), _token_pitch(vf), ssm_state.data_ptr(),
             cu.data_ptr(), idx.data_ptr(), idx_stride, n_seq, H, HV, K, V, float(K) ** -0.5, time_tile,
             _lib.current_stream(dev)), "ix_gdn_scan")
     if rc != _lib.IX_OK:
         raise RuntimeError(f"[isoexec-amd] ix_gdn_scan declined K={K} V={V} dtype={io}")
+    if o is None:
+        return None
     return o.view(B, T, HV, V) if cu_seqlens is None else o.unsqueeze(0)
 
 

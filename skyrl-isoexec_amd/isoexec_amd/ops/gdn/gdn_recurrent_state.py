@@ -475,6 +475,16 @@ class RecurrentGDN:
         prefill_query_start_loc: torch.Tensor | None = None,
     ) -> torch.Tensor:
         """Prefill a packed batch of N prompts (or prompt chunks). Returns ``o [T, HV, V]``."""
+        rows, is_cont, rows_out, cu, q, k, v, g, beta = self._prefill_prepare(
+            slots_cpu, x, a, b, qsl, has_initial_state, prefill_query_start_loc)
+        o = gdn_recurrent_kernel(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), g.unsqueeze(0), beta.unsqueeze(0),
+                                 ssm_state=self.ssm_state, state_indices=rows_out, cu_seqlens=cu)
+        return o[0]
+
+    def _prefill_prepare(self, slots_cpu, x, a, b, qsl, has_initial_state, prefill_query_start_loc):
+        """Everything of a prefill in front of the scan: rows assigned (fresh rows zeroed), the convolution with
+        its window carried in the pool, q/k normalised, gate and beta. Returns ``(rows, is_cont, rows_out int32
+        device, cu int32 device, q, k, v, g, beta)`` with q, k ``[T, H, K]``, v ``[T, HV, V]``, g, beta ``[T, HV]``."""
         N = len(slots_cpu)
         dev = x.device
         if len(qsl) != N + 1 or qsl[-1] != x.shape[0]:
@@ -506,14 +516,16 @@ class RecurrentGDN:
         if cu is None:
             cu = torch.from_numpy(np.asarray(qsl, dtype=np.int32)).to(dev, non_blocking=True)
         # A fresh row must start from zero; a resumed row keeps what the previous chunk left.
-        self.ssm_state.index_fill_(0, meta_t[2].long(), 0.0)
+        self._zero_fresh_rows(meta_t[2].long())
         y = conv_packed(x, self.conv_weight, self.conv_bias, cu_seqlens=cu, conv_state=self.conv_state,
                         rows_in=rows_in, rows_out=rows_out, activation=self.activation)
         q, k, v = self._split_qkv(y)
         g, beta = self._gate_and_beta(a, b)
-        o = gdn_recurrent_kernel(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), g.unsqueeze(0), beta.unsqueeze(0),
-                                 ssm_state=self.ssm_state, state_indices=rows_out, cu_seqlens=cu)
-        return o[0]
+        return rows, is_cont, rows_out, cu, q, k, v, g, beta
+
+    def _zero_fresh_rows(self, fresh_rows: torch.Tensor) -> None:
+        """Rows that start a new request (device int64, 0 = none)."""
+        self.ssm_state.index_fill_(0, fresh_rows, 0.0)
 
     @torch.no_grad()
     def decode(self, slots: torch.Tensor, x: torch.Tensor, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:

@@ -24,6 +24,8 @@ import torch
 
 from ..ops.attention.varlen_attn import KVCache, varlen_attention
 from ..ops.gdn.gdn_ops import conv_packed, gdn_native_core
+from ..ops.gdn.gdn_cpr import gdn_native_cpr_fwd
+from ..ops.gdn.gdn_cpr_state import CprGDN
 from ..ops.gdn.gdn_recurrent_state import RecurrentGDN
 from ..ops.logprobs.rowinv import leaves, sampled_forward
 from ..ops.mm.mm_hip import linear_nt
@@ -43,6 +45,10 @@ class HybridConfig:
     gdn_v_heads: int = 32
     gdn_head_dim: int = 128
     conv_width: int = 4
+    # delta-rule kernel of every site: "recurrent", or "cpr" (fp32 chain at chunk boundaries, running state
+    # re-snapshotted in the wire dtype every gdn_chunk tokens); trainer and engine must run the same one
+    gdn_kernel: str = "recurrent"
+    gdn_chunk: int = 64
     # attention
     q_heads: int = 32
     kv_heads: int = 4
@@ -213,7 +219,11 @@ class TrainerModel:
             q = y[:, :kd].unflatten(1, (c.gdn_k_heads, c.gdn_head_dim))
             k = y[:, kd : 2 * kd].unflatten(1, (c.gdn_k_heads, c.gdn_head_dim))
             v = y[:, 2 * kd :].unflatten(1, (c.gdn_v_heads, c.gdn_head_dim))
-            o = gdn_native_core(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), a, bb, lw["A_log"], lw["dt_bias"], cu_seqlens=cu)
+            if c.gdn_kernel == "cpr":
+                o = gdn_native_cpr_fwd(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), a, bb, lw["A_log"], lw["dt_bias"],
+                                       cu_seqlens=cu, chunk_size=c.gdn_chunk)
+            else:
+                o = gdn_native_core(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), a, bb, lw["A_log"], lw["dt_bias"], cu_seqlens=cu)
             return b.gdn_out(i, o[0], z)
 
         return b.run_layers(b.embed(tokens), mixer)
@@ -245,10 +255,11 @@ class RolloutEngine:
             if cfg.is_attention(i):
                 self.kv[i] = KVCache(max_num_seqs, max_len, cfg.kv_heads, cfg.head_dim, device=dev)
             else:
-                self.gdn[i] = RecurrentGDN(
-                    capacity=max_num_seqs, conv_weight=lw["conv_weight"], conv_bias=lw["conv_bias"], A_log=lw["A_log"],
-                    dt_bias=lw["dt_bias"], num_k_heads=cfg.gdn_k_heads, head_k_dim=cfg.gdn_head_dim,
-                    num_v_heads=cfg.gdn_v_heads, head_v_dim=cfg.gdn_head_dim, device=dev, driver_managed=True)
+                kw = dict(capacity=max_num_seqs, conv_weight=lw["conv_weight"], conv_bias=lw["conv_bias"],
+                          A_log=lw["A_log"], dt_bias=lw["dt_bias"], num_k_heads=cfg.gdn_k_heads,
+                          head_k_dim=cfg.gdn_head_dim, num_v_heads=cfg.gdn_v_heads, head_v_dim=cfg.gdn_head_dim,
+                          device=dev, driver_managed=True)
+                self.gdn[i] = CprGDN(chunk_size=cfg.gdn_chunk, **kw) if cfg.gdn_kernel == "cpr" else RecurrentGDN(**kw)
         # One row table names a request's place in the key/value caches; the GatedDeltaNet layers keep
         # their own (identical) tables so each can be released or evicted with its pool.
         self.kv_rows: dict[int, int] = {}

@@ -1,0 +1,201 @@
+"""GPU parity of the boundary-form engine state (``CprGDN``; reference gdn_cpr_state.py:379-1245) with the
+boundary-form forward (``gdn_cpr_fwd``): whatever way a request's tokens are cut into a packed prefill, resumed
+prefill chunks and single-token decode steps, mixed with other requests and padded lanes, the layer's outputs equal
+the one-pass forward's bit for bit, and its entry states, running states, buffers and positions are what the
+definition says."""
+
+import numpy as np
+import pytest
+import torch
+
+from _util import cpu_gen, same_bits
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+H, K, HV, V, W = 2, 64, 4, 64, 4
+KD = H * K
+D = 2 * KD + HV * V
+C = 16
+
+
+def params():
+    g = cpu_gen(11)
+    bf = lambda t: t.to(torch.bfloat16)
+    return dict(conv_weight=bf(torch.randn(D, W, generator=g) * 0.4).to(DEV), conv_bias=bf(torch.randn(D, generator=g) * 0.1).to(DEV),
+                A_log=(torch.randn(HV, generator=g) * 0.3).to(DEV), dt_bias=(torch.randn(HV, generator=g) * 0.3).to(DEV))
+
+
+def make_layer(capacity=6, chunk=C):
+    from isoexec_amd.ops.gdn.gdn_cpr_state import CprGDN
+
+    return CprGDN(capacity=capacity, chunk_size=chunk, num_k_heads=H, head_k_dim=K, num_v_heads=HV, head_v_dim=V,
+                  device=DEV, **params())
+
+
+def request(seed, n):
+    g = cpu_gen(seed)
+    bf = lambda t: t.to(torch.bfloat16).to(DEV)
+    return bf(torch.randn(n, D, generator=g)), bf(torch.randn(n, HV, generator=g)), bf(torch.randn(n, HV, generator=g))
+
+
+def one_pass(layer, x, a, b, chunk=C):
+    """The forward over a whole request from nothing: conv, normalisation, gate, then gdn_cpr_fwd; also the chain
+    state at the last boundary and the running state after the last token."""
+    from isoexec_amd.ops.gdn.gdn_cpr import chunk_boundary_states, gdn_cpr_fwd
+    from isoexec_amd.ops.gdn.gdn_ops import conv_packed, gdn_recurrent_kernel
+
+    n = x.shape[0]
+    cu = torch.tensor([0, n], dtype=torch.int32, device=DEV)
+    y = conv_packed(x, layer.conv_weight, layer.conv_bias, cu_seqlens=cu)
+    q, k, v = layer._split_qkv(y)
+    g, beta = layer._gate_and_beta(a, b)
+    u = lambda t: t.unsqueeze(0)
+    o = gdn_cpr_fwd(u(q), u(k), u(v), u(g), u(beta), cu_seqlens=cu, chunk_size=chunk)[0]
+    nfull = (n // chunk) * chunk
+    entry = torch.zeros(HV, V, K, device=DEV)
+    if nfull:
+        cuf = torch.tensor([0, nfull], dtype=torch.int32, device=DEV)
+        _, fin, _ = chunk_boundary_states(None, u(k[:nfull]), u(v[:nfull]), u(g[:nfull]), u(beta[:nfull]), cuf, chunk,
+                                          output_final_state=True)
+        entry = fin[0]
+    running = entry.to(torch.bfloat16).float().unsqueeze(0).contiguous()
+    pool = torch.cat([torch.zeros_like(running), running])
+    if n > nfull:
+        cut = torch.tensor([0, n - nfull], dtype=torch.int32, device=DEV)
+        gdn_recurrent_kernel(u(q[nfull:]), u(k[nfull:]), u(v[nfull:]), u(g[nfull:]), u(beta[nfull:]), ssm_state=pool,
+                             state_indices=torch.tensor([1], dtype=torch.int32, device=DEV), cu_seqlens=cut)
+    return o, entry, pool[1], (k, v, g, beta)
+
+
+def check_row(layer, slot, n, want):
+    o_want, entry, running, (k, v, g, beta) = want
+    row = layer.require_row(slot)
+    assert int(layer.pos[row]) == n
+    assert same_bits(layer.entry_state[row], entry)
+    assert same_bits(layer.ssm_state[row], running)
+    r = n % layer.chunk_size
+    if r:
+        assert same_bits(layer.k_buf[row, :r], k[n - r:n].contiguous()) and same_bits(layer.v_buf[row, :r], v[n - r:n].contiguous())
+        assert same_bits(layer.g_buf[row, :r], g[n - r:n]) and same_bits(layer.b_buf[row, :r], beta[n - r:n])
+
+
+@pytest.mark.parametrize("cuts", [
+    {"prefill": [(0, 37), (1, 16), (2, 5)], "decode_to": 70},          # ends inside, on, and before a boundary
+    {"prefill": [(0, 1), (1, 32), (2, 47)], "decode_to": 50},
+])
+def test_prefill_then_decode_equals_the_one_pass_forward(cuts):
+    layer = make_layer()
+    total = cuts["decode_to"]
+    reqs = {s: request(100 + s, total) for s, _ in cuts["prefill"]}
+    want = {s: one_pass(layer, *reqs[s]) for s in reqs}
+    slots = [s for s, _ in cuts["prefill"]]
+    lens = [n for _, n in cuts["prefill"]]
+    x = torch.cat([reqs[s][0][:n] for s, n in cuts["prefill"]])
+    a = torch.cat([reqs[s][1][:n] for s, n in cuts["prefill"]])
+    b = torch.cat([reqs[s][2][:n] for s, n in cuts["prefill"]])
+    qsl = [0] + list(np.cumsum(lens))
+    o = layer.prefill(torch.tensor(slots, device=DEV), slots, x, a, b, qsl)
+    at = 0
+    for s, n in cuts["prefill"]:
+        assert same_bits(o[at:at + n], want[s][0][:n]), (s, "prefill")
+        at += n
+    have = dict(cuts["prefill"])
+    # decode: all live requests plus one padded lane (an unknown slot id -> the null row)
+    st = torch.tensor(slots + [4000], dtype=torch.int64, device=DEV)
+    step = 0
+    while any(have[s] < total for s in slots):
+        xs = torch.stack([reqs[s][0][min(have[s], total - 1)] for s in slots] + [reqs[slots[0]][0][0]])
+        as_ = torch.stack([reqs[s][1][min(have[s], total - 1)] for s in slots] + [reqs[slots[0]][1][0]])
+        bs = torch.stack([reqs[s][2][min(have[s], total - 1)] for s in slots] + [reqs[slots[0]][2][0]])
+        live = [s for s in slots if have[s] < total]
+        if len(live) < len(slots):  # finished requests drop out of the batch
+            keep = [i for i, s in enumerate(slots) if s in live] + [len(slots)]
+            xs, as_, bs = xs[keep], as_[keep], bs[keep]
+            stt = st[keep]
+        else:
+            stt = st
+        od = layer.decode(stt, xs.contiguous(), as_.contiguous(), bs.contiguous())
+        for i, s in enumerate(live):
+            assert same_bits(od[i], want[s][0][have[s]]), (s, have[s], "decode")
+            have[s] += 1
+        assert not od[len(live)].any()  # the padded lane returns zeros
+        step += 1
+    for s in slots:
+        full = one_pass(layer, *(t[:total] for t in reqs[s]))
+        check_row(layer, s, total, full)
+    assert int(layer.pos[0]) == 0 and not layer._due.any()
+
+
+def test_chunked_prefill_resumes_inside_and_on_boundaries(monkeypatch):
+    monkeypatch.setenv("SKYRL_ISOEXEC_GDN_CHUNKED_PREFILL", "1")
+    layer = make_layer()
+    n = 75
+    req = request(7, n)
+    want = one_pass(layer, *req)
+    slot = 3
+    st = torch.tensor([slot], device=DEV)
+    got = []
+    for lo, hi in ((0, 9), (9, 16), (16, 17), (17, 60), (60, 64), (64, 75)):  # inside, onto, off, across, onto, off
+        got.append(layer.prefill(st, [slot], req[0][lo:hi], req[1][lo:hi], req[2][lo:hi], [0, hi - lo],
+                                 has_initial_state=[lo > 0]))
+        part = one_pass(layer, *(t[:hi] for t in req))
+        check_row(layer, slot, hi, part)
+    assert same_bits(torch.cat(got), want[0])
+    # a reissued slot starts from nothing
+    layer.release_slot(slot)
+    o2 = layer.prefill(st, [slot], req[0][:20], req[1][:20], req[2][:20], [0, 20])
+    assert same_bits(o2, want[0][:20])
+
+
+def test_cpr_state_refuses_engine_owned_tensors():
+    from isoexec_amd.ops.gdn.gdn_cpr_state import CprGDN
+
+    with pytest.raises(ValueError, match="owns its state pool"):
+        CprGDN(capacity=2, chunk_size=16, num_k_heads=H, head_k_dim=K, num_v_heads=HV, head_v_dim=V, device=DEV,
+               ssm_state=torch.zeros(3, HV, V, K, device=DEV), conv_state=torch.zeros(3, D, W - 1, device=DEV), **params())
+
+
+def test_decode_step_replays_from_a_graph_across_boundaries():
+    """The decode step reads nothing on the host (due rows are marked and consumed on the device), so it can be
+    recorded once and replayed: 40 replayed steps, crossing chunk boundaries at different steps per request, against
+    the same steps run eagerly on a twin layer. Every replay is compared, with host work between replays."""
+    eager, graphed = make_layer(), make_layer()
+    slots = [0, 1, 2]
+    lens = [5, 14, 16]
+    total = 60
+    reqs = {s: request(300 + s, total) for s in slots}
+    x = torch.cat([reqs[s][0][:n] for s, n in zip(slots, lens)])
+    a = torch.cat([reqs[s][1][:n] for s, n in zip(slots, lens)])
+    b = torch.cat([reqs[s][2][:n] for s, n in zip(slots, lens)])
+    qsl = [0] + list(np.cumsum(lens))
+    st = torch.tensor(slots, dtype=torch.int64, device=DEV)
+    for layer in (eager, graphed):
+        layer.prefill(st, slots, x, a, b, qsl)
+    have = dict(zip(slots, lens))
+    feed = lambda: tuple(torch.stack([reqs[s][j][have[s]] for s in slots]).contiguous() for j in range(3))
+    # one eager step on both, so every kernel has been launched once before the capture
+    xs, as_, bs = feed()
+    assert same_bits(eager.decode(st, xs, as_, bs), graphed.decode(st, xs.clone(), as_.clone(), bs.clone()))
+    for s in slots:
+        have[s] += 1
+    sx, sa, sb = (t.clone() for t in feed())
+    graphed.flush_slot_map()
+    graph = torch.cuda.CUDAGraph()
+    keep = [t.clone() for t in (graphed.ssm_state, graphed.entry_state, graphed.conv_state, graphed.pos, graphed.k_buf,
+                                graphed.v_buf, graphed.g_buf, graphed.b_buf, graphed.last_used, graphed._clock)]
+    with torch.cuda.graph(graph):
+        out = graphed.decode(st, sx, sa, sb)
+    for t, k in zip((graphed.ssm_state, graphed.entry_state, graphed.conv_state, graphed.pos, graphed.k_buf, graphed.v_buf,
+                     graphed.g_buf, graphed.b_buf, graphed.last_used, graphed._clock), keep):
+        t.copy_(k)  # capture may have run nothing or something: start the replays from the saved state
+    for step in range(40):
+        xs, as_, bs = feed()
+        sx.copy_(xs); sa.copy_(as_); sb.copy_(bs)
+        graph.replay()
+        want = eager.decode(st, xs, as_, bs)
+        torch.cuda.synchronize()
+        assert same_bits(out, want), step
+        for s in slots:
+            have[s] += 1
+    for t, u in ((graphed.ssm_state, eager.ssm_state), (graphed.entry_state, eager.entry_state), (graphed.pos, eager.pos)):
+        assert same_bits(t, u)

@@ -68,6 +68,34 @@ def test_reduced_model_ratio_is_exactly_one():
         assert same_bits(again[j], scored[i])
 
 
+def test_boundary_kernel_ratio_is_exactly_one_too():
+    """The cpr composition (fp32 chain at chunk boundaries, bf16 snapshot as the running state): the engine's
+    prefill + decode out of CprGDN state and the trainer's boundary-form forward are the same function, so the
+    ratio is exactly one -- and it is a different function from the recurrent composition."""
+    import dataclasses
+
+    base = small_config()
+    cfg = dataclasses.replace(base, gdn_kernel="cpr", gdn_chunk=16)
+    prompt_lens, steps = [37, 5, 64, 1, 16], 40   # prompts ending inside, before and exactly on chunk boundaries
+    w, engine, trainer, packed, lens, toks, lps = rollout_then_score(cfg, prompt_lens, steps, seed=0)
+    scored = trainer.response_logprobs(packed, lens, prompt_lens)
+    for i in range(len(lens)):
+        assert same_bits(scored[i], lps[i]), f"sequence {i}"
+    # the graph-replayed decode gives the same tokens and logprobs
+    engine2 = type(engine)(cfg, w, max_num_seqs=len(lens) + 2, max_len=max(prompt_lens) + steps)
+    g = torch.Generator(device=DEV)
+    g.manual_seed(1)
+    prompts = torch.randint(0, cfg.vocab, (sum(prompt_lens),), device=DEV, generator=g)
+    toks2, lps2 = engine2.generate([11 + 3 * i for i in range(len(lens))], prompts, prompt_lens, steps, seed=0, use_graph=True)
+    assert torch.equal(toks2, toks) and same_bits(lps2, lps)
+    # not the recurrent function: scoring the same sequences with the recurrent kernel moves some bits
+    from isoexec_amd.runtimes.hybrid import TrainerModel
+
+    other = TrainerModel(base, w).response_logprobs(packed, lens, prompt_lens)
+    assert any(not same_bits(a, b) for a, b in zip(other, scored))
+    assert max(float((a - b).abs().max()) for a, b in zip(other, scored)) < 0.25
+
+
 def test_rollout_bits_do_not_depend_on_batch_or_chunked_prefill(monkeypatch):
     """The same request decoded alone, inside a batch, and after a prefill cut into chunks."""
     from isoexec_amd.runtimes.hybrid import HybridWeights, RolloutEngine
