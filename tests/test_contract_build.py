@@ -296,8 +296,13 @@ def test_shipped_registry_and_policy_agree():
     assert policy.policy_matches_registry_capabilities(qwen3_5.PROFILE, reg) == []
     full = policy.derive_selections(qwen3_5.PROFILE)
     assert full[("attention.varlen", "engine_decode")].pinned_constants == {"num_splits": 1}
+    # ops absorbed by another op's impl (the fused GatedDeltaNet core; the permutation's block map; the fc1 epilogue
+    # and the single expert-weight buffer of the grouped GEMMs) are registered but get no entry of their own
+    absorbed = ("gdn.l2norm", "gdn.gating", "moe.blockmap", "moe.epilogue", "moe.weights")
     assert ("rope.rope", "trainer_fwd") in full and frozenset(full) == reg.installed_keys() - {
-        (op, s) for op in ("gdn.l2norm", "gdn.gating") for s in ALL}
+        (op, s) for op in absorbed for s in ALL}
+    assert set(reg.ops["moe.dispatch"].impls["hip_bitmask_index"].subsumes) == {"moe.blockmap"}
+    assert set(reg.ops["moe.experts"].impls["hip_grouped_mfma"].subsumes) == {"moe.epilogue", "moe.weights"}
     sels = policy.derive_selections(qwen3_5.PATH_PROFILE)
     assert ("gdn.l2norm", "trainer_fwd") not in sels and ("gdn.state", "trainer_fwd") not in sels
     assert sels[("logprobs.log_softmax", "engine_decode")].pinned_constants == {"leaves": 8, "block": 4096, "accum": "kahan_fp32"}
