@@ -1,42 +1,52 @@
-"""The GatedDeltaNet delta-rule kernel selector: one vocabulary, one default, one parser
-(reference: core/gdn_kernel_env.py:1-56). The declaration site and the read sites must parse
-``SKYRL_ISOEXEC_GDN_KERNEL`` identically, so the parsing lives in one place."""
+"""Which delta-rule kernel the GatedDeltaNet sites run, as named by the environment.
+
+Counterpart of the reference's core/gdn_kernel_env.py:1-56. The declaration side (what the contract pins) and the
+read side (what ``ops/gdn`` dispatches on) both ask this module, so a spelling is interpreted once. An unknown
+spelling is an error and not the default: both runtimes would make the same mistake and then agree with each other.
+"""
 from __future__ import annotations
 
 import os
+from typing import Mapping, Optional
 
 KERNEL_ENV = "SKYRL_ISOEXEC_GDN_KERNEL"
-# Trainer-only ablation override; a run that sets it is not an IsoExec configuration.
-TRAINER_KERNEL_ENV = "SKYRL_ISOEXEC_GDN_TRAINER_KERNEL"
+TRAINER_KERNEL_ENV = "SKYRL_ISOEXEC_GDN_TRAINER_KERNEL"  # ablation switch for the trainer's door only
 
-# "cpr": boundary states per chunk, recurrent inside a chunk. "chunk" (the chunk-parallel form) is in the
-# vocabulary because launch scripts may name it; this library does not serve it and says so when asked.
-KERNELS = ("chunk", "cpr", "recurrent")
+# name -> (served here, what it is)
+_VOCABULARY: Mapping[str, tuple] = {
+    "chunk": (False, "chunk-parallel form; its bits depend on the chunk length"),
+    "cpr": (True, "fp32 chain at chunk boundaries, recurrent inside a chunk"),
+    "recurrent": (True, "token-by-token recurrence"),
+}
+KERNELS = tuple(sorted(_VOCABULARY))
+SERVED_KERNELS = tuple(k for k in KERNELS if _VOCABULARY[k][0])
 DEFAULT_KERNEL = "recurrent"
-SERVED_KERNELS = ("cpr", "recurrent")
-
-_RENAMED = {"chunk_synced": "cpr"}
+_FORMER_NAMES = {"chunk_synced": "cpr"}
 
 
 def parse_gdn_kernel(value, env: str = KERNEL_ENV) -> str:
-    """Normalise one environment value to a kernel name. Unknown names refuse; empty or absent gives the
-    default. A typo that fell back would be the same typo on both runtimes, and they would agree on a wrong
-    composition."""
-    name = (value or "").strip().lower()
-    if not name:
+    """One environment value -> a kernel name; nothing set -> the default; anything else raises."""
+    text = "" if value is None else str(value).strip().lower()
+    if text in _VOCABULARY:
+        return text
+    if not text:
         return DEFAULT_KERNEL
-    if name not in KERNELS:
-        successor = f" {name!r} was renamed to {_RENAMED[name]!r}." if name in _RENAMED else ""
-        raise ValueError(f"{env}={value!r} names no delta-rule kernel; the vocabulary is {list(KERNELS)}.{successor}")
-    return name
+    message = f"{env}={value!r} names no delta-rule kernel; the vocabulary is {list(KERNELS)}."
+    if text in _FORMER_NAMES:
+        message += f" {text!r} was renamed to {_FORMER_NAMES[text]!r}."
+    raise ValueError(message)
+
+
+def _lookup(env: str) -> Optional[str]:
+    raw = os.environ.get(env)
+    return None if raw is None or not raw.strip() else parse_gdn_kernel(raw, env)
 
 
 def gdn_kernel_mode() -> str:
-    """The delta-rule kernel this process runs, read from the environment at call time."""
-    return parse_gdn_kernel(os.environ.get(KERNEL_ENV), KERNEL_ENV)
+    """The kernel of this process, looked up when asked (not at import)."""
+    return _lookup(KERNEL_ENV) or DEFAULT_KERNEL
 
 
-def gdn_trainer_kernel_override():
-    """The trainer-only kernel override, or None when unset (the supported configuration)."""
-    raw = os.environ.get(TRAINER_KERNEL_ENV, "")
-    return parse_gdn_kernel(raw, TRAINER_KERNEL_ENV) if raw.strip() else None
+def gdn_trainer_kernel_override() -> Optional[str]:
+    """The trainer-door override if one is set, else None. A run that sets it is an ablation."""
+    return _lookup(TRAINER_KERNEL_ENV)

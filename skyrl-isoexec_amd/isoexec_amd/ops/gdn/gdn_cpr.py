@@ -35,24 +35,19 @@ def host_meta_enabled() -> bool:
 def host_chunk_meta(lens, chunk_size: int, device, dtype=torch.int32):
     """``(chunk_indices [M, 2] = (sequence, chunk within it), chunk_offsets [N+1] int64)`` for host-known
     lengths (gdn_cpr.py:25-51). Offsets are int64 whatever ``dtype`` is."""
-    key = (tuple(int(x) for x in lens), int(chunk_size), str(device), dtype)
-    hit = _META_CACHE.get(key)
-    if hit is not None:
+    key = (tuple(int(n) for n in lens), int(chunk_size), str(device), dtype)
+    if key in _META_CACHE:
         _META_CACHE.move_to_end(key)
-        return hit
-    nb = np.asarray([-(-int(n) // chunk_size) for n in lens], dtype=np.int64)
-    if nb.size:
-        seq = np.repeat(np.arange(nb.size, dtype=np.int64), nb)
-        first = np.repeat(np.cumsum(nb) - nb, nb)
-        idx_np = np.stack([seq, np.arange(int(nb.sum()), dtype=np.int64) - first], 1)
-        off_np = np.concatenate([[0], np.cumsum(nb)])
-    else:
-        idx_np = np.zeros((0, 2), dtype=np.int64)
-        off_np = np.zeros(1, dtype=np.int64)
-    idx = torch.from_numpy(idx_np).to(device=device, dtype=dtype)
-    off = torch.from_numpy(off_np).to(device=device, dtype=torch.int64)
+        return _META_CACHE[key]
+    pairs, starts = [], [0]
+    for s, n in enumerate(key[0]):
+        count = -(-n // chunk_size)
+        pairs.extend((s, c) for c in range(count))
+        starts.append(starts[-1] + count)
+    idx = torch.tensor(pairs, dtype=dtype, device=device).reshape(-1, 2)
+    off = torch.tensor(starts, dtype=torch.int64, device=device)
     _META_CACHE[key] = (idx, off)
-    if len(_META_CACHE) > _META_CACHE_MAX:
+    while len(_META_CACHE) > _META_CACHE_MAX:
         _META_CACHE.popitem(last=False)
     return idx, off
 
@@ -66,22 +61,18 @@ def chunked_cu_seqlens_and_indices(cu_seqlens: torch.Tensor, chunk_size: int, de
     """Split a packed batch at every chunk boundary: ``(cu_chunked [M+1] int32, state_indices [M, chunk_size]
     int32, n_chunks)`` (gdn_cpr.py:187-213). Only column 0 of the map is set (the chunk's pool row, counted from
     1: row 0 is the null row); the map is full width because the scan indexes it by token."""
-    if lens is None:
-        lens = packed_lens(cu_seqlens)
-    offsets, rows = [0], []
-    row = 1
+    lens = packed_lens(cu_seqlens) if lens is None else lens
+    cuts = [0]
     for n in lens:
-        pos = 0
-        while pos < n:
-            seg = min(chunk_size, n - pos)
-            offsets.append(offsets[-1] + seg)
-            rows.append(row)
-            row += 1
-            pos += seg
-    cu_chunked = torch.tensor(offsets, dtype=torch.int32, device=device)
-    state_indices = torch.zeros(len(rows), chunk_size, dtype=torch.int32, device=device)
-    state_indices[:, 0] = torch.tensor(rows, dtype=torch.int32, device=device)
-    return cu_chunked, state_indices, row - 1
+        n = int(n)
+        whole, rest = divmod(n, chunk_size)
+        for seg in [chunk_size] * whole + ([rest] if rest else []):
+            cuts.append(cuts[-1] + seg)
+    m = len(cuts) - 1
+    state_indices = torch.zeros(m, chunk_size, dtype=torch.int32, device=device)
+    if m:
+        state_indices[:, 0] = torch.arange(1, m + 1, dtype=torch.int32, device=device)
+    return torch.tensor(cuts, dtype=torch.int32, device=device), state_indices, m
 
 
 # Per-forward memo of the above, keyed on the identity and version of cu_seqlens (gdn_cpr.py:54-107).
@@ -99,27 +90,26 @@ def seq_meta_census() -> dict:
 
 
 def sequence_metadata(cu_seqlens: torch.Tensor, chunk_size: int, device):
-    """``(lens, cu_fla, cu_chunked, state_indices, n_chunks)``, memoized while ``cu_seqlens`` is unchanged."""
-    key = None
+    """``(lens, cu_fla, cu_chunked, state_indices, n_chunks)``, memoized while ``cu_seqlens`` is unchanged
+    (same object, same version counter); the memo holds the tensor, so its id cannot be reissued meanwhile."""
+    memo_key = None
     if seq_meta_cache_enabled() and torch.is_tensor(cu_seqlens) and cu_seqlens.numel() <= 8192:
-        key = (id(cu_seqlens), cu_seqlens._version, int(chunk_size), str(cu_seqlens.device))
-    if key is not None:
-        hit = _SEQ_CACHE.get(key)
-        if hit is not None:
-            _SEQ_CACHE.move_to_end(key)
+        memo_key = (id(cu_seqlens), cu_seqlens._version, int(chunk_size), str(cu_seqlens.device))
+        held = _SEQ_CACHE.get(memo_key)
+        if held is not None:
+            _SEQ_CACHE.move_to_end(memo_key)
             _SEQ_STATS["served"] += 1
-            return hit[1]
+            return held[1]
     lens = packed_lens(cu_seqlens)
-    cu_chunked, state_indices, n_chunks = chunked_cu_seqlens_and_indices(cu_seqlens, chunk_size, device, lens=lens)
-    entry = (lens, cu_seqlens.clone(), cu_chunked, state_indices, n_chunks)
-    if key is None:
+    built = (lens, cu_seqlens.clone()) + chunked_cu_seqlens_and_indices(cu_seqlens, chunk_size, device, lens=lens)
+    if memo_key is None:
         _SEQ_STATS["declined"] += 1
-        return entry
-    _SEQ_CACHE[key] = (cu_seqlens, entry)  # the strong reference keeps id() from being reissued
-    _SEQ_STATS["built"] += 1
-    if len(_SEQ_CACHE) > _SEQ_CACHE_MAX:
-        _SEQ_CACHE.popitem(last=False)
-    return entry
+    else:
+        _SEQ_STATS["built"] += 1
+        _SEQ_CACHE[memo_key] = (cu_seqlens, built)
+        while len(_SEQ_CACHE) > _SEQ_CACHE_MAX:
+            _SEQ_CACHE.popitem(last=False)
+    return built
 
 
 def chunk_boundary_states(q, k, v, g, beta, cu_seqlens, chunk_size: int, initial_state=None,
