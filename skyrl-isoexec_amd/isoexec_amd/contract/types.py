@@ -1,155 +1,108 @@
-"""The ExecutionContract record types: immutable data, no I/O, no registry access.
+"""The records an ExecutionContract is made of: immutable data, no I/O, no registry access.
 
-Field names and their order are the wire format (reference: isoexec/contract/types.py:1-132), so a
-contract frozen by the reference decodes here and hashes to the same three identities. Each field
-carries a ``wire`` tag that the codec in ``serialize.py`` interprets; that table is the single description
-of the format, used for encoding, strict decoding and the identity projections alike.
+The records are GENERATED from the schema table below. A record's field names and their order are the wire format
+of the reference (isoexec/contract/types.py:1-132), so a contract frozen there decodes here and hashes to the same
+three identities; the table adds to every field the ``wire`` tag that ``serialize.py`` encodes, strictly decodes and
+projects identities by, which makes the table the one description of the format.
 
-Wire tags:
-    "val"        a JSON scalar (str / int / bool / None), stored as is
-    "strs"       a tuple of scalars, written as a JSON list
-    "map"        sorted (key, value) pairs, written as a JSON object; a BitPattern value is an object
-    "pair"       exactly two strings, written as a two-element list
-    <class>      a nested record
-    [<class>]    a tuple of nested records
-    ?<class>     a nested record or None (spelled ("opt", <class>))
+Wire tags: ``"val"`` a JSON scalar (str, int, bool, None) stored as is; ``"strs"`` a tuple of scalars, a JSON list;
+``"map"`` (key, value) pairs in key order, a JSON object whose values may be BitPattern objects; ``"pair"`` exactly
+two strings; a record class = a nested record; ``[cls]`` = a tuple of records; ``("opt", cls)`` = a record or None.
 """
 
 from __future__ import annotations
 
+import dataclasses
 from collections.abc import Mapping
-from dataclasses import dataclass, field
 
 # Closed vocabularies (reference: contract/types.py:6-14).
-ROUTES = frozenset({"reference_preserving", "composition_defining", "protected", "canonical"})
-DISCHARGE_KINDS = frozenset({"bitwise_equal_to", "equivalence_proof", "neutrality_proof"})
-COVERAGE_KINDS = frozenset({"enumerated_shapes", "symbolic_domain"})
-HALVES = frozenset({"function", "deployment"})
-TOPOLOGY_KINDS = frozenset({"pinned", "invariant"})
-# Only lifecycle events that some boundary observes; anything else would be hashed prose.
-STATE_EVENTS = frozenset({"weight_sync", "sleep_wake"})
+ROUTES = frozenset(("canonical", "composition_defining", "protected", "reference_preserving"))
+HALVES = frozenset(("deployment", "function"))
+DISCHARGE_KINDS = frozenset(("bitwise_equal_to", "equivalence_proof", "neutrality_proof"))
+COVERAGE_KINDS = frozenset(("enumerated_shapes", "symbolic_domain"))
+TOPOLOGY_KINDS = frozenset(("invariant", "pinned"))
+# A lifecycle event belongs here only if some boundary of the system observes it; anything else would be prose
+# that gets hashed.
+STATE_EVENTS = frozenset(("sleep_wake", "weight_sync"))
 
-
-def _w(tag, **kw):
-    return field(metadata={"wire": tag}, **kw)
+_REQUIRED = object()
 
 
 def sorted_pairs(m) -> tuple:
-    """A Mapping or an iterable of pairs -> a tuple of (str key, value) pairs in key order."""
-    items = m.items() if isinstance(m, Mapping) else tuple(m)
-    return tuple(sorted((str(k), v) for k, v in items))
+    """A mapping, or any iterable of pairs, as a tuple of (str key, value) pairs ordered by key."""
+    pairs = m.items() if isinstance(m, Mapping) else m
+    return tuple(sorted(((str(k), v) for k, v in pairs), key=lambda kv: kv[0]))
 
 
-@dataclass(frozen=True)
-class BitPattern:
-    """The only carrier a floating-point constant may travel in: hex bits plus the dtype name."""
-
-    bits: str = _w("val")
-    dtype: str = _w("val")
-
-
-@dataclass(frozen=True)
-class ImplRef:
-    id: str = _w("val")
-    version: int = _w("val")
-    arch: str = _w("val")
-
-
-@dataclass(frozen=True)
-class EquivalenceProof:
-    kind: str = _w("val")
-    ref: str = _w("val")
-
-
-@dataclass(frozen=True)
-class Coverage:
-    kind: str = _w("val")
-    description: str = _w("val")
-
-
-@dataclass(frozen=True)
-class ModelRef:
-    family: str = _w("val")
-    architectures: tuple = _w("strs")
-    profile_ref: str = _w("val")
+def _record(name: str, doc: str, columns, normalise=()):
+    """A frozen dataclass ``name`` with one field per (field name, wire tag, default) column. ``normalise`` names the
+    "map" fields that are put into key order on construction."""
+    specs = []
+    for column in columns:
+        field_name, tag = column[0], column[1]
+        default = column[2] if len(column) > 2 else _REQUIRED
+        options = {"metadata": {"wire": tag}}
+        if default is dataclasses.MISSING or default is _REQUIRED:
+            pass
+        elif callable(default):
+            options["default_factory"] = default
+        else:
+            options["default"] = default
+        specs.append((field_name, object, dataclasses.field(**options)))
+    namespace = {"__doc__": doc}
+    if normalise:
+        def __post_init__(self, _fields=tuple(normalise)):
+            for f in _fields:
+                object.__setattr__(self, f, sorted_pairs(getattr(self, f)))
+        namespace["__post_init__"] = __post_init__
+    cls = dataclasses.make_dataclass(name, specs, frozen=True, namespace=namespace)
+    cls.__module__ = __name__
+    return cls
 
 
-@dataclass(frozen=True)
-class Identities:
-    semantic: str = _w("val")
-    numerical_policy: str = _w("val")
-    deployment: str = _w("val")
+BitPattern = _record("BitPattern", "The only way a floating-point constant travels: its bits in hex and the dtype's name.",
+                     [("bits", "val"), ("dtype", "val")])
 
+ImplRef = _record("ImplRef", "An implementation by id, version and the architecture it was resolved for.",
+                  [("id", "val"), ("version", "val"), ("arch", "val")])
 
-@dataclass(frozen=True)
-class ExecutionCase:
-    id: str = _w("val")
-    runtime_role: str = _w("val")
-    grad_mode: str = _w("val")
-    state_mode: str = _w("val")
-    shape_domain: str = _w("val")
-    constraints: tuple = _w("strs", default=())
+EquivalenceProof = _record("EquivalenceProof", "A discharge: what kind of argument, and where it lives.",
+                           [("kind", "val"), ("ref", "val")])
 
+Coverage = _record("Coverage", "What an entry's claim ranges over.", [("kind", "val"), ("description", "val")])
 
-@dataclass(frozen=True)
-class CompositionEntry:
-    """One partition unit: a sorted group of logical ops run by one impl under a set of cases."""
+ModelRef = _record("ModelRef", "The model the contract was derived for.",
+                   [("family", "val"), ("architectures", "strs"), ("profile_ref", "val")])
 
-    region: tuple = _w("strs")
-    cases: tuple = _w("strs")
-    impl: ImplRef = _w(ImplRef)
-    route: str = _w("val")
-    constants: tuple = _w("map", default=())
-    artifact: str | None = _w("val", default=None)
-    reference: ImplRef | None = _w(("opt", ImplRef), default=None)
-    coverage: Coverage | None = _w(("opt", Coverage), default=None)
-    discharge: EquivalenceProof | None = _w(("opt", EquivalenceProof), default=None)
-    half: str = _w("val", default="function")
+Identities = _record("Identities", "The three hashes of a contract.",
+                     [("semantic", "val"), ("numerical_policy", "val"), ("deployment", "val")])
 
-    def __post_init__(self):
-        object.__setattr__(self, "constants", sorted_pairs(self.constants))
+ExecutionCase = _record("ExecutionCase", "A situation the model runs in (who, with or without gradients, which state, which shapes).",
+                        [("id", "val"), ("runtime_role", "val"), ("grad_mode", "val"), ("state_mode", "val"),
+                         ("shape_domain", "val"), ("constraints", "strs", ())])
 
+CompositionEntry = _record(
+    "CompositionEntry", "One unit of the partition: a sorted group of logical ops that one impl runs under a set of cases.",
+    [("region", "strs"), ("cases", "strs"), ("impl", ImplRef), ("route", "val"), ("constants", "map", ()),
+     ("artifact", "val", None), ("reference", ("opt", ImplRef), None), ("coverage", ("opt", Coverage), None),
+     ("discharge", ("opt", EquivalenceProof), None), ("half", "val", "function")],
+    normalise=("constants",))
 
-@dataclass(frozen=True)
-class TopologyClaim:
-    axis: str = _w("val")
-    kind: str = _w("val")
-    degree: int | None = _w("val", default=None)
-    collective_plan: str | None = _w("val", default=None)
-    domain: tuple = _w("strs", default=())
-    proof: str | None = _w("val", default=None)
+TopologyClaim = _record("TopologyClaim", "A parallelism axis, either pinned to a degree or claimed invariant over a domain.",
+                        [("axis", "val"), ("kind", "val"), ("degree", "val", None), ("collective_plan", "val", None),
+                         ("domain", "strs", ()), ("proof", "val", None)])
 
+StateClaim = _record("StateClaim", "A piece of carried state and the events that invalidate it.",
+                     [("state_id", "val"), ("invalidated_by", "strs"), ("replay_safe", "val"), ("ref", "val")])
 
-@dataclass(frozen=True)
-class StateClaim:
-    state_id: str = _w("val")
-    invalidated_by: tuple = _w("strs")
-    replay_safe: bool = _w("val")
-    ref: str = _w("val")
+ToleranceClaim = _record("ToleranceClaim", "An accepted envelope between two cases; bounds are decimal strings, hashed as written.",
+                         [("case_pair", "pair"), ("bounds", "map", ()), ("attributed_to", "strs", ())],
+                         normalise=("bounds",))
 
+Claims = _record("Claims", "Everything a contract claims beyond its composition.",
+                 [("topology", [TopologyClaim], ()), ("state", [StateClaim], ()), ("tolerances", [ToleranceClaim], ())])
 
-@dataclass(frozen=True)
-class ToleranceClaim:
-    case_pair: tuple = _w("pair")
-    bounds: tuple = _w("map", default=())  # values are decimal strings, hashed as written
-    attributed_to: tuple = _w("strs", default=())
-
-    def __post_init__(self):
-        object.__setattr__(self, "bounds", sorted_pairs(self.bounds))
-
-
-@dataclass(frozen=True)
-class Claims:
-    topology: tuple = _w([TopologyClaim], default=())
-    state: tuple = _w([StateClaim], default=())
-    tolerances: tuple = _w([ToleranceClaim], default=())
-
-
-@dataclass(frozen=True)
-class ExecutionContract:
-    schema_version: str = _w("val")
-    model: ModelRef = _w(ModelRef)
-    identities: Identities = _w(Identities)
-    cases: tuple = _w([ExecutionCase])
-    composition: tuple = _w([CompositionEntry])
-    claims: Claims = _w(Claims, default_factory=Claims)
+ExecutionContract = _record(
+    "ExecutionContract", "The frozen contract.",
+    [("schema_version", "val"), ("model", ModelRef), ("identities", Identities), ("cases", [ExecutionCase]),
+     ("composition", [CompositionEntry]), ("claims", Claims, Claims)])

@@ -1,13 +1,16 @@
-"""Structural invariants of a frozen contract, checked at build time and in CI.
+"""Structural checks on a frozen contract (build time and CI).
 
-Each rule is a generator of human-readable violations; ``validate`` runs all of them and returns the
-list (empty = valid). The rule set follows the reference's (isoexec/contract/validate.py:38-167).
+``validate`` returns every complaint as text, an empty list meaning the contract is well formed. The checks are
+grouped by what they look at -- the header, each entry on its own, who owns which op inside a case, regions served
+by several impls, and the three claim families -- and the rule set is the reference's
+(isoexec/contract/validate.py:35-175).
 """
 
 from __future__ import annotations
 
 import math
 import re
+from collections import defaultdict
 from collections.abc import Mapping
 
 from .identity import compute_identities
@@ -23,186 +26,181 @@ from .types import (
     ExecutionContract,
 )
 
-_HEX_BITS = re.compile(r"^0x[0-9a-fA-F]+$")
-
 
 class ValidationError(Exception):
     pass
 
 
-def _finite_decimal(text) -> bool:
-    # "nan" and "inf" parse as floats and would make a threshold comparison admit everything.
+class _Complaints(list):
+    """Collects complaints; ``unless(ok, text)`` records ``text`` when ``ok`` does not hold."""
+
+    def unless(self, ok, text: str) -> bool:
+        if not ok:
+            self.append(text)
+        return bool(ok)
+
+
+def _is_hex_word(text: str) -> bool:
+    return re.fullmatch(r"0x[0-9a-fA-F]+", text) is not None
+
+
+def _is_finite_number(text) -> bool:
+    """A threshold must compare: "nan" and "inf" parse as numbers and would let everything through."""
     try:
         return math.isfinite(float(text))
     except (TypeError, ValueError):
         return False
 
 
-def _label(entry) -> str:
-    return f"entry {entry.region}@{entry.impl.id}"
+# ---- one entry at a time -------------------------------------------------------------------------------------
+def _entry_shape(out: _Complaints, tag: str, e) -> None:
+    out.unless(len(e.region) > 0, f"{tag}: empty region")
+    out.unless(list(e.region) == sorted(e.region), f"{tag}: region tuple must be sorted")
+    out.unless(e.route in ROUTES, f"{tag}: unknown route {e.route!r}")
+    out.unless(e.half in HALVES, f"{tag}: unknown half {e.half!r}")
+    proof = e.discharge
+    if proof is not None:
+        out.unless(proof.kind in DISCHARGE_KINDS, f"{tag}: unknown discharge kind {proof.kind!r}")
+        out.unless(proof.ref.strip() != "", f"{tag}: {proof.kind} discharge with an empty ref")
+    if e.coverage is not None:
+        out.unless(e.coverage.kind in COVERAGE_KINDS, f"{tag}: unknown coverage kind {e.coverage.kind!r}")
 
 
-def _rule_header(c, case_ids, required):
-    if c.schema_version not in SUPPORTED_SCHEMA_VERSIONS:
-        yield f"unsupported schema_version {c.schema_version!r}"
-    if len(case_ids) != len(c.cases):
-        yield "duplicate case ids"
-    if not c.composition:
-        yield (
-            "empty composition: a contract naming no entry claims nothing, and two processes that both "
-            "failed to derive a composition would agree perfectly"
-        )
+def _entry_obligations(out: _Complaints, tag: str, e) -> None:
+    """What a route or a half obliges an entry to carry."""
+    if e.route == "composition_defining":
+        out.unless(e.artifact is not None, f"{tag}: composition_defining requires an artifact")
+    if e.route == "reference_preserving":
+        out.unless(e.reference is not None, f"{tag}: reference_preserving requires a reference")
+    if e.half == "deployment":
+        neutral = e.discharge is not None and e.discharge.kind == "neutrality_proof"
+        out.unless(neutral, f"{tag}: deployment-half entry requires a neutrality_proof discharge")
 
 
-def _rule_entries(c, case_ids, required):
-    claimed = set()
-    for e in c.composition:
-        who = _label(e)
-        if not e.region:
-            yield f"{who}: empty region"
-        if tuple(sorted(e.region)) != tuple(e.region):
-            yield f"{who}: region tuple must be sorted"
-        if e.route not in ROUTES:
-            yield f"{who}: unknown route {e.route!r}"
-        if e.half not in HALVES:
-            yield f"{who}: unknown half {e.half!r}"
-        if e.discharge is not None:
-            if e.discharge.kind not in DISCHARGE_KINDS:
-                yield f"{who}: unknown discharge kind {e.discharge.kind!r}"
-            if not e.discharge.ref.strip():
-                yield f"{who}: {e.discharge.kind} discharge with an empty ref"
-        if e.coverage is not None and e.coverage.kind not in COVERAGE_KINDS:
-            yield f"{who}: unknown coverage kind {e.coverage.kind!r}"
-        for cid in e.cases:
-            if cid not in case_ids:
-                yield f"{who}: unknown case {cid!r}"
-            if (e.region, cid) in claimed:
-                yield f"{who}: duplicate (region, case) claim for {cid!r}"
-            claimed.add((e.region, cid))
-        if e.route == "composition_defining" and e.artifact is None:
-            yield f"{who}: composition_defining requires an artifact"
-        if e.route == "reference_preserving" and e.reference is None:
-            yield f"{who}: reference_preserving requires a reference"
-        if e.half == "deployment" and (e.discharge is None or e.discharge.kind != "neutrality_proof"):
-            yield f"{who}: deployment-half entry requires a neutrality_proof discharge"
-        for key, const in e.constants:
-            if isinstance(const, float):
-                yield f"{who}: constant {key!r} is a raw float"
-            if isinstance(const, BitPattern) and not _HEX_BITS.match(const.bits):
-                yield f"{who}: constant {key!r} has invalid bit pattern {const.bits!r}"
+def _entry_constants(out: _Complaints, tag: str, e) -> None:
+    for name, value in e.constants:
+        out.unless(not isinstance(value, float), f"{tag}: constant {name!r} is a raw float")
+        if isinstance(value, BitPattern):
+            out.unless(_is_hex_word(value.bits), f"{tag}: constant {name!r} has invalid bit pattern {value.bits!r}")
 
 
-def _rule_ownership(c, case_ids, required):
-    # Within one case a logical op belongs to at most one region; required ops must all be owned.
-    for cid in case_ids:
+def _entries(out: _Complaints, contract, case_ids) -> None:
+    claims = set()
+    for e in contract.composition:
+        tag = f"entry {e.region}@{e.impl.id}"
+        _entry_shape(out, tag, e)
+        for case in e.cases:
+            out.unless(case in case_ids, f"{tag}: unknown case {case!r}")
+            out.unless((e.region, case) not in claims, f"{tag}: duplicate (region, case) claim for {case!r}")
+            claims.add((e.region, case))
+        _entry_obligations(out, tag, e)
+        _entry_constants(out, tag, e)
+
+
+# ---- across entries ------------------------------------------------------------------------------------------
+def _ownership(out: _Complaints, contract, case_ids, required) -> None:
+    """Inside one case an op has one owning region, and every op the case needs has an owner."""
+    for case in case_ids:
         owner = {}
-        for e in c.composition:
-            if cid not in e.cases:
-                continue
-            for op in e.region:
-                if op in owner and owner[op] != e.region:
-                    yield f"case {cid!r}: op {op!r} owned by both {owner[op]} and {e.region}"
-                owner[op] = e.region
-        if required is not None and cid in required:
-            uncovered = required[cid] - set(owner)
-            if uncovered:
-                yield f"case {cid!r}: uncovered required op(s) {sorted(uncovered)}"
+        for e in contract.composition:
+            if case in e.cases:
+                for op in e.region:
+                    prior = owner.setdefault(op, e.region)
+                    out.unless(prior == e.region, f"case {case!r}: op {op!r} owned by both {prior} and {e.region}")
+                    owner[op] = e.region
+        needed = (required or {}).get(case)
+        if needed is not None:
+            orphans = sorted(set(needed) - owner.keys())
+            out.unless(not orphans, f"case {case!r}: uncovered required op(s) {orphans}")
 
 
-def _rule_asymmetry(c, case_ids, required):
-    # One region run by different impls under different cases: every such entry carries its proof.
-    impls_of = {}
-    for e in c.composition:
-        impls_of.setdefault(e.region, []).append(e)
-    for region, group in impls_of.items():
-        if len({e.impl.id for e in group}) > 1:
-            for e in group:
-                if e.discharge is None:
-                    yield f"entry {region}@{e.impl.id}: asymmetric region requires a discharge"
+def _asymmetry(out: _Complaints, contract) -> None:
+    """A region that different cases run with different impls owes a discharge on every one of its entries."""
+    by_region = defaultdict(list)
+    for e in contract.composition:
+        by_region[e.region].append(e)
+    for region, group in by_region.items():
+        if len({e.impl.id for e in group}) < 2:
+            continue
+        for e in group:
+            out.unless(e.discharge is not None, f"entry {region}@{e.impl.id}: asymmetric region requires a discharge")
 
 
-def _rule_tolerances(c, case_ids, required):
-    for t in c.claims.tolerances:
-        for cid in t.case_pair:
-            if cid not in case_ids:
-                yield f"tolerance {t.case_pair}: unknown case {cid!r}"
-        if not t.bounds:
-            yield f"tolerance {t.case_pair}: no bounds (an envelope with no threshold admits everything)"
-        for key, bound in t.bounds:
-            if not _finite_decimal(bound):
-                yield f"tolerance {t.case_pair}: bound {key}={bound!r} is not a finite threshold"
+# ---- claims --------------------------------------------------------------------------------------------------
+def _tolerances(out: _Complaints, contract, case_ids) -> None:
+    for t in contract.claims.tolerances:
+        tag = f"tolerance {t.case_pair}"
+        for case in t.case_pair:
+            out.unless(case in case_ids, f"{tag}: unknown case {case!r}")
+        out.unless(len(t.bounds) > 0, f"{tag}: no bounds (an envelope without a threshold admits everything)")
+        for name, bound in t.bounds:
+            out.unless(_is_finite_number(bound), f"{tag}: bound {name}={bound!r} is not a finite threshold")
 
 
-def _rule_state(c, case_ids, required):
-    for s in c.claims.state:
-        if not s.ref.strip():
-            yield f"state {s.state_id!r}: empty ref (the claim names no implementing hook)"
-        if not s.invalidated_by:
-            yield f"state {s.state_id!r}: empty invalidated_by (a state invalidated by nothing is not a claim)"
-        stray = sorted(set(s.invalidated_by) - STATE_EVENTS)
-        if stray:
-            yield (
-                f"state {s.state_id!r}: unknown lifecycle event(s) {stray}; the vocabulary is "
-                f"{sorted(STATE_EVENTS)} -- an event no boundary observes cannot be enforced"
-            )
+def _state_claims(out: _Complaints, contract) -> None:
+    for s in contract.claims.state:
+        tag = f"state {s.state_id!r}"
+        out.unless(s.ref.strip() != "", f"{tag}: empty ref (no hook is named that implements the claim)")
+        out.unless(len(s.invalidated_by) > 0, f"{tag}: empty invalidated_by (nothing ever invalidates this state?)")
+        unknown = sorted(set(s.invalidated_by) - STATE_EVENTS)
+        out.unless(not unknown, f"{tag}: unknown lifecycle event(s) {unknown}; the vocabulary is {sorted(STATE_EVENTS)} "
+                                f"(an event no boundary observes cannot be enforced)")
 
 
-def _rule_topology(c, case_ids, required):
-    axes = [t.axis for t in c.claims.topology]
-    if len(axes) != len(set(axes)):
-        yield "duplicate topology axes"
-    for t in c.claims.topology:
-        if t.proof is not None and not t.proof.strip():
-            yield f"topology {t.axis!r}: empty proof ref (a proof that names nothing is not a proof)"
-        if t.kind not in TOPOLOGY_KINDS:
-            yield f"topology {t.axis!r}: unknown kind {t.kind!r}"
-        elif t.kind == "pinned":
-            if t.degree is None or t.collective_plan is None:
-                yield f"topology {t.axis!r}: pinned requires degree and collective_plan"
-            elif t.degree < 1:
-                yield f"topology {t.axis!r}: pinned degree {t.degree} is not a deployable degree (>= 1)"
-        elif not t.domain or not t.proof:
-            yield f"topology {t.axis!r}: invariant requires a non-empty domain and a proof"
-        elif len(set(t.domain)) < 2:
-            yield (
-                f"topology {t.axis!r}: invariant over the single degree {sorted(set(t.domain))} is a "
-                f"tautology, not an invariance claim; pin the axis instead"
-            )
-
-
-def _rule_identities(c, case_ids, required):
-    try:
-        fresh = compute_identities(c)
-    except SerializationError as exc:
-        yield f"identity recomputation failed: {exc}"
+def _one_topology_claim(out: _Complaints, t) -> None:
+    tag = f"topology {t.axis!r}"
+    if t.proof is not None:
+        out.unless(t.proof.strip() != "", f"{tag}: empty proof ref (it names nothing)")
+    if not out.unless(t.kind in TOPOLOGY_KINDS, f"{tag}: unknown kind {t.kind!r}"):
         return
-    if c.identities != fresh:
-        yield "stored identities do not match recomputed identities"
+    if t.kind == "pinned":
+        if out.unless(t.degree is not None and t.collective_plan is not None,
+                      f"{tag}: pinned requires degree and collective_plan"):
+            out.unless(t.degree >= 1, f"{tag}: pinned degree {t.degree} is not a deployable degree (>= 1)")
+        return
+    if out.unless(bool(t.domain) and bool(t.proof), f"{tag}: invariant requires a non-empty domain and a proof"):
+        degrees = sorted(set(t.domain))
+        out.unless(len(degrees) >= 2, f"{tag}: invariant over the single degree {degrees} is a tautology, not an "
+                                      f"invariance claim; pin the axis instead")
 
 
-_RULES = (
-    _rule_header,
-    _rule_entries,
-    _rule_ownership,
-    _rule_asymmetry,
-    _rule_tolerances,
-    _rule_state,
-    _rule_topology,
-    _rule_identities,
-)
+def _topology(out: _Complaints, contract) -> None:
+    axes = [t.axis for t in contract.claims.topology]
+    out.unless(len(set(axes)) == len(axes), "duplicate topology axes")
+    for t in contract.claims.topology:
+        _one_topology_claim(out, t)
+
+
+def _identities(out: _Complaints, contract) -> None:
+    try:
+        recomputed = compute_identities(contract)
+    except SerializationError as exc:
+        out.append(f"identity recomputation failed: {exc}")
+        return
+    out.unless(contract.identities == recomputed, "stored identities do not match recomputed identities")
 
 
 def validate(contract: ExecutionContract, required_ops: Mapping | None = None) -> list:
-    """Every violation of the structural rules, as text. ``required_ops`` maps a case id to the set
-    of logical ops that case must have an owner for."""
+    """Every complaint about ``contract``, as text. ``required_ops`` maps a case id to the ops that case must
+    have an owner for."""
+    out = _Complaints()
     case_ids = {c.id for c in contract.cases}
-    found = []
-    for rule in _RULES:
-        found.extend(rule(contract, case_ids, required_ops))
-    return found
+    out.unless(contract.schema_version in SUPPORTED_SCHEMA_VERSIONS, f"unsupported schema_version {contract.schema_version!r}")
+    out.unless(len(case_ids) == len(contract.cases), "duplicate case ids")
+    out.unless(len(contract.composition) > 0,
+               "empty composition: a contract with no entry claims nothing, and two processes that both failed to "
+               "derive a composition would then agree perfectly")
+    _entries(out, contract, case_ids)
+    _ownership(out, contract, case_ids, required_ops)
+    _asymmetry(out, contract)
+    _tolerances(out, contract, case_ids)
+    _state_claims(out, contract)
+    _topology(out, contract)
+    _identities(out, contract)
+    return list(out)
 
 
 def validate_or_raise(contract: ExecutionContract, required_ops: Mapping | None = None) -> None:
-    problems = validate(contract, required_ops)
-    if problems:
-        raise ValidationError("; ".join(problems))
+    complaints = validate(contract, required_ops)
+    if complaints:
+        raise ValidationError("; ".join(complaints))

@@ -1,70 +1,81 @@
-"""Resolve the references a claim names (a state hook, a proof gate) to code that exists in the tree.
+"""Does a reference written into a claim point at something that exists?
 
-Reference: isoexec/core/claim_refs.py:19-76. Paths are containment-checked so a ``../`` reference
-cannot reach outside the package, and symbols are found by parsing rather than by text search.
-Gates are the parity tests: the package's own ``ops/*/tests`` and the repository's ``tests`` folder.
+Two kinds of reference appear in a contract: ``file.py::symbol`` for the hook that implements a state claim, and a
+proof pointer for an invariance or equivalence claim, which names a gate (a parity test) either by file or by a word
+that occurs in a gate. Files are looked up inside this package only (a path that climbs out of it is refused), and a
+symbol counts only if the file defines it at module level -- a mention in a comment does not. Gates are the
+package's ``ops/*/tests`` and the repository's ``tests`` folder. (Reference: isoexec/core/claim_refs.py:19-76.)
 """
 
 from __future__ import annotations
 
 import ast
-import pathlib
+from pathlib import Path
+from typing import Dict, Optional
 
-PACKAGE_DIR = pathlib.Path(__file__).resolve().parents[1]
-_GATE_GLOBS = ((PACKAGE_DIR, "ops/*/tests/*.py"), (PACKAGE_DIR.parents[1], "tests/*.py"))
-_gate_text: dict | None = None
+PACKAGE_DIR = Path(__file__).resolve().parent.parent
+_REPO_DIR = PACKAGE_DIR.parent.parent
 
 
-def _inside_package(path: str):
+class _GateIndex:
+    """Path and text of every gate file, read on first use."""
+
+    where = ((PACKAGE_DIR, "ops/*/tests/*.py"), (_REPO_DIR, "tests/*.py"))
+
+    def __init__(self):
+        self._files: Optional[Dict[str, str]] = None
+
+    def mentions(self, word: str) -> bool:
+        if self._files is None:
+            self._files = {}
+            for base, pattern in self.where:
+                for f in sorted(base.glob(pattern)):
+                    self._files[f.relative_to(base).as_posix()] = f.read_text(errors="replace")
+        return any(word in name or word in text for name, text in self._files.items())
+
+
+_gates = _GateIndex()
+
+
+def _package_file(relative: str) -> Optional[Path]:
+    """``relative`` as a path under the package, or None if it leaves the package or cannot be resolved."""
     try:
-        full = (PACKAGE_DIR / path).resolve()
-        full.relative_to(PACKAGE_DIR)
-        return full
-    except (ValueError, OSError):
+        candidate = (PACKAGE_DIR / relative).resolve()
+    except OSError:
         return None
+    return candidate if PACKAGE_DIR in candidate.parents or candidate == PACKAGE_DIR else None
 
 
-def _top_level_names(source: str) -> set:
+def _module_level_definitions(path: Path) -> set:
     try:
-        body = ast.parse(source).body
+        module = ast.parse(path.read_text(errors="replace"))
     except SyntaxError:
         return set()
-    return {n.name for n in body if isinstance(n, (ast.FunctionDef, ast.AsyncFunctionDef, ast.ClassDef))}
+    kinds = (ast.FunctionDef, ast.AsyncFunctionDef, ast.ClassDef)
+    return {node.name for node in module.body if isinstance(node, kinds)}
 
 
-def hook_ref_problem(ref: str):
-    """Why ``path::symbol`` names no code in this package, or None when it does."""
-    path, _, symbol = ref.partition("::")
-    target = _inside_package(path)
-    if target is None:
-        return f"ref path {path!r} escapes the package, so it names no code this tree ships"
-    if not target.is_file():
-        return f"ref file {path!r} missing"
-    if symbol not in _top_level_names(target.read_text(errors="replace")):
-        return f"hook {symbol!r} not defined in {path}"
-    return None
+def hook_ref_problem(ref: str) -> Optional[str]:
+    """None if ``path::symbol`` names a definition in this package, else what is wrong with it."""
+    relative, _sep, symbol = ref.partition("::")
+    path = _package_file(relative)
+    if path is None:
+        return f"ref path {relative!r} escapes the package, so it names no code this tree ships"
+    if not path.is_file():
+        return f"ref file {relative!r} missing"
+    if symbol in _module_level_definitions(path):
+        return None
+    return f"hook {symbol!r} not defined in {relative}"
 
 
-def _gates() -> dict:
-    global _gate_text
-    if _gate_text is None:
-        _gate_text = {}
-        for root, pattern in _GATE_GLOBS:
-            for p in sorted(root.glob(pattern)):
-                _gate_text[str(p.relative_to(root))] = p.read_text(errors="replace")
-    return _gate_text
-
-
-def proof_ref_problem(ref: str):
-    """Why a proof pointer resolves to no gate, or None when it does. The pointer is a path inside
-    the package, or ``"<gate name>: <what it shows>"`` where the name appears in a gate's path or text."""
-    words = ref.strip().split(":")[0].split()
-    if not words:
+def proof_ref_problem(ref: str) -> Optional[str]:
+    """None if the pointer resolves to a gate, else why not. A pointer is a file path inside the package, or
+    ``"<gate word>: <what the gate shows>"``; only the first word before the colon is looked up."""
+    head = ref.strip().partition(":")[0].split()
+    if not head:
         return "empty proof ref"
-    name = words[0]
-    target = _inside_package(name)
-    if target is not None and target.is_file():
+    word = head[0]
+    path = _package_file(word)
+    if (path is not None and path.is_file()) or _gates.mentions(word):
         return None
-    if any(name in path or name in text for path, text in _gates().items()):
-        return None
-    return f"proof ref {ref!r} resolves to no gate: {name!r} names no file and appears in no test source"
+    return f"proof ref {ref!r} resolves to no gate: {word!r} names no file and appears in no test source"

@@ -1,7 +1,7 @@
-"""The per-process contract: built once from the registry and the model's selections, then compared.
+"""This process's contract: derived once from the registry and the model declaration, kept for the life of the
+process, and compared with the peer's by hash (a disagreement is a refusal to run).
 
-Reference: isoexec/core/process_contract.py:17-226. Both runtimes build the same contract at start-up;
-``assert_contract_agreement`` turns a disagreement into a refusal to run.
+Reference: isoexec/core/process_contract.py:17-226.
 """
 
 from __future__ import annotations
@@ -14,92 +14,94 @@ import struct
 
 logger = logging.getLogger(__name__)
 
+
+# What the process holds once the contract exists, and the named digests (name -> callable) of components outside
+# the op registry that both sides must also agree on.
 _CONTRACT = None
 _VIEW = None
-# Named components outside the model registry that must also agree across the pair. With none
-# registered the handshake hash is the numerical_policy identity itself.
 _EXTENSIONS: dict = {}
 
 
 def register_contract_extension(name: str, digest_fn) -> None:
-    """Fold ``digest_fn() -> str`` into the handshake hash; it is evaluated at every hash read."""
+    """Make ``digest_fn()`` part of the handshake hash. It is called every time the hash is read."""
     _EXTENSIONS[name] = digest_fn
 
 
 def composite_hash(base):
+    """``base`` folded with every registered extension's digest (``base`` itself when there are none)."""
     if base is None or not _EXTENSIONS:
         return base
-    folded = {}
-    for name in sorted(_EXTENSIONS):
+    digests = {}
+    for name, fn in sorted(_EXTENSIONS.items()):
         try:
-            folded[name] = str(_EXTENSIONS[name]())
-        except Exception as exc:  # noqa: BLE001 -- a broken extension must not fake agreement
-            folded[name] = f"EXTENSION-ERROR:{type(exc).__name__}"
-    text = json.dumps({"base": base, "extensions": folded}, sort_keys=True, separators=(",", ":"))
-    return hashlib.sha256(text.encode("utf-8")).hexdigest()
+            digests[name] = str(fn())
+        except Exception as exc:  # noqa: BLE001 -- a failing extension must never look like agreement
+            digests[name] = "EXTENSION-ERROR:" + type(exc).__name__
+    blob = json.dumps({"base": base, "extensions": digests}, sort_keys=True, separators=(",", ":")).encode("utf-8")
+    return hashlib.sha256(blob).hexdigest()
 
 
-def _plain_constant(value):
-    # Floats travel as fp64 bit patterns; the fingerprint compares plain values.
+def _as_plain_value(constant):
+    """A contract stores a float as the bit pattern of its fp64; the installed-state comparison wants the number."""
     from ..contract import BitPattern
 
-    if isinstance(value, BitPattern) and value.dtype == "fp64":
-        return struct.unpack("<d", struct.pack("<Q", int(value.bits, 16)))[0]
-    return value
+    if isinstance(constant, BitPattern) and constant.dtype == "fp64":
+        (number,) = struct.unpack("<d", struct.pack("<Q", int(constant.bits, 16)))
+        return number
+    return constant
 
 
 def build_contract_view(contract, registry) -> dict:
-    """``{(op, site): {impl_id, version, pinned_constants, half}}`` for the fingerprint comparison."""
+    """The contract flattened to ``{(op, site): {impl_id, version, pinned_constants, half}}``, the shape the
+    installed-state fingerprint is compared in."""
     from .contract_delivery import primary_op
 
-    view = {}
+    flat = {}
     for entry in contract.composition:
-        op = primary_op(registry, entry)
-        row = {
-            "impl_id": entry.impl.id,
-            "version": entry.impl.version,
-            "pinned_constants": {k: _plain_constant(v) for k, v in entry.constants},
-            "half": entry.half,
-        }
-        for case in entry.cases:
-            view[(op, case)] = dict(row)
-    return view
+        owner = primary_op(registry, entry)
+        constants = {name: _as_plain_value(value) for name, value in entry.constants}
+        for site in entry.cases:
+            flat[(owner, site)] = {"impl_id": entry.impl.id, "version": entry.impl.version,
+                                   "pinned_constants": dict(constants), "half": entry.half}
+    return flat
+
+
+def _publish(contract) -> None:
+    """Write the artifact where ``ISOEXEC_CONTRACT_PATH`` says, if it says anything; failure is logged, not fatal."""
+    where = os.environ.get("ISOEXEC_CONTRACT_PATH")
+    if not where:
+        return
+    try:
+        from .contract_delivery import write_contract_file
+
+        write_contract_file(contract, where)
+    except Exception as exc:  # noqa: BLE001
+        logger.warning("[ISOEXEC-CONTRACT] artifact write to %s skipped: %s", where, exc)
 
 
 def get_process_contract(model_path=None, *, arch=None):
-    """Build (once) and return this process's contract; None when none exists and no model is named.
-    With ``ISOEXEC_CONTRACT_PATH`` set, the first build also writes the canonical artifact there."""
+    """The process's contract, building it on the first call that names a model (None before that)."""
     global _CONTRACT, _VIEW
-    if _CONTRACT is not None:
+    if _CONTRACT is not None or not model_path:
         return _CONTRACT
-    if not model_path:
-        return None
     from .. import models
     from . import enforce
     from .registry_build import build_registry
 
+    obligation = f"{enforce.BUILD_VALID}:contract"
     registry = build_registry(strict=False)
     try:
         contract = models.build_for(model_path, registry, arch=arch)
     except Exception as exc:
-        enforce.report(f"{enforce.BUILD_VALID}:contract", enforce.INSTALL, enforce.VIOLATION, f"{type(exc).__name__}: {exc}")
+        enforce.report(obligation, enforce.INSTALL, enforce.VIOLATION, f"{type(exc).__name__}: {exc}")
         raise
     _CONTRACT, _VIEW = contract, build_contract_view(contract, registry)
     ids = contract.identities
-    enforce.report(f"{enforce.BUILD_VALID}:contract", enforce.INSTALL, enforce.OK, f"numerical_policy={ids.numerical_policy}")
-    logger.info(
-        "[ISOEXEC-CONTRACT] model=%s arch=%s numerical_policy=%s semantic=%s deployment=%s entries=%d",
-        contract.model.family, contract.composition[0].impl.arch, ids.numerical_policy, ids.semantic,
-        ids.deployment, len(contract.composition),
-    )
-    path = os.environ.get("ISOEXEC_CONTRACT_PATH")
-    if path:
-        try:
-            from .contract_delivery import write_contract_file
-
-            write_contract_file(contract, path)
-        except Exception as exc:  # noqa: BLE001 -- the artifact is best-effort
-            logger.warning("[ISOEXEC-CONTRACT] artifact write to %s skipped: %s", path, exc)
+    enforce.report(obligation, enforce.INSTALL, enforce.OK, f"numerical_policy={ids.numerical_policy}")
+    logger.info("[ISOEXEC-CONTRACT] model=%s arch=%s numerical_policy=%s semantic=%s deployment=%s entries=%d",
+                contract.model.family, contract.composition[0].impl.arch, ids.numerical_policy, ids.semantic,
+                ids.deployment, len(contract.composition))
+    _publish(contract)
     return contract
 
 
@@ -118,41 +120,44 @@ def _reset_for_tests() -> None:
 
 
 def contract_hash(model_path=None):
-    """The handshake hash: numerical_policy folded with the registered extensions."""
+    """What the two sides exchange: the numerical-policy identity folded with the extensions."""
     contract = get_process_contract(model_path)
-    return None if contract is None else composite_hash(contract.identities.numerical_policy)
+    if contract is None:
+        return None
+    return composite_hash(contract.identities.numerical_policy)
 
 
 def assert_contract_agreement(other_hash: str, *, other_side: str = "peer") -> bool:
-    """The peer's handshake hash must equal ours. A mismatch is recorded and refuses unless demoted."""
+    """Compare the peer's hash with ours. Equal: recorded as met. Different: recorded as a violation and refused
+    (unless enforcement is demoted). No local contract yet: recorded as skipped."""
     from . import enforce
 
-    oid = f"{enforce.HANDSHAKE}:numerical_policy"
-    ours = contract_hash()
-    if ours is None:
-        enforce.report(oid, enforce.WEIGHT_SYNC, enforce.SKIPPED, f"{enforce.SKIP_NO_LOCAL_CONTRACT}: local contract not built")
+    obligation = f"{enforce.HANDSHAKE}:numerical_policy"
+    mine = contract_hash()
+    if mine is None:
+        enforce.report(obligation, enforce.WEIGHT_SYNC, enforce.SKIPPED,
+                       f"{enforce.SKIP_NO_LOCAL_CONTRACT}: local contract not built")
         return True
-    if other_hash == ours:
-        enforce.report(oid, enforce.WEIGHT_SYNC, enforce.OK, f"MATCH hash={ours} ({other_side})")
+    if mine == other_hash:
+        enforce.report(obligation, enforce.WEIGHT_SYNC, enforce.OK, f"MATCH hash={mine} ({other_side})")
         return True
-    msg = (
-        f"[ISOEXEC-CONTRACT-HANDSHAKE] MISMATCH: local={ours} {other_side}={other_hash}. The two runtimes "
-        "resolved different numerical policies; running on would compare outputs of different functions."
-    )
-    enforce.report(oid, enforce.WEIGHT_SYNC, enforce.VIOLATION, msg)
-    return enforce.refuse(msg)
+    complaint = (f"[ISOEXEC-CONTRACT-HANDSHAKE] MISMATCH: local={mine} {other_side}={other_hash}. The two runtimes "
+                 "resolved different numerical policies; carrying on would compare the outputs of two functions.")
+    enforce.report(obligation, enforce.WEIGHT_SYNC, enforce.VIOLATION, complaint)
+    return enforce.refuse(complaint)
 
 
 def assert_init_info_contract(init_info, *, other_side: str = "trainer") -> bool:
-    """Receiver side: compare against the hash a peer stamped on ``init_info.contract_hash``."""
+    """The receiving side of the handshake: the peer's hash arrives as ``init_info.contract_hash``."""
     from . import enforce
 
-    oid = f"{enforce.HANDSHAKE}:numerical_policy"
-    stamped = getattr(init_info, "contract_hash", None)
-    if stamped is None:
-        enforce.report(oid, enforce.WEIGHT_SYNC, enforce.SKIPPED, f"{enforce.SKIP_NO_PEER_STAMP}: {other_side} stamped no contract_hash")
-        return True
-    if contract_hash() is None:
-        enforce.report(oid, enforce.WEIGHT_SYNC, enforce.SKIPPED, f"{enforce.SKIP_NO_LOCAL_CONTRACT}: local contract not built")
-        return True
-    return assert_contract_agreement(stamped, other_side=other_side)
+    obligation = f"{enforce.HANDSHAKE}:numerical_policy"
+    theirs = getattr(init_info, "contract_hash", None)
+    if theirs is None:
+        reason = f"{enforce.SKIP_NO_PEER_STAMP}: {other_side} stamped no contract_hash"
+    elif contract_hash() is None:
+        reason = f"{enforce.SKIP_NO_LOCAL_CONTRACT}: local contract not built"
+    else:
+        return assert_contract_agreement(theirs, other_side=other_side)
+    enforce.report(obligation, enforce.WEIGHT_SYNC, enforce.SKIPPED, reason)
+    return True

@@ -1,8 +1,10 @@
-"""Ops, implementations and their rounding schedules: the table a model's selections resolve against.
+"""The table of ops and their implementations that a model's selections are resolved against.
 
-Reference: isoexec/core/registry.py:14-247. An op's identity is its rounding schedule. Sites and
-hazards come from closed vocabularies; there is no layer dimension (an op resolves identically at
-every layer).
+An implementation is identified by WHAT IT COMPUTES, written down as a rounding schedule; an op lists the execution
+sites it exists at (a site it does not list does not exist for it -- nothing is defaulted); hazards are the
+situations an implementation's parity tests promise to exercise. Sites, hazards and routes are closed vocabularies.
+There is no per-layer dimension: an op resolves the same way at every layer.
+(Reference: isoexec/core/registry.py:14-247.)
 """
 
 from __future__ import annotations
@@ -10,32 +12,30 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Callable, Dict, List, Optional, Sequence
 
-# Execution sites. A site an op does not list does not exist for it; there is no default.
-_BASE_SITES = frozenset({"trainer_fwd", "trainer_score", "engine_prefill", "engine_decode"})
-
-# What a parity test may claim to exercise (and must then show it did).
-HAZARDS = frozenset(
-    {
-        "null_lanes",        # padded / inert lanes under graph replay
-        "t_zero",            # an empty sequence
-        "non_contiguous",    # strided inputs
-        "e_mismatch",        # expert count differs from the expected one
-        "profiling_shapes",  # shapes the engine profiles at start-up
-        "tie_boundaries",    # ties in top-k
-        "subnormals",        # denormal inputs on flush-to-zero paths
-        "signed_zero",       # +0.0 versus -0.0
-    }
-)
-
-_ROUTES = frozenset({"reference_preserving", "composition_defining", "protected", "canonical"})
-
 
 class RegistryError(ValueError):
     pass
 
 
+# ---- vocabularies --------------------------------------------------------------------------------------------
+_BASE_SITES = frozenset(("trainer_fwd", "trainer_score", "engine_prefill", "engine_decode"))
+_ROUTES = frozenset(("reference_preserving", "composition_defining", "protected", "canonical"))
+_HAZARD_NOTES = {
+    "null_lanes": "padded lanes that must stay inert when a graph is replayed",
+    "t_zero": "a sequence with no tokens",
+    "non_contiguous": "inputs that are strided views",
+    "e_mismatch": "an expert count other than the expected one",
+    "profiling_shapes": "the shapes an engine probes at start-up",
+    "tie_boundaries": "equal scores in a top-k",
+    "subnormals": "denormal inputs where a path flushes to zero",
+    "signed_zero": "the sign of a zero",
+}
+HAZARDS = frozenset(_HAZARD_NOTES)
+
+
+# ---- values a schedule may hold ------------------------------------------------------------------------------
 class _PerModel:
-    """Marks a schedule key whose value is a fact of the model, supplied by the pin itself."""
+    """Placeholder for a schedule value that is a fact of the model: the pin supplies it."""
 
     __slots__ = ()
 
@@ -47,20 +47,19 @@ PER_MODEL = _PerModel()
 
 
 def pin_values_equal(a, b) -> bool:
-    """Equality between a declared schedule value and a pin: a list equals the same tuple (JSON turns
-    one into the other), and a bool never equals an int."""
-    if isinstance(a, bool) != isinstance(b, bool):
-        return False
-    seq = (list, tuple)
-    if isinstance(a, seq) and isinstance(b, seq):
-        return len(a) == len(b) and all(map(pin_values_equal, a, b))
+    """Do a declared value and a pinned value agree? Lists and tuples compare by content (a round trip through
+    JSON turns one into the other), mappings key by key, and True is not 1."""
+    if isinstance(a, bool) or isinstance(b, bool):
+        return isinstance(a, bool) and isinstance(b, bool) and a == b
+    if isinstance(a, (list, tuple)) and isinstance(b, (list, tuple)):
+        return len(a) == len(b) and all(pin_values_equal(x, y) for x, y in zip(a, b))
     if isinstance(a, dict) and isinstance(b, dict):
-        return a.keys() == b.keys() and all(pin_values_equal(a[k], b[k]) for k in a)
+        return set(a) == set(b) and all(pin_values_equal(a[k], b[k]) for k in a)
     return a == b
 
 
 class OneOf:
-    """A schedule value restricted to an enumerated set."""
+    """A schedule value that may be any one of the listed alternatives."""
 
     __slots__ = ("values",)
 
@@ -68,41 +67,47 @@ class OneOf:
         self.values = tuple(values)
 
     def __contains__(self, candidate) -> bool:
-        return any(pin_values_equal(v, candidate) for v in self.values)
+        for allowed in self.values:
+            if pin_values_equal(allowed, candidate):
+                return True
+        return False
 
     def __repr__(self) -> str:
-        return f"OneOf{self.values!r}"
+        return "OneOf" + repr(self.values)
 
 
 @dataclass(frozen=True)
 class RoundingSchedule:
-    """What an impl computes, as data. ``machine_assertable`` holds literals, ``PER_MODEL`` or
-    ``OneOf``; its keys are exactly the pins the impl accepts. Changing either half is a new version."""
+    """What an implementation computes. ``machine_assertable`` maps a key to a literal, ``PER_MODEL`` or a
+    ``OneOf``; these keys are also the only pins the implementation accepts. ``documentary`` is prose. A change to
+    either is a new version of the implementation."""
 
     machine_assertable: Dict[str, object] = field(default_factory=dict)
     documentary: str = ""
 
     def check_pin(self, key: str, value) -> Optional[str]:
-        """None when the pin is consistent with the schedule, else the reason it is not. A key the
-        schedule never declared refuses: such a pin would hash and match while constraining nothing."""
-        if key not in self.machine_assertable:
-            known = sorted(str(k) for k in self.machine_assertable)
-            return (
-                f"the impl's machine_assertable rounding schedule declares no such key (declared: {known}). "
-                "A pin the impl never declared constrains nothing -- declare it (a literal, PER_MODEL, "
-                "or OneOf(...)) or drop the pin."
-            )
-        declared = self.machine_assertable[key]
+        """Why pinning ``key`` to ``value`` contradicts this schedule, or None if it does not. Pinning a key the
+        schedule does not have is refused too: it would be hashed and compared while constraining nothing."""
+        try:
+            declared = self.machine_assertable[key]
+        except KeyError:
+            have = sorted(map(str, self.machine_assertable))
+            return (f"the impl's machine_assertable rounding schedule declares no such key (declared: {have}). "
+                    "A pin the impl never declared constrains nothing -- declare it (a literal, PER_MODEL, or "
+                    "OneOf(...)) or drop the pin.")
         if declared is PER_MODEL:
             return None
-        fits = (value in declared) if isinstance(declared, OneOf) else pin_values_equal(declared, value)
-        return None if fits else f"the impl declares {key}={declared!r}"
+        if isinstance(declared, OneOf):
+            agrees = value in declared
+        else:
+            agrees = pin_values_equal(declared, value)
+        return None if agrees else f"the impl declares {key}={declared!r}"
 
 
 @dataclass(frozen=True)
 class StateInvalidation:
-    """When a stateful op's state must be rebound; ``hook(state, ctx) -> bool`` is the host-only
-    check (True while the state is still valid)."""
+    """For an op that keeps state: the condition under which the state has to be rebound, and optionally a
+    host-side ``hook(state, ctx) -> bool`` that is True while the state is still good."""
 
     condition: str
     hook: Optional[Callable[..., bool]] = None
@@ -110,8 +115,8 @@ class StateInvalidation:
 
 @dataclass(frozen=True)
 class ImplSpec:
-    """One implementation of an op at a pinned version. ``subsumes`` lists the ops it absorbs;
-    ``hazards`` is the floor its parity tests exercise."""
+    """An implementation of an op at one version. ``subsumes``: ops it absorbs (they then install nothing of their
+    own). ``hazards``: the least its parity tests exercise."""
 
     impl_id: str
     version: int
@@ -124,16 +129,14 @@ class ImplSpec:
     route: str = "protected"
 
     def __post_init__(self) -> None:
+        me = f"impl {self.impl_id!r}"
         if self.route not in _ROUTES:
-            raise RegistryError(f"impl {self.impl_id!r} declares unknown route {self.route!r}")
-        stray = set(self.hazards) - HAZARDS
-        if stray:
-            raise RegistryError(
-                f"impl {self.impl_id!r} declares unknown hazard(s) {sorted(stray)}; the hazard "
-                f"vocabulary is {sorted(HAZARDS)}"
-            )
-        if not self.supported_archs:
-            raise RegistryError(f"impl {self.impl_id!r} must declare at least one supported arch")
+            raise RegistryError(f"{me} declares unknown route {self.route!r}")
+        unknown = sorted(set(self.hazards).difference(HAZARDS))
+        if unknown:
+            raise RegistryError(f"{me} declares unknown hazard(s) {unknown}; the hazard vocabulary is {sorted(HAZARDS)}")
+        if len(self.supported_archs) == 0:
+            raise RegistryError(f"{me} must declare at least one supported arch")
 
 
 @dataclass
@@ -144,60 +147,62 @@ class OpSpec:
     per_layer_uniform: bool = True
 
     def add_impl(self, impl: ImplSpec) -> "OpSpec":
-        if impl.impl_id in self.impls:
+        """Chainable. One impl id, one impl."""
+        if self.impls.setdefault(impl.impl_id, impl) is not impl:
             raise RegistryError(f"op {self.name!r} already has impl {impl.impl_id!r}")
-        self.impls[impl.impl_id] = impl
         return self
 
 
 class Registry:
-    def __init__(self) -> None:
-        self._sites = set(_BASE_SITES)
-        self._ops: Dict[str, OpSpec] = {}
+    """Ops by name, plus the site vocabulary (which a deployment may extend before registering ops)."""
 
+    def __init__(self) -> None:
+        self._ops: Dict[str, OpSpec] = {}
+        self._sites = set(_BASE_SITES)
+
+    # -- sites
     @property
     def sites(self) -> frozenset:
         return frozenset(self._sites)
 
-    @property
-    def ops(self) -> Dict[str, OpSpec]:
-        return dict(self._ops)
-
     def register_site(self, name: str) -> None:
-        if not name or not name.replace("_", "").isalnum():
+        looks_like_identifier = bool(name) and name.replace("_", "").isalnum()
+        if not looks_like_identifier:
             raise RegistryError(f"invalid site name {name!r}: must be a non-empty identifier")
         self._sites.add(name)
 
-    def register_op(self, op: OpSpec) -> OpSpec:
-        if op.name in self._ops:
-            raise RegistryError(f"op {op.name!r} already registered")
-        stray = set(op.sites) - self._sites
-        if stray:
-            raise RegistryError(
-                f"op {op.name!r} declares unknown site(s) {sorted(stray)}; register them first via "
-                f"register_site(). Known sites: {sorted(self._sites)}"
-            )
-        self._ops[op.name] = op
-        return op
+    # -- ops
+    @property
+    def ops(self) -> Dict[str, OpSpec]:
+        return dict(self._ops)
 
     def has_op(self, name: str) -> bool:
         return name in self._ops
 
     def get_op(self, name: str) -> OpSpec:
-        try:
-            return self._ops[name]
-        except KeyError:
-            raise RegistryError(f"unknown op {name!r}") from None
+        if name not in self._ops:
+            raise RegistryError(f"unknown op {name!r}")
+        return self._ops[name]
+
+    def register_op(self, op: OpSpec) -> OpSpec:
+        if self.has_op(op.name):
+            raise RegistryError(f"op {op.name!r} already registered")
+        unknown = sorted(set(op.sites).difference(self._sites))
+        if unknown:
+            raise RegistryError(f"op {op.name!r} declares unknown site(s) {unknown}; register them first via "
+                                f"register_site(). Known sites: {sorted(self._sites)}")
+        self._ops[op.name] = op
+        return op
 
     def installed_keys(self) -> frozenset:
-        return frozenset((op.name, site) for op in self._ops.values() for site in op.sites)
+        """Every (op, site) pair that exists."""
+        return frozenset((name, site) for name, op in self._ops.items() for site in op.sites)
 
     def assert_subsumption_closed(self) -> None:
-        for op in self._ops.values():
-            for impl in op.impls.values():
-                for absorbed in impl.subsumes:
-                    if absorbed not in self._ops:
-                        raise RegistryError(
-                            f"impl {op.name}:{impl.impl_id} subsumes unregistered op {absorbed!r}; "
-                            f"its passthrough cannot be derived"
-                        )
+        """An absorbed op must itself be registered, or nothing can say what was absorbed."""
+        for name, op in self._ops.items():
+            for impl_id, impl in op.impls.items():
+                missing = [a for a in impl.subsumes if a not in self._ops]
+                if missing:
+                    raise RegistryError(f"impl {name}:{impl_id} subsumes unregistered op {missing[0]!r}; its "
+                                        f"passthrough cannot be derived")
