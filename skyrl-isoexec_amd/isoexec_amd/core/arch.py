@@ -1,9 +1,10 @@
-"""The architecture tag: one dimension of every implementation's identity (``impl@version x arch``).
+"""The architecture tag.
 
-Reference: isoexec/core/arch.py:14-88. Kernel bit patterns are arch-specific, so the tag is written
-into every contract entry, and a trainer/engine pair on different tags refuses to run. On this
-library's target the tag is ``gfx950`` (the leading component of ``gcnArchName``); a host with no
-visible accelerator gets the sentinel ``cpu``, which the contract builder refuses to key on.
+Kernels give different bits on different architectures, so the tag is part of what an implementation IS
+(``impl@version`` on an arch): every contract entry carries it, and a trainer and an engine that report different
+tags refuse to pair up -- no claim is ever made across architectures. On the hardware this library targets the tag is
+``gfx950``, the first component of the device's ``gcnArchName``; a process that sees no accelerator gets the
+sentinel ``cpu``, which the contract builder will not accept as a key. (Reference: isoexec/core/arch.py:14-88.)
 """
 
 from __future__ import annotations
@@ -13,64 +14,68 @@ from dataclasses import dataclass
 NON_ACCELERATOR_ARCH: str = "cpu"
 
 
+class ArchMismatchError(RuntimeError):
+    """Raised when the two sides of a handshake are on different architectures."""
+
+
 def is_accelerator_arch(arch: str) -> bool:
-    """True when ``arch`` names a real accelerator: non-empty and not the sentinel."""
-    return bool(arch) and arch != NON_ACCELERATOR_ARCH
+    """Is ``arch`` the tag of a real accelerator (neither empty nor the sentinel)?"""
+    return arch not in ("", None, NON_ACCELERATOR_ARCH)
 
 
 def _tag_from_gcn_name(name: str) -> str:
-    # "gfx950:sramecc+:xnack-" -> "gfx950". Feature suffixes do not change kernel bit patterns.
-    return name.split(":", 1)[0].strip()
+    """``gfx950:sramecc+:xnack-`` -> ``gfx950``: the feature flags after the colon do not change what a kernel
+    computes."""
+    head, _colon, _flags = name.partition(":")
+    return head.strip()
+
+
+def _visible_device():
+    """The torch module if it can see an accelerator, else None. Any failure up to and including the visibility
+    question means "no accelerator"."""
+    try:
+        import torch
+
+        return torch if torch.cuda.is_available() else None
+    except Exception:
+        return None
 
 
 def detect_arch() -> str:
-    """The visible accelerator's tag, or the sentinel when none is visible.
-
-    Once the runtime reports a device, failing to read its name is a detection bug and propagates:
-    collapsing it to the sentinel would be baked into a contract identity.
-    """
-    try:
-        import torch
-    except Exception:
+    """The tag of the accelerator this process sees, else the sentinel. Once a device IS visible, failing to read
+    its name is a bug and is allowed to propagate: quietly answering ``cpu`` would end up inside a contract."""
+    torch = _visible_device()
+    if torch is None:
         return NON_ACCELERATOR_ARCH
-    try:
-        if not torch.cuda.is_available():
-            return NON_ACCELERATOR_ARCH
-    except Exception:
-        return NON_ACCELERATOR_ARCH
-    props = torch.cuda.get_device_properties(torch.cuda.current_device())
-    name = getattr(props, "gcnArchName", "") or ""
-    if name:
-        return _tag_from_gcn_name(name)
-    major, minor = torch.cuda.get_device_capability()
-    return f"sm{major}{minor}"
+    properties = torch.cuda.get_device_properties(torch.cuda.current_device())
+    gcn_name = getattr(properties, "gcnArchName", None)
+    if gcn_name:
+        return _tag_from_gcn_name(gcn_name)
+    return "sm%d%d" % tuple(torch.cuda.get_device_capability())
 
 
 ARCH: str = detect_arch()
 
 
-class ArchMismatchError(RuntimeError):
-    """The two runtimes report different arch tags; no cross-arch bitwise claim is ever made."""
+def assert_homogeneous(arch_a: str, arch_b: str) -> None:
+    if arch_a == arch_b:
+        return
+    raise ArchMismatchError(f"arch handshake failed: this side is {arch_a!r}, other side is {arch_b!r}; trainer and "
+                            f"engine must run the same architecture.")
 
 
 @dataclass(frozen=True)
 class HardwareTarget:
+    """An architecture, with the two questions asked of it."""
+
     arch: str
 
     @classmethod
     def current(cls) -> "HardwareTarget":
-        return cls(arch=ARCH)
+        return cls(ARCH)
 
     def supports(self, supported_archs) -> bool:
-        return self.arch in set(supported_archs)
+        return any(self.arch == a for a in supported_archs)
 
     def assert_homogeneous(self, other_arch: str) -> None:
         assert_homogeneous(self.arch, other_arch)
-
-
-def assert_homogeneous(arch_a: str, arch_b: str) -> None:
-    if arch_a != arch_b:
-        raise ArchMismatchError(
-            f"arch handshake failed: this side is {arch_a!r}, other side is {arch_b!r}; trainer and "
-            f"engine must run the same architecture."
-        )

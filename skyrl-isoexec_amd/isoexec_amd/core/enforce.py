@@ -1,9 +1,9 @@
-"""The obligation ledger: every agreement check reports here, and refusals funnel through ``refuse``.
+"""The ledger of obligations. Every agreement check in this package files its verdict here, and every refusal to
+run goes through ``refuse``, so that one switch decides whether a violation stops the process or is only recorded.
 
-A reduced form of the reference's enforcement module (isoexec/core/enforce.py:25-62, 252-410): the
-phase and result vocabularies, an append-only ledger of (obligation, phase, result, evidence)
-records, and the strict / demoted switch. The plan derivation and verdict artifacts of the reference
-belong to its trainer/engine installers and are not part of this path.
+This is the part of the reference's enforcement module that the contract path needs (isoexec/core/enforce.py:25-62,
+252-410): the vocabularies of phases and results, an append-only list of (obligation, phase, result, evidence), and
+the strict/demoted switch. Its plan derivation and verdict files serve the reference's installers and are not here.
 """
 
 from __future__ import annotations
@@ -11,19 +11,24 @@ from __future__ import annotations
 import logging
 import os
 from dataclasses import dataclass
-from typing import Dict, List, Tuple
+from typing import Dict, List, Optional, Tuple
 
 logger = logging.getLogger(__name__)
 
-INSTALL, FIRST_FORWARD, WEIGHT_SYNC, STEP1 = "INSTALL", "FIRST_FORWARD", "WEIGHT_SYNC", "STEP1"
+# when a verdict is filed
+INSTALL = "INSTALL"
+FIRST_FORWARD = "FIRST_FORWARD"
+WEIGHT_SYNC = "WEIGHT_SYNC"
+STEP1 = "STEP1"
 PHASES = (INSTALL, FIRST_FORWARD, WEIGHT_SYNC, STEP1)
 
-BUILD_VALID = "build_valid"
-INSTALL_ATTEST = "install_attest"
-FINGERPRINT = "fingerprint"
-HANDSHAKE = "handshake"
+# what the verdict is about (prefix of an obligation id)
+BUILD_VALID, INSTALL_ATTEST, FINGERPRINT, HANDSHAKE = "build_valid", "install_attest", "fingerprint", "handshake"
 
-OK, VIOLATION, SKIPPED = "ok", "violation", "skipped"
+# the verdict, least to most severe
+OK, SKIPPED, VIOLATION = "ok", "skipped", "violation"
+_SEVERITY = {OK: 0, SKIPPED: 1, VIOLATION: 2}
+# the reasons a check may be skipped for
 SKIP_NO_PEER_STAMP = "no-peer-stamp"
 SKIP_NO_LOCAL_CONTRACT = "no-local-contract"
 RECOGNIZED_SKIPS = (SKIP_NO_PEER_STAMP, SKIP_NO_LOCAL_CONTRACT)
@@ -38,31 +43,31 @@ class Record:
 
 
 class ObligationLedger:
+    """Append-only."""
+
     def __init__(self) -> None:
         self.records: List[Record] = []
 
     def report(self, obligation_id: str, phase: str, result: str, evidence: str = "") -> None:
-        if phase not in PHASES:
-            raise ValueError(f"unknown phase {phase!r}")
-        if result not in (OK, VIOLATION, SKIPPED):
-            raise ValueError(f"unknown result {result!r}")
+        for what, value, allowed in (("phase", phase, PHASES), ("result", result, _SEVERITY)):
+            if value not in allowed:
+                raise ValueError(f"unknown {what} {value!r}")
         self.records.append(Record(obligation_id, phase, result, evidence))
 
     def status(self) -> Dict[Tuple[str, str], str]:
-        """Worst result per (obligation, phase): a violation is never overwritten by a later ok."""
-        rank = {OK: 0, SKIPPED: 1, VIOLATION: 2}
-        out: Dict[Tuple[str, str], str] = {}
-        for r in self.records:
-            key = (r.obligation_id, r.phase)
-            if key not in out or rank[r.result] > rank[out[key]]:
-                out[key] = r.result
-        return out
+        """The most severe result filed for each (obligation, phase): a later ``ok`` never hides a violation."""
+        worst: Dict[Tuple[str, str], str] = {}
+        for record in self.records:
+            slot = (record.obligation_id, record.phase)
+            if _SEVERITY[record.result] > _SEVERITY.get(worst.get(slot), -1):
+                worst[slot] = record.result
+        return worst
 
     def violations(self) -> List[Record]:
-        return [r for r in self.records if r.result == VIOLATION]
+        return [record for record in self.records if record.result == VIOLATION]
 
 
-_LEDGER: ObligationLedger | None = None
+_LEDGER: Optional[ObligationLedger] = None
 
 
 def ledger() -> ObligationLedger:
@@ -76,23 +81,27 @@ def _reset_for_tests() -> None:
     global _LEDGER
     _LEDGER = None
     try:
-        from .fingerprint import _ATTESTED
+        from . import fingerprint
 
-        _ATTESTED.clear()
+        fingerprint._ATTESTED.clear()
     except Exception:  # noqa: BLE001
         pass
 
 
 def report(obligation_id: str, phase: str, result: str, evidence: str = "") -> None:
-    """Record one verdict. Fail-safe: a reporting bug never breaks the check it wraps."""
+    """File one verdict. A bug in filing must not break the check that files, so nothing escapes from here."""
     try:
         ledger().report(obligation_id, phase, result, evidence)
     except Exception as exc:  # noqa: BLE001
         logger.warning("[ISOEXEC-ENFORCE] report(%s, %s, %s) skipped: %s", obligation_id, phase, result, exc)
 
 
+def _flag(name: str, default: str) -> bool:
+    return os.environ.get(name, default).lower() not in ("", "0", "false", "no")
+
+
 def _strict() -> bool:
-    return os.environ.get("SKYRL_ISOEXEC_MANIFEST_STRICT", "1").lower() not in ("", "0", "false", "no")
+    return _flag("SKYRL_ISOEXEC_MANIFEST_STRICT", "1")
 
 
 def debug_demoted() -> bool:
@@ -100,14 +109,14 @@ def debug_demoted() -> bool:
 
 
 def demoted() -> bool:
-    """True when a refusal logs and continues instead of raising."""
-    return not _strict() or debug_demoted()
+    """When True a refusal is logged and the run goes on."""
+    return debug_demoted() or not _strict()
 
 
 def refuse(msg: str) -> bool:
-    """Raise ``msg`` as the refusal, or log it and return False when demoted. The ledger entry that
-    preceded the call stays red either way."""
-    if demoted():
-        logger.error("%s (demoted: violation recorded, run continues)", msg)
-        return False
-    raise RuntimeError(msg)
+    """Stop the run with ``msg`` -- or, when demoted, log it and return False. Either way the violation that was
+    filed before calling this stays in the ledger."""
+    if not demoted():
+        raise RuntimeError(msg)
+    logger.error("%s (demoted: violation recorded, run continues)", msg)
+    return False
