@@ -82,8 +82,8 @@ class RoundingSchedule:
     ``OneOf``; these keys are also the only pins the implementation accepts. ``documentary`` is prose. A change to
     either is a new version of the implementation."""
 
-    machine_assertable: Dict[str, object] = field(default_factory=dict)
-    documentary: str = ""
+    machine_assertable: "dict[str, object]" = field(default_factory=dict)
+    documentary: str = ""           # prose; hashed with the rest
 
     def check_pin(self, key: str, value) -> Optional[str]:
         """Why pinning ``key`` to ``value`` contradicts this schedule, or None if it does not. Pinning a key the
@@ -109,8 +109,8 @@ class StateInvalidation:
     """For an op that keeps state: the condition under which the state has to be rebound, and optionally a
     host-side ``hook(state, ctx) -> bool`` that is True while the state is still good."""
 
-    condition: str
-    hook: Optional[Callable[..., bool]] = None
+    condition: str                                  # in words
+    hook: "Callable[..., bool] | None" = None       # host-side check, optional
 
 
 @dataclass(frozen=True)
@@ -118,15 +118,15 @@ class ImplSpec:
     """An implementation of an op at one version. ``subsumes``: ops it absorbs (they then install nothing of their
     own). ``hazards``: the least its parity tests exercise."""
 
-    impl_id: str
-    version: int
-    supported_archs: frozenset
-    rounding: RoundingSchedule = field(default_factory=RoundingSchedule)
-    capabilities: Dict[str, object] = field(default_factory=dict)
-    subsumes: Sequence[str] = ()
-    state_invalidation: Optional[StateInvalidation] = None
-    hazards: Sequence[str] = ()
-    route: str = "protected"
+    impl_id: str                    # unique within its op
+    version: int                    # bumped whenever the rounding schedule changes
+    supported_archs: frozenset      # architecture tags the bits were established on
+    rounding: "RoundingSchedule" = field(default_factory=lambda: RoundingSchedule())
+    capabilities: "dict[str, object]" = field(default_factory=dict)
+    subsumes: "tuple[str, ...]" = ()
+    state_invalidation: "StateInvalidation | None" = None
+    hazards: "tuple[str, ...]" = ()
+    route: str = "protected"        # one of _ROUTES
 
     def __post_init__(self) -> None:
         me = f"impl {self.impl_id!r}"
@@ -141,10 +141,10 @@ class ImplSpec:
 
 @dataclass
 class OpSpec:
-    name: str
-    sites: List[str]
-    impls: Dict[str, ImplSpec] = field(default_factory=dict)
-    per_layer_uniform: bool = True
+    name: str                                   # "family.op"
+    sites: "list[str]"                          # where the op exists
+    impls: "dict[str, ImplSpec]" = field(default_factory=dict)
+    per_layer_uniform: bool = True              # resolved once, for every layer
 
     def add_impl(self, impl: ImplSpec) -> "OpSpec":
         """Chainable. One impl id, one impl."""
@@ -157,7 +157,7 @@ class Registry:
     """Ops by name, plus the site vocabulary (which a deployment may extend before registering ops)."""
 
     def __init__(self) -> None:
-        self._ops: Dict[str, OpSpec] = {}
+        self._ops: "dict[str, OpSpec]" = dict()
         self._sites = set(_BASE_SITES)
 
     # -- sites
@@ -173,8 +173,9 @@ class Registry:
 
     # -- ops
     @property
-    def ops(self) -> Dict[str, OpSpec]:
-        return dict(self._ops)
+    def ops(self) -> "dict[str, OpSpec]":
+        """A copy: registering goes through ``register_op``."""
+        return {name: op for name, op in self._ops.items()}
 
     def has_op(self, name: str) -> bool:
         return name in self._ops
