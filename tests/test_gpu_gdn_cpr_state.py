@@ -199,3 +199,47 @@ def test_decode_step_replays_from_a_graph_across_boundaries():
             have[s] += 1
     for t, u in ((graphed.ssm_state, eager.ssm_state), (graphed.entry_state, eager.entry_state), (graphed.pos, eager.pos)):
         assert same_bits(t, u)
+
+
+def test_wide_heads_take_the_lane_pair_scan_in_the_boundary_pass():
+    """K = V = 128 and a pool of more than 128 rows: the state-only boundary scan over the buffer pool then runs in
+    the lane-pair layout (every row that is not due a null lane). Same check as above: prefill, decode across
+    boundaries, against the one-pass forward."""
+    from isoexec_amd.ops.gdn.gdn_cpr import gdn_cpr_fwd
+    from isoexec_amd.ops.gdn.gdn_cpr_state import CprGDN
+    from isoexec_amd.ops.gdn.gdn_ops import conv_packed
+
+    h, k_, hv, v_, w_, c_ = 2, 128, 4, 128, 4, 16
+    d = 2 * h * k_ + hv * v_
+    g = cpu_gen(41)
+    bf = lambda t: t.to(torch.bfloat16).to(DEV)
+    layer = CprGDN(capacity=140, chunk_size=c_, num_k_heads=h, head_k_dim=k_, num_v_heads=hv, head_v_dim=v_, device=DEV,
+                   conv_weight=bf(torch.randn(d, w_, generator=g) * 0.4), conv_bias=bf(torch.randn(d, generator=g) * 0.1),
+                   A_log=(torch.randn(hv, generator=g) * 0.3).to(DEV), dt_bias=(torch.randn(hv, generator=g) * 0.3).to(DEV))
+    total, lens, slots = 40, [13, 16, 30], [5, 6, 7]
+    reqs = [(bf(torch.randn(total, d, generator=g)), bf(torch.randn(total, hv, generator=g)), bf(torch.randn(total, hv, generator=g)))
+            for _ in slots]
+    want = []
+    for x, a, b in reqs:
+        cu = torch.tensor([0, total], dtype=torch.int32, device=DEV)
+        y = conv_packed(x, layer.conv_weight, layer.conv_bias, cu_seqlens=cu)
+        q, k, v = layer._split_qkv(y)
+        gate, beta = layer._gate_and_beta(a, b)
+        u = lambda t: t.unsqueeze(0)
+        want.append(gdn_cpr_fwd(u(q), u(k), u(v), u(gate), u(beta), cu_seqlens=cu, chunk_size=c_)[0])
+    st = torch.tensor(slots, dtype=torch.int64, device=DEV)
+    cat = lambda j: torch.cat([r[j][:n] for r, n in zip(reqs, lens)])
+    o = layer.prefill(st, slots, cat(0), cat(1), cat(2), [0] + list(np.cumsum(lens)))
+    at = 0
+    for i, n in enumerate(lens):
+        assert same_bits(o[at:at + n], want[i][:n])
+        at += n
+    have = list(lens)
+    while min(have) < total:
+        live = [i for i in range(3) if have[i] < total]
+        pick = lambda j: torch.stack([reqs[i][j][have[i]] for i in live]).contiguous()
+        od = layer.decode(st[live], pick(0), pick(1), pick(2))
+        for row, i in enumerate(live):
+            assert same_bits(od[row], want[i][have[i]]), (i, have[i])
+            have[i] += 1
+    assert not layer._due.any()
