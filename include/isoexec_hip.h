@@ -133,8 +133,10 @@ int ix_gemm_f32_nt(const void* A, int a_dtype, long lda, const void* W, long ldw
  * the sequence. stride 0 is the compact form: state_indices [N] holds one row per sequence, loaded
  * before its first token and stored once after its last. HV % H == 0 (GQA: head hv reads q/k
  * head hv / (HV/H)). K in {32,64,128,256}.
- * time_tile: bits 0-7 = tokens staged per LDS fill (<= 64, 0 = default); bits 8.. = state rows held per
- * lane group (1, 2 or 4; 0 = chosen from the grid size). Neither changes results. */
+ * time_tile: bits 0-7 = tokens staged per LDS fill (<= 64, 0 = default; 1 also tells the launcher that every
+ * sequence has one token, a decode step); bits 8.. = the layout: state rows held per group of 16 lanes (1, 2 or 4),
+ * or 16 for the lane-pair layout (K = 128, compact state form, V % 128 == 0; declined otherwise); 0 = chosen from the
+ * grid size. Neither changes results. */
 int ix_gdn_scan(const void* q, const void* k, const void* v, const float* g, const void* beta, void* o,
                 int io_dtype, long q_pitch, long k_pitch, long v_pitch, float* state_pool,
                 const int* cu_seqlens, const int* state_indices, long state_indices_stride, long N, long H,
