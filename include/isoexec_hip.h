@@ -250,6 +250,32 @@ int ix_moe_experts(const void* x, long ldx, const int* sorted_token, const float
 int ix_moe_combine(const void* expert_out, const int* combine_rows, void* out, long T, long Hd, long k,
                    int fp32_acc, void* stream);
 
+/* ---- order-invariant digests: debug/thash ------------------------------------------------- */
+
+#define IX_DIGEST_MAX_MASKS 8
+
+/* The weighted modular sums behind tensor_digest / digest_ladder (thash.py:180-217,251-301; the kernel
+ * thash_kernels.py:49-90): out[j] = SUM_i (sext(x_i) & masks[j]) * w(i) mod 2^64 for j < nmask <= 8, with
+ * w(i) = (mix64((i >> 3) ^ salt) ^ ((i & 7) * 0x9E3779B97F4A7C15)) | 1 and mix64 the splitmix64 finaliser.
+ * x = n integers of elem_bytes (1, 2, 4 or 8) each, read as signed; masks = nmask values in HOST memory, read
+ * during the call; out = nmask words in device memory; workspace = device words, at least
+ * ix_digest_workspace_words(1, n, nmask) of them (may be NULL when that is 0). All nmask sums come from one
+ * pass over x. n = 0 gives zeros. */
+int ix_digest_sums(const void* x, int elem_bytes, long n, uint64_t salt, const uint64_t* masks, int nmask,
+                   uint64_t* workspace, size_t workspace_words, uint64_t* out, void* stream);
+
+/* The per-segment sums behind segment_digests (thash.py:319-354; thash_kernels.py:93-104): x is cut into nseg
+ * runs of seg_numel elements (the last may be short; nseg = ceil(n / seg_numel)); out[s] is the sum above over
+ * run s alone, positions counted from the run's start, with
+ * salt_s = mix64(seed ^ mix64(s * seg_numel + 1)) ^ 0x9E3779B97F4A7C15. One launch covers every segment.
+ * workspace as above with ix_digest_workspace_words(nseg, seg_numel, 1). */
+int ix_digest_segment_sums(const void* x, int elem_bytes, long n, long nseg, long seg_numel, uint64_t seed,
+                           uint64_t mask, uint64_t* workspace, size_t workspace_words, uint64_t* out,
+                           void* stream);
+
+/* Host arithmetic only: device words of workspace the two calls above need (0 = none). */
+size_t ix_digest_workspace_words(long nseg, long seg_numel, int nmask);
+
 #ifdef __cplusplus
 }
 #endif

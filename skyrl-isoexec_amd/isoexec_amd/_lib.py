@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_float, c_int, c_long, c_size_t, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_long, c_size_t, c_uint64, c_void_p
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC_DIR = os.path.normpath(os.path.join(_PKG_DIR, "..", "csrc"))
@@ -82,6 +82,9 @@ SIGNATURES = {
         [P, c_long, P, P, P, P, P, c_long, c_long, P, P, c_long, c_long, c_long, c_long, P],
     ),
     "ix_moe_combine": (c_int, [P, P, P, c_long, c_long, c_long, c_int, P]),
+    "ix_digest_sums": (c_int, [P, c_int, c_long, c_uint64, P, c_int, P, c_size_t, P, P]),
+    "ix_digest_segment_sums": (c_int, [P, c_int, c_long, c_long, c_long, c_uint64, c_uint64, P, c_size_t, P, P]),
+    "ix_digest_workspace_words": (c_size_t, [c_long, c_long, c_int]),
 }
 
 _LIB = None
