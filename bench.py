@@ -5,7 +5,7 @@ Default workload (``dense_head``, BASELINE.json configs[1]): M = 4096 hidden sta
 log-softmax + target gather. One step = one pass over the 4096 tokens; inputs are resident in HBM
 before the timed region. Prints ONE JSON line.
 
-Other workloads (``--workload gdn_decode | moe | hybrid``) time configs[2], configs[3] and configs[4] with
+Other workloads (``--workload gdn_decode | moe | hybrid | attention | digest``) time configs[2], configs[3] and configs[4] with
 the same contract; they are extra lines for profiling, not the headline.
 """
 
@@ -369,12 +369,73 @@ def hybrid(args):
                         "graph_decode_tokens_per_s": n / t_graph, "batch": n}}
 
 
+def digest(args):
+    """Order-invariant digest of a [tokens, 151936] bf16 logits matrix: the full-precision digest (one mask) and the
+    five-mask ladder, each one pass over the tensor. The kernel is timed with events through the C ABI; ``value``
+    is whole calls of tensor_digest, host read-back included."""
+    import ctypes
+
+    import torch
+
+    from isoexec_amd._lib import check, current_stream, lib
+    from isoexec_amd.debug import thash
+
+    dev = "cuda:0"
+    rows, vocab = args.tokens, 151936
+    x = torch.empty(rows, vocab, dtype=torch.bfloat16, device=dev).normal_()
+    n, nbytes = x.numel(), x.numel() * 2
+    handle = lib()
+    out = torch.empty(8, dtype=torch.int64, device=dev)
+    timers = {}
+    for label, masks in (("one mask", [0xFFFF]), ("ladder of 5", [0xFFFF, 0xFFFE, 0xFFF8, 0xFFE0, 0xFF80])):
+        need = handle.ix_digest_workspace_words(1, n, len(masks))
+        work = torch.empty(max(1, need), dtype=torch.int64, device=dev)
+        arr = (ctypes.c_uint64 * 8)(*masks)
+        call = lambda: check(handle.ix_digest_sums(x.data_ptr(), 2, n, 0x1234, arr, len(masks), work.data_ptr(), need,
+                                                   out.data_ptr(), current_stream(x.device)), "ix_digest_sums")
+        timers[label] = KernelTimer()
+        for _ in range(args.warmup):
+            call()
+        for _ in range(args.steps):
+            timers[label](call)
+        torch.cuda.synchronize()
+    for _ in range(args.warmup):
+        thash.tensor_digest(x)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        thash.tensor_digest(x)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms = timers["one mask"].mean_ms()
+    res = {"metric": "digest GB/s", "value": nbytes * args.steps / dt / 1e9, "unit": "GB/s", "n_gpus": 1,
+           "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "u64", "data": "synthetic",
+           "config": {"workload": f"digest: [{rows}, {vocab}] bf16 ({nbytes / 1e9:.2f} GB), tensor_digest per step"},
+           "roofline": {"bound": "hbm", "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                        "frac": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                        "kernel": "k_digest_partial<2,1> + k_digest_finish", "kernel_ms": ms,
+                        "ladder_of_5_ms": timers["ladder of 5"].mean_ms()}}
+    if not args.no_cpu_baseline:
+        from oracle import thash as OT
+
+        sample_rows = max(1, min(rows, 4096))          # about 10 s of numpy work
+        iv = x[:sample_rows].cpu().view(torch.int16).numpy()
+        t0 = time.perf_counter()
+        OT.tensor_digest(iv, "bfloat16", (sample_rows, vocab))
+        cpu = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": sample_rows * vocab * 2 / cpu / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": f"first {sample_rows} rows of the same matrix ({cpu:.1f} s of CPU work; "
+                                         "numpy restatement of the digest)"}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="dense_head", choices=["dense_head", "gdn_decode", "moe", "hybrid", "attention"])
+    ap.add_argument("--workload", default="dense_head", choices=["dense_head", "gdn_decode", "moe", "hybrid", "attention", "digest"])
     ap.add_argument("--seqs", type=int, default=64)
     ap.add_argument("--prompt", type=int, default=2048)
     ap.add_argument("--response", type=int, default=512)
@@ -394,7 +455,7 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(3)
-    out = {"dense_head": dense_head, "gdn_decode": gdn_decode, "moe": moe, "hybrid": hybrid, "attention": attention}[args.workload](args)
+    out = {"dense_head": dense_head, "gdn_decode": gdn_decode, "moe": moe, "hybrid": hybrid, "attention": attention, "digest": digest}[args.workload](args)
     print(json.dumps(out))
 
 

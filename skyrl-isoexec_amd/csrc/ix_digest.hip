@@ -15,7 +15,8 @@
 #include "../../include/isoexec_hip.h"
 
 #define DG_THREADS 256
-#define DG_MAX_BLOCKS 4096   // upper bound on workgroups per launch along x and on partial rows per segment
+#define DG_UNROLL 4          // groups whose loads are in flight together
+#define DG_MAX_BLOCKS 2048   // upper bound on workgroups per launch along x and on partial rows per segment
 
 static constexpr uint64_t DG_MIX1 = 0xBF58476D1CE4E5B9ull;
 static constexpr uint64_t DG_MIX2 = 0x94D049BB133111EBull;
@@ -82,6 +83,23 @@ __device__ __forceinline__ void dg_load8(const char* __restrict__ p, int cnt, bo
   }
 }
 
+// Adds group g's eight elements, each times its weight, to the NM sums. Absent elements are zero and add nothing.
+template <int EB, int NM>
+__device__ __forceinline__ void dg_fold(long g, uint64_t salt, const uint32_t (&lo)[8], const uint32_t (&hi)[8],
+                                        const DgMasks& masks, uint64_t (&acc)[NM]) {
+  const uint64_t wbase = dg_mix((uint64_t)g ^ salt);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const uint64_t w = (wbase ^ ((uint64_t)i * DG_GOLDEN)) | 1ull;
+    const uint32_t sign = EB == 8 ? hi[i] : (uint32_t)((int32_t)lo[i] >> 31);
+#pragma unroll
+    for (int j = 0; j < NM; ++j) {
+      acc[j] += (uint64_t)(lo[i] & masks.lo[j]) * w;
+      if (masks.hi[j]) acc[j] += (uint64_t)((sign & masks.hi[j]) * (uint32_t)w) << 32;
+    }
+  }
+}
+
 // One workgroup's share of one segment: groups of eight elements dealt to threads, then a fixed tree over the
 // workgroup (any order would do). partials[(segment * nb + blockIdx.x) * NM + j]; with nb == 1 that IS the result.
 template <int EB, int NM>
@@ -102,22 +120,24 @@ __global__ __launch_bounds__(DG_THREADS) void k_digest_partial(const char* __res
     uint64_t acc[NM];
 #pragma unroll
     for (int j = 0; j < NM; ++j) acc[j] = 0;
-    for (long g = (long)blockIdx.x * DG_THREADS + threadIdx.x; g < ngroups; g += (long)nb * DG_THREADS) {
-      const long off = g << 3;
-      const int cnt = (len - off) < 8 ? (int)(len - off) : 8;
-      uint32_t lo[8], hi[8];
-      dg_load8<EB>(xs + off * EB, cnt, vec, lo, hi);
-      const uint64_t wbase = dg_mix((uint64_t)g ^ salt);
+    const long stride = (long)nb * DG_THREADS;
+    long g = (long)blockIdx.x * DG_THREADS + threadIdx.x;
+    // DG_UNROLL groups per trip: their loads are issued together, then each is folded into the sums
+    // (only while all of them are whole groups behind an aligned start: no branch between the loads)
+    if (vec) {
+      for (; ((g + (DG_UNROLL - 1) * stride) << 3) + 8 <= len; g += DG_UNROLL * stride) {
+        uint32_t lo[DG_UNROLL][8], hi[DG_UNROLL][8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const uint64_t w = (wbase ^ ((uint64_t)i * DG_GOLDEN)) | 1ull;   // absent elements are zero: they add nothing
-        const uint32_t sign = EB == 8 ? hi[i] : (uint32_t)((int32_t)lo[i] >> 31);
+        for (int u = 0; u < DG_UNROLL; ++u) dg_load8<EB>(xs + ((g + u * stride) << 3) * EB, 8, true, lo[u], hi[u]);
 #pragma unroll
-        for (int j = 0; j < NM; ++j) {
-          acc[j] += (uint64_t)(lo[i] & masks.lo[j]) * w;
-          if (masks.hi[j]) acc[j] += (uint64_t)((sign & masks.hi[j]) * (uint32_t)w) << 32;
-        }
+        for (int u = 0; u < DG_UNROLL; ++u) dg_fold<EB, NM>(g + u * stride, salt, lo[u], hi[u], masks, acc);
       }
+    }
+    for (; g < ngroups; g += stride) {
+      const long off = g << 3;
+      uint32_t lo[8], hi[8];
+      dg_load8<EB>(xs + off * EB, (len - off) < 8 ? (int)(len - off) : 8, vec, lo, hi);
+      dg_fold<EB, NM>(g, salt, lo, hi, masks, acc);
     }
 #pragma unroll
     for (int j = 0; j < NM; ++j) {
@@ -137,19 +157,26 @@ __global__ __launch_bounds__(DG_THREADS) void k_digest_partial(const char* __res
   }
 }
 
-// out[r] = SUM_b partials[(r / nm * nb + b) * nm + r % nm]: one wave per result.
+// out[r] = SUM_b partials[(r / nm * nb + b) * nm + r % nm]: one workgroup per result, its loads independent.
 __global__ __launch_bounds__(DG_THREADS) void k_digest_finish(const uint64_t* __restrict__ partials, int nb, int nm,
-                                                              long results, uint64_t* __restrict__ out) {
-  const int lane = threadIdx.x & (IX_WAVE - 1);
-  const long r = (long)blockIdx.x * (DG_THREADS / IX_WAVE) + threadIdx.x / IX_WAVE;
-  if (r >= results) return;
+                                                              uint64_t* __restrict__ out) {
+  __shared__ uint64_t s_part[DG_THREADS / IX_WAVE];
+  const int lane = threadIdx.x & (IX_WAVE - 1), wave = threadIdx.x / IX_WAVE;
+  const long r = blockIdx.x;
   const long seg = r / nm;
   const int j = (int)(r % nm);
   uint64_t v = 0;
-  for (int b = lane; b < nb; b += IX_WAVE) v += partials[(seg * nb + b) * nm + j];
+  for (int b = threadIdx.x; b < nb; b += DG_THREADS) v += partials[(seg * nb + b) * nm + j];
 #pragma unroll
   for (int d = IX_WAVE / 2; d >= 1; d >>= 1) v += __shfl_xor((unsigned long long)v, d, IX_WAVE);
-  if (lane == 0) out[r] = v;
+  if (lane == 0) s_part[wave] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint64_t total = 0;
+#pragma unroll
+    for (int w = 0; w < DG_THREADS / IX_WAVE; ++w) total += s_part[w];
+    out[r] = total;
+  }
 }
 
 // Workgroups per segment: enough that a thread sees about four groups, few enough that all segments together stay
@@ -216,10 +243,8 @@ static int dg_run(const void* x, int elem_bytes, long n, long nseg, long seg_num
   }
   int rc = ix_launch_status();
   if (rc != IX_OK || nb == 1) return rc;
-  const long results = nseg * nmask;
-  const long grid = (results + DG_THREADS / IX_WAVE - 1) / (DG_THREADS / IX_WAVE);
-  if (grid > 0x7fffffffL) return IX_DECLINED;
-  hipLaunchKernelGGL(k_digest_finish, dim3((unsigned)grid), dim3(DG_THREADS), 0, st, workspace, nb, nmask, results,
+  // nb > 1 only when nseg <= DG_MAX_BLOCKS / 2, so the grid is small
+  hipLaunchKernelGGL(k_digest_finish, dim3((unsigned)(nseg * nmask)), dim3(DG_THREADS), 0, st, workspace, nb, nmask,
                      out);
   return ix_launch_status();
 }
