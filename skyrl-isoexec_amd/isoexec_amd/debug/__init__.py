@@ -1,13 +1,15 @@
-"""Debug aids for locating a trainer/engine mismatch: on-device digests of tensors (``thash``).
+"""Debug aids for locating a trainer/engine mismatch: on-device digests of tensors (``thash``) and per-region logs of
+them with their comparison (``regions``).
 
 Nothing is imported until a name is asked for, so importing the package costs nothing in a run that never digests.
-(The reference's ``isoexec/debug`` package re-exports the same digest names lazily: debug/__init__.py:8-35.)
+(The reference's ``isoexec/debug`` package re-exports its names lazily in the same way: debug/__init__.py:8-35.)
 """
 
 _DIGEST_NAMES = ("tensor_digest", "digest_ladder", "ladder_for", "segment_axis", "segment_digests",
                  "first_divergent_segments", "iter_tensor_outputs", "digest_backend")
+_REGION_NAMES = ("RegionLog", "wrap_region", "compare", "render", "ladder_verdict", "segment_note")
 
-__all__ = sorted(_DIGEST_NAMES + ("preload_digest",))
+__all__ = sorted(_DIGEST_NAMES + _REGION_NAMES + ("preload_digest",))
 
 
 def __getattr__(name):
@@ -15,4 +17,8 @@ def __getattr__(name):
         from . import thash
 
         return thash.preload if name == "preload_digest" else getattr(thash, name)
+    if name in _REGION_NAMES:
+        from . import regions
+
+        return getattr(regions, name)
     raise AttributeError(f"module {__name__!r} has no attribute {name!r}")

@@ -130,6 +130,13 @@ class _Blocks:
         self.cfg, self.w = cfg, weights
         dev = weights.embed.device
         self.cos, self.sin = rope_tables(cfg.max_positions, cfg.head_dim, cfg.rope_theta, device=dev)
+        # a debug.regions.RegionLog, or None: when set, the residual stream's per-layer outputs are digested on the
+        # device as they are produced, so that two runtimes' passes over the same tokens can be compared region by region
+        self.region_log = None
+
+    def _note(self, region: str, layer, out) -> None:
+        if self.region_log is not None:
+            self.region_log.record(region, out, layer=layer)
 
     def embed(self, tokens: torch.Tensor) -> torch.Tensor:
         return self.w.embed.index_select(0, tokens)
@@ -174,10 +181,14 @@ class _Blocks:
         x = fused_rms_norm_gamma(h, self.w.layers[0]["pre_norm"], c.eps)
         for i in range(c.layers):
             lw = self.w.layers[i]
-            x, h = fused_add_rms_norm_gamma(mixer(i, x), h, lw["post_norm"], c.eps)
+            mixed = mixer(i, x)
+            self._note("attention.varlen" if c.is_attention(i) else "gdn.core", i, mixed)
+            x, h = fused_add_rms_norm_gamma(mixed, h, lw["post_norm"], c.eps)
             delta = self.moe(i, x)
+            self._note("moe.combine", i, delta)
             nxt = self.w.layers[i + 1]["pre_norm"] if i + 1 < c.layers else self.w.final_norm
             x, h = fused_add_rms_norm_gamma(delta, h, nxt, c.eps)
+            self._note("norms.rms", i, (x, h))
         return x  # final-normed hidden states
 
     def logits(self, x: torch.Tensor, want_row_max: bool = False):
