@@ -100,7 +100,7 @@ def derive_selections(profile: ModelProfile) -> Dict[Key, Selection]:
         put("moe.router", ALL_SITES, impl="hip_fused_topk", pinned={"topk": r.topk, "experts": r.num_experts, "score": r.order})
         put("moe.dispatch", ALL_SITES, impl="hip_bitmask_index")
         put("moe.experts", ALL_SITES, impl="hip_grouped_mfma")
-        put("moe.combine", ALL_SITES, impl="hip_fixed_order", pinned={"leaf_dtype": "fp32"})
+        put("moe.combine", ALL_SITES, impl="hip_fixed_order", pinned={"leaf_dtype": profile.moe_combine_dtype})
 
     if profile.tensor_parallel:
         raise ContractBuildError(

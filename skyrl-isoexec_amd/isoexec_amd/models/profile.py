@@ -148,6 +148,7 @@ class ModelProfile:
     ssm_cache_dtype: str = "float32"
     pik_leaves: int = 8
     pik_leaf_dtype: str = "bf16"
+    moe_combine_dtype: str = "fp32"   # what a token's k expert rows are summed in: "fp32" (one rounding) or "bf16" (one per add)
     topology: tuple = field(default=(), compare=False)
     states: tuple = field(default=(), compare=False)
     tolerances: tuple = field(default=(), compare=False)
@@ -158,6 +159,8 @@ class ModelProfile:
         me = repr(self.model)
         if self.attention not in _ATTENTIONS:
             raise ProfileError(f"unknown attention family {self.attention!r}; expected one of {sorted(_ATTENTIONS)}")
+        if self.moe_combine_dtype not in ("fp32", "bf16"):
+            _refuse(me, f"unknown moe_combine_dtype {self.moe_combine_dtype!r}")
         if self.has_moe != (self.router is not None):
             _refuse(me, "has_moe=True requires a RouterProfile" if self.has_moe else "router declared but has_moe=False")
         declared_axes = [fact.axis for fact in self.topology]

@@ -59,10 +59,23 @@ class HybridConfig:
     experts: int = 128
     topk: int = 8
     expert_inter: int = 768
+    # what a token's k expert rows are summed in by the combine: "fp32" (the contract's default) or "bf16"
+    moe_combine_dtype: str = "fp32"
     eps: float = 1.0e-6
 
     def is_attention(self, layer: int) -> bool:
         return (layer + 1) % self.attention_every == 0
+
+    def profile(self):
+        """The model declaration of THIS configuration: the production declaration with the widths and kernel
+        choices that reach the contract replaced by this configuration's."""
+        from ..models import qwen3_5
+        from ..models.profile import RouterProfile
+
+        return qwen3_5.PROFILE.with_overrides(
+            model=f"hybrid-{self.layers}l-{self.experts}e", name_patterns=(),
+            router=RouterProfile(topk=self.topk, num_experts=self.experts),
+            gdn_kernel=self.gdn_kernel, gdn_chunk_size=self.gdn_chunk, moe_combine_dtype=self.moe_combine_dtype)
 
     @property
     def gdn_qkv(self) -> int:
@@ -173,7 +186,8 @@ class _Blocks:
 
     def moe(self, layer: int, x: torch.Tensor) -> torch.Tensor:
         lw = self.w.layers[layer]
-        return moe_ffn_forward(x, lw["router"], lw["w1"], lw["w2"], self.cfg.topk, pre_softmax=True)
+        return moe_ffn_forward(x, lw["router"], lw["w1"], lw["w2"], self.cfg.topk, pre_softmax=True,
+                               fp32_combine=self.cfg.moe_combine_dtype == "fp32")
 
     def run_layers(self, h: torch.Tensor, mixer) -> torch.Tensor:
         """The residual stream over all layers; ``mixer(layer, x)`` is the runtime's own part."""
@@ -201,6 +215,45 @@ class _Blocks:
         logits, row_max = self.logits(x, want_row_max=True)
         lp, _ = sampled_forward(logits, targets, leaves(), row_max=row_max)
         return lp
+
+
+def bound_implementations(cfg: HybridConfig) -> dict:
+    """op -> (impl id, the callable these runtimes bind for it, the constants it runs with). Written from what the
+    code above calls, not read back from a contract, so that comparing it with a contract says something."""
+    scan = gdn_native_cpr_fwd if cfg.gdn_kernel == "cpr" else gdn_native_core
+    from ..ops.logprobs.rowinv import BLOCK
+
+    return {
+        "mm": ("hip_mfma_batch_invariant", linear_nt, None),
+        "norms.rms": ("hip_fused", fused_add_rms_norm_gamma, None),
+        "norms.gated_out": ("hip_fused", fused_gated_out_norm, None),
+        "attention.varlen": ("hip_varlen_ns1", varlen_attention, {"num_splits": 1}),
+        "rope.rope": ("hip_rope", apply_rope_, None),
+        "gdn.conv": ("hip_causal_conv", conv_packed, None),
+        "gdn.core": ("hip_fused_recurrent", scan, {"kernel": cfg.gdn_kernel}),
+        "gdn.state": ("hip_private_pool", CprGDN if cfg.gdn_kernel == "cpr" else RecurrentGDN, {"ssm_cache_dtype": "float32"}),
+        "moe.router": ("hip_fused_topk", moe_ffn_forward, {"topk": cfg.topk, "experts": cfg.experts, "score": "softmax_then_topk"}),
+        "moe.dispatch": ("hip_bitmask_index", moe_ffn_forward, None),
+        "moe.experts": ("hip_grouped_mfma", moe_ffn_forward, None),
+        "moe.combine": ("hip_fixed_order", moe_ffn_forward, {"leaf_dtype": cfg.moe_combine_dtype}),
+        "logprobs.log_softmax": ("hip_rowinv_leaftree", sampled_forward, {"leaves": leaves(), "block": BLOCK, "accum": "kahan_fp32"}),
+        "logprobs.lm_head_slice": ("sampled_rows", _Blocks.sampled_logprobs, None),
+    }
+
+
+def record_runtime_installs(cfg: HybridConfig, side: str, registry=None) -> int:
+    """File, for every op above, an install record at each site of ``side`` ("trainer" / "engine") the op exists at.
+    Returns the number of (op, site) keys recorded."""
+    from ..core import enforce, fingerprint
+    from ..core.registry_build import build_registry
+
+    registry = registry or build_registry()
+    count = 0
+    for op, (impl_id, fn, pins) in bound_implementations(cfg).items():
+        sites = [site for site in registry.get_op(op).sites if site in enforce.SIDES[side]]
+        fingerprint.record_installs(op, sites, impl_id, fn, pins)
+        count += len(sites)
+    return count
 
 
 class TrainerModel:
