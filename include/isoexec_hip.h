@@ -244,6 +244,14 @@ int ix_moe_experts(const void* x, long ldx, const int* sorted_token, const float
                    const void* W1, const void* W2, const int* tile_meta, long max_tiles, long BM, void* inter,
                    void* expert_out, long T, long rows, long Hd, long F, void* stream);
 
+/* The same product with the weight-tile width chosen by the caller: BN = 256 (what ix_moe_experts uses), or
+ * BN = 128 with BM = 128 (square 128 x 128 tiles, two workgroups per CU). The tile shape decides which
+ * workgroup computes an element, never how: results are bit-identical for every (BM, BN). The reference's
+ * counterpart is the BLOCK_M / BLOCK_N choice of its fused expert kernel (moe_fused_experts.py:292-503). */
+int ix_moe_experts_tile(const void* x, long ldx, const int* sorted_token, const float* permuted_prob,
+                        const void* W1, const void* W2, const int* tile_meta, long max_tiles, long BM, long BN,
+                        void* inter, void* expert_out, long T, long rows, long Hd, long F, void* stream);
+
 /* _fixed_order_combine / _combine_topk_kernel (moe_batch_invariant.py:276-320,
  * moe_combine_kernel.py:36-76): out bf16 [T, Hd] = the token's k rows of expert_out summed in
  * ascending expert order; fp32_acc 0 = bf16 adds (a round per add), 1 = fp32 sum, one round. */

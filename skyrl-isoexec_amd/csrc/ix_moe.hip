@@ -153,6 +153,123 @@ __global__ __launch_bounds__(256) void k_moe_router(const float* __restrict__ lo
   }
 }
 
+// E <= 128: a token takes 16 lanes (a row of the wave, so every exchange is a row-local lane control) and a wave
+// routes 4 tokens. Lane i of the row holds experts 4i .. 4i+3 and 64+4i .. 64+4i+3. Same function as k_moe_router
+// bit for bit: the winner under ix_beats does not depend on the exchange network, and the softmax denominator is
+// built as there -- s[v] + s[v + 64] per v = e mod 64, then the adjacent-pairwise tree over v (two levels inside the
+// lane, four across the row).
+__global__ __launch_bounds__(256) void k_moe_router_row16(const float* __restrict__ logits, long ld, int T, int E,
+                                                          int k, int mode, float scaling, int* __restrict__ topk_idx,
+                                                          float* __restrict__ topk_prob,
+                                                          float* __restrict__ dense_probs,
+                                                          uint8_t* __restrict__ dense_map) {
+  const int li = threadIdx.x & 15;
+  const long t = (long)blockIdx.x * 16 + (threadIdx.x >> 4);
+  if (t >= T) return;  // whole rows leave together; the lane controls below stay inside a row
+  float s[8];
+  int eid[8];
+  bool live[8];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int e0 = 64 * h + 4 * li;
+    float4 v4 = make_float4(IX_NEG_INF, IX_NEG_INF, IX_NEG_INF, IX_NEG_INF);
+    if (e0 + 4 <= E && (ld & 3) == 0 && (reinterpret_cast<uintptr_t>(logits) & 15) == 0) {
+      v4 = *reinterpret_cast<const float4*>(logits + t * ld + e0);
+    } else {
+      if (e0 + 0 < E) v4.x = logits[t * ld + e0 + 0];
+      if (e0 + 1 < E) v4.y = logits[t * ld + e0 + 1];
+      if (e0 + 2 < E) v4.z = logits[t * ld + e0 + 2];
+      if (e0 + 3 < E) v4.w = logits[t * ld + e0 + 3];
+    }
+    const float q[4] = {v4.x, v4.y, v4.z, v4.w};
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int e = e0 + c;
+      eid[4 * h + c] = e;
+      live[4 * h + c] = e < E;
+      float v = live[4 * h + c] ? q[c] : IX_NEG_INF;
+      if (v != v) v = IX_NEG_INF;
+      s[4 * h + c] = v;
+    }
+  }
+  if (mode == 1) {
+    float m = IX_NEG_INF;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) m = fmaxf(m, s[c]);
+    m = ix_lane_max<16>(m);
+    float zl[4];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) s[c] = live[c] ? ix_exp(s[c] - m) : 0.0f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) zl[c] = s[c] + s[4 + c];
+    float z = (zl[0] + zl[1]) + (zl[2] + zl[3]);
+    z = ix_lane_tree<16>(z);
+#pragma unroll
+    for (int c = 0; c < 8; ++c) s[c] = s[c] / z;
+  }
+  float vals[IX_MOE_KMAX];
+  int idxs[IX_MOE_KMAX];
+#pragma unroll
+  for (int j = 0; j < IX_MOE_KMAX; ++j) {
+    vals[j] = 0.0f;
+    idxs[j] = 0;
+    if (j < k) {
+      float bv = 0.0f;
+      int bi = E;
+#pragma unroll
+      for (int c = 0; c < 8; ++c)
+        if (live[c] && ix_beats(s[c], eid[c], bv, bi, E)) { bv = s[c]; bi = eid[c]; }
+      ix_best_step<1>(bv, bi, E);
+      ix_best_step<2>(bv, bi, E);
+      ix_best_step<4>(bv, bi, E);
+      ix_best_step<8>(bv, bi, E);
+      bi = min(bi, E - 1);
+      vals[j] = bv;
+      idxs[j] = bi;
+#pragma unroll
+      for (int c = 0; c < 8; ++c)
+        if (eid[c] == bi) live[c] = false;
+    }
+  }
+  float p[IX_MOE_KMAX], tmp[IX_MOE_KMAX];
+  if (mode == 0) {
+    const float m = vals[0];
+#pragma unroll
+    for (int j = 0; j < IX_MOE_KMAX; ++j) { p[j] = (j < k) ? ix_exp(vals[j] - m) : 0.0f; tmp[j] = p[j]; }
+  } else {
+#pragma unroll
+    for (int j = 0; j < IX_MOE_KMAX; ++j) { p[j] = (j < k) ? vals[j] : 0.0f; tmp[j] = p[j]; }
+  }
+  const float den = ix_tree_k(tmp, k);
+#pragma unroll
+  for (int j = 0; j < IX_MOE_KMAX; ++j) {
+    p[j] = p[j] / den;
+    if (scaling != 0.0f) p[j] = p[j] * scaling;
+  }
+#pragma unroll
+  for (int j = 0; j < IX_MOE_KMAX; ++j) {
+    if (j < k && li == j) {
+      topk_idx[t * k + j] = idxs[j];
+      topk_prob[t * k + j] = p[j];
+    }
+  }
+  if (dense_probs || dense_map) {
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const int e = eid[c];
+      if (e < E) {
+        float dp = 0.0f;
+        uint8_t dm = 0;
+#pragma unroll
+        for (int j = 0; j < IX_MOE_KMAX; ++j)
+          if (j < k && idxs[j] == e) { dp = p[j]; dm = 1; }
+        if (dense_probs) dense_probs[t * E + e] = dp;
+        if (dense_map) dense_map[t * E + e] = dm;
+      }
+    }
+  }
+}
+
 extern "C" int ix_moe_router_topk(const float* logits, long ld, long T, long E, long k, int mode, float scaling,
                                   int* topk_idx, float* topk_prob, float* dense_probs, uint8_t* dense_map,
                                   void* stream) {
@@ -166,8 +283,11 @@ extern "C" int ix_moe_router_topk(const float* logits, long ld, long T, long E, 
 #define IX_ROUTER(EC_)                                                                                            \
   hipLaunchKernelGGL(k_moe_router<EC_>, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, logits, ld,      \
                      (int)T, (int)E, (int)k, mode, scaling, topk_idx, topk_prob, dense_probs, dense_map)
-  if (E <= 128) IX_ROUTER(2);
-  else if (E <= 256) IX_ROUTER(4);
+  if (E <= 128) {
+    const long grid16 = (T + 15) / 16;
+    hipLaunchKernelGGL(k_moe_router_row16, dim3((unsigned)grid16), dim3(256), 0, (hipStream_t)stream, logits, ld,
+                       (int)T, (int)E, (int)k, mode, scaling, topk_idx, topk_prob, dense_probs, dense_map);
+  } else if (E <= 256) IX_ROUTER(4);
   else IX_ROUTER(IX_MOE_EC);
 #undef IX_ROUTER
   return ix_launch_status();
@@ -222,8 +342,11 @@ __global__ __launch_bounds__(256) void k_moe_offsets(const int* __restrict__ til
   const int tid = threadIdx.x;
   for (int e = tid; e < E; e += 256) s_cnt[e] = 0;
   __syncthreads();
-  for (int t0 = 0; t0 < ntiles; t0 += IX_MOE_SCAN_TILES) {
-    const int nt = min(IX_MOE_SCAN_TILES, ntiles - t0);
+  // as many token tiles per stage as the staging array holds for this E (64 for 128 experts): each stage costs a
+  // round trip to memory and three barriers
+  const int stage_tiles = (IX_MOE_SCAN_TILES * IX_MOE_EMAX) / E;
+  for (int t0 = 0; t0 < ntiles; t0 += stage_tiles) {
+    const int nt = min(stage_tiles, ntiles - t0);
     for (int i = tid; i < nt * E; i += 256) s_stage[i] = tile_counts[(long)t0 * E + i];
     __syncthreads();
     for (int e = tid; e < E; e += 256) {
@@ -239,18 +362,42 @@ __global__ __launch_bounds__(256) void k_moe_offsets(const int* __restrict__ til
     for (int i = tid; i < nt * E; i += 256) tile_base[(long)t0 * E + i] = s_stage[i];
     __syncthreads();
   }
-  if (tid == 0) {
-    int run = 0, trun = 0;
-    for (int e = 0; e < E; ++e) {
-      s_off[e] = run;
-      s_toff[e] = trun;
-      run += s_cnt[e];
-      trun += (s_cnt[e] + BM - 1) / BM;
+  // exclusive scan over the experts (rows and row tiles): lane owns experts 2 tid and 2 tid + 1 (E <= 512)
+  {
+    __shared__ int s_rows[256], s_tiles[256];
+    int c[2], tl[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int e = 2 * tid + h;
+      c[h] = e < E ? s_cnt[e] : 0;
+      tl[h] = (c[h] + BM - 1) / BM;
     }
-    s_off[E] = run;
-    s_toff[E] = trun;
-    offsets[E] = run;
-    meta[0] = min(trun, max_tiles);
+    s_rows[tid] = c[0] + c[1];
+    s_tiles[tid] = tl[0] + tl[1];
+    __syncthreads();
+    for (int d = 1; d < 256; d <<= 1) {
+      const int a = tid >= d ? s_rows[tid - d] : 0;
+      const int b = tid >= d ? s_tiles[tid - d] : 0;
+      __syncthreads();
+      s_rows[tid] += a;
+      s_tiles[tid] += b;
+      __syncthreads();
+    }
+    int row0 = s_rows[tid] - (c[0] + c[1]);
+    int tile0 = s_tiles[tid] - (tl[0] + tl[1]);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int e = 2 * tid + h;
+      if (e < E) { s_off[e] = row0; s_toff[e] = tile0; }
+      row0 += c[h];
+      tile0 += tl[h];
+    }
+    if (tid == 255) {
+      s_off[E] = s_rows[255];
+      s_toff[E] = s_tiles[255];
+      offsets[E] = s_rows[255];
+      meta[0] = min(s_tiles[255], max_tiles);
+    }
   }
   __syncthreads();
   int* tile_expert = meta + 1;
@@ -625,9 +772,10 @@ static int ix_moe_experts_launch(const bf16_t* x, long ldx, int T, const int* so
   return ix_launch_status();
 }
 
-extern "C" int ix_moe_experts(const void* x, long ldx, const int* sorted_token, const float* permuted_prob,
-                              const void* W1, const void* W2, const int* tile_meta, long max_tiles, long BM,
-                              void* inter, void* expert_out, long T, long rows, long Hd, long F, void* stream) {
+extern "C" int ix_moe_experts_tile(const void* x, long ldx, const int* sorted_token, const float* permuted_prob,
+                                   const void* W1, const void* W2, const int* tile_meta, long max_tiles, long BM,
+                                   long BN, void* inter, void* expert_out, long T, long rows, long Hd, long F,
+                                   void* stream) {
   if (!x || !sorted_token || !permuted_prob || !W1 || !W2 || !tile_meta || !inter || !expert_out)
     return IX_ERR_ARG;
   if (T < 0 || rows < 0 || Hd <= 0 || F <= 0 || max_tiles < 0 || ldx < Hd) return IX_ERR_ARG;
@@ -640,6 +788,10 @@ extern "C" int ix_moe_experts(const void* x, long ldx, const int* sorted_token, 
   hipStream_t st = (hipStream_t)stream;
   const bf16_t *xx = (const bf16_t*)x, *w1 = (const bf16_t*)W1, *w2 = (const bf16_t*)W2;
   bf16_t *it = (bf16_t*)inter, *eo = (bf16_t*)expert_out;
+  if (BN != 256 && !(BN == 128 && BM == 128)) return IX_ERR_ARG;
+  if (BN == 128)
+    return ix_moe_experts_launch<128, 128, 2, 2>(xx, ldx, (int)T, sorted_token, permuted_prob, w1, w2, tile_meta,
+                                                 max_tiles, it, eo, (int)Hd, (int)F, st);
   switch (BM) {
     case 32:
       return ix_moe_experts_launch<32, 256, 1, 4>(xx, ldx, (int)T, sorted_token, permuted_prob, w1, w2, tile_meta,
@@ -652,6 +804,13 @@ extern "C" int ix_moe_experts(const void* x, long ldx, const int* sorted_token, 
                                                    max_tiles, it, eo, (int)Hd, (int)F, st);
     default: return IX_ERR_ARG;
   }
+}
+
+extern "C" int ix_moe_experts(const void* x, long ldx, const int* sorted_token, const float* permuted_prob,
+                              const void* W1, const void* W2, const int* tile_meta, long max_tiles, long BM,
+                              void* inter, void* expert_out, long T, long rows, long Hd, long F, void* stream) {
+  return ix_moe_experts_tile(x, ldx, sorted_token, permuted_prob, W1, W2, tile_meta, max_tiles, BM, 256, inter,
+                             expert_out, T, rows, Hd, F, stream);
 }
 
 // ---------------------------------------------------------------------------------------------

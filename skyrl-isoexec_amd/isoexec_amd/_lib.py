@@ -81,6 +81,10 @@ SIGNATURES = {
         c_int,
         [P, c_long, P, P, P, P, P, c_long, c_long, P, P, c_long, c_long, c_long, c_long, P],
     ),
+    "ix_moe_experts_tile": (
+        c_int,
+        [P, c_long, P, P, P, P, P, c_long, c_long, c_long, P, P, c_long, c_long, c_long, c_long, P],
+    ),
     "ix_moe_combine": (c_int, [P, P, P, c_long, c_long, c_long, c_int, P]),
     "ix_digest_sums": (c_int, [P, c_int, c_long, c_uint64, P, c_int, P, c_size_t, P, P]),
     "ix_digest_segment_sums": (c_int, [P, c_int, c_long, c_long, c_long, c_uint64, c_uint64, P, c_size_t, P, P]),

@@ -47,11 +47,12 @@ def fused_router_dense(logits: torch.Tensor, k: int, *, scaling_factor: float | 
 class Permutation:
     """Device-side routing plan: everything the grouped GEMMs and the combine need."""
 
-    __slots__ = ("T", "E", "k", "BM", "counts", "offsets", "sorted_token", "permuted_prob", "combine_rows",
+    __slots__ = ("T", "E", "k", "BM", "BN", "counts", "offsets", "sorted_token", "permuted_prob", "combine_rows",
                  "tile_meta", "max_tiles")
 
 
-def permute(topk_idx: torch.Tensor, topk_prob: torch.Tensor, E: int, *, BM: int | None = None) -> Permutation:
+def permute(topk_idx: torch.Tensor, topk_prob: torch.Tensor, E: int, *, BM: int | None = None,
+            BN: int | None = None) -> Permutation:
     """Expert-major, token-ascending permutation + block map (integer only, no host sync)."""
     _lib.require_device(topk_idx, topk_prob)
     T, k = topk_idx.shape
@@ -60,6 +61,7 @@ def permute(topk_idx: torch.Tensor, topk_prob: torch.Tensor, E: int, *, BM: int 
     p = Permutation()
     p.T, p.E, p.k = T, E, k
     p.BM = int(BM or L.ix_moe_pick_bm(T, k, E))
+    p.BN = int(BN or 256)          # weight-tile width of the grouped GEMMs: 256, or 128 with BM = 128
     p.max_tiles = int(L.ix_moe_max_tiles(T, k, E, p.BM))
     i32 = dict(dtype=torch.int32, device=dev)
     p.counts = torch.empty(E, **i32)
@@ -102,10 +104,11 @@ def experts_forward(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, p: Perm
     out = torch.empty(rows, H, dtype=torch.bfloat16, device=dev)
     xc = x if x.stride(1) == 1 else x.contiguous()
     rc = _lib.check(
-        _lib.lib().ix_moe_experts(xc.data_ptr(), xc.stride(0), p.sorted_token.data_ptr(),
-                                  p.permuted_prob.data_ptr(), w1.contiguous().data_ptr(),
-                                  w2.contiguous().data_ptr(), p.tile_meta.data_ptr(), p.max_tiles, p.BM,
-                                  inter.data_ptr(), out.data_ptr(), T, rows, H, F, _lib.current_stream(dev)),
+        _lib.lib().ix_moe_experts_tile(xc.data_ptr(), xc.stride(0), p.sorted_token.data_ptr(),
+                                       p.permuted_prob.data_ptr(), w1.contiguous().data_ptr(),
+                                       w2.contiguous().data_ptr(), p.tile_meta.data_ptr(), p.max_tiles, p.BM,
+                                       p.BN, inter.data_ptr(), out.data_ptr(), T, rows, H, F,
+                                       _lib.current_stream(dev)),
         "ix_moe_experts")
     if rc != _lib.IX_OK:
         raise RuntimeError(f"[isoexec-amd] ix_moe_experts declined H={H} F={F}")

@@ -119,6 +119,12 @@ def test_moe_ffn_parity_and_batch_invariance(dprims):
     ref = moe_ffn_forward(xd, wrd, w1d, w2d, k, BM=256)
     for BM in (32, 128):
         assert same_bits(moe_ffn_forward(xd, wrd, w1d, w2d, k, BM=BM), ref)
+    # the square 128 x 128 tile (two workgroups per CU) through ix_moe_experts_tile: same rows, same bits
+    idx, prob, _, _ = router_topk(router_gemm(xd, wrd), k)
+    rows = experts_forward(xd, w1d, w2d, permute(idx, prob, E, BM=128))
+    assert same_bits(experts_forward(xd, w1d, w2d, permute(idx, prob, E, BM=128, BN=128)), rows)
+    with pytest.raises(RuntimeError):
+        experts_forward(xd, w1d, w2d, permute(idx, prob, E, BM=256, BN=128))   # only the square pairing exists
     for t in (0, 17, 299):
         assert same_bits(moe_ffn_forward(xd[t:t + 1], wrd, w1d, w2d, k), ref[t:t + 1])
     assert same_bits(moe_ffn_forward(xd[:33], wrd, w1d, w2d, k), ref[:33])
