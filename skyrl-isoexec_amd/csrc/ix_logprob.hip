@@ -26,12 +26,61 @@
 #define IX_LP_SPLIT_BELOW 192
 #define IX_LP_SEG 8192  // columns per partial-max / full-row-write workgroup in the split shape
 
+// Eight consecutive elements as they lie in memory (a 16-byte-aligned group of bf16, a 32-byte-aligned group of
+// fp32): loading and widening are separate steps so that several loads can be in flight before the first is used.
+template <typename T>
+struct IxRaw8;
+template <>
+struct IxRaw8<bf16_t> {
+  uint4 v;
+  __device__ __forceinline__ void load(const bf16_t* __restrict__ p) { v = *reinterpret_cast<const uint4*>(p); }
+  __device__ __forceinline__ void widen(float (&o)[8]) const { ix_unpack8(v, o); }
+};
+template <>
+struct IxRaw8<float> {
+  float4 a, b;
+  __device__ __forceinline__ void load(const float* __restrict__ p) {
+    a = *reinterpret_cast<const float4*>(p);
+    b = *reinterpret_cast<const float4*>(p + 4);
+  }
+  __device__ __forceinline__ void widen(float (&o)[8]) const {
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+  }
+};
+
 // One wave sums one block. `blk` points at the block's first column, n_valid <= 4096 columns
 // exist. Returns the block sum in every lane.
-template <typename T>
-__device__ __forceinline__ float ix_block_expsum(const T* __restrict__ blk, int n_valid, float m, bool vec,
-                                                 int lane) {
+// `row_max()` yields the row maximum; it is called after the block's loads are issued, so a maximum that is itself
+// read from memory does not put its latency in front of theirs.
+template <typename T, typename MaxFn>
+__device__ __forceinline__ float ix_block_expsum_with(const T* __restrict__ blk, int n_valid, const MaxFn& row_max,
+                                                      bool vec, int lane) {
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (vec) {
+    // vec implies that the leaf length is a multiple of 8, so a group of 8 columns is whole or absent. All eight
+    // groups are requested before the first is used: a lane has eight independent loads in flight instead of one
+    // (a load, its wait and its sum per group is bound by memory latency). An absent group reads the block's first
+    // columns instead (no branch between the loads) and adds +0.0. The sums are the ones below: slot i adds its
+    // groups in ascending c.
+    IxRaw8<T> raw[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const int off = c * 512 + lane * 8;
+      raw[c].load(blk + ((n_valid - off >= 8) ? off : 0));
+    }
+    __builtin_amdgcn_sched_barrier(0);  // the loads are issued back to back; widening waits with the sums
+    const float m = row_max();
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const bool whole = n_valid - (c * 512 + lane * 8) >= 8;
+      float x[8];
+      raw[c].widen(x);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] = acc[i] + (whole ? ix_exp_fast(x[i] - m) : 0.0f);
+    }
+    return ix_lane_tree<64>(ix_tree8(acc));
+  }
+  const float m = row_max();
 #pragma unroll
   for (int c = 0; c < 8; ++c) {
     const int off = c * 512 + lane * 8;
@@ -47,6 +96,12 @@ __device__ __forceinline__ float ix_block_expsum(const T* __restrict__ blk, int 
     }
   }
   return ix_lane_tree<64>(ix_tree8(acc));
+}
+
+template <typename T>
+__device__ __forceinline__ float ix_block_expsum(const T* __restrict__ blk, int n_valid, float m, bool vec,
+                                                 int lane) {
+  return ix_block_expsum_with(blk, n_valid, [m]() { return m; }, vec, lane);
 }
 
 __device__ __forceinline__ float ix_kahan_blocks(const float* __restrict__ bsum, int nb) {
@@ -192,11 +247,11 @@ __global__ __launch_bounds__(256) void k_lp_blocksums(const T* __restrict__ x, l
   const int units = G * NB;
   const int u = blockIdx.y * 4 + wave;
   if (u >= units) return;
-  const float m = ix_row_max_from_parts(pmax + row * P, P, lane);
   const int g = u / NB, b = u - g * NB;
   const long base = (long)g * L + (long)b * IX_LP_BLOCK;
   const int nv = min(IX_LP_BLOCK, L - b * IX_LP_BLOCK);
-  const float bs = ix_block_expsum(x + row * row_stride + base, nv, m, vec != 0, lane);
+  const float bs = ix_block_expsum_with(
+      x + row * row_stride + base, nv, [&]() { return ix_row_max_from_parts(pmax + row * P, P, lane); }, vec != 0, lane);
   if (lane == 0) bsum[row * units + u] = bs;
 }
 
