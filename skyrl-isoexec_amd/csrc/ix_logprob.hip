@@ -212,8 +212,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void k_lp_partmax(const T* __restrict__ x, long row_stride, int V, int P,
                                                     float* __restrict__ pmax, int vec) {
   __shared__ float s_w[4];
-  const long row = blockIdx.x;
-  const int p = blockIdx.y;
+  const long row = blockIdx.x / P;  // parts fastest: consecutive workgroups read consecutive memory
+  const int p = blockIdx.x % P;
   const T* xr = x + row * row_stride;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const long lo = (long)p * IX_LP_SEG;
@@ -236,16 +236,19 @@ __device__ __forceinline__ float ix_row_max_from_parts(const float* __restrict__
   return ix_lane_max<64>(m);
 }
 
+// Workgroup -> (row, group of 4 units) with the units fastest: consecutive workgroups read consecutive memory
+// (with the rows fastest they read addresses a row pitch apart: 0.234 -> 0.219 ms on 4096 x 151936 bf16).
 template <typename T>
 __global__ __launch_bounds__(256) void k_lp_blocksums(const T* __restrict__ x, long row_stride, int V, int G,
                                                       int P, const float* __restrict__ pmax,
-                                                      float* __restrict__ bsum, int vec) {
-  const long row = blockIdx.x;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+                                                      float* __restrict__ bsum, int vec, int ny) {
+  const long row = blockIdx.x / ny;
+  const int by = blockIdx.x % ny;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int L = V / G;
   const int NB = (L + IX_LP_BLOCK - 1) / IX_LP_BLOCK;
   const int units = G * NB;
-  const int u = blockIdx.y * 4 + wave;
+  const int u = by * 4 + wave;
   if (u >= units) return;
   const int g = u / NB, b = u - g * NB;
   const long base = (long)g * L + (long)b * IX_LP_BLOCK;
@@ -281,12 +284,12 @@ __global__ __launch_bounds__(64) void k_lp_finalize(const T* __restrict__ x, lon
 template <typename T>
 __global__ __launch_bounds__(256) void k_lp_fullwrite(const T* __restrict__ x, long row_stride, int V,
                                                       const float* __restrict__ fin, float* __restrict__ out_full,
-                                                      long full_stride, int vec) {
-  const long row = blockIdx.x;
+                                                      long full_stride, int vec, int PW) {
+  const long row = blockIdx.x / PW;  // segments fastest
   const T* xr = x + row * row_stride;
   float* orow = out_full + row * full_stride;
   const float mm = fin[row * 2], ls = fin[row * 2 + 1];
-  const long lo = (long)blockIdx.y * IX_LP_SEG;
+  const long lo = (long)(blockIdx.x % PW) * IX_LP_SEG;
   const long hi = min((long)V, lo + IX_LP_SEG);
   for (long off = lo + (long)threadIdx.x * 8; off < hi; off += 256 * 8) {
     float o[8];
@@ -352,7 +355,8 @@ static int ix_lp_launch(const T* x, long rows, long V, long row_stride, int G, c
                        out_lp, out_lse, out_full, full_stride, vec);
     return ix_launch_status();
   }
-  if (rows > 65535L * 1024) return IX_DECLINED;
+  if (rows * (long)((V + IX_LP_SEG - 1) / IX_LP_SEG) > 0x7fffffffL || rows * (long)(G * ((L + IX_LP_BLOCK - 1) / IX_LP_BLOCK)) > 0x7fffffffL)
+    return IX_DECLINED;
   if (!ws || ws_bytes < ix_logprob_workspace_bytes(rows, V, G)) return IX_ERR_ARG;
   const int NB = (int)((L + IX_LP_BLOCK - 1) / IX_LP_BLOCK);
   const int PW = (int)((V + IX_LP_SEG - 1) / IX_LP_SEG);  // workspace layout always reserves PW parts
@@ -363,15 +367,16 @@ static int ix_lp_launch(const T* x, long rows, long V, long row_stride, int G, c
   const int P = row_max_in ? 1 : PW;
   const float* pmax = row_max_in ? row_max_in : ws_pmax;
   if (!row_max_in)
-    hipLaunchKernelGGL((k_lp_partmax<T>), dim3((unsigned)rows, P), dim3(256), 0, st, x, row_stride, (int)V, P,
+    hipLaunchKernelGGL((k_lp_partmax<T>), dim3((unsigned)(rows * P)), dim3(256), 0, st, x, row_stride, (int)V, P,
                        ws_pmax, vec);
-  hipLaunchKernelGGL((k_lp_blocksums<T>), dim3((unsigned)rows, (U + 3) / 4), dim3(256), 0, st, x, row_stride,
-                     (int)V, G, P, pmax, bsum, vec);
+  const int ny = (U + 3) / 4;
+  hipLaunchKernelGGL((k_lp_blocksums<T>), dim3((unsigned)(rows * ny)), dim3(256), 0, st, x, row_stride, (int)V, G, P,
+                     pmax, bsum, vec, ny);
   hipLaunchKernelGGL((k_lp_finalize<T>), dim3((unsigned)rows), dim3(64), 0, st, x, row_stride, (int)V, G, P, pmax,
                      bsum, fin, target, out_lp, out_lse);
   if (out_full)
-    hipLaunchKernelGGL((k_lp_fullwrite<T>), dim3((unsigned)rows, PW), dim3(256), 0, st, x, row_stride, (int)V, fin,
-                       out_full, full_stride, vec);
+    hipLaunchKernelGGL((k_lp_fullwrite<T>), dim3((unsigned)(rows * PW)), dim3(256), 0, st, x, row_stride, (int)V, fin,
+                       out_full, full_stride, vec, PW);
   return ix_launch_status();
 }
 
