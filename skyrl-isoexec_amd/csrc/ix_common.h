@@ -180,6 +180,19 @@ __device__ __forceinline__ void ix_store8_bf16(bf16_t* __restrict__ p, long vali
   }
 }
 
+// Workgroup id -> position in a linear work order, for kernels that stream memory in that order. Hardware deals
+// consecutive workgroup ids to the 8 XCDs round-robin; here the order is cut into 8 equal runs and XCD x walks run x,
+// so every XCD (its own L2, its own path to memory) streams one contiguous region instead of every eighth piece of
+// all of them. Launch ix_xcd_run_grid(total) workgroups; a workgroup past its run's end gets false and exits.
+__device__ __forceinline__ bool ix_xcd_run_position(unsigned bid, unsigned total, unsigned* pos) {
+  const unsigned xcd = bid & 7u, idx = bid >> 3;
+  const unsigned q = total >> 3, r = total & 7u;
+  const unsigned lo = q * xcd + ((r * xcd) >> 3), hi = q * (xcd + 1) + ((r * (xcd + 1)) >> 3);
+  *pos = lo + idx;
+  return lo + idx < hi;
+}
+static inline unsigned ix_xcd_run_grid(unsigned total) { return 8u * ((total + 7u) / 8u); }
+
 static inline int ix_launch_status() {
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? IX_OK : IX_ERR_LAUNCH;
