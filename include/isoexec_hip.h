@@ -33,6 +33,7 @@ extern "C" {
 #define IX_DECLINED 1
 #define IX_ERR_ARG (-1)
 #define IX_ERR_LAUNCH (-2)
+#define IX_ERR_SIZE (-3) /* input larger than a fixed internal buffer */
 #define IX_DT_F32 0
 #define IX_DT_BF16 1
 #endif
@@ -234,6 +235,19 @@ int ix_moe_pick_bm(long T, long k, long E);               /* 32, 128 or 256 */
 int ix_moe_permute(const int* topk_idx, const float* topk_prob, long T, long E, long k, long BM, int* counts,
                    int* offsets, int* sorted_token, float* permuted_prob, int* combine_rows, int* tile_meta,
                    long max_tiles, int* scratch, void* stream);
+
+/* ix_moe_permute for callers that cannot allocate device memory or bring a workspace: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid allocation. No counterpart in the reference (its permutation
+ * allocates its tables with torch on every call). Same arguments, same kernels and same integers as ix_moe_permute,
+ * minus `scratch`: the two internal tables live in a 1 MiB file-scope device array that each GPU holds until the
+ * process ends. The call allocates and frees nothing. Limit: ix_moe_permute_scratch_ints(T, E) <=
+ * ix_moe_permute_static_max_ints() (262,144 ints: 262,144 tokens at E = 128), else IX_ERR_SIZE and nothing is
+ * launched. All calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads) race;
+ * calls in stream order do not, and no call depends on what an earlier one left in the array. */
+size_t ix_moe_permute_static_max_ints(void);
+int ix_moe_permute_static(const int* topk_idx, const float* topk_prob, long T, long E, long k, long BM, int* counts,
+                          int* offsets, int* sorted_token, float* permuted_prob, int* combine_rows, int* tile_meta,
+                          long max_tiles, void* stream);
 
 /* _batched_experts_forward / _fused_forward (moe_batched_experts.py:301-531,
  * moe_fused_experts.py:292-503): grouped fc1 + SwiGLU + prob epilogue, then grouped fc2.

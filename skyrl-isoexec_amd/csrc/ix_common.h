@@ -15,6 +15,7 @@
 #define IX_DECLINED 1
 #define IX_ERR_ARG (-1)
 #define IX_ERR_LAUNCH (-2)
+#define IX_ERR_SIZE (-3)
 
 #define IX_DT_F32 0
 #define IX_DT_BF16 1

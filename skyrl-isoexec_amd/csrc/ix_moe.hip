@@ -571,6 +571,48 @@ extern "C" int ix_moe_permute(const int* topk_idx, const float* topk_prob, long 
 }
 
 // ---------------------------------------------------------------------------------------------
+// The permutation for callers that cannot allocate (code under graph capture, serving loops, harnesses that forbid
+// it): the two integer tables ix_moe_permute takes as `scratch` live in a file-scope device array instead. Every GPU
+// the library runs on holds its own copy of the array, at its own address, until the process ends; the address is
+// resolved once per device, with that device current, on the first call there. Kernels receive that address as an
+// argument, exactly as they receive the caller's workspace in ix_moe_permute. Both tables are fully rewritten by
+// every call before they are read (k_moe_tile_counts writes [ntiles, E], k_moe_offsets writes the bases), so nothing
+// has to start at zero; two calls that overlap on one GPU share the array and race.
+#define IX_MOE_STATIC_SCRATCH_INTS (256 * 1024)  // 1 MiB: 2 * ceil(T / 256) * E ints, e.g. 262,144 tokens at E = 128
+#define IX_MAX_DEVICES 64
+static __device__ __align__(256) int ix_moe_static_scratch[IX_MOE_STATIC_SCRATCH_INTS];
+static int* volatile ix_moe_static_scratch_ptr[IX_MAX_DEVICES];  // per device, 0 = not resolved yet
+
+static int ix_moe_static_scratch_for_current_device(int** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= IX_MAX_DEVICES) return IX_ERR_LAUNCH;
+  int* p = ix_moe_static_scratch_ptr[dev];
+  if (!p) {
+    // Two threads resolving at once store the same address: the lookup has no side effect on the array.
+    void* sym = nullptr;
+    if (hipGetSymbolAddress(&sym, HIP_SYMBOL(ix_moe_static_scratch)) != hipSuccess || !sym) return IX_ERR_LAUNCH;
+    p = static_cast<int*>(sym);
+    ix_moe_static_scratch_ptr[dev] = p;
+  }
+  *out = p;
+  return IX_OK;
+}
+
+extern "C" size_t ix_moe_permute_static_max_ints(void) { return (size_t)IX_MOE_STATIC_SCRATCH_INTS; }
+
+extern "C" int ix_moe_permute_static(const int* topk_idx, const float* topk_prob, long T, long E, long k, long BM,
+                                     int* counts, int* offsets, int* sorted_token, float* permuted_prob,
+                                     int* combine_rows, int* tile_meta, long max_tiles, void* stream) {
+  if (T < 0 || E <= 0) return IX_ERR_ARG;
+  if (ix_moe_permute_scratch_ints(T, E) > (size_t)IX_MOE_STATIC_SCRATCH_INTS) return IX_ERR_SIZE;
+  int* scratch = nullptr;
+  const int rc = ix_moe_static_scratch_for_current_device(&scratch);
+  if (rc != IX_OK) return rc;
+  return ix_moe_permute(topk_idx, topk_prob, T, E, k, BM, counts, offsets, sorted_token, permuted_prob, combine_rows,
+                        tile_meta, max_tiles, scratch, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
 // Grouped GEMMs over the block map. A workgroup past the device-side tile count exits at once,
 // so the host never reads the routing back.
 //

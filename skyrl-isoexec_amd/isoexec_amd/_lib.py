@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(CSRC_DIR, "libisoexec_hip.so")
 
 IX_OK = 0
 IX_DECLINED = 1
+IX_ERR_SIZE = -3
 DT_F32 = 0
 DT_BF16 = 1
 
@@ -76,6 +77,11 @@ SIGNATURES = {
     "ix_moe_permute": (
         c_int,
         [P, P, c_long, c_long, c_long, c_long, P, P, P, P, P, P, c_long, P, P],
+    ),
+    "ix_moe_permute_static_max_ints": (c_size_t, []),
+    "ix_moe_permute_static": (
+        c_int,
+        [P, P, c_long, c_long, c_long, c_long, P, P, P, P, P, P, c_long, P],
     ),
     "ix_moe_experts": (
         c_int,

@@ -52,8 +52,11 @@ class Permutation:
 
 
 def permute(topk_idx: torch.Tensor, topk_prob: torch.Tensor, E: int, *, BM: int | None = None,
-            BN: int | None = None) -> Permutation:
-    """Expert-major, token-ascending permutation + block map (integer only, no host sync)."""
+            BN: int | None = None, static_scratch: bool = False) -> Permutation:
+    """Expert-major, token-ascending permutation + block map (integer only, no host sync).
+
+    ``static_scratch=True`` keeps the kernels' internal tables in the library's file-scope device array instead of a
+    torch allocation (``ix_moe_permute_static``; calls that overlap on one GPU race on that array)."""
     _lib.require_device(topk_idx, topk_prob)
     T, k = topk_idx.shape
     dev = topk_idx.device
@@ -70,6 +73,17 @@ def permute(topk_idx: torch.Tensor, topk_prob: torch.Tensor, E: int, *, BM: int 
     p.permuted_prob = torch.empty(T * k, dtype=torch.float32, device=dev)
     p.combine_rows = torch.empty(T, k, **i32)
     p.tile_meta = torch.empty(1 + 3 * p.max_tiles, **i32)
+    if static_scratch:
+        rc = L.ix_moe_permute_static(topk_idx.contiguous().data_ptr(), topk_prob.contiguous().data_ptr(), T, E, k, p.BM,
+                                     p.counts.data_ptr(), p.offsets.data_ptr(), p.sorted_token.data_ptr(),
+                                     p.permuted_prob.data_ptr(), p.combine_rows.data_ptr(), p.tile_meta.data_ptr(),
+                                     p.max_tiles, _lib.current_stream(dev))
+        if rc == _lib.IX_ERR_SIZE:
+            raise RuntimeError(
+                f"[isoexec-amd] ix_moe_permute_static: T={T}, E={E} needs {int(L.ix_moe_permute_scratch_ints(T, E))} "
+                f"table entries, the static array holds {int(L.ix_moe_permute_static_max_ints())}")
+        _lib.check(rc, "ix_moe_permute_static")
+        return p
     scratch = torch.empty(max(1, int(L.ix_moe_permute_scratch_ints(T, E))), **i32)
     _lib.check(
         L.ix_moe_permute(topk_idx.contiguous().data_ptr(), topk_prob.contiguous().data_ptr(), T, E, k, p.BM,
