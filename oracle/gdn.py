@@ -1,7 +1,7 @@
 """Oracle: GatedDeltaNet conv, l2norm, gating and the delta-rule scan (reference
 ops/gdn/gdn_ops.py:74-170, :173-213, :261-315, :400-441, :1197-1210).
 
-Pinned by (tests/test_oracle_gdn.py): the textbook fp64 recurrence ``scan_fp64`` (written from the
+Pinned by (tests/test_oracle_gdn_moe.py): the textbook fp64 recurrence ``scan_fp64`` (written from the
 math, independent of the lane structure); the chunked WY form ``chunk_fp64`` (the same algorithm
 as the reference's fp32 ``_torch_chunk_gdr_one``, gdn_ops.py:261-315, in float64); closed forms
 (beta = 0: pure decay ``S_T = exp(sum g) S_0``; g = 0, beta = 1, orthonormal keys: associative

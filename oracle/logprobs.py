@@ -1,6 +1,6 @@
 """Oracle: row-invariant log-softmax + target gather (reference ops/logprobs/rowinv.py:136-245,547-570).
 
-Pinned by (tests/test_oracle_logprobs.py): fp64 ``x_t - logsumexp(x)`` truth on random and
+Pinned by (tests/test_oracle_dense.py): fp64 ``x_t - logsumexp(x)`` truth on random and
 adversarial rows (the reference's own probe, rowinv_gpu.py:112-131 and tolerance rowinv.py:21-22);
 the closed form for a constant row (S == V exactly); ``combine_order`` against the schedule the
 reference documents for G=8 (pik/plan.py:104-119); invariance to row count and to which rows

@@ -5,7 +5,7 @@ products, one bf16 round).
 The fp32 accumulation ORDER inside a matrix instruction is hardware-defined, so this function is
 a tolerance reference only: products of bf16 values are exact in fp32, and the result of any
 accumulation order lies within the bound ``gemm_tolerance`` of the float64 sum. Pinned by
-(tests/test_oracle_mm.py and the GPU tests): ``numpy.matmul`` in float64; the exact-arithmetic
+(tests/test_oracle_dense.py and the GPU tests): ``numpy.matmul`` in float64; the exact-arithmetic
 special case (small-integer operands make every partial sum exact, so every order gives the same
 bits: a bit-exact known answer); row m independent of M.
 """

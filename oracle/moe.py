@@ -2,7 +2,7 @@
 ops/moe/moe_router_o2_kernel.py:87-174,369-397; ops/moe/moe_batched_experts.py:496-503;
 ops/moe/moe_batch_invariant.py:276-320; ops/moe/moe_combine_kernel.py:36-76).
 
-Pinned by (tests/test_oracle_moe.py): ``torch.topk`` / ``torch.softmax`` on CPU for the router
+Pinned by (tests/test_oracle_gdn_moe.py): ``torch.topk`` / ``torch.softmax`` on CPU for the router
 (mode 1 is the HF Qwen3-MoE form: softmax over all experts, top-k, renormalise); tie and NaN
 cases from the reference kernel's comments (lowest index wins, NaN -> -inf); the eager
 ``argsort(stable)`` permutation of ``ref_permute_index``; a brute-force per-expert loop with

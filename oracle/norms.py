@@ -2,7 +2,7 @@
 ops/norms/fused_outnorm.py:113-232, ops/norms/zero_centered_norm.py:36-37,
 runtimes/megatron/gdn_fla_shim.py:390-425).
 
-Pinned by (tests/test_oracle_norms.py): ``torch.nn.functional.rms_norm`` on CPU plus the bf16
+Pinned by (tests/test_oracle_dense.py): ``torch.nn.functional.rms_norm`` on CPU plus the bf16
 rounds of the eager expression (a library routine, <= 1 bf16 ulp apart because its fp32 sum runs
 in another order); an fp64 brute force on tiny rows; invariance of a row's bits to the row count.
 """

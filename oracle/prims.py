@@ -10,7 +10,7 @@ F32 = np.float32
 
 def round_bf16(x: np.ndarray) -> np.ndarray:
     """fp32 -> bf16 (round to nearest even, NaN -> 0x7fc0) -> fp32. Pinned against
-    ``torch.Tensor.to(torch.bfloat16)`` in tests/test_oracle_prims.py."""
+    ``torch.Tensor.to(torch.bfloat16)`` in tests/test_oracle_dense.py."""
     x = np.ascontiguousarray(x, dtype=np.float32)
     u = x.view(np.uint32).astype(np.uint64)
     nan = (u & 0x7FFFFFFF) > 0x7F800000

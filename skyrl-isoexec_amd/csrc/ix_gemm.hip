@@ -69,9 +69,6 @@ __global__ __launch_bounds__((WM * WN + PW) * 64) void k_gemm_bf16_nt(const bf16
   extern __shared__ __align__(16) char ix_lds[];
   int tm, tn;
   if (!ix_tile_of_block(blockIdx.x, nb_m, nb_n, &tm, &tn)) return;
-#ifdef IX_EXPERIMENT_SAME_TILE
-  tm = 0; tn = tn & 7;
-#endif
   const long m0 = (long)tm * BM;
   const long n0 = (long)tn * BN;
   const int m_valid = (int)min((long)BM, (long)M - m0);
@@ -85,16 +82,6 @@ __global__ __launch_bounds__((WM * WN + PW) * 64) void k_gemm_bf16_nt(const bf16
 
   ix_f32x16 acc[Cfg::MI][Cfg::NI];
   ix_acc_zero<Cfg>(acc);
-#ifdef IX_EXPERIMENT_RANDOM_LDS
-  {  // fill the whole LDS allocation with pseudo-random bf16 of magnitude ~1 (timing experiments without the fetch)
-    uint32_t h = (threadIdx.x + 1) * 2654435761u + blockIdx.x * 40503u;
-    for (int i = threadIdx.x; i < Cfg::LDS_BYTES / 4; i += Cfg::NTT) {
-      h ^= h << 13; h ^= h >> 17; h ^= h << 5;
-      reinterpret_cast<uint32_t*>(ix_lds)[i] = (h & 0x807f807fu) | 0x3f003f00u;
-    }
-    __syncthreads();
-  }
-#endif
   ix_gemm_mainloop<Cfg>(x_rsrc, x_row, w_rsrc, w_row, K, ix_lds, acc);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;

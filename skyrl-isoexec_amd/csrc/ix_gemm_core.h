@@ -27,13 +27,6 @@ typedef __attribute__((ext_vector_type(16))) float ix_f32x16;
 typedef __attribute__((address_space(3))) void ix_lds_void;
 
 #define IX_BK 64
-// Differential-profiling switches, never defined by the Makefile: IX_EXPERIMENT_NO_DMA drops the memory -> LDS
-// fetches, IX_EXPERIMENT_NO_FRAG the LDS fragment reads, IX_EXPERIMENT_NO_MFMA the matrix instructions (results are
-// then meaningless; only the timing of what remains is of interest), IX_EXPERIMENT_NO_VMWAIT the wait for the
-// fetched units before each barrier (unit ring), IX_EXPERIMENT_SAME_TILE (dense kernel) points
-// every workgroup at the same few tiles so that all fetches hit L2, IX_EXPERIMENT_RANDOM_LDS (dense kernel) fills the
-// LDS with random bf16 before the loop (for timing the loop without the fetch on realistic operand values),
-// IX_NO_UNIT_RING selects the half-tile ring for square tiles.
 #define IX_OOB 0x7FFFF000u  // a byte offset no buffer descriptor here admits (all are < 1 GiB)
 
 // LDS tiles are [rows][k] bf16 with the 16-byte chunks of a row permuted by an XOR swizzle so that
@@ -74,7 +67,6 @@ struct IxGemmCfg {
   static constexpr int HALF_STAGES =
       (IX_HALF_STAGES_MAX * (STAGE_BYTES / 2) <= 160 * 1024) ? IX_HALF_STAGES_MAX : 4;
   // Square tiles may instead use a ring of whole-k-tile operand units (pipeline C).
-#ifndef IX_NO_UNIT_RING
   // Five units (the two being consumed, three in flight) for every square tile: the 256-row tile fills the LDS
   // with them, and the 128-row tile's 80 KiB let two workgroups share a CU, each behind its own barrier (measured:
   // +27 % over nine units and one workgroup per CU).
@@ -83,10 +75,6 @@ struct IxGemmCfg {
 #endif
   static constexpr int UNITS = (160 * 1024) / (BM * 128) > IX_UNITS_MAX ? IX_UNITS_MAX : (160 * 1024) / (BM * 128);
   static constexpr bool UNIT_RING = BM == BN && UNITS >= 5 && X_CH >= 1;
-#else
-  static constexpr int UNITS = 0;
-  static constexpr bool UNIT_RING = false;
-#endif
   // Pipeline D (fetching waves): as many whole stages as fit in 144 KiB; a small tile stops at
   // IX_SPLIT_STAGES_SMALL so that two workgroups share a CU.
 #ifndef IX_SPLIT_STAGES_SMALL
@@ -121,9 +109,6 @@ __device__ __forceinline__ ix_rsrc_t ix_make_rsrc(const void* base, uint32_t byt
 // every LDS read, and the ring of stages below relies on waiting only for the oldest group
 // (explicit s_waitcnt vmcnt(N); vector loads retire in order).
 __device__ __forceinline__ void ix_dma16(ix_rsrc_t rsrc, uint32_t lds_addr, uint32_t voff, int soff) {
-#ifdef IX_EXPERIMENT_NO_DMA
-  return;
-#endif
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                :
                : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
@@ -284,10 +269,6 @@ __device__ __forceinline__ void ix_gemm_mainloop_h4(ix_rsrc_t x_rsrc, const XRow
     for (int ni = 0; ni < Cfg::NI; ++ni) wf[ni] = *reinterpret_cast<const ix_bf16x8*>(sb + (w_foff[ni] ^ (ls << 4)));
   };
   auto mfmas = [&](const ix_bf16x8* xf, const ix_bf16x8* wf) {
-#ifdef IX_EXPERIMENT_NO_MFMA
-    asm volatile("" ::"v"(xf[0]), "v"(wf[0]));
-    return;
-#endif
 #pragma unroll
     for (int mi = 0; mi < Cfg::MI; ++mi)
 #pragma unroll
@@ -367,19 +348,12 @@ __device__ __forceinline__ void ix_gemm_mainloop_units(ix_rsrc_t x_rsrc, const X
 
   ix_bf16x8 xa[Cfg::MI], wa[Cfg::NI], xb[Cfg::MI], wb[Cfg::NI];
   auto frags = [&](const char* xs, const char* ws, int s, ix_bf16x8* xf, ix_bf16x8* wf) {
-#ifdef IX_EXPERIMENT_NO_FRAG
-    return;
-#endif
 #pragma unroll
     for (int mi = 0; mi < Cfg::MI; ++mi) xf[mi] = *reinterpret_cast<const ix_bf16x8*>(xs + (x_foff[mi] ^ (s << 4)));
 #pragma unroll
     for (int ni = 0; ni < Cfg::NI; ++ni) wf[ni] = *reinterpret_cast<const ix_bf16x8*>(ws + (w_foff[ni] ^ (s << 4)));
   };
   auto mfmas = [&](const ix_bf16x8* xf, const ix_bf16x8* wf) {
-#ifdef IX_EXPERIMENT_NO_MFMA
-    asm volatile("" ::"v"(xf[0]), "v"(wf[0]));
-    return;
-#endif
 #pragma unroll
     for (int mi = 0; mi < Cfg::MI; ++mi)
 #pragma unroll
@@ -397,9 +371,7 @@ __device__ __forceinline__ void ix_gemm_mainloop_units(ix_rsrc_t x_rsrc, const X
   int cs = 0;            // slot of the W unit being consumed
   int nu = NU - 2;       // index of the next unit to issue
   for (int kt = 0; kt < KT; ++kt) {
-#ifndef IX_EXPERIMENT_NO_VMWAIT
     __builtin_amdgcn_s_waitcnt(IX_VMCNT((NU - 4) * CH));  // units 2kt and 2kt+1 have landed
-#endif
     __syncthreads();
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
