@@ -53,6 +53,15 @@ __device__ __forceinline__ uint32_t ix_pack_bf2_hw(float lo, float hi) {
   return *reinterpret_cast<const uint32_t*>(&r);
 }
 
+// One value through the same instruction (the other half is a constant zero).
+__device__ __forceinline__ bf16_t ix_f2bf_hw(float f) { return (bf16_t)(ix_pack_bf2_hw(f, 0.0f) & 0xffffu); }
+// bf16-round two floats and widen them back: three instructions for the pair.
+__device__ __forceinline__ void ix_rbf2_hw(float a, float b, float& ra, float& rb) {
+  const uint32_t u = ix_pack_bf2_hw(a, b);
+  ra = __uint_as_float(u << 16);
+  rb = __uint_as_float(u & 0xffff0000u);
+}
+
 // ---- the transcendental primitives -------------------------------------------------------
 // One definition each; every kernel of an op family calls these and nothing else, so prefill
 // and decode, M=1 and M=4096, see the same function. ix_prim_unary (ix_prims.hip) exports

@@ -90,53 +90,76 @@ __global__ __launch_bounds__((WM * WN + PW) * 64) void k_gemm_bf16_nt(const bf16
   float rmax[Cfg::MI];
   // A whole bf16 tile with 16-byte aligned rows takes the wide stores (same values, same places).
   const bool wide = sizeof(TC) == 2 && m_valid == BM && n_valid == BN && (ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(C) % 16 == 0);
+  // Compile-time indices throughout: a rolled loop over mi would index the accumulators dynamically and push them to
+  // memory. The whole-tile path is instantiated with and without a bias: at 256 values per lane the epilogue is bound by
+  // vector-ALU issue, not by the stores (the row maximum costs three instructions per four values and is always taken).
 #pragma unroll
-  for (int mi = 0; mi < Cfg::MI; ++mi) {
-    rmax[mi] = IX_NEG_INF;
-    if (!computes) continue;
-    const long m = m0 + wm * Cfg::TM + mi * 32 + (lane & 31);
-#pragma unroll
-    for (int ni = 0; ni < Cfg::NI; ++ni) {
-      if (wide) {
+  for (int mi = 0; mi < Cfg::MI; ++mi) rmax[mi] = IX_NEG_INF;
+  if constexpr (Cfg::MI * Cfg::NI == 16) {
+    // the matrix pipeline has drained before the accumulation registers are read by hand below
+    asm volatile("s_nop 15\n\ts_nop 15");
+  }
+  auto whole_tile = [&](auto has_bias_c) {
+    constexpr bool HAS_BIAS = decltype(has_bias_c)::value;
+    ix_static_for<0, Cfg::MI>([&](auto mic) {
+      constexpr int mi = decltype(mic)::value;
+      const long m = m0 + wm * Cfg::TM + mi * 32 + (lane & 31);
+      ix_static_for<0, Cfg::NI>([&](auto nic) {
+        constexpr int ni = decltype(nic)::value;
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
           uint2 pk[2];
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
             const int q = 2 * p + h;
-            const long n = n0 + wn * Cfg::TN + ni * 32 + ix_acc_row(q * 4, lane);
             float v[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              v[e] = acc[mi][ni][q * 4 + e];
-              if (bias) v[e] = v[e] + ix_bf2f(bias[n + e]);
-              rmax[mi] = fmaxf(rmax[mi], v[e]);
+            for (int e = 0; e < 4; ++e) v[e] = ix_acc_read<(Cfg::MI * Cfg::NI == 16)>(acc[mi][ni], q * 4 + e);
+            if constexpr (HAS_BIAS) {
+              const long n = n0 + wn * Cfg::TN + ni * 32 + ix_acc_row(q * 4, lane);
+              const uint2 b4 = *reinterpret_cast<const uint2*>(bias + n);  // n % 4 == 0 and bias is 8-byte aligned
+              v[0] = v[0] + __uint_as_float(b4.x << 16);
+              v[1] = v[1] + __uint_as_float(b4.x & 0xffff0000u);
+              v[2] = v[2] + __uint_as_float(b4.y << 16);
+              v[3] = v[3] + __uint_as_float(b4.y & 0xffff0000u);
             }
-            pk[h].x = ix_pack_bf2(v[0], v[1]);
-            pk[h].y = ix_pack_bf2(v[2], v[3]);
+            rmax[mi] = fmaxf(rmax[mi], fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
+            pk[h].x = ix_pack_bf2_hw(v[0], v[1]);
+            pk[h].y = ix_pack_bf2_hw(v[2], v[3]);
           }
           const uint4 w = ix_join_halves(pk[0], pk[1]);
           const long n = n0 + wn * Cfg::TN + ni * 32 + 16 * p + (lane >> 5) * 8;
           *reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(C) + m * ldc + n) = w;
         }
-        continue;
-      }
+      });
+    });
+  };
+  if (!computes) {
+  } else if (wide && (!bias || (reinterpret_cast<uintptr_t>(bias) % 8 == 0))) {
+    if (bias) whole_tile(std::true_type{}); else whole_tile(std::false_type{});
+  } else {
+    ix_static_for<0, Cfg::MI>([&](auto mic) {
+      constexpr int mi = decltype(mic)::value;
+      const long m = m0 + wm * Cfg::TM + mi * 32 + (lane & 31);
+      ix_static_for<0, Cfg::NI>([&](auto nic) {
+        constexpr int ni = decltype(nic)::value;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const long n = n0 + wn * Cfg::TN + ni * 32 + ix_acc_row(q * 4, lane);
-        const int valid = (int)min(4L, (long)N - n);
-        if (valid <= 0 || m >= M) continue;
-        float v[4];
+        for (int q = 0; q < 4; ++q) {
+          const long n = n0 + wn * Cfg::TN + ni * 32 + ix_acc_row(q * 4, lane);
+          const int valid = (int)min(4L, (long)N - n);
+          if (valid <= 0 || m >= M) continue;
+          float v[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          v[e] = acc[mi][ni][q * 4 + e];
-          // addmm: the bias joins in fp32 before the single bf16 round.
-          if (bias && e < valid) v[e] = v[e] + ix_bf2f(bias[n + e]);
-          if (e < valid) rmax[mi] = fmaxf(rmax[mi], v[e]);
+          for (int e = 0; e < 4; ++e) {
+            v[e] = acc[mi][ni][q * 4 + e];
+            // addmm: the bias joins in fp32 before the single bf16 round.
+            if (bias && e < valid) v[e] = v[e] + ix_bf2f(bias[n + e]);
+            if (e < valid) rmax[mi] = fmaxf(rmax[mi], v[e]);
+          }
+          ix_store4(C + m * ldc + n, valid, vec_store != 0, v);
         }
-        ix_store4(C + m * ldc + n, valid, vec_store != 0, v);
-      }
-    }
+      });
+    });
   }
   if (row_max_parts) {
     float* s_max = reinterpret_cast<float*>(ix_lds);  // [WN][BM]

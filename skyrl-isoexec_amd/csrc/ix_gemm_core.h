@@ -21,6 +21,7 @@
 // has no branches.
 #pragma once
 #include "ix_common.h"
+#include <type_traits>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 ix_bf16x8;
 typedef __attribute__((ext_vector_type(16))) float ix_f32x16;
@@ -406,6 +407,134 @@ __device__ __forceinline__ void ix_gemm_mainloop_units(ix_rsrc_t x_rsrc, const X
   __builtin_amdgcn_s_waitcnt(IX_VMCNT(0));
 }
 
+// Compile-time loop: f(integral_constant<int, I>) for I = B .. E-1, so that every index derived from I is a constant
+// expression where it is used (arrays indexed this way are split into registers before any loop is unrolled).
+template <int B, int E, typename F>
+__device__ __forceinline__ void ix_static_for(F&& f) {
+  if constexpr (B < E) {
+    f(std::integral_constant<int, B>{});
+    ix_static_for<B + 1, E>(f);
+  }
+}
+
+// ---- pipeline E: four waves, one per SIMD, 128 x 128 per wave, statically interleaved ------------------------------
+// The 256 x 256 tile on four waves reads a third less from LDS than on eight (each fragment feeds four matrix
+// instructions instead of two or four), but a lone wave per SIMD has nobody to hide its fetch bursts and LDS latencies
+// behind. So the k-tile is written as four phases of 16 matrix instructions, and after each matrix instruction
+// exactly one other instruction is placed: one of the 8 fragment reads for the NEXT phase, or one of the 16 fetches
+// of the k-tile (unit ring of pipeline C: five units, W two k-tiles ahead, X one). The phase that follows the barrier
+// multiplies the last quarter of the previous k-tile while the first fragments of the new one travel from LDS.
+// Same K order as every other pipeline.
+template <typename Cfg, typename XRow, typename WRow, typename Acc>
+__device__ __forceinline__ void ix_gemm_mainloop_units4(ix_rsrc_t x_rsrc, const XRow& x_row,
+                                                        ix_rsrc_t w_rsrc, const WRow& w_row, int K,
+                                                        char* lds, Acc& acc) {
+  constexpr int NT = Cfg::NT, CH = Cfg::X_CH, UNIT = Cfg::BM * 128, NU = 5;
+  static_assert(Cfg::BM == Cfg::BN && Cfg::MI == 4 && Cfg::NI == 4 && CH == 8 && Cfg::UNITS == NU,
+                "four waves of 128 x 128 over a 256 x 256 tile");
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+  const int KT = (K + IX_BK - 1) / IX_BK;
+  const uint32_t lds_base = __builtin_amdgcn_readfirstlane(ix_lds_addr(lds) + (wave * 64) * 16);
+  const int K2 = K * 2;
+
+  uint32_t x_voff[CH], w_voff[CH];
+  int kb[CH];
+#pragma unroll
+  for (int j = 0; j < CH; ++j) {
+    const int r = (tid + j * NT) >> 3;
+    kb[j] = ((tid & 7) ^ ix_swz8(r)) * 16;
+    x_voff[j] = x_row(r) + kb[j];
+    w_voff[j] = w_row(r) + kb[j];
+  }
+  // chunk j of the X (or W) rows of k-tile t into ring slot `slot`
+  auto fetch = [&](bool is_x, int t, int slot, int j) {
+    const int soff = t * (IX_BK * 2);
+    const uint32_t dead = (uint32_t)((K2 - 1 - (soff + kb[j])) >> 31) & IX_OOB;
+    if (is_x) ix_dma16(x_rsrc, lds_base + slot * UNIT + j * NT * 16, x_voff[j] | dead, soff);
+    else ix_dma16(w_rsrc, lds_base + slot * UNIT + j * NT * 16, w_voff[j] | dead, soff);
+  };
+  const int frow = lane & 31, fg = lane >> 5;
+  int x_foff[4], w_foff[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    x_foff[i] = ix_lds_off(wm * Cfg::TM + i * 32 + frow, fg * 4);
+    w_foff[i] = ix_lds_off(wn * Cfg::TN + i * 32 + frow, fg * 4);
+  }
+  ix_bf16x8 fa[8], fb[8];  // [0..3] activation fragments, [4..7] weight fragments; two buffers
+#define IX_READ_FRAG(F, XS, WS, S, I)                                                                   \
+  F[I] = (I) < 4 ? *reinterpret_cast<const ix_bf16x8*>((XS) + (x_foff[(I) & 3] ^ ((S) << 4)))          \
+                 : *reinterpret_cast<const ix_bf16x8*>((WS) + (w_foff[(I) & 3] ^ ((S) << 4)))
+#define IX_MFMA(F, J)                                                                                   \
+  acc[(J) >> 2][(J) & 3] =                                                                              \
+      __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[4 + ((J) & 3)], F[(J) >> 2], acc[(J) >> 2][(J) & 3], 0, 0, 0)
+
+  // One phase: 16 matrix instructions on fragment buffer FM; after the even ones a fragment read of step S of the
+  // k-tile at (XS, WS) into buffer FR (x0, w0..w3, x1..x3: the order in which the next phase needs them), after
+  // instructions 1, 5, 9, 13 one fetch (chunks J0..J0+3 of the X or W rows of k-tile T into ring slot SLOT).
+#define IX_PHASE(FM, FR, XS, WS, S, IS_X, T, SLOT, J0)                                                  \
+  ix_static_for<0, 16>([&](auto jc) {                                                                   \
+    constexpr int j = decltype(jc)::value;                                                              \
+    IX_MFMA(FM, j);                                                                                     \
+    __builtin_amdgcn_sched_barrier(0);                                                                  \
+    if constexpr ((j & 1) == 0) {                                                                       \
+      constexpr int f = (j >> 1) == 0 ? 0 : ((j >> 1) <= 4 ? 3 + (j >> 1) : (j >> 1) - 4);              \
+      IX_READ_FRAG(FR, XS, WS, S, f);                                                                   \
+    } else if constexpr ((j & 3) == 1) {                                                                \
+      fetch(IS_X, T, SLOT, (J0) + (j >> 2));                                                            \
+    }                                                                                                   \
+    __builtin_amdgcn_sched_barrier(0);                                                                  \
+  })
+
+  // units in ring order: W(0), X(0), W(1), X(1), ...; the prologue fetches the first three and half of the fourth
+#pragma unroll
+  for (int j = 0; j < CH; ++j) fetch(false, 0, 0, j);
+#pragma unroll
+  for (int j = 0; j < CH; ++j) fetch(true, 0, 1, j);
+#pragma unroll
+  for (int j = 0; j < CH; ++j) fetch(false, 1, 2, j);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) fetch(true, 1, 3, j);
+  int slot = 3;  // ring slot of X(kt + 1)
+  __builtin_amdgcn_s_waitcnt(IX_VMCNT(CH + 4));  // units 0 and 1 have landed
+  __syncthreads();
+  int cs = 0;  // slot of the W unit of the k-tile being read
+  {
+    const char* ws = lds;
+    const char* xs = lds + UNIT;
+    ix_static_for<0, 8>([&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      IX_READ_FRAG(fa, xs, ws, 0, i);
+    });
+  }
+  for (int kt = 0; kt < KT; ++kt) {
+    const char* ws = lds + cs * UNIT;
+    const int xsl = cs + 1 == NU ? 0 : cs + 1;
+    const char* xs = lds + xsl * UNIT;
+    cs = xsl + 1 == NU ? 0 : xsl + 1;
+    const int slot_x = slot, slot_w = slot + 1 == NU ? 0 : slot + 1;  // X(kt+1), W(kt+2)
+    slot = slot_w + 1 == NU ? 0 : slot_w + 1;                         // X(kt+2): the slot W(kt) leaves
+    IX_PHASE(fa, fb, xs, ws, 1, true, kt + 1, slot_x, 4);   // multiply step 0, read step 1
+    IX_PHASE(fb, fa, xs, ws, 2, false, kt + 2, slot_w, 0);  // multiply step 1, read step 2
+    IX_PHASE(fa, fb, xs, ws, 3, false, kt + 2, slot_w, 4);  // multiply step 2, read step 3
+    // Every fragment of this k-tile is in registers (so its two slots may be overwritten by whoever passes the
+    // barrier first), and all fetches but the last eight (the W rows of k-tile kt+2) have landed: k-tile kt+1 is
+    // complete.
+    __builtin_amdgcn_s_waitcnt(IX_VMCNT(CH) & 0xF0FF);  // also lgkmcnt(0)
+    __syncthreads();
+    // multiply step 3 while the first fragments of the next k-tile travel from LDS (past the end: stale bytes that
+    // nothing multiplies)
+    const char* ws1 = lds + cs * UNIT;
+    const char* xs1 = lds + (cs + 1 == NU ? 0 : cs + 1) * UNIT;
+    IX_PHASE(fb, fa, xs1, ws1, 0, true, kt + 2, slot, 0);
+  }
+#undef IX_PHASE
+#undef IX_READ_FRAG
+#undef IX_MFMA
+  __builtin_amdgcn_s_waitcnt(IX_VMCNT(0));
+}
+
 // ---- pipeline D: fetching waves and computing waves (small tiles) -----------------------------------------------
 // A tile with one or two MFMAs per wave and step is bound by instruction issue (a lone wave issues one instruction
 // every four cycles, and a k-tile costs it the fetch instructions, the ring bookkeeping, the LDS reads and the
@@ -508,6 +637,8 @@ __device__ __forceinline__ void ix_gemm_mainloop(ix_rsrc_t x_rsrc, const XRow& x
                                                  Acc& acc) {
   if constexpr (Cfg::PW > 0)
     ix_gemm_mainloop_split<Cfg>(x_rsrc, x_row, w_rsrc, w_row, K, lds, acc);
+  else if constexpr (Cfg::UNIT_RING && Cfg::NT == 256 && Cfg::MI == 4 && Cfg::NI == 4)
+    ix_gemm_mainloop_units4<Cfg>(x_rsrc, x_row, w_rsrc, w_row, K, lds, acc);
   else if constexpr (Cfg::UNIT_RING)
     ix_gemm_mainloop_units<Cfg>(x_rsrc, x_row, w_rsrc, w_row, K, lds, acc);
   else if constexpr (Cfg::HALF_RING)
@@ -526,6 +657,20 @@ __device__ __forceinline__ void ix_acc_zero(Acc& acc) {
       for (int i = 0; i < 16; ++i) acc[mi][ni][i] = 0.0f;
 }
 
+// Element e of an accumulator block. With 256 accumulator registers per lane (four waves on a 256 x 256 tile) the
+// blocks live in the accumulation registers; read there, at the point of use, a value goes straight into a vector
+// register instead of being copied out early and spilled by the register allocator.
+template <bool FROM_AGPR>
+__device__ __forceinline__ float ix_acc_read(const ix_f32x16& a, int e) {
+  if constexpr (FROM_AGPR) {
+    float r;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(r) : "a"(a[e]));
+    return r;
+  } else {
+    return a[e];
+  }
+}
+
 // A 32x32 accumulator holds, for the token of this lane, output columns (i/4)*8 + hf*4 + i%4. For the column
 // blocks q = 2p and 2p+1 the two half-waves swap one packed pair each, after which the lower half holds columns
 // 16p .. 16p+7 and the upper half 16p+8 .. 16p+15 of the token: one 16-byte store per lane instead of two
@@ -536,18 +681,20 @@ __device__ __forceinline__ uint4 ix_join_halves(uint2 lo, uint2 hi) {
   return make_uint4(x[0], y[0], x[1], y[1]);
 }
 
-// Store 4 consecutive output columns of one token (8 bytes when aligned and in range).
+// Store 4 consecutive output columns of one token (8 bytes when aligned and in range). Rounding is the hardware
+// pack-convert everywhere in the GEMM epilogues (round to nearest even; a NaN stays a NaN and keeps its payload),
+// so that wide and narrow stores of the same value give the same bits.
 __device__ __forceinline__ void ix_store4_bf16(bf16_t* __restrict__ p, int valid, bool vec, float a, float b,
                                                float c, float d) {
   if (vec && valid >= 4) {
     uint2 u;
-    u.x = ix_pack_bf2(a, b);
-    u.y = ix_pack_bf2(c, d);
+    u.x = ix_pack_bf2_hw(a, b);
+    u.y = ix_pack_bf2_hw(c, d);
     *reinterpret_cast<uint2*>(p) = u;
   } else {
-    if (valid > 0) p[0] = ix_f2bf(a);
-    if (valid > 1) p[1] = ix_f2bf(b);
-    if (valid > 2) p[2] = ix_f2bf(c);
-    if (valid > 3) p[3] = ix_f2bf(d);
+    if (valid > 0) p[0] = ix_f2bf_hw(a);
+    if (valid > 1) p[1] = ix_f2bf_hw(b);
+    if (valid > 2) p[2] = ix_f2bf_hw(c);
+    if (valid > 3) p[3] = ix_f2bf_hw(d);
   }
 }

@@ -672,8 +672,18 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc1_glu(const bf16_t* __res
   // the wave's 32 columns all exist and rows are 16-byte aligned: two half-waves join their column blocks into
   // 16-byte stores (same values, same places)
   const bool wide = n0h + wn * 32 + 32 <= F && (reinterpret_cast<uintptr_t>(inter) % 16 == 0);
-#pragma unroll
-  for (int mi = 0; mi < Cfg::MI; ++mi) {
+  // bf16(gate), bf16(up) -> s = bf16(silu(gate)) -> h = bf16(s * up) -> bf16(h * prob), two columns at a time so that
+  // each rounding is one hardware pack-convert for the pair (round to nearest even; a NaN stays a NaN).
+  auto chain2 = [&](float g0, float g1, float u0, float u1, float prob) -> uint32_t {
+    float gate0, gate1, up0, up1, s0, s1, h0, h1;
+    ix_rbf2_hw(g0, g1, gate0, gate1);
+    ix_rbf2_hw(u0, u1, up0, up1);
+    ix_rbf2_hw(ix_silu_div(gate0), ix_silu_div(gate1), s0, s1);
+    ix_rbf2_hw(s0 * up0, s1 * up1, h0, h1);
+    return ix_pack_bf2_hw(h0 * prob, h1 * prob);
+  };
+  ix_static_for<0, Cfg::MI>([&](auto mic) {
+    constexpr int mi = decltype(mic)::value;
     const int r = wm * Cfg::TM + mi * 32 + (lane & 31);
     const bool live = r < nrows;  // the same for the two lanes that share a row
     const long m = row0 + (live ? r : 0);
@@ -685,42 +695,35 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc1_glu(const bf16_t* __res
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
           const int q = 2 * p + h;
-          float v[4];
-#pragma unroll
-          for (int c = 0; c < 4; ++c) {
-            const float gate = ix_rbf(acc[mi][0][q * 4 + c]);
-            const float up = ix_rbf(acc[mi][1][q * 4 + c]);
-            const float s = ix_rbf(ix_silu_div(gate));
-            const float h2 = ix_rbf(s * up);
-            v[c] = h2 * prob;
-          }
-          pk[h].x = ix_pack_bf2(v[0], v[1]);
-          pk[h].y = ix_pack_bf2(v[2], v[3]);
+          pk[h].x = chain2(acc[mi][0][q * 4], acc[mi][0][q * 4 + 1], acc[mi][1][q * 4], acc[mi][1][q * 4 + 1], prob);
+          pk[h].y = chain2(acc[mi][0][q * 4 + 2], acc[mi][0][q * 4 + 3], acc[mi][1][q * 4 + 2], acc[mi][1][q * 4 + 3],
+                           prob);
         }
         const uint4 w = ix_join_halves(pk[0], pk[1]);
         const int col = n0h + wn * 32 + 16 * p + (lane >> 5) * 8;
         if (live) *reinterpret_cast<uint4*>(inter + m * F + col) = w;
       }
-      continue;
+      return;
     }
-    if (!live) continue;
+    if (!live) return;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int col = n0h + wn * 32 + ix_acc_row(q * 4, lane);
       const int valid = min(4, F - col);
       if (valid <= 0) continue;
-      float v[4];
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const float gate = ix_rbf(acc[mi][0][q * 4 + c]);
-        const float up = ix_rbf(acc[mi][1][q * 4 + c]);
-        const float s = ix_rbf(ix_silu_div(gate));
-        const float h = ix_rbf(s * up);
-        v[c] = h * prob;
+      const uint32_t lo = chain2(acc[mi][0][q * 4], acc[mi][0][q * 4 + 1], acc[mi][1][q * 4], acc[mi][1][q * 4 + 1], prob);
+      const uint32_t hi = chain2(acc[mi][0][q * 4 + 2], acc[mi][0][q * 4 + 3], acc[mi][1][q * 4 + 2],
+                                 acc[mi][1][q * 4 + 3], prob);
+      bf16_t* dst = inter + m * F + col;
+      if (valid >= 4) {
+        *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);  // col % 4 == 0, F % 8 == 0, inter 16-byte aligned
+      } else {
+        if (valid > 0) dst[0] = (bf16_t)(lo & 0xffffu);
+        if (valid > 1) dst[1] = (bf16_t)(lo >> 16);
+        if (valid > 2) dst[2] = (bf16_t)(hi & 0xffffu);
       }
-      ix_store4_bf16(inter + m * F + col, valid, true, v[0], v[1], v[2], v[3]);
     }
-  }
+  });
 }
 
 template <int BM, int BN, int WM, int WN>
@@ -750,13 +753,13 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc2(const bf16_t* __restric
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WN, wn = wave % WN;
   const bool wide = n_valid == BN && (Hd % 8 == 0) && (reinterpret_cast<uintptr_t>(out) % 16 == 0);
-#pragma unroll
-  for (int mi = 0; mi < Cfg::MI; ++mi) {
+  ix_static_for<0, Cfg::MI>([&](auto mic) {
+    constexpr int mi = decltype(mic)::value;
     const int r = wm * Cfg::TM + mi * 32 + (lane & 31);
     const bool live = r < nrows;  // the same for the two lanes that share a row
     const long m = row0 + r;
-#pragma unroll
-    for (int ni = 0; ni < Cfg::NI; ++ni) {
+    ix_static_for<0, Cfg::NI>([&](auto nic) {
+      constexpr int ni = decltype(nic)::value;
       if (wide) {
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
@@ -764,16 +767,16 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc2(const bf16_t* __restric
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
             const int q = 2 * p + h;
-            pk[h].x = ix_pack_bf2(acc[mi][ni][q * 4], acc[mi][ni][q * 4 + 1]);
-            pk[h].y = ix_pack_bf2(acc[mi][ni][q * 4 + 2], acc[mi][ni][q * 4 + 3]);
+            pk[h].x = ix_pack_bf2_hw(acc[mi][ni][q * 4], acc[mi][ni][q * 4 + 1]);
+            pk[h].y = ix_pack_bf2_hw(acc[mi][ni][q * 4 + 2], acc[mi][ni][q * 4 + 3]);
           }
           const uint4 w = ix_join_halves(pk[0], pk[1]);
           const long n = n0 + wn * Cfg::TN + ni * 32 + 16 * p + (lane >> 5) * 8;
           if (live) *reinterpret_cast<uint4*>(out + m * Hd + n) = w;
         }
-        continue;
+        return;
       }
-      if (!live) continue;
+      if (!live) return;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const long n = n0 + wn * Cfg::TN + ni * 32 + ix_acc_row(q * 4, lane);
@@ -782,8 +785,8 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc2(const bf16_t* __restric
         ix_store4_bf16(out + m * Hd + n, valid, true, acc[mi][ni][q * 4], acc[mi][ni][q * 4 + 1],
                        acc[mi][ni][q * 4 + 2], acc[mi][ni][q * 4 + 3]);
       }
-    }
-  }
+    });
+  });
 }
 
 template <int BM, int BN, int WM, int WN>
