@@ -31,8 +31,11 @@ def _tree_k(t: np.ndarray) -> np.ndarray:
     return pairwise_tree(t)
 
 
-def router_topk(logits: np.ndarray, k: int, mode: int = 0, scaling: float | None = None, prims: Prims = DEFAULT):
-    """Returns ``(idx [T,k] int32 in rank order, prob [T,k] fp32)``.
+def router_topk(logits: np.ndarray, k: int, mode: int = 0, scaling: float | None = None, prims: Prims = DEFAULT,
+                forced_idx: np.ndarray | None = None):
+    """Returns ``(idx [T,k] int32 in rank order, prob [T,k] fp32)``. ``forced_idx [T,k]`` replaces the selection
+    (the winners and their rank order are taken from it; every value is still computed here), for comparing a
+    composed model whose discrete choices must be like for like.
     mode 0: top-k on logits, softmax over the winners (``ref_router_dense``);
     mode 1: softmax over all E (sum: per-lane columns e % 64 left to right over e // 64, then the
     adjacent-pairwise tree over the 64 lanes), top-k on the probabilities, renormalise."""
@@ -51,7 +54,11 @@ def router_topk(logits: np.ndarray, k: int, mode: int = 0, scaling: float | None
             z = (z + pad[:, c]).astype(F32)
         z = pairwise_tree(z)
         s = (e / z[:, None]).astype(F32)
-    idx, vals = _topk_rank(s, k)
+    if forced_idx is None:
+        idx, vals = _topk_rank(s, k)
+    else:
+        idx = np.asarray(forced_idx).astype(np.int32)
+        vals = np.take_along_axis(s, idx.astype(np.int64), axis=1)
     if mode == 0:
         p = prims.exp((vals - vals[:, :1]).astype(F32))
     else:

@@ -141,13 +141,18 @@ def combine(expert_out: torch.Tensor, p: Permutation, *, fp32_acc: bool = False)
 
 def moe_ffn_forward(x: torch.Tensor, router_weight: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, k: int, *,
                     pre_softmax: bool = False, logit_bias: torch.Tensor | None = None,
-                    scaling_factor: float | None = None, fp32_combine: bool = False, BM: int | None = None):
-    """Router GEMM (fp32) -> top-k -> permutation -> grouped experts -> combine. ``x [T, H]`` bf16."""
+                    scaling_factor: float | None = None, fp32_combine: bool = False, BM: int | None = None,
+                    routing_out: list | None = None):
+    """Router GEMM (fp32) -> top-k -> permutation -> grouped experts -> combine. ``x [T, H]`` bf16.
+    ``routing_out``: a list that receives this call's ``topk_idx [T, k]`` (for comparing composed models whose
+    discrete choices must be like for like)."""
     logits = router_gemm(x, router_weight)
     if logits is None:
         raise RuntimeError("[isoexec-amd] router GEMM declined")
     if logit_bias is not None:
         logits = logits + logit_bias  # elementwise, per token
     idx, prob, _, _ = router_topk(logits, k, pre_softmax=pre_softmax, scaling_factor=scaling_factor)
+    if routing_out is not None:
+        routing_out.append(idx)
     p = permute(idx, prob, router_weight.shape[0], BM=BM)
     return combine(experts_forward(x, w1, w2, p), p, fp32_acc=fp32_combine)

@@ -146,6 +146,8 @@ class _Blocks:
         # a debug.regions.RegionLog, or None: when set, the residual stream's per-layer outputs are digested on the
         # device as they are produced, so that two runtimes' passes over the same tokens can be compared region by region
         self.region_log = None
+        # a list, or None: when set, every mixture call appends its top-k expert ids [T, k] (layer order)
+        self.routing_log = None
 
     def _note(self, region: str, layer, out) -> None:
         if self.region_log is not None:
@@ -187,7 +189,7 @@ class _Blocks:
     def moe(self, layer: int, x: torch.Tensor) -> torch.Tensor:
         lw = self.w.layers[layer]
         return moe_ffn_forward(x, lw["router"], lw["w1"], lw["w2"], self.cfg.topk, pre_softmax=True,
-                               fp32_combine=self.cfg.moe_combine_dtype == "fp32")
+                               fp32_combine=self.cfg.moe_combine_dtype == "fp32", routing_out=self.routing_log)
 
     def run_layers(self, h: torch.Tensor, mixer) -> torch.Tensor:
         """The residual stream over all layers; ``mixer(layer, x)`` is the runtime's own part."""
