@@ -87,7 +87,18 @@ class HybridConfig:
 
 
 def _normal(shape, std, gen, device, dtype=torch.bfloat16):
-    return (torch.randn(shape, generator=gen, device=device) * std).to(dtype)
+    """N(0, std) drawn from ``gen``. A generator that lives on the host draws on the host (in pieces of at most 64 M
+    values, so the fp32 staging stays small) and the pieces are cast on the device: the values then do not depend on
+    which GPU, or which vendor's GPU, runs the model."""
+    if gen.device.type == torch.device(device).type:
+        return (torch.randn(shape, generator=gen, device=device) * std).to(dtype)
+    out = torch.empty(shape, dtype=dtype, device=device)
+    flat = out.view(-1)
+    step = 1 << 26
+    for lo in range(0, flat.numel(), step):
+        n = min(step, flat.numel() - lo)
+        flat[lo : lo + n] = (torch.randn(n, generator=gen).to(device, non_blocking=False) * std).to(dtype)
+    return out
 
 
 @dataclass
@@ -100,8 +111,8 @@ class HybridWeights:
     layers: list = field(default_factory=list)
 
     @classmethod
-    def make(cls, cfg: HybridConfig, seed: int = 0, device="cuda") -> "HybridWeights":
-        g = torch.Generator(device=device)
+    def make(cls, cfg: HybridConfig, seed: int = 0, device="cuda", host_rng: bool = False) -> "HybridWeights":
+        g = torch.Generator(device="cpu" if host_rng else device)
         g.manual_seed(seed)
         H = cfg.hidden
         w = cls(embed=_normal((cfg.vocab, H), 1.0, g, device), lm_head=_normal((cfg.vocab, H), 0.02, g, device),
