@@ -55,6 +55,15 @@ __device__ __forceinline__ void ix_store4(float* p, int valid, bool vec, const f
   }
 }
 
+#ifdef LAB_STAMPS
+__device__ unsigned long long lab_stamps[16384 * 8];
+extern "C" int lab_read_stamps(unsigned long long* host, int n) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(lab_stamps), (size_t)n * 8 * sizeof(unsigned long long));
+}
+#define LAB_STAMP(i) if (threadIdx.x == 0 && blockIdx.x < 16384) lab_stamps[blockIdx.x * 8 + (i)] = __builtin_amdgcn_s_memrealtime()
+#else
+#define LAB_STAMP(i)
+#endif
 // TC = bf16_t: C is the bf16 round of the fp32 accumulator; TC = float: the accumulator itself.
 // row_max_parts (optional): [M, parts_ld] fp32, entry (m, tn) = max over the tile's columns of the
 // values stored to C (exact, order-free), so a consumer can skip its own max pass over C.
@@ -68,6 +77,14 @@ __global__ __launch_bounds__((WM * WN + PW) * 64) void k_gemm_bf16_nt(const bf16
   using Cfg = IxGemmCfg<BM, BN, WM, WN, PW>;
   extern __shared__ __align__(16) char ix_lds[];
   int tm, tn;
+  LAB_STAMP(0);
+#ifdef LAB_STAMPS
+  if (threadIdx.x == 0 && blockIdx.x < 16384) {
+    unsigned hw = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));   // HW_REG_HW_ID, all 32 bits
+    unsigned xcc = __builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (3 << 11));  // HW_REG_XCC_ID, bits 0-3
+    lab_stamps[blockIdx.x * 8 + 7] = ((unsigned long long)xcc << 32) | hw;
+  }
+#endif
   if (!ix_tile_of_block(blockIdx.x, nb_m, nb_n, &tm, &tn)) return;
   const long m0 = (long)tm * BM;
   const long n0 = (long)tn * BN;
@@ -82,7 +99,9 @@ __global__ __launch_bounds__((WM * WN + PW) * 64) void k_gemm_bf16_nt(const bf16
 
   ix_f32x16 acc[Cfg::MI][Cfg::NI];
   ix_acc_zero<Cfg>(acc);
+  LAB_STAMP(1);
   ix_gemm_mainloop<Cfg>(x_rsrc, x_row, w_rsrc, w_row, K, ix_lds, acc);
+  LAB_STAMP(2);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WN, wn = wave % WN;
@@ -101,11 +120,15 @@ __global__ __launch_bounds__((WM * WN + PW) * 64) void k_gemm_bf16_nt(const bf16
   }
   auto whole_tile = [&](auto has_bias_c) {
     constexpr bool HAS_BIAS = decltype(has_bias_c)::value;
+    constexpr int NPIECE = Cfg::NI * 2;
+    char* buf = ix_lds + wave * ix_store_block32_lds_bytes<NPIECE>();
     ix_static_for<0, Cfg::MI>([&](auto mic) {
       constexpr int mi = decltype(mic)::value;
-      const long m = m0 + wm * Cfg::TM + mi * 32 + (lane & 31);
+      uint4 pieces[NPIECE];
       ix_static_for<0, Cfg::NI>([&](auto nic) {
         constexpr int ni = decltype(nic)::value;
+        float a16[16];
+        ix_acc_read16<(Cfg::MI * Cfg::NI == 16)>(acc[mi][ni], a16);
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
           uint2 pk[2];
@@ -114,7 +137,7 @@ __global__ __launch_bounds__((WM * WN + PW) * 64) void k_gemm_bf16_nt(const bf16
             const int q = 2 * p + h;
             float v[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = ix_acc_read<(Cfg::MI * Cfg::NI == 16)>(acc[mi][ni], q * 4 + e);
+            for (int e = 0; e < 4; ++e) v[e] = a16[q * 4 + e];
             if constexpr (HAS_BIAS) {
               const long n = n0 + wn * Cfg::TN + ni * 32 + ix_acc_row(q * 4, lane);
               const uint2 b4 = *reinterpret_cast<const uint2*>(bias + n);  // n % 4 == 0 and bias is 8-byte aligned
@@ -127,13 +150,17 @@ __global__ __launch_bounds__((WM * WN + PW) * 64) void k_gemm_bf16_nt(const bf16
             pk[h].x = ix_pack_bf2_hw(v[0], v[1]);
             pk[h].y = ix_pack_bf2_hw(v[2], v[3]);
           }
-          const uint4 w = ix_join_halves(pk[0], pk[1]);
-          const long n = n0 + wn * Cfg::TN + ni * 32 + 16 * p + (lane >> 5) * 8;
-          *reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(C) + m * ldc + n) = w;
+          pieces[ni * 2 + p] = ix_join_halves(pk[0], pk[1]);
         }
       });
+      // whole rows of the wave's TN columns per store instruction instead of 32-byte pieces of 32 rows
+      ix_store_block32_via_lds<NPIECE>(buf, pieces,
+                                       reinterpret_cast<bf16_t*>(C) + (m0 + wm * Cfg::TM + mi * 32) * ldc + n0 + wn * Cfg::TN,
+                                       ldc, 32);
     });
   };
+  // Late zero-fills of the ring by other waves' past-the-end fetches must not land on the store buffers.
+  if (wide) __syncthreads();
   if (!computes) {
   } else if (wide && (!bias || (reinterpret_cast<uintptr_t>(bias) % 8 == 0))) {
     if (bias) whole_tile(std::true_type{}); else whole_tile(std::false_type{});
@@ -161,6 +188,7 @@ __global__ __launch_bounds__((WM * WN + PW) * 64) void k_gemm_bf16_nt(const bf16
       });
     });
   }
+  LAB_STAMP(3);
   if (row_max_parts) {
     float* s_max = reinterpret_cast<float*>(ix_lds);  // [WN][BM]
     __syncthreads();                                  // every wave has left the main loop's LDS reads
@@ -211,22 +239,24 @@ static int ix_gemm_bf16_launch(const bf16_t* A, long lda, const bf16_t* W, long 
 static int ix_gemm_tile_for(long M, long N, long K, int tile) {
   if (tile != 0) return tile;
   if (M > 128 && N <= 128) return 2;  // one 128-wide column of tiles (the router's gating product)
-  // slots: workgroups resident on the chip at once; us_per_ktile: with the CU to itself / shared with a second one
-  struct Shape { int id, bm, bn; double slots, us_per_ktile, us_per_ktile_shared; };
-  // preference order on ties: larger tiles first
-  static const Shape shapes[] = {{3, 256, 256, 256.0, 1.5, 1.5},  {5, 128, 256, 256.0, 0.75, 0.75},
-                                 {2, 128, 128, 512.0, 0.6, 1.0},  {1, 32, 256, 256.0, 0.55, 0.55},
-                                 {6, 64, 32, 512.0, 0.16, 0.16}};
+  // slots: workgroups resident on the chip at once; us_per_ktile: with the CU to itself / shared with a second one;
+  // us_fixed: launch, first fetches and the store phase of one workgroup
+  struct Shape { int id, bm, bn; double slots, us_per_ktile, us_per_ktile_shared, us_fixed; };
+  // preference order on ties: larger tiles first. The 256 x 256 tile runs on four waves (id 4: a third fewer LDS reads,
+  // 1.4 us per k-tile) unless the product is short in K, where the eight-wave form's shorter store phase wins.
+  static const Shape shapes[] = {{4, 256, 256, 256.0, 1.4, 1.4, 8.0},   {5, 128, 256, 256.0, 0.75, 0.75, 6.0},
+                                 {2, 128, 128, 512.0, 0.6, 1.0, 6.0},   {1, 32, 256, 256.0, 0.55, 0.55, 6.0},
+                                 {6, 64, 32, 512.0, 0.16, 0.16, 6.0}};
   const double kt = (double)((K + 63) / 64);
   const double stream_us = (double)(N + M) * (double)K * 2.0 / 5.0e6;  // both operands once at 5 TB/s
-  int best = 3;
+  int best = 4;
   double best_cost = 1e300, big_cost = 0.0;
   for (const Shape& sh : shapes) {
     const double tiles = (double)((M + sh.bm - 1) / sh.bm) * (double)((N + sh.bn - 1) / sh.bn);
     const double waves = (double)(long)((tiles + sh.slots - 1.0) / sh.slots);
-    double cost = waves * (6.0 + kt * (tiles > 256.0 ? sh.us_per_ktile_shared : sh.us_per_ktile));
+    double cost = waves * (sh.us_fixed + kt * (tiles > 256.0 ? sh.us_per_ktile_shared : sh.us_per_ktile));
     if (cost < stream_us) cost = sh.id == 2 ? 0.9 * stream_us : stream_us;  // two workgroups per CU stream best
-    if (sh.id == 3) big_cost = cost;
+    if (sh.id == 4) big_cost = cost;
     if (cost < best_cost * 0.97) {  // a later (smaller) shape must win by a margin
       best_cost = cost;
       best = sh.id;
@@ -234,14 +264,14 @@ static int ix_gemm_tile_for(long M, long N, long K, int tile) {
   }
   // With more than half a big tile of rows, the big tile keeps its place unless another shape is clearly ahead:
   // at scale the smaller shapes pull more bytes through L2 than the per-k-tile rates above say.
-  if (M > 128 && big_cost <= 1.25 * best_cost) return 3;
+  if (M > 128 && big_cost <= 1.25 * best_cost) best = 4;
   return best;
 }
 
 // Row-max parts per row of C: one per column tile of the shape that runs.
 extern "C" long ix_gemm_bf16_n_tiles(long M, long N, long K, int tile) {
   const int t = ix_gemm_tile_for(M, N, K, tile);
-  const long bn = (t == 2) ? 128 : (t == 6) ? 32 : 256;
+  const long bn = (t == 2) ? 128 : (t == 6) ? 32 : 256;  // ids 1, 3, 4, 5 are 256 wide
   return N <= 0 ? 0 : (N + bn - 1) / bn;
 }
 

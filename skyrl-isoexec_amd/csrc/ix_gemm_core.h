@@ -419,12 +419,14 @@ __device__ __forceinline__ void ix_static_for(F&& f) {
 
 // ---- pipeline E: four waves, one per SIMD, 128 x 128 per wave, statically interleaved ------------------------------
 // The 256 x 256 tile on four waves reads a third less from LDS than on eight (each fragment feeds four matrix
-// instructions instead of two or four), but a lone wave per SIMD has nobody to hide its fetch bursts and LDS latencies
-// behind. So the k-tile is written as four phases of 16 matrix instructions, and after each matrix instruction
-// exactly one other instruction is placed: one of the 8 fragment reads for the NEXT phase, or one of the 16 fetches
-// of the k-tile (unit ring of pipeline C: five units, W two k-tiles ahead, X one). The phase that follows the barrier
-// multiplies the last quarter of the previous k-tile while the first fragments of the new one travel from LDS.
-// Same K order as every other pipeline.
+// instructions instead of two), but a lone wave per SIMD has nobody to hide behind: whenever it waits, its matrix
+// pipeline idles. So the k-tile is written as four phases of 16 matrix instructions with exactly one other
+// instruction placed after each: the 8 fragment reads of the NEXT phase after instructions 0..7, one fetch after
+// instructions 8, 10, 12, 14 (16 fetches per k-tile, evenly spread so that the four waves never hand the address
+// unit a burst). Unit ring of pipeline C: five units, W two k-tiles ahead, X one. The phase that follows the k-tile's
+// barrier multiplies the last quarter of the previous k-tile while the first fragments of the new one travel from LDS.
+// Same K order as every other pipeline. Measured on MI355X, LM head 4096 x 4096 x 151936: 3.9 ms against 4.3 ms for
+// the eight-wave form.
 template <typename Cfg, typename XRow, typename WRow, typename Acc>
 __device__ __forceinline__ void ix_gemm_mainloop_units4(ix_rsrc_t x_rsrc, const XRow& x_row,
                                                         ix_rsrc_t w_rsrc, const WRow& w_row, int K,
@@ -449,9 +451,23 @@ __device__ __forceinline__ void ix_gemm_mainloop_units4(ix_rsrc_t x_rsrc, const 
     w_voff[j] = w_row(r) + kb[j];
   }
   // chunk j of the X (or W) rows of k-tile t into ring slot `slot`
+#ifdef LAB_NO_DMA_LOOP
+  bool lab_prologue = true;
+#endif
   auto fetch = [&](bool is_x, int t, int slot, int j) {
+#ifdef LAB_NO_DMA
+    return;
+#endif
+#ifdef LAB_NO_DMA_LOOP
+    if (!lab_prologue) return;
+#endif
+#ifdef LAB_NO_DEAD
+    const int soff = min(t, KT - 1) * (IX_BK * 2);
+    const uint32_t dead = 0;
+#else
     const int soff = t * (IX_BK * 2);
     const uint32_t dead = (uint32_t)((K2 - 1 - (soff + kb[j])) >> 31) & IX_OOB;
+#endif
     if (is_x) ix_dma16(x_rsrc, lds_base + slot * UNIT + j * NT * 16, x_voff[j] | dead, soff);
     else ix_dma16(w_rsrc, lds_base + slot * UNIT + j * NT * 16, w_voff[j] | dead, soff);
   };
@@ -463,26 +479,56 @@ __device__ __forceinline__ void ix_gemm_mainloop_units4(ix_rsrc_t x_rsrc, const 
     w_foff[i] = ix_lds_off(wn * Cfg::TN + i * 32 + frow, fg * 4);
   }
   ix_bf16x8 fa[8], fb[8];  // [0..3] activation fragments, [4..7] weight fragments; two buffers
-#define IX_READ_FRAG(F, XS, WS, S, I)                                                                   \
+#ifdef LAB_NO_FRAG
+#define IX_READ_FRAG(F, XS, WS, S, I) if (lab_first) IX_READ_FRAG_(F, XS, WS, S, I)
+  bool lab_first = true;
+#else
+#define IX_READ_FRAG IX_READ_FRAG_
+#endif
+#define IX_READ_FRAG_(F, XS, WS, S, I)                                                                   \
   F[I] = (I) < 4 ? *reinterpret_cast<const ix_bf16x8*>((XS) + (x_foff[(I) & 3] ^ ((S) << 4)))          \
                  : *reinterpret_cast<const ix_bf16x8*>((WS) + (w_foff[(I) & 3] ^ ((S) << 4)))
-#define IX_MFMA(F, J)                                                                                   \
+#ifdef LAB_NO_MFMA
+#define IX_MFMA(F, J) asm volatile("" ::"v"(F[4 + ((J) & 3)]), "v"(F[(J) >> 2]))
+#elif defined(LAB_MFMA16)
+  // timing only: the same register traffic expressed as 16x16x32 instructions (two per 32x32x16: same flops)
+  typedef __attribute__((ext_vector_type(4))) float lab_f32x4;
+#define IX_MFMA(F, J)                                                                                              \
+  {                                                                                                                \
+    lab_f32x4* q_ = reinterpret_cast<lab_f32x4*>(&acc[(J) >> 2][(J) & 3]);                                         \
+    q_[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(F[4 + ((J) & 3)], F[(J) >> 2], q_[0], 0, 0, 0);                \
+    q_[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(F[4 + ((J) & 3)], F[(J) >> 2], q_[1], 0, 0, 0);                \
+  }
+#else
+#define IX_MFMA IX_MFMA_
+#endif
+#define IX_MFMA_(F, J)                                                                                   \
   acc[(J) >> 2][(J) & 3] =                                                                              \
       __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[4 + ((J) & 3)], F[(J) >> 2], acc[(J) >> 2][(J) & 3], 0, 0, 0)
 
   // One phase: 16 matrix instructions on fragment buffer FM; after the even ones a fragment read of step S of the
   // k-tile at (XS, WS) into buffer FR (x0, w0..w3, x1..x3: the order in which the next phase needs them), after
   // instructions 1, 5, 9, 13 one fetch (chunks J0..J0+3 of the X or W rows of k-tile T into ring slot SLOT).
+#if defined(LAB_SCHED_EVEN)
+#define IX_PHASE_READ_SLOT(j) (((j) & 1) == 0 ? (j) >> 1 : -1)
+#define IX_PHASE_FETCH_SLOT(j) (((j) & 3) == 1 ? (j) >> 2 : -1)
+#else
+  // fragment reads after matrix instructions 0..7, fetches after 8, 10, 12, 14: the last read is eight matrix
+  // instructions old when the k-tile's closing wait asks for it
+#define IX_PHASE_READ_SLOT(j) ((j) < 8 ? (j) : -1)
+#define IX_PHASE_FETCH_SLOT(j) ((j) >= 8 && ((j) & 1) == 0 ? ((j) - 8) >> 1 : -1)
+#endif
 #define IX_PHASE(FM, FR, XS, WS, S, IS_X, T, SLOT, J0)                                                  \
   ix_static_for<0, 16>([&](auto jc) {                                                                   \
     constexpr int j = decltype(jc)::value;                                                              \
     IX_MFMA(FM, j);                                                                                     \
     __builtin_amdgcn_sched_barrier(0);                                                                  \
-    if constexpr ((j & 1) == 0) {                                                                       \
-      constexpr int f = (j >> 1) == 0 ? 0 : ((j >> 1) <= 4 ? 3 + (j >> 1) : (j >> 1) - 4);              \
+    if constexpr (IX_PHASE_READ_SLOT(j) >= 0) {                                                         \
+      constexpr int r = IX_PHASE_READ_SLOT(j);                                                          \
+      constexpr int f = r == 0 ? 0 : (r <= 4 ? 3 + r : r - 4);                                          \
       IX_READ_FRAG(FR, XS, WS, S, f);                                                                   \
-    } else if constexpr ((j & 3) == 1) {                                                                \
-      fetch(IS_X, T, SLOT, (J0) + (j >> 2));                                                            \
+    } else if constexpr (IX_PHASE_FETCH_SLOT(j) >= 0) {                                                 \
+      fetch(IS_X, T, SLOT, (J0) + IX_PHASE_FETCH_SLOT(j));                                              \
     }                                                                                                   \
     __builtin_amdgcn_sched_barrier(0);                                                                  \
   })
@@ -496,6 +542,14 @@ __device__ __forceinline__ void ix_gemm_mainloop_units4(ix_rsrc_t x_rsrc, const 
   for (int j = 0; j < CH; ++j) fetch(false, 1, 2, j);
 #pragma unroll
   for (int j = 0; j < 4; ++j) fetch(true, 1, 3, j);
+#ifdef LAB_NO_DMA_LOOP
+#pragma unroll
+  for (int j = 4; j < CH; ++j) fetch(true, 1, 3, j);
+#pragma unroll
+  for (int j = 0; j < CH; ++j) fetch(false, 2, 4, j);
+  __builtin_amdgcn_s_waitcnt(IX_VMCNT(0));
+  lab_prologue = false;
+#endif
   int slot = 3;  // ring slot of X(kt + 1)
   __builtin_amdgcn_s_waitcnt(IX_VMCNT(CH + 4));  // units 0 and 1 have landed
   __syncthreads();
@@ -508,6 +562,9 @@ __device__ __forceinline__ void ix_gemm_mainloop_units4(ix_rsrc_t x_rsrc, const 
       IX_READ_FRAG(fa, xs, ws, 0, i);
     });
   }
+#ifdef LAB_NO_FRAG
+  lab_first = false;
+#endif
   for (int kt = 0; kt < KT; ++kt) {
     const char* ws = lds + cs * UNIT;
     const int xsl = cs + 1 == NU ? 0 : cs + 1;
@@ -521,8 +578,12 @@ __device__ __forceinline__ void ix_gemm_mainloop_units4(ix_rsrc_t x_rsrc, const 
     // Every fragment of this k-tile is in registers (so its two slots may be overwritten by whoever passes the
     // barrier first), and all fetches but the last eight (the W rows of k-tile kt+2) have landed: k-tile kt+1 is
     // complete.
+#ifndef LAB_NO_VMWAIT
     __builtin_amdgcn_s_waitcnt(IX_VMCNT(CH) & 0xF0FF);  // also lgkmcnt(0)
+#endif
+#ifndef LAB_NO_BARRIER
     __syncthreads();
+#endif
     // multiply step 3 while the first fragments of the next k-tile travel from LDS (past the end: stale bytes that
     // nothing multiplies)
     const char* ws1 = lds + cs * UNIT;
@@ -530,8 +591,12 @@ __device__ __forceinline__ void ix_gemm_mainloop_units4(ix_rsrc_t x_rsrc, const 
     IX_PHASE(fb, fa, xs1, ws1, 0, true, kt + 2, slot, 0);
   }
 #undef IX_PHASE
+#undef IX_PHASE_READ_SLOT
+#undef IX_PHASE_FETCH_SLOT
 #undef IX_READ_FRAG
 #undef IX_MFMA
+#undef IX_READ_FRAG_
+#undef IX_MFMA_
   __builtin_amdgcn_s_waitcnt(IX_VMCNT(0));
 }
 
@@ -671,6 +736,14 @@ __device__ __forceinline__ float ix_acc_read(const ix_f32x16& a, int e) {
   }
 }
 
+// All 16 values of an accumulator block, read before any of them is used: the reads are independent of each other, so a
+// lone wave issues them back to back instead of stalling on each read -> convert pair.
+template <bool FROM_AGPR>
+__device__ __forceinline__ void ix_acc_read16(const ix_f32x16& a, float (&v)[16]) {
+#pragma unroll
+  for (int e = 0; e < 16; ++e) v[e] = ix_acc_read<FROM_AGPR>(a, e);
+}
+
 // A 32x32 accumulator holds, for the token of this lane, output columns (i/4)*8 + hf*4 + i%4. For the column
 // blocks q = 2p and 2p+1 the two half-waves swap one packed pair each, after which the lower half holds columns
 // 16p .. 16p+7 and the upper half 16p+8 .. 16p+15 of the token: one 16-byte store per lane instead of two
@@ -680,6 +753,34 @@ __device__ __forceinline__ uint4 ix_join_halves(uint2 lo, uint2 hi) {
   const auto y = __builtin_amdgcn_permlane32_swap(lo.y, hi.y, false, false);
   return make_uint4(x[0], y[0], x[1], y[1]);
 }
+
+// A 32-row block of a wave's output, NPIECE * 16 columns wide, stored in whole rows. After ix_join_halves a lane holds,
+// for token row lane % 32, the 16-byte pieces i = 0 .. NPIECE-1 = columns 16 i + 8 (lane / 32) .. + 7: stored directly,
+// one instruction would touch 32 rows with 32 bytes each. Here the pieces pass through a wave-private LDS buffer
+// (32 rows of NPIECE * 32 + 16 bytes; the 16 bytes of padding spread the rows over the banks) and come back with
+// 2 NPIECE lanes per row, so that an instruction stores 64 / (2 NPIECE) whole rows of NPIECE * 32 contiguous bytes.
+// Rows at or past live_rows are not stored. dst = the block's row 0 at the wave's first column; 16-byte aligned, ld % 8
+// == 0. No barrier: only this wave touches buf, and a wave's LDS operations complete in order.
+template <int NPIECE>
+__device__ __forceinline__ void ix_store_block32_via_lds(char* buf, const uint4 (&pc)[NPIECE], bf16_t* dst, long ld,
+                                                         int live_rows) {
+  constexpr int PITCH = NPIECE * 32 + 16, CPR = NPIECE * 2, RPI = 64 / CPR;
+  static_assert(64 % CPR == 0 && 32 % RPI == 0, "pieces per row must divide the wave");
+  const int lane = threadIdx.x & 63;
+  char* mine = buf + (lane & 31) * PITCH + (lane >> 5) * 16;
+#pragma unroll
+  for (int i = 0; i < NPIECE; ++i) *reinterpret_cast<uint4*>(mine + i * 32) = pc[i];
+  const int rr = lane / CPR, cc = lane % CPR;
+#pragma unroll
+  for (int j = 0; j < 32 / RPI; ++j) {
+    const int row = j * RPI + rr;
+    const uint4 v = *reinterpret_cast<const uint4*>(buf + row * PITCH + cc * 16);
+    if (row < live_rows) *reinterpret_cast<uint4*>(dst + (long)row * ld + cc * 8) = v;
+  }
+}
+// bytes of LDS one wave needs for it
+template <int NPIECE>
+constexpr int ix_store_block32_lds_bytes() { return 32 * (NPIECE * 32 + 16); }
 
 // Store 4 consecutive output columns of one token (8 bytes when aligned and in range). Rounding is the hardware
 // pack-convert everywhere in the GEMM epilogues (round to nearest even; a NaN stays a NaN and keeps its payload),

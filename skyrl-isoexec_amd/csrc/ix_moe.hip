@@ -16,6 +16,9 @@
 // is fixed (ix_gemm_core.h).
 #include "ix_gemm_core.h"
 #include "../../include/isoexec_hip.h"
+#ifdef LAB_ENV
+#include <cstdlib>
+#endif
 
 #define IX_MOE_KMAX 16
 #define IX_MOE_EC 8  // experts per lane: E <= 512
@@ -641,7 +644,8 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc1_glu(const bf16_t* __res
                                                              const int* __restrict__ meta, int max_tiles,
                                                              bf16_t* __restrict__ inter, int Hd, int F, int nb_n) {
   using Cfg = IxGemmCfg<BM, BN, WM, WN>;
-  static_assert(Cfg::NI == 2, "a wave must hold one gate tile and its up tile");
+  static_assert(Cfg::NI % 2 == 0, "a wave must hold gate tiles and their up tiles");
+  constexpr int NP = Cfg::NI / 2;  // (gate, up) pairs of 32 columns per wave
   extern __shared__ __align__(16) char ix_lds[];
   int mt, nt;
   if (!ix_moe_tile_of_block(blockIdx.x, meta[0], nb_n, &mt, &nt)) return;
@@ -651,19 +655,20 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc1_glu(const bf16_t* __res
   const int n0h = nt * (BN / 2);
 
   // activations: gathered token rows of x; weights: the expert's [2F, Hd] fc1 matrix with the
-  // tile's rows interleaved so that each wave holds a gate tile (ni = 0) and its up tile (ni = 1):
-  // tile row r -> wave r/64, half (r/32)&1, column n0h + 32*(r/64) + r%32.
+  // tile's rows interleaved so that each wave holds NP gate tiles (ni < NP) and their up tiles (ni >= NP):
+  // tile row r -> wave r / TN, block b = (r % TN) / 32, half b / NP, column n0h + 32 * NP * wave + 32 * (b % NP) + r % 32.
   const ix_rsrc_t x_rsrc = ix_make_rsrc(x, (uint32_t)(((long)(T - 1) * ldx + Hd) * 2));
   const ix_rsrc_t w_rsrc = ix_make_rsrc(W1 + (long)e * 2 * F * Hd, (uint32_t)((long)2 * F * Hd * 2));
   auto x_row = [&](int r) -> uint32_t {
     return (r < nrows) ? (uint32_t)((long)sorted_token[row0 + r] * ldx * 2) : IX_OOB;
   };
   auto w_row = [&](int r) -> uint32_t {
-    const int col = n0h + (r >> 6) * 32 + (r & 31);
-    return (col < F) ? (uint32_t)(((long)((r >> 5) & 1) * F + col) * Hd * 2) : IX_OOB;
+    const int b = (r % Cfg::TN) >> 5;
+    const int col = n0h + (r / Cfg::TN) * (32 * NP) + (b % NP) * 32 + (r & 31);
+    return (col < F) ? (uint32_t)(((long)(b / NP) * F + col) * Hd * 2) : IX_OOB;
   };
 
-  ix_f32x16 acc[Cfg::MI][2];
+  ix_f32x16 acc[Cfg::MI][Cfg::NI];
   ix_acc_zero<Cfg>(acc);
   ix_gemm_mainloop<Cfg>(x_rsrc, x_row, w_rsrc, w_row, Hd, ix_lds, acc);
 
@@ -671,7 +676,13 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc1_glu(const bf16_t* __res
   const int wm = wave / WN, wn = wave % WN;
   // the wave's 32 columns all exist and rows are 16-byte aligned: two half-waves join their column blocks into
   // 16-byte stores (same values, same places)
-  const bool wide = n0h + wn * 32 + 32 <= F && (reinterpret_cast<uintptr_t>(inter) % 16 == 0);
+  // the same for every wave of the workgroup (a barrier depends on it): the whole tile's columns exist
+  const bool wide = n0h + BN / 2 <= F && (F % 8 == 0) && (reinterpret_cast<uintptr_t>(inter) % 16 == 0);
+  // late zero-fills of the ring by other waves' past-the-end fetches must not land on the store buffers
+  if (wide) __syncthreads();
+  char* buf = ix_lds + wave * ix_store_block32_lds_bytes<2 * NP>();
+  if constexpr (Cfg::MI * Cfg::NI == 16) asm volatile("s_nop 15\n\ts_nop 15");  // matrix pipeline drained before the
+                                                                                  // accumulation registers are read by hand
   // bf16(gate), bf16(up) -> s = bf16(silu(gate)) -> h = bf16(s * up) -> bf16(h * prob), two columns at a time so that
   // each rounding is one hardware pack-convert for the pair (round to nearest even; a NaN stays a NaN).
   auto chain2 = [&](float g0, float g1, float u0, float u1, float prob) -> uint32_t {
@@ -688,41 +699,56 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc1_glu(const bf16_t* __res
     const bool live = r < nrows;  // the same for the two lanes that share a row
     const long m = row0 + (live ? r : 0);
     const float prob = live ? permuted_prob[m] : 0.0f;
+    constexpr bool AG = Cfg::MI * Cfg::NI == 16;
     if (wide) {
+      uint4 pieces[2 * NP];
+      ix_static_for<0, NP>([&](auto cbc) {
+        constexpr int cb = decltype(cbc)::value;  // gate block cb, up block NP + cb
+        float g16[16], u16[16];
+        ix_acc_read16<AG>(acc[mi][cb], g16);
+        ix_acc_read16<AG>(acc[mi][NP + cb], u16);
+        auto G = [&](int i) { return g16[i]; };
+        auto U = [&](int i) { return u16[i]; };
 #pragma unroll
-      for (int p = 0; p < 2; ++p) {
-        uint2 pk[2];
+        for (int p = 0; p < 2; ++p) {
+          uint2 pk[2];
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const int q = 2 * p + h;
-          pk[h].x = chain2(acc[mi][0][q * 4], acc[mi][0][q * 4 + 1], acc[mi][1][q * 4], acc[mi][1][q * 4 + 1], prob);
-          pk[h].y = chain2(acc[mi][0][q * 4 + 2], acc[mi][0][q * 4 + 3], acc[mi][1][q * 4 + 2], acc[mi][1][q * 4 + 3],
-                           prob);
+          for (int h = 0; h < 2; ++h) {
+            const int q = 2 * p + h;
+            pk[h].x = chain2(G(q * 4), G(q * 4 + 1), U(q * 4), U(q * 4 + 1), prob);
+            pk[h].y = chain2(G(q * 4 + 2), G(q * 4 + 3), U(q * 4 + 2), U(q * 4 + 3), prob);
+          }
+          pieces[cb * 2 + p] = ix_join_halves(pk[0], pk[1]);
         }
-        const uint4 w = ix_join_halves(pk[0], pk[1]);
-        const int col = n0h + wn * 32 + 16 * p + (lane >> 5) * 8;
-        if (live) *reinterpret_cast<uint4*>(inter + m * F + col) = w;
-      }
+      });
+      const int first = wm * Cfg::TM + mi * 32;  // whole rows of the wave's 32 NP columns per store instruction
+      ix_store_block32_via_lds<2 * NP>(buf, pieces, inter + (row0 + first) * F + n0h + wn * (32 * NP), F,
+                                       min(32, nrows - first));
       return;
     }
     if (!live) return;
+    ix_static_for<0, NP>([&](auto cbc) {
+      constexpr int cb = decltype(cbc)::value;
+      const int c0 = n0h + wn * (32 * NP) + cb * 32;
+      auto G = [&](int i) { return ix_acc_read<AG>(acc[mi][cb], i); };
+      auto U = [&](int i) { return ix_acc_read<AG>(acc[mi][NP + cb], i); };
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int col = n0h + wn * 32 + ix_acc_row(q * 4, lane);
-      const int valid = min(4, F - col);
-      if (valid <= 0) continue;
-      const uint32_t lo = chain2(acc[mi][0][q * 4], acc[mi][0][q * 4 + 1], acc[mi][1][q * 4], acc[mi][1][q * 4 + 1], prob);
-      const uint32_t hi = chain2(acc[mi][0][q * 4 + 2], acc[mi][0][q * 4 + 3], acc[mi][1][q * 4 + 2],
-                                 acc[mi][1][q * 4 + 3], prob);
-      bf16_t* dst = inter + m * F + col;
-      if (valid >= 4) {
-        *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);  // col % 4 == 0, F % 8 == 0, inter 16-byte aligned
-      } else {
-        if (valid > 0) dst[0] = (bf16_t)(lo & 0xffffu);
-        if (valid > 1) dst[1] = (bf16_t)(lo >> 16);
-        if (valid > 2) dst[2] = (bf16_t)(hi & 0xffffu);
+      for (int q = 0; q < 4; ++q) {
+        const int col = c0 + ix_acc_row(q * 4, lane);
+        const int valid = min(4, F - col);
+        if (valid <= 0) continue;
+        const uint32_t lo = chain2(G(q * 4), G(q * 4 + 1), U(q * 4), U(q * 4 + 1), prob);
+        const uint32_t hi = chain2(G(q * 4 + 2), G(q * 4 + 3), U(q * 4 + 2), U(q * 4 + 3), prob);
+        bf16_t* dst = inter + m * F + col;
+        if (valid >= 4) {
+          *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);  // col % 4 == 0, F % 8 == 0, inter 16-byte aligned
+        } else {
+          if (valid > 0) dst[0] = (bf16_t)(lo & 0xffffu);
+          if (valid > 1) dst[1] = (bf16_t)(lo >> 16);
+          if (valid > 2) dst[2] = (bf16_t)(hi & 0xffffu);
+        }
       }
-    }
+    });
   });
 }
 
@@ -753,30 +779,43 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc2(const bf16_t* __restric
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WN, wn = wave % WN;
   const bool wide = n_valid == BN && (Hd % 8 == 0) && (reinterpret_cast<uintptr_t>(out) % 16 == 0);
+  constexpr bool AG = Cfg::MI * Cfg::NI == 16;
+  if constexpr (AG) asm volatile("s_nop 15\n\ts_nop 15");
+  // late zero-fills of the ring by other waves' past-the-end fetches must not land on the store buffers
+  if (wide) __syncthreads();
+  constexpr int NPIECE = Cfg::NI * 2;
+  char* buf = ix_lds + wave * ix_store_block32_lds_bytes<NPIECE>();
   ix_static_for<0, Cfg::MI>([&](auto mic) {
     constexpr int mi = decltype(mic)::value;
     const int r = wm * Cfg::TM + mi * 32 + (lane & 31);
     const bool live = r < nrows;  // the same for the two lanes that share a row
     const long m = row0 + r;
-    ix_static_for<0, Cfg::NI>([&](auto nic) {
-      constexpr int ni = decltype(nic)::value;
-      if (wide) {
+    if (wide) {
+      uint4 pieces[NPIECE];
+      ix_static_for<0, Cfg::NI>([&](auto nic) {
+        constexpr int ni = decltype(nic)::value;
+        float a16[16];
+        ix_acc_read16<AG>(acc[mi][ni], a16);
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
           uint2 pk[2];
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
             const int q = 2 * p + h;
-            pk[h].x = ix_pack_bf2_hw(acc[mi][ni][q * 4], acc[mi][ni][q * 4 + 1]);
-            pk[h].y = ix_pack_bf2_hw(acc[mi][ni][q * 4 + 2], acc[mi][ni][q * 4 + 3]);
+            pk[h].x = ix_pack_bf2_hw(a16[q * 4], a16[q * 4 + 1]);
+            pk[h].y = ix_pack_bf2_hw(a16[q * 4 + 2], a16[q * 4 + 3]);
           }
-          const uint4 w = ix_join_halves(pk[0], pk[1]);
-          const long n = n0 + wn * Cfg::TN + ni * 32 + 16 * p + (lane >> 5) * 8;
-          if (live) *reinterpret_cast<uint4*>(out + m * Hd + n) = w;
+          pieces[ni * 2 + p] = ix_join_halves(pk[0], pk[1]);
         }
-        return;
-      }
-      if (!live) return;
+      });
+      const int first = wm * Cfg::TM + mi * 32;  // whole rows of the wave's TN columns per store instruction
+      ix_store_block32_via_lds<NPIECE>(buf, pieces, out + (row0 + first) * Hd + n0 + wn * Cfg::TN, Hd,
+                                       min(32, nrows - first));
+      return;
+    }
+    if (!live) return;
+    ix_static_for<0, Cfg::NI>([&](auto nic) {
+      constexpr int ni = decltype(nic)::value;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const long n = n0 + wn * Cfg::TN + ni * 32 + ix_acc_row(q * 4, lane);
@@ -845,7 +884,12 @@ extern "C" int ix_moe_experts_tile(const void* x, long ldx, const int* sorted_to
       return ix_moe_experts_launch<128, 256, 2, 4>(xx, ldx, (int)T, sorted_token, permuted_prob, w1, w2, tile_meta,
                                                    max_tiles, it, eo, (int)Hd, (int)F, st);
     case 256:
-      return ix_moe_experts_launch<256, 256, 2, 4>(xx, ldx, (int)T, sorted_token, permuted_prob, w1, w2, tile_meta,
+#ifdef LAB_ENV
+      if (getenv("IX_LAB_MOE_WAVES8"))
+        return ix_moe_experts_launch<256, 256, 2, 4>(xx, ldx, (int)T, sorted_token, permuted_prob, w1, w2, tile_meta,
+                                                     max_tiles, it, eo, (int)Hd, (int)F, st);
+#endif
+      return ix_moe_experts_launch<256, 256, 2, 2>(xx, ldx, (int)T, sorted_token, permuted_prob, w1, w2, tile_meta,
                                                    max_tiles, it, eo, (int)Hd, (int)F, st);
     default: return IX_ERR_ARG;
   }
