@@ -55,15 +55,6 @@ __device__ __forceinline__ void ix_store4(float* p, int valid, bool vec, const f
   }
 }
 
-#ifdef LAB_STAMPS
-__device__ unsigned long long lab_stamps[16384 * 8];
-extern "C" int lab_read_stamps(unsigned long long* host, int n) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(lab_stamps), (size_t)n * 8 * sizeof(unsigned long long));
-}
-#define LAB_STAMP(i) if (threadIdx.x == 0 && blockIdx.x < 16384) lab_stamps[blockIdx.x * 8 + (i)] = __builtin_amdgcn_s_memrealtime()
-#else
-#define LAB_STAMP(i)
-#endif
 // TC = bf16_t: C is the bf16 round of the fp32 accumulator; TC = float: the accumulator itself.
 // row_max_parts (optional): [M, parts_ld] fp32, entry (m, tn) = max over the tile's columns of the
 // values stored to C (exact, order-free), so a consumer can skip its own max pass over C.
@@ -77,14 +68,6 @@ __global__ __launch_bounds__((WM * WN + PW) * 64) void k_gemm_bf16_nt(const bf16
   using Cfg = IxGemmCfg<BM, BN, WM, WN, PW>;
   extern __shared__ __align__(16) char ix_lds[];
   int tm, tn;
-  LAB_STAMP(0);
-#ifdef LAB_STAMPS
-  if (threadIdx.x == 0 && blockIdx.x < 16384) {
-    unsigned hw = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));   // HW_REG_HW_ID, all 32 bits
-    unsigned xcc = __builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (3 << 11));  // HW_REG_XCC_ID, bits 0-3
-    lab_stamps[blockIdx.x * 8 + 7] = ((unsigned long long)xcc << 32) | hw;
-  }
-#endif
   if (!ix_tile_of_block(blockIdx.x, nb_m, nb_n, &tm, &tn)) return;
   const long m0 = (long)tm * BM;
   const long n0 = (long)tn * BN;
@@ -99,9 +82,7 @@ __global__ __launch_bounds__((WM * WN + PW) * 64) void k_gemm_bf16_nt(const bf16
 
   ix_f32x16 acc[Cfg::MI][Cfg::NI];
   ix_acc_zero<Cfg>(acc);
-  LAB_STAMP(1);
   ix_gemm_mainloop<Cfg>(x_rsrc, x_row, w_rsrc, w_row, K, ix_lds, acc);
-  LAB_STAMP(2);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WN, wn = wave % WN;
@@ -188,7 +169,6 @@ __global__ __launch_bounds__((WM * WN + PW) * 64) void k_gemm_bf16_nt(const bf16
       });
     });
   }
-  LAB_STAMP(3);
   if (row_max_parts) {
     float* s_max = reinterpret_cast<float*>(ix_lds);  // [WN][BM]
     __syncthreads();                                  // every wave has left the main loop's LDS reads

@@ -451,23 +451,9 @@ __device__ __forceinline__ void ix_gemm_mainloop_units4(ix_rsrc_t x_rsrc, const 
     w_voff[j] = w_row(r) + kb[j];
   }
   // chunk j of the X (or W) rows of k-tile t into ring slot `slot`
-#ifdef LAB_NO_DMA_LOOP
-  bool lab_prologue = true;
-#endif
   auto fetch = [&](bool is_x, int t, int slot, int j) {
-#ifdef LAB_NO_DMA
-    return;
-#endif
-#ifdef LAB_NO_DMA_LOOP
-    if (!lab_prologue) return;
-#endif
-#ifdef LAB_NO_DEAD
-    const int soff = min(t, KT - 1) * (IX_BK * 2);
-    const uint32_t dead = 0;
-#else
     const int soff = t * (IX_BK * 2);
     const uint32_t dead = (uint32_t)((K2 - 1 - (soff + kb[j])) >> 31) & IX_OOB;
-#endif
     if (is_x) ix_dma16(x_rsrc, lds_base + slot * UNIT + j * NT * 16, x_voff[j] | dead, soff);
     else ix_dma16(w_rsrc, lds_base + slot * UNIT + j * NT * 16, w_voff[j] | dead, soff);
   };
@@ -479,45 +465,20 @@ __device__ __forceinline__ void ix_gemm_mainloop_units4(ix_rsrc_t x_rsrc, const 
     w_foff[i] = ix_lds_off(wn * Cfg::TN + i * 32 + frow, fg * 4);
   }
   ix_bf16x8 fa[8], fb[8];  // [0..3] activation fragments, [4..7] weight fragments; two buffers
-#ifdef LAB_NO_FRAG
-#define IX_READ_FRAG(F, XS, WS, S, I) if (lab_first) IX_READ_FRAG_(F, XS, WS, S, I)
-  bool lab_first = true;
-#else
-#define IX_READ_FRAG IX_READ_FRAG_
-#endif
-#define IX_READ_FRAG_(F, XS, WS, S, I)                                                                   \
+#define IX_READ_FRAG(F, XS, WS, S, I)                                                                   \
   F[I] = (I) < 4 ? *reinterpret_cast<const ix_bf16x8*>((XS) + (x_foff[(I) & 3] ^ ((S) << 4)))          \
                  : *reinterpret_cast<const ix_bf16x8*>((WS) + (w_foff[(I) & 3] ^ ((S) << 4)))
-#ifdef LAB_NO_MFMA
-#define IX_MFMA(F, J) asm volatile("" ::"v"(F[4 + ((J) & 3)]), "v"(F[(J) >> 2]))
-#elif defined(LAB_MFMA16)
-  // timing only: the same register traffic expressed as 16x16x32 instructions (two per 32x32x16: same flops)
-  typedef __attribute__((ext_vector_type(4))) float lab_f32x4;
-#define IX_MFMA(F, J)                                                                                              \
-  {                                                                                                                \
-    lab_f32x4* q_ = reinterpret_cast<lab_f32x4*>(&acc[(J) >> 2][(J) & 3]);                                         \
-    q_[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(F[4 + ((J) & 3)], F[(J) >> 2], q_[0], 0, 0, 0);                \
-    q_[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(F[4 + ((J) & 3)], F[(J) >> 2], q_[1], 0, 0, 0);                \
-  }
-#else
-#define IX_MFMA IX_MFMA_
-#endif
-#define IX_MFMA_(F, J)                                                                                   \
+#define IX_MFMA(F, J)                                                                                   \
   acc[(J) >> 2][(J) & 3] =                                                                              \
       __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[4 + ((J) & 3)], F[(J) >> 2], acc[(J) >> 2][(J) & 3], 0, 0, 0)
 
   // One phase: 16 matrix instructions on fragment buffer FM; after the even ones a fragment read of step S of the
   // k-tile at (XS, WS) into buffer FR (x0, w0..w3, x1..x3: the order in which the next phase needs them), after
   // instructions 1, 5, 9, 13 one fetch (chunks J0..J0+3 of the X or W rows of k-tile T into ring slot SLOT).
-#if defined(LAB_SCHED_EVEN)
-#define IX_PHASE_READ_SLOT(j) (((j) & 1) == 0 ? (j) >> 1 : -1)
-#define IX_PHASE_FETCH_SLOT(j) (((j) & 3) == 1 ? (j) >> 2 : -1)
-#else
   // fragment reads after matrix instructions 0..7, fetches after 8, 10, 12, 14: the last read is eight matrix
   // instructions old when the k-tile's closing wait asks for it
 #define IX_PHASE_READ_SLOT(j) ((j) < 8 ? (j) : -1)
 #define IX_PHASE_FETCH_SLOT(j) ((j) >= 8 && ((j) & 1) == 0 ? ((j) - 8) >> 1 : -1)
-#endif
 #define IX_PHASE(FM, FR, XS, WS, S, IS_X, T, SLOT, J0)                                                  \
   ix_static_for<0, 16>([&](auto jc) {                                                                   \
     constexpr int j = decltype(jc)::value;                                                              \
@@ -542,14 +503,6 @@ __device__ __forceinline__ void ix_gemm_mainloop_units4(ix_rsrc_t x_rsrc, const 
   for (int j = 0; j < CH; ++j) fetch(false, 1, 2, j);
 #pragma unroll
   for (int j = 0; j < 4; ++j) fetch(true, 1, 3, j);
-#ifdef LAB_NO_DMA_LOOP
-#pragma unroll
-  for (int j = 4; j < CH; ++j) fetch(true, 1, 3, j);
-#pragma unroll
-  for (int j = 0; j < CH; ++j) fetch(false, 2, 4, j);
-  __builtin_amdgcn_s_waitcnt(IX_VMCNT(0));
-  lab_prologue = false;
-#endif
   int slot = 3;  // ring slot of X(kt + 1)
   __builtin_amdgcn_s_waitcnt(IX_VMCNT(CH + 4));  // units 0 and 1 have landed
   __syncthreads();
@@ -562,9 +515,6 @@ __device__ __forceinline__ void ix_gemm_mainloop_units4(ix_rsrc_t x_rsrc, const 
       IX_READ_FRAG(fa, xs, ws, 0, i);
     });
   }
-#ifdef LAB_NO_FRAG
-  lab_first = false;
-#endif
   for (int kt = 0; kt < KT; ++kt) {
     const char* ws = lds + cs * UNIT;
     const int xsl = cs + 1 == NU ? 0 : cs + 1;
@@ -578,12 +528,8 @@ __device__ __forceinline__ void ix_gemm_mainloop_units4(ix_rsrc_t x_rsrc, const 
     // Every fragment of this k-tile is in registers (so its two slots may be overwritten by whoever passes the
     // barrier first), and all fetches but the last eight (the W rows of k-tile kt+2) have landed: k-tile kt+1 is
     // complete.
-#ifndef LAB_NO_VMWAIT
     __builtin_amdgcn_s_waitcnt(IX_VMCNT(CH) & 0xF0FF);  // also lgkmcnt(0)
-#endif
-#ifndef LAB_NO_BARRIER
     __syncthreads();
-#endif
     // multiply step 3 while the first fragments of the next k-tile travel from LDS (past the end: stale bytes that
     // nothing multiplies)
     const char* ws1 = lds + cs * UNIT;
@@ -595,8 +541,6 @@ __device__ __forceinline__ void ix_gemm_mainloop_units4(ix_rsrc_t x_rsrc, const 
 #undef IX_PHASE_FETCH_SLOT
 #undef IX_READ_FRAG
 #undef IX_MFMA
-#undef IX_READ_FRAG_
-#undef IX_MFMA_
   __builtin_amdgcn_s_waitcnt(IX_VMCNT(0));
 }
 

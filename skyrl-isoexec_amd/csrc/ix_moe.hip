@@ -16,9 +16,6 @@
 // is fixed (ix_gemm_core.h).
 #include "ix_gemm_core.h"
 #include "../../include/isoexec_hip.h"
-#ifdef LAB_ENV
-#include <cstdlib>
-#endif
 
 #define IX_MOE_KMAX 16
 #define IX_MOE_EC 8  // experts per lane: E <= 512
@@ -884,11 +881,6 @@ extern "C" int ix_moe_experts_tile(const void* x, long ldx, const int* sorted_to
       return ix_moe_experts_launch<128, 256, 2, 4>(xx, ldx, (int)T, sorted_token, permuted_prob, w1, w2, tile_meta,
                                                    max_tiles, it, eo, (int)Hd, (int)F, st);
     case 256:
-#ifdef LAB_ENV
-      if (getenv("IX_LAB_MOE_WAVES8"))
-        return ix_moe_experts_launch<256, 256, 2, 4>(xx, ldx, (int)T, sorted_token, permuted_prob, w1, w2, tile_meta,
-                                                     max_tiles, it, eo, (int)Hd, (int)F, st);
-#endif
       return ix_moe_experts_launch<256, 256, 2, 2>(xx, ldx, (int)T, sorted_token, permuted_prob, w1, w2, tile_meta,
                                                    max_tiles, it, eo, (int)Hd, (int)F, st);
     default: return IX_ERR_ARG;
