@@ -117,6 +117,12 @@ int ix_gemm_bf16_nt(const void* A, long lda, const void* W, long ldw, const void
                     void* stream);
 long ix_gemm_bf16_n_tiles(long M, long N, long K, int tile);
 
+/* aten::bmm of the same override (moe_batch_invariant.py:453-464): `batch` independent products A_b [M,K] . W_b [N,K]^T
+ * -> C_b [M,N] (bf16) in ONE launch, each computed exactly as ix_gemm_bf16_nt computes it (same bits). Matrix b of an
+ * operand starts b * stride elements after matrix 0 (stride_w = 0 shares one weight). batch <= 65535. */
+int ix_gemm_bf16_nt_batched(const void* A, long lda, long stride_a, const void* W, long ldw, long stride_w, void* C,
+                            long ldc, long stride_c, long batch, long M, long N, long K, int tile, void* stream);
+
 /* Router gating GEMM (moe/_register.py:59-66): C fp32 [M,N] = A[M,K] . W[N,K]^T with W fp32 and
  * A fp32 or bf16 (a_dtype), fp32 accumulate in a fixed K order. */
 int ix_gemm_f32_nt(const void* A, int a_dtype, long lda, const void* W, long ldw, void* C, long ldc, long M,
@@ -235,6 +241,14 @@ int ix_moe_pick_bm(long T, long k, long E);               /* 32, 128 or 256 */
 int ix_moe_permute(const int* topk_idx, const float* topk_prob, long T, long E, long k, long BM, int* counts,
                    int* offsets, int* sorted_token, float* permuted_prob, int* combine_rows, int* tile_meta,
                    long max_tiles, int* scratch, void* stream);
+
+/* _block_map / fused_block_map (moe_fused_experts.py:156-205, moe_blockmap_kernel.py): the block map for rows that
+ * are ALREADY grouped by expert (SequentialMLP.forward's tokens_per_expert, moe_batched_experts.py:301-330). counts
+ * int32 or int64 [E] (counts_i64) in device memory; offsets int32 [E+1] (may be NULL) receives the exclusive scan;
+ * tile_meta as in ix_moe_permute, max_tiles >= ix_moe_max_tiles(rows, 1, E, BM). Integer work only, one launch, nothing
+ * read back by the host. */
+int ix_moe_block_map(const void* counts, int counts_i64, long E, long BM, int* offsets, int* tile_meta, long max_tiles,
+                     void* stream);
 
 /* ix_moe_permute for callers that cannot allocate device memory or bring a workspace: code under HIP graph
  * capture, tight serving loops, harnesses that forbid allocation. No counterpart in the reference (its permutation

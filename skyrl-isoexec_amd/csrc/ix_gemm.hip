@@ -64,9 +64,14 @@ __global__ __launch_bounds__((WM * WN + PW) * 64) void k_gemm_bf16_nt(const bf16
                                                               const bf16_t* __restrict__ bias,
                                                               TC* __restrict__ C, long ldc, int M, int N, int K,
                                                               int nb_m, int nb_n, int vec_store,
-                                                              float* __restrict__ row_max_parts, long parts_ld) {
+                                                              float* __restrict__ row_max_parts, long parts_ld,
+                                                              long batch_a, long batch_w, long batch_c) {
   using Cfg = IxGemmCfg<BM, BN, WM, WN, PW>;
   extern __shared__ __align__(16) char ix_lds[];
+  // a batch of independent products (bmm): workgroup row blockIdx.y works on matrices batch strides further on
+  A += (long)blockIdx.y * batch_a;
+  W += (long)blockIdx.y * batch_w;
+  C += (long)blockIdx.y * batch_c;
   int tm, tn;
   if (!ix_tile_of_block(blockIdx.x, nb_m, nb_n, &tm, &tn)) return;
   const long m0 = (long)tm * BM;
@@ -191,7 +196,8 @@ __global__ __launch_bounds__((WM * WN + PW) * 64) void k_gemm_bf16_nt(const bf16
 
 template <int BM, int BN, int WM, int WN, typename TC, int PW = 0>
 static int ix_gemm_bf16_launch(const bf16_t* A, long lda, const bf16_t* W, long ldw, const bf16_t* bias, TC* C,
-                               long ldc, long M, long N, long K, float* parts, long parts_ld, hipStream_t st) {
+                               long ldc, long M, long N, long K, float* parts, long parts_ld, hipStream_t st,
+                               long batch = 1, long batch_a = 0, long batch_w = 0, long batch_c = 0) {
   using Cfg = IxGemmCfg<BM, BN, WM, WN, PW>;
   const long nb_m = (M + BM - 1) / BM, nb_n = (N + BN - 1) / BN;
   const long grid = 8 * ((nb_m * nb_n + 7) / 8);  // 8 XCD runs of the tile order, the longest one sets the count
@@ -206,8 +212,10 @@ static int ix_gemm_bf16_launch(const bf16_t* A, long lda, const bf16_t* W, long 
     attr_set = true;
   }
   const int vec = (ldc % 4 == 0) && ix_aligned(C, 4 * sizeof(TC));
-  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(Cfg::NTT), Cfg::LDS_BYTES, st, A, lda, W, ldw, bias, C, ldc,
-                     (int)M, (int)N, (int)K, (int)nb_m, (int)nb_n, vec, parts, parts_ld);
+  if (batch > 65535) return IX_DECLINED;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid, (unsigned)batch), dim3(Cfg::NTT), Cfg::LDS_BYTES, st, A, lda, W, ldw,
+                     bias, C, ldc, (int)M, (int)N, (int)K, (int)nb_m, (int)nb_n, vec, parts, parts_ld, batch_a, batch_w,
+                     batch_c);
   return ix_launch_status();
 }
 
@@ -258,17 +266,19 @@ extern "C" long ix_gemm_bf16_n_tiles(long M, long N, long K, int tile) {
 template <typename TC>
 static int ix_gemm_bf16_dispatch(const bf16_t* a, long lda, const bf16_t* w, long ldw, const bf16_t* b, TC* c,
                                  long ldc, long M, long N, long K, int tile, float* parts, long parts_ld,
-                                 hipStream_t st) {
+                                 hipStream_t st, long batch = 1, long sa = 0, long sw = 0, long sc = 0) {
   // `tile` only picks which workgroup owns an element (0 = by M); the bits do not depend on it.
-  switch (ix_gemm_tile_for(M, N, K, tile)) {
-    case 1: return ix_gemm_bf16_launch<32, 256, 1, 4, TC, 4>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
-    case 2: return ix_gemm_bf16_launch<128, 128, 2, 2, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
-    case 3: return ix_gemm_bf16_launch<256, 256, 2, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
-    case 4: return ix_gemm_bf16_launch<256, 256, 2, 2, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
-    case 5: return ix_gemm_bf16_launch<128, 256, 2, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
-    case 6: return ix_gemm_bf16_launch<64, 32, 2, 1, TC, 2>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st);
+#define IX_BATCH_ARGS , batch, sa, sw, sc
+  switch (ix_gemm_tile_for(M * (batch > 1 ? batch : 1), N, K, tile)) {
+    case 1: return ix_gemm_bf16_launch<32, 256, 1, 4, TC, 4>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st IX_BATCH_ARGS);
+    case 2: return ix_gemm_bf16_launch<128, 128, 2, 2, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st IX_BATCH_ARGS);
+    case 3: return ix_gemm_bf16_launch<256, 256, 2, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st IX_BATCH_ARGS);
+    case 4: return ix_gemm_bf16_launch<256, 256, 2, 2, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st IX_BATCH_ARGS);
+    case 5: return ix_gemm_bf16_launch<128, 256, 2, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st IX_BATCH_ARGS);
+    case 6: return ix_gemm_bf16_launch<64, 32, 2, 1, TC, 2>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st IX_BATCH_ARGS);
     default: return IX_ERR_ARG;
   }
+#undef IX_BATCH_ARGS
 }
 
 extern "C" int ix_gemm_bf16_nt(const void* A, long lda, const void* W, long ldw, const void* bias, void* C,
@@ -287,6 +297,23 @@ extern "C" int ix_gemm_bf16_nt(const void* A, long lda, const void* W, long ldw,
   if (c_dtype == IX_DT_BF16)
     return ix_gemm_bf16_dispatch(a, lda, w, ldw, b, (bf16_t*)C, ldc, M, N, K, tile, row_max_parts, parts_ld, st);
   return ix_gemm_bf16_dispatch(a, lda, w, ldw, b, (float*)C, ldc, M, N, K, tile, row_max_parts, parts_ld, st);
+}
+
+// aten::bmm of the override (ops/moe/moe_batch_invariant.py:453-464): `batch` independent products in ONE launch, each
+// exactly the product ix_gemm_bf16_nt computes (same tiles, same K order, same bits); matrix b of an operand starts
+// b * stride elements after matrix 0. The tile shape is chosen for the whole batch (rows M * batch).
+extern "C" int ix_gemm_bf16_nt_batched(const void* A, long lda, long stride_a, const void* W, long ldw, long stride_w,
+                                       void* C, long ldc, long stride_c, long batch, long M, long N, long K, int tile,
+                                       void* stream) {
+  if (!A || !W || !C || batch < 0 || M < 0 || N <= 0 || K <= 0) return IX_ERR_ARG;
+  if (lda < K || ldw < K || ldc < N) return IX_ERR_ARG;
+  if ((K % 8) || (lda % 8) || (ldw % 8) || (stride_a % 8) || (stride_w % 8) || !ix_aligned(A, 16) || !ix_aligned(W, 16))
+    return IX_DECLINED;
+  if (M > 0x7fffffffL || N > 0x7fffffffL || K > 0x7fffffffL) return IX_DECLINED;
+  if (lda * 2 * 256 >= 0x40000000L || ldw * 2 * 256 >= 0x40000000L) return IX_DECLINED;
+  if (M == 0 || batch == 0) return IX_OK;
+  return ix_gemm_bf16_dispatch((const bf16_t*)A, lda, (const bf16_t*)W, ldw, (const bf16_t*)nullptr, (bf16_t*)C, ldc, M,
+                               N, K, tile, (float*)nullptr, 0, (hipStream_t)stream, batch, stride_a, stride_w, stride_c);
 }
 
 // ---------------------------------------------------------------------------------------------

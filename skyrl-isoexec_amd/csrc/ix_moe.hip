@@ -524,6 +524,71 @@ __global__ __launch_bounds__(256) void k_moe_permute_one_tile(const int* __restr
   }
 }
 
+// Block map for rows that are ALREADY grouped by expert (the caller holds tokens_per_expert, e.g. a dispatcher's
+// output): exclusive scan of the counts, then every expert writes its own row tiles. One workgroup, integer only.
+template <typename TI>
+__global__ __launch_bounds__(256) void k_moe_block_map(const TI* __restrict__ counts_in, int E, int BM, int max_tiles,
+                                                       int* __restrict__ offsets, int* __restrict__ meta) {
+  __shared__ int s_rows[256], s_tiles[256];
+  const int tid = threadIdx.x;
+  int c[2], tl[2];  // lane owns experts 2 tid and 2 tid + 1 (E <= 512)
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int e = 2 * tid + h;
+    c[h] = e < E ? max(0, (int)counts_in[e]) : 0;
+    tl[h] = (c[h] + BM - 1) / BM;
+  }
+  s_rows[tid] = c[0] + c[1];
+  s_tiles[tid] = tl[0] + tl[1];
+  __syncthreads();
+  for (int d = 1; d < 256; d <<= 1) {
+    const int a = tid >= d ? s_rows[tid - d] : 0;
+    const int b = tid >= d ? s_tiles[tid - d] : 0;
+    __syncthreads();
+    s_rows[tid] += a;
+    s_tiles[tid] += b;
+    __syncthreads();
+  }
+  int row0 = s_rows[tid] - (c[0] + c[1]);
+  int tile0 = s_tiles[tid] - (tl[0] + tl[1]);
+  int* tile_expert = meta + 1;
+  int* tile_row0 = tile_expert + max_tiles;
+  int* tile_nrows = tile_row0 + max_tiles;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int e = 2 * tid + h;
+    if (e < E) {
+      if (offsets) offsets[e] = row0;
+      int nt = tile0;
+      for (int r0 = 0; r0 < c[h] && nt < max_tiles; r0 += BM, ++nt) {
+        tile_expert[nt] = e;
+        tile_row0[nt] = row0 + r0;
+        tile_nrows[nt] = min(BM, c[h] - r0);
+      }
+    }
+    row0 += c[h];
+    tile0 += tl[h];
+  }
+  if (tid == 255) {
+    if (offsets) offsets[E] = s_rows[255];
+    meta[0] = min(s_tiles[255], max_tiles);
+  }
+}
+
+extern "C" int ix_moe_block_map(const void* counts, int counts_i64, long E, long BM, int* offsets, int* tile_meta,
+                                long max_tiles, void* stream) {
+  if (!counts || !tile_meta || E <= 0 || BM <= 0 || max_tiles <= 0) return IX_ERR_ARG;
+  if (E > IX_MOE_EMAX) return IX_DECLINED;
+  hipStream_t st = (hipStream_t)stream;
+  if (counts_i64)
+    hipLaunchKernelGGL(k_moe_block_map<long>, dim3(1), dim3(256), 0, st, (const long*)counts, (int)E, (int)BM,
+                       (int)max_tiles, offsets, tile_meta);
+  else
+    hipLaunchKernelGGL(k_moe_block_map<int>, dim3(1), dim3(256), 0, st, (const int*)counts, (int)E, (int)BM,
+                       (int)max_tiles, offsets, tile_meta);
+  return ix_launch_status();
+}
+
 extern "C" long ix_moe_max_tiles(long T, long k, long E, long BM) {
   if (T < 0 || k <= 0 || E <= 0 || BM <= 0) return 0;
   return (T * k + BM - 1) / BM + E;

@@ -56,6 +56,10 @@ SIGNATURES = {
         [P, c_long, P, c_long, P, P, c_int, c_long, c_long, c_long, c_long, c_int, P, c_long, P],
     ),
     "ix_gemm_bf16_n_tiles": (c_long, [c_long, c_long, c_long, c_int]),
+    "ix_gemm_bf16_nt_batched": (
+        c_int,
+        [P, c_long, c_long, P, c_long, c_long, P, c_long, c_long, c_long, c_long, c_long, c_long, c_int, P],
+    ),
     "ix_gemm_f32_nt": (c_int, [P, c_int, c_long, P, c_long, P, c_long, c_long, c_long, c_long, P]),
     "ix_gdn_scan": (
         c_int,
@@ -78,6 +82,7 @@ SIGNATURES = {
         c_int,
         [P, P, c_long, c_long, c_long, c_long, P, P, P, P, P, P, c_long, P, P],
     ),
+    "ix_moe_block_map": (c_int, [P, c_int, c_long, c_long, P, P, c_long, P]),
     "ix_moe_permute_static_max_ints": (c_size_t, []),
     "ix_moe_permute_static": (
         c_int,

@@ -13,11 +13,18 @@ import torch
 from ... import _lib
 
 _LIBRARY = None
-_COUNTS = {"mm": 0, "addmm": 0, "bmm": 0, "declined": 0}
+_COUNTS = {"mm": 0, "addmm": 0, "bmm": 0, "declined": 0, "operand_copies": 0}
 
 
 def stats() -> dict:
+    """Calls served per primitive since import, calls handed to the stock kernel, operands copied to reach the
+    kernel's K-contiguous layout."""
     return dict(_COUNTS)
+
+
+def reset_stats() -> None:
+    for key in _COUNTS:
+        _COUNTS[key] = 0
 
 
 def linear_nt(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *, tile: int = 0,
@@ -86,57 +93,139 @@ def linear_f32_nt(x: torch.Tensor, weight: torch.Tensor):
 
 
 def _as_nt(b: torch.Tensor):
-    """``b [K, N]`` as a K-contiguous ``[N, K]`` matrix (free for the transposed view of a
-    ``[N, K]`` weight, which is what ``F.linear`` hands to ``aten::mm``)."""
-    bt = b.t()
-    return bt if bt.stride(1) == 1 else bt.contiguous()
+    """``b [K, N]`` as a K-contiguous ``[N, K]`` matrix: free for the transposed view of a ``[N, K]`` weight (what
+    ``F.linear`` hands to ``aten::mm``); a ``[K, N]`` operand that is itself row-major (a backward-pass product) is
+    copied, and the copy is counted in ``stats()["operand_copies"]``."""
+    bt = b.transpose(-1, -2)
+    if bt.stride(-1) == 1:
+        return bt
+    _COUNTS["operand_copies"] += 1
+    return bt.contiguous()
+
+
+def _rows(a: torch.Tensor):
+    if a.stride(-1) == 1:
+        return a
+    _COUNTS["operand_copies"] += 1
+    return a.contiguous()
 
 
 def mm_batch_invariant(a: torch.Tensor, b: torch.Tensor):
-    out = None
+    """``a [M, K] @ b [K, N]`` on the fixed-order kernels, or ``None`` for a signature they do not serve."""
+    if a.ndim != 2 or b.ndim != 2 or not a.is_cuda or not b.is_cuda:
+        return None
     if a.dtype is torch.bfloat16 and b.dtype is torch.bfloat16:
-        out = linear_nt(a if a.stride(1) == 1 else a.contiguous(), _as_nt(b))
-    elif a.dtype is torch.float32 and b.dtype is torch.float32:
-        out = linear_f32_nt(a if a.stride(1) == 1 else a.contiguous(), _as_nt(b))
+        return linear_nt(_rows(a), _as_nt(b))
+    if a.dtype is torch.float32 and b.dtype is torch.float32:
+        return linear_f32_nt(_rows(a), _as_nt(b))
+    return None
+
+
+def addmm_batch_invariant(bias, a, b, *, beta=1, alpha=1):
+    """``bias [N] + a @ b`` (bf16, alpha = beta = 1: what ``F.linear`` with a bias dispatches), else ``None``."""
+    if beta != 1 or alpha != 1 or bias.ndim != 1 or a.ndim != 2 or b.ndim != 2:
+        return None
+    if not (a.dtype is b.dtype is bias.dtype is torch.bfloat16) or bias.shape[0] != b.shape[1]:
+        return None
+    return linear_nt(_rows(a), _as_nt(b), bias.contiguous())
+
+
+def bmm_batch_invariant(a: torch.Tensor, b: torch.Tensor):
+    """``a [B, M, K] @ b [B, K, N]``: ONE launch over the batch, every product computed exactly as ``mm`` computes
+    it (same bits as a loop of ``mm_batch_invariant``); ``None`` for a signature the kernel does not serve."""
+    if a.ndim != 3 or b.ndim != 3 or a.dtype is not torch.bfloat16 or b.dtype is not torch.bfloat16:
+        return None
+    if not a.is_cuda or a.shape[0] != b.shape[0] or a.shape[2] != b.shape[1]:
+        return None
+    ar, bt = _rows(a), _as_nt(b)          # [B, M, K], [B, N, K], rows K-contiguous
+    if ar.stride(1) < ar.shape[2] or bt.stride(1) < bt.shape[2]:
+        return None
+    B, M, K = ar.shape
+    N = bt.shape[1]
+    out = torch.empty(B, M, N, dtype=torch.bfloat16, device=a.device)
+    if B == 0 or M == 0:
+        return out
+    rc = _lib.check(
+        _lib.lib().ix_gemm_bf16_nt_batched(ar.data_ptr(), ar.stride(1), ar.stride(0), bt.data_ptr(), bt.stride(1),
+                                           bt.stride(0), out.data_ptr(), N, M * N, B, M, N, K, 0,
+                                           _lib.current_stream(a.device)), "ix_gemm_bf16_nt_batched")
+    return out if rc == _lib.IX_OK else None
+
+
+# ---- the operator override (moe_batch_invariant.py:422-473) -------------------------------------------------------
+# aten::mm / addmm / bmm on the device dispatch key are replaced, so every F.linear / torch.matmul of the process
+# lands on the fixed-order kernels (matmul and linear are composite: only these three primitives need replacing).
+# A signature the kernels do not serve (other dtypes, K or a row pitch that is not a multiple of 8, alpha/beta forms)
+# is handed to the kernel that was registered before, counted under "declined" and named once on stderr: the process
+# keeps working, and the count says whether anything on the hot path escaped. ``strict=True`` raises instead.
+_STOCK = {}
+_STRICT = False
+_NAMED = set()
+
+
+def _fall_through(name, keyset, args, kwargs):
+    _COUNTS["declined"] += 1
+    sig = (name,) + tuple((tuple(t.shape), str(t.dtype)) for t in args if isinstance(t, torch.Tensor))
+    if _STRICT:
+        raise RuntimeError(f"[isoexec-amd] {name} override: no batch-invariant kernel for {sig[1:]}")
+    if sig not in _NAMED and len(_NAMED) < 32:
+        _NAMED.add(sig)
+        import sys
+
+        print(f"[isoexec-amd] {name}: {sig[1:]} is not served by the batch-invariant kernels; stock kernel used",
+              file=sys.stderr, flush=True)
+    return _STOCK[name].call_boxed(keyset, *args, **kwargs)
+
+
+def _mm_impl(keyset, a, b):
+    out = mm_batch_invariant(a, b)
     if out is None:
-        _COUNTS["declined"] += 1
-        raise RuntimeError(
-            f"[isoexec-amd] mm override declined {tuple(a.shape)}x{tuple(b.shape)} {a.dtype}/{b.dtype}: "
-            "no batch-invariant kernel for this signature")
+        return _fall_through("mm", keyset, (a, b), {})
     _COUNTS["mm"] += 1
     return out
 
 
-def addmm_batch_invariant(bias, a, b, *, beta=1, alpha=1):
-    if beta != 1 or alpha != 1 or bias.ndim != 1 or a.dtype is not torch.bfloat16:
-        raise RuntimeError("[isoexec-amd] addmm override serves bias[N] + a@b with alpha=beta=1 in bf16 only")
-    out = linear_nt(a if a.stride(1) == 1 else a.contiguous(), _as_nt(b), bias.contiguous())
+def _addmm_impl(keyset, bias, a, b, *, beta=1, alpha=1):
+    out = addmm_batch_invariant(bias, a, b, beta=beta, alpha=alpha)
     if out is None:
-        _COUNTS["declined"] += 1
-        raise RuntimeError("[isoexec-amd] addmm override declined")
+        return _fall_through("addmm", keyset, (bias, a, b), {"beta": beta, "alpha": alpha})
     _COUNTS["addmm"] += 1
     return out
 
 
-def bmm_batch_invariant(a, b):
+def _bmm_impl(keyset, a, b):
+    out = bmm_batch_invariant(a, b)
+    if out is None:
+        return _fall_through("bmm", keyset, (a, b), {})
     _COUNTS["bmm"] += 1
-    return torch.stack([mm_batch_invariant(a[i], b[i]) for i in range(a.shape[0])])
+    return out
 
 
-def install_mm_override() -> bool:
-    """Route ``aten::mm/addmm/bmm`` on device tensors to the kernel (moe_batch_invariant.py:453-464)."""
-    global _LIBRARY
+def install_mm_override(strict: bool = False) -> bool:
+    """Route ``aten::mm/addmm/bmm`` on device tensors to the kernels (moe_batch_invariant.py:453-464)."""
+    global _LIBRARY, _STRICT
+    _STRICT = bool(strict)
     if _LIBRARY is not None:
         return True
     _lib.lib()
+    for name in ("mm", "addmm", "bmm"):
+        _STOCK[name] = torch.library.get_kernel(f"aten::{name}", "CUDA")
     library = torch.library.Library("aten", "IMPL")
-    library.impl("aten::mm", mm_batch_invariant, "CUDA")
-    library.impl("aten::addmm", addmm_batch_invariant, "CUDA")
-    library.impl("aten::bmm", bmm_batch_invariant, "CUDA")
+    library.impl("mm", _mm_impl, "CUDA", with_keyset=True)
+    library.impl("addmm", _addmm_impl, "CUDA", with_keyset=True)
+    library.impl("bmm", _bmm_impl, "CUDA", with_keyset=True)
     _LIBRARY = library
     return True
 
 
 def uninstall_mm_override() -> None:
+    """Remove the override: the kernels registered before serve again."""
     global _LIBRARY
-    _LIBRARY = None
+    if _LIBRARY is not None:
+        _LIBRARY._destroy()
+        _LIBRARY = None
+    _STOCK.clear()
+
+
+def mm_override_installed() -> bool:
+    return _LIBRARY is not None

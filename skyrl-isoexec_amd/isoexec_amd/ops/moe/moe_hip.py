@@ -103,9 +103,10 @@ def fused_permute_index(routing_map: torch.Tensor, routing_probs: torch.Tensor, 
     return p.sorted_token.long(), p.permuted_prob, p.counts.long()
 
 
-def experts_forward(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, p: Permutation):
+def experts_forward(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, p: Permutation, *, return_inter: bool = False):
     """Grouped fc1 + SwiGLU + prob epilogue + fc2 over the permuted rows. ``x [T, H]`` bf16,
-    ``w1 [E, 2F, H]``, ``w2 [E, H, F]``. Returns ``expert_out [T*k, H]`` in permuted order."""
+    ``w1 [E, 2F, H]``, ``w2 [E, H, F]``. Returns ``expert_out [T*k, H]`` in permuted order; with ``return_inter`` also
+    the activation that enters fc2, ``inter [T*k, F]`` = bf16(bf16(bf16(silu(gate)) * up) * prob)."""
     _lib.require_device(x, w1, w2)
     if x.dtype is not torch.bfloat16 or w1.dtype is not torch.bfloat16 or w2.dtype is not torch.bfloat16:
         raise RuntimeError("[isoexec-amd] experts serve bf16 only")
@@ -126,7 +127,7 @@ def experts_forward(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, p: Perm
         "ix_moe_experts")
     if rc != _lib.IX_OK:
         raise RuntimeError(f"[isoexec-amd] ix_moe_experts declined H={H} F={F}")
-    return out
+    return (out, inter) if return_inter else out
 
 
 def combine(expert_out: torch.Tensor, p: Permutation, *, fp32_acc: bool = False) -> torch.Tensor:

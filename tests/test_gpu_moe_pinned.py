@@ -1,0 +1,177 @@
+"""GPU: the grouped expert kernels pinned bit for bit, and the MoE doors with the reference's call shapes.
+
+The grouped GEMMs share the dense kernel's core (one instruction, one K order), so each expert's rows must equal, bit
+for bit, what the dense entry point gives for the same rows: fc1 = ``linear_nt(x[rows_e], W1[e])`` followed by the
+oracle's SwiGLU * prob epilogue (device transcendentals plugged in), fc2 = ``linear_nt(inter_e, W2[e])``
+(reference chain: ops/moe/moe_batched_experts.py:496-503; its invariance gate :652-708)."""
+
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+from _util import DevicePrims, bf16_to_np, cpu_gen, np_to_bf16, same_bits
+from oracle.prims import round_bf16
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+F32 = np.float32
+
+
+def make(T, H, E, F, seed):
+    g = cpu_gen(seed)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(DEV)
+    wr = (0.02 * torch.randn(E, H, generator=g)).to(torch.bfloat16).to(DEV)
+    w1 = (0.02 * torch.randn(E, 2 * F, H, generator=g)).to(torch.bfloat16).to(DEV)
+    w2 = (0.02 * torch.randn(E, H, F, generator=g)).to(torch.bfloat16).to(DEV)
+    return x, wr, w1, w2
+
+
+@pytest.mark.parametrize("T,H,E,F,k,BM", [(300, 256, 16, 128, 4, None), (300, 256, 16, 96, 4, 256), (77, 512, 8, 192, 2, 128),
+                                          (33, 2048, 128, 768, 8, None), (600, 2048, 8, 768, 2, 256)])
+def test_grouped_kernels_equal_the_dense_kernel_per_expert(T, H, E, F, k, BM):
+    from isoexec_amd.ops.mm.mm_hip import linear_nt, router_gemm
+    from isoexec_amd.ops.moe.moe_hip import experts_forward, permute, router_topk
+
+    prims = DevicePrims(DEV)
+    x, wr, w1, w2 = make(T, H, E, F, seed=T + F)
+    logits = router_gemm(x, wr)
+    logits[:, :2] += 2.0          # skewed load: some experts get ragged multi-tile segments, some get nothing
+    idx, prob, _, _ = router_topk(logits, k, pre_softmax=True)
+    p = permute(idx, prob, E, BM=BM)
+    eo, inter = experts_forward(x, w1, w2, p, return_inter=True)
+    offsets = p.offsets.cpu().numpy()
+    st = p.sorted_token.long()
+    pp = p.permuted_prob.cpu().numpy()
+    checked = 0
+    for e in range(E):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        if hi == lo:
+            continue
+        xe = x.index_select(0, st[lo:hi])
+        lin = bf16_to_np(linear_nt(xe, w1[e]))                      # bf16(x W1^T): gate columns then up columns
+        gate, up = lin[:, :F], lin[:, F:]
+        s = round_bf16(prims.silu_div(gate))
+        h = round_bf16((s * up).astype(F32))
+        a = round_bf16((h * pp[lo:hi, None]).astype(F32))
+        assert same_bits(inter[lo:hi].cpu(), np_to_bf16(a)), f"fc1 epilogue, expert {e} rows {lo}:{hi}"
+        assert same_bits(eo[lo:hi], linear_nt(inter[lo:hi].contiguous(), w2[e])), f"fc2, expert {e}"
+        checked += hi - lo
+    assert checked == T * k
+
+
+def fake_sequential_mlp(w1, w2, stacked=True):
+    """What ``_batched_experts_forward`` reads of a ``SequentialMLP`` (the reference's own stand-in,
+    ops/moe/tests/moe_fused_vs_bmm_gpu.py:26-44)."""
+    cfg = SimpleNamespace(activation_func=torch.nn.functional.silu, activation_func_clamp_value=None, glu_linear_offset=0.0,
+                          fp8=False, bias_activation_fusion=False, gated_linear_unit=True, add_bias_linear=False)
+    pick = (lambda w, e: w[e]) if stacked else (lambda w, e: w[e].clone())
+    experts = [SimpleNamespace(linear_fc1=SimpleNamespace(weight=pick(w1, e)), linear_fc2=SimpleNamespace(weight=pick(w2, e)))
+               for e in range(w1.shape[0])]
+    return SimpleNamespace(config=cfg, num_local_experts=w1.shape[0], local_experts=experts)
+
+
+@pytest.mark.parametrize("stacked", [True, False])
+def test_doors_with_the_reference_call_shapes(stacked):
+    from isoexec_amd.ops.mm.mm_hip import router_gemm
+    from isoexec_amd.ops.moe import moe_doors
+    from isoexec_amd.ops.moe.moe_hip import combine, experts_forward, fused_router_dense, permute, router_topk
+
+    T, H, E, F, k = 300, 256, 16, 128, 4
+    x, wr, w1, w2 = make(T, H, E, F, seed=9)
+    logits = router_gemm(x, wr)
+    # TopKRouter.routing(logits) -> (routing_probs, routing_map)
+    router = SimpleNamespace(topk=k, config=SimpleNamespace(moe_router_pre_softmax=False, moe_router_topk_scaling_factor=None))
+    rprobs, rmap = moe_doors._make_sorted_topk_routing(None)(router, logits)
+    dprobs, dmap = fused_router_dense(logits, k)
+    assert same_bits(rprobs, dprobs) and torch.equal(rmap, dmap) and int(rmap.sum()) == T * k
+    # dispatcher: dispatch_postprocess(hidden, probs) -> (permuted hidden, tokens_per_expert, permuted probs)
+    disp = SimpleNamespace(routing_map=rmap, local_expert_indices=list(range(E)), config=SimpleNamespace(moe_router_topk=k))
+    hidden, tpe, pprobs = moe_doors._dispatch_postprocess_fixed_shape(disp, x, rprobs)
+    idx, prob, _, _ = router_topk(logits, k)
+    p = permute(idx, prob, E)
+    assert torch.equal(disp.reversed_local_input_permutation_mapping, p.sorted_token.long())
+    assert torch.equal(tpe, p.counts.long()) and same_bits(pprobs, p.permuted_prob)
+    assert same_bits(hidden, x.index_select(0, p.sorted_token.long()))
+    # SequentialMLP.forward(permuted hidden, tokens_per_expert, permuted probs) -> (out, None)
+    mlp = fake_sequential_mlp(w1, w2, stacked)
+    out, bias = moe_doors._batched_experts_forward(mlp, hidden, tpe, pprobs)
+    assert bias is None and same_bits(out, experts_forward(x, w1, w2, p))
+    out_host_counts, _ = moe_doors._batched_experts_forward(mlp, hidden, tpe.cpu().to(torch.int32), pprobs)
+    assert same_bits(out_host_counts, out)
+    empty, _ = moe_doors._batched_experts_forward(mlp, hidden[:0], torch.zeros(E, dtype=torch.int64), pprobs[:0])
+    assert empty.shape == (0, H)
+    # moe_utils.unpermute(permuted_tokens, sorted_indices, restore_shape)
+    got = moe_doors._deterministic_unpermute(out, disp.reversed_local_input_permutation_mapping, x.shape)
+    assert same_bits(got, combine(out, p))
+    assert moe_doors._deterministic_unpermute(out, disp.reversed_local_input_permutation_mapping, x.shape,
+                                              isoexec_out_dtype=torch.float32).dtype is torch.float32
+    assert moe_doors._fixed_order_combine(out[:-1], disp.reversed_local_input_permutation_mapping[:-1], x.shape) is None
+    with pytest.raises(RuntimeError):
+        moe_doors._deterministic_unpermute(out, disp.reversed_local_input_permutation_mapping, x.shape, fused=True)
+    # a SequentialMLP the kernels do not serve says so
+    mlp.config.add_bias_linear = True
+    with pytest.raises(RuntimeError):
+        moe_doors._batched_experts_forward(mlp, hidden, tpe, pprobs)
+
+
+def test_operator_override_door():
+    """aten::mm / addmm / bmm on the device key land on the fixed-order kernels: F.linear, torch.mm, torch.addmm,
+    torch.bmm, 2-D and 3-D, with and without bias, forward and backward; what the kernels do not serve goes to the
+    stock kernel and is counted; uninstalling brings the stock kernels back."""
+    import torch.nn.functional as Fn
+
+    from isoexec_amd.ops.mm import mm_hip
+
+    g = cpu_gen(21)
+    x = torch.randn(37, 256, generator=g).to(torch.bfloat16).to(DEV)
+    w = (0.05 * torch.randn(96, 256, generator=g)).to(torch.bfloat16).to(DEV)
+    b = torch.randn(96, generator=g).to(torch.bfloat16).to(DEV)
+    want = mm_hip.linear_nt(x, w)
+    want_b = mm_hip.linear_nt(x, w, b)
+    stock = Fn.linear(x, w)
+    mm_hip.reset_stats()
+    assert mm_hip.install_mm_override() and mm_hip.mm_override_installed()
+    try:
+        assert same_bits(Fn.linear(x, w), want) and mm_hip.stats()["mm"] == 1
+        assert same_bits(torch.mm(x, w.t()), want) and same_bits(x @ w.t(), want) and mm_hip.stats()["mm"] == 3
+        assert same_bits(Fn.linear(x, w, b), want_b) and same_bits(torch.addmm(b, x, w.t()), want_b)
+        assert mm_hip.stats()["addmm"] == 2
+        x3 = x.view(1, 37, 256).expand(3, 37, 256).contiguous()
+        assert same_bits(Fn.linear(x3, w), want.expand(3, 37, 96))           # 3-D input folds into one mm
+        w3 = torch.stack([w, w.roll(1, 0), w.flip(0)])
+        got = torch.bmm(x3, w3.transpose(1, 2))
+        assert mm_hip.stats()["bmm"] == 1
+        for i in range(3):
+            assert same_bits(got[i], mm_hip.linear_nt(x, w3[i]))              # bmm == mm, product by product
+        assert mm_hip.stats()["operand_copies"] == 0                          # nothing above needed a copy
+        # row m does not depend on how many rows share the call (the point of the override)
+        assert same_bits(Fn.linear(x[5:6], w), want[5:6]) and same_bits(Fn.linear(x[:20], w), want[:20])
+        # backward through the override: grad products are mm calls too (their row-major operands are copied)
+        xg, wg = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+        Fn.linear(xg, wg).float().square().sum().backward()
+        assert xg.grad.shape == x.shape and wg.grad.shape == w.shape and bool(torch.isfinite(wg.grad.float()).all())
+        ref_gx = (2 * want.float()).to(torch.bfloat16).float() @ w.float()
+        assert float((xg.grad.float() - ref_gx).abs().max()) <= 0.05 * float(ref_gx.abs().max())
+        assert mm_hip.stats()["operand_copies"] >= 1
+        # not served: fp16, and a K that is not a multiple of 8 -> the stock kernel, counted, same answer as stock
+        before = mm_hip.stats()["declined"]
+        h = torch.randn(4, 24, generator=g).to(DEV).half()
+        assert torch.equal(h @ h.t(), torch.mm(h, h.t())) and mm_hip.stats()["declined"] == before + 2
+        odd = torch.randn(5, 20, generator=g).to(torch.bfloat16).to(DEV)
+        assert (odd @ odd.t()).shape == (5, 5) and mm_hip.stats()["declined"] == before + 3
+        # fp32 products take the fp32 kernel (the router's gating product)
+        f = torch.randn(9, 64, generator=g).to(DEV)
+        served = mm_hip.stats()["mm"]
+        assert same_bits(f @ f.t(), mm_hip.linear_f32_nt(f, f)) and mm_hip.stats()["mm"] == served + 1
+        # strict mode refuses instead of falling through
+        mm_hip.install_mm_override(strict=True)
+        with pytest.raises(RuntimeError):
+            h @ h.t()
+        mm_hip.install_mm_override(strict=False)
+    finally:
+        mm_hip.uninstall_mm_override()
+    assert not mm_hip.mm_override_installed()
+    served = dict(mm_hip.stats())
+    assert same_bits(Fn.linear(x, w), stock) and mm_hip.stats() == served          # the stock kernel is back
