@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define IX_ABI_VERSION 1
+#define IX_ABI_VERSION 2
 
 #ifndef IX_OK
 #define IX_OK 0
@@ -166,9 +166,10 @@ int ix_attn_varlen(const void* q, long q_pitch, const void* k, const void* v, lo
 /* rope.rope (ops/rope/_register.py:17-77; rope_fused.py:66-108): rotate-half rotary embedding over the
  * first R lanes of every head, in place, with the three-round bf16 multiply-add
  * bf16(bf16(x*cos) + bf16(rot*sin)). x [tokens, heads, D] with token pitch x_pitch; cos/sin bf16
- * [positions, R]; positions int32 [tokens]. */
-int ix_rope_inplace(void* x, long x_pitch, const void* cos_table, const void* sin_table, const int* positions,
-                    long tokens, long heads, long D, long R, void* stream);
+ * [table_rows, R]; positions int32 [tokens]. A position outside [0, table_rows) reads nothing and makes that
+ * token's rotated lanes NaN (positions live on the device, so the host cannot refuse them without a sync). */
+int ix_rope_inplace(void* x, long x_pitch, const void* cos_table, const void* sin_table, long table_rows,
+                    const int* positions, long tokens, long heads, long D, long R, void* stream);
 
 /* gdn_l2norm (gdn_ops.py:202-213): y = x * (1/sqrt(sum x^2 + eps)) over rows of K.
  * x [tokens, H, K] with token pitch x_pitch; y [tokens, H, K] contiguous. */

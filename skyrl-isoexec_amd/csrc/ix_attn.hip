@@ -391,7 +391,7 @@ extern "C" int ix_attn_varlen(const void* q, long q_pitch, const void* k, const 
 // bf16 tables; pos[t] picks the row.
 __global__ __launch_bounds__(256) void k_rope(bf16_t* __restrict__ x, long x_pitch, const bf16_t* __restrict__ cs,
                                               const bf16_t* __restrict__ sn, const int* __restrict__ pos, long total,
-                                              int heads, int D, int R) {
+                                              int heads, int D, int R, int table_rows) {
   const long i = (long)blockIdx.x * 256 + threadIdx.x;
   if (i >= total) return;
   const int half = R >> 1;
@@ -400,7 +400,14 @@ __global__ __launch_bounds__(256) void k_rope(bf16_t* __restrict__ x, long x_pit
   const int hd = (int)(th % heads);
   const long t = th / heads;
   bf16_t* row = x + t * x_pitch + (long)hd * D;
-  const long tab = (long)pos[t] * R;
+  const int p = pos[t];
+  if (p < 0 || p >= table_rows) {
+    // a position the tables do not hold: no read past them, and a result nobody can mistake for a rotation
+    row[d] = (bf16_t)0x7fc0;
+    row[d + half] = (bf16_t)0x7fc0;
+    return;
+  }
+  const long tab = (long)p * R;
   const float a = ix_bf2f(row[d]), b = ix_bf2f(row[d + half]);
   const float c0 = ix_bf2f(cs[tab + d]), c1 = ix_bf2f(cs[tab + d + half]);
   const float s0 = ix_bf2f(sn[tab + d]), s1 = ix_bf2f(sn[tab + d + half]);
@@ -410,15 +417,17 @@ __global__ __launch_bounds__(256) void k_rope(bf16_t* __restrict__ x, long x_pit
   row[d + half] = ix_f2bf(hi);
 }
 
-extern "C" int ix_rope_inplace(void* x, long x_pitch, const void* cos_table, const void* sin_table,
+extern "C" int ix_rope_inplace(void* x, long x_pitch, const void* cos_table, const void* sin_table, long table_rows,
                                const int* positions, long tokens, long heads, long D, long R, void* stream) {
   if (!x || !cos_table || !sin_table || !positions || tokens < 0 || heads <= 0 || D <= 0) return IX_ERR_ARG;
+  if (table_rows <= 0 || table_rows > 0x7fffffffL) return IX_ERR_ARG;
   if (R <= 0 || R % 2 != 0 || R > D) return IX_ERR_ARG;
   const long total = tokens * heads * (R / 2);
   if (total == 0) return IX_OK;
   const long grid = (total + 255) / 256;
   if (grid > (1L << 24)) return IX_DECLINED;
   hipLaunchKernelGGL(k_rope, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, (bf16_t*)x, x_pitch,
-                     (const bf16_t*)cos_table, (const bf16_t*)sin_table, positions, total, (int)heads, (int)D, (int)R);
+                     (const bf16_t*)cos_table, (const bf16_t*)sin_table, positions, total, (int)heads, (int)D, (int)R,
+                     (int)table_rows);
   return ix_launch_status();
 }

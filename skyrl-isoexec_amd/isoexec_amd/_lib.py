@@ -73,7 +73,7 @@ SIGNATURES = {
     "ix_gdn_gate": (c_int, [P, c_long, P, c_long, P, P, P, P, c_int, c_long, c_long, P]),
     "ix_gdn_conv": (c_int, [P, c_long, P, P, P, P, P, P, P, c_long, c_long, c_long, c_long, c_int, P]),
     "ix_attn_varlen": (c_int, [P, c_long, P, P, c_long, P, P, P, P, c_long, c_long, c_long, c_long, c_long, c_float, P]),
-    "ix_rope_inplace": (c_int, [P, c_long, P, P, P, c_long, c_long, c_long, c_long, P]),
+    "ix_rope_inplace": (c_int, [P, c_long, P, P, c_long, P, c_long, c_long, c_long, c_long, P]),
     "ix_moe_router_topk": (c_int, [P, c_long, c_long, c_long, c_long, c_int, c_float, P, P, P, P, P]),
     "ix_moe_max_tiles": (c_long, [c_long, c_long, c_long, c_long]),
     "ix_moe_permute_scratch_ints": (c_size_t, [c_long, c_long]),

@@ -30,7 +30,6 @@ def varlen_attention(
 ) -> torch.Tensor:
     """Returns ``o [Tq, HQ, D]`` bf16. Sequence n attends to key tokens
     ``kv_start[n] + (0 .. q_pos0[n] + len_q[n] - 1)``, causally."""
-    _lib.require_device(q, k, v, cu_seqlens_q, kv_start, q_pos0)
     if q.ndim != 3 or k.ndim != 3 or v.shape != k.shape:
         raise RuntimeError(f"[isoexec-amd] attention expects q [T,HQ,D], k/v [T,HKV,D]; got {tuple(q.shape)} {tuple(k.shape)} {tuple(v.shape)}")
     if q.dtype is not torch.bfloat16 or k.dtype is not torch.bfloat16 or v.dtype is not torch.bfloat16:
@@ -45,6 +44,14 @@ def varlen_attention(
     if cu_seqlens_q.dtype is not torch.int32:
         raise RuntimeError("[isoexec-amd] cu_seqlens_q must be int32")
     n_seq = cu_seqlens_q.numel() - 1
+    if kv_start is None:
+        # keys packed beside the queries: sequence n's keys are tokens cu[n] .. cu[n+1]-1 of k, so k must hold a key
+        # for every query token (the kernel addresses keys from the queries' offsets)
+        if k.shape[0] < Tq:
+            raise RuntimeError(f"[isoexec-amd] attention: packed keys hold {k.shape[0]} tokens for {Tq} queries")
+        if q_pos0 is not None:
+            raise RuntimeError("[isoexec-amd] attention: q_pos0 (context before the first query) needs kv_start")
+    _lib.require_device(q, k, v, cu_seqlens_q, kv_start, q_pos0)
     if kv_start is None:
         kv_start = cu_seqlens_q[:-1].to(torch.int64)
     if kv_start.dtype is not torch.int64 or kv_start.numel() != n_seq:

@@ -28,8 +28,8 @@ def rope_tables(max_positions: int, rotary_dim: int, theta: float = 1.0e6, devic
 
 def apply_rope_(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
     """Rotate ``x [T, heads, D]`` in place (a strided slice of a projection output is fine: only the
-    heads of one token must be contiguous). ``positions`` int32 [T] index the tables."""
-    _lib.require_device(x, cos, sin, positions)
+    heads of one token must be contiguous). ``positions`` int32 [T] index the tables; a position the tables do not
+    hold turns that token's rotated lanes into NaN (the kernel never reads past the tables)."""
     if x.dtype is not torch.bfloat16 or cos.dtype is not torch.bfloat16 or sin.dtype is not torch.bfloat16:
         raise RuntimeError("[isoexec-amd] rope serves bf16 only")
     T, heads, D = x.shape
@@ -40,8 +40,12 @@ def apply_rope_(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions
         raise RuntimeError("[isoexec-amd] rope: cos/sin must be contiguous [positions, R]")
     if positions.dtype is not torch.int32 or positions.numel() != T:
         raise RuntimeError("[isoexec-amd] rope: positions must be int32 [T]")
+    if cos.ndim != 2 or R % 2 != 0 or R > D:
+        raise RuntimeError(f"[isoexec-amd] rope: tables must be [positions, R] with even R <= D, got {tuple(cos.shape)}")
+    _lib.require_device(x, cos, sin, positions)
     rc = _lib.check(
-        _lib.lib().ix_rope_inplace(x.data_ptr(), x.stride(0), cos.data_ptr(), sin.data_ptr(), positions.contiguous().data_ptr(),
+        _lib.lib().ix_rope_inplace(x.data_ptr(), x.stride(0), cos.data_ptr(), sin.data_ptr(), cos.shape[0],
+                                   positions.contiguous().data_ptr(),
                                    T, heads, D, R, _lib.current_stream(x.device)),
         "ix_rope_inplace")
     if rc != _lib.IX_OK:

@@ -140,6 +140,14 @@ class HybridWeights:
         return w
 
 
+def check_lengths(cfg: "HybridConfig", lens, what: str) -> None:
+    """Every sequence must fit the rotary tables (``cfg.max_positions`` rows): positions are 0 .. len-1."""
+    longest = int(max(lens)) if len(lens) else 0
+    if longest > cfg.max_positions:
+        raise ValueError(f"[isoexec-amd] {what}: a sequence of {longest} tokens exceeds max_positions = "
+                         f"{cfg.max_positions} (the rotary tables hold that many positions)")
+
+
 def _linear(x, w):
     out = linear_nt(x, w)
     if out is None:
@@ -226,8 +234,11 @@ class _Blocks:
 
     def sampled_logprobs(self, x: torch.Tensor, targets: torch.Tensor) -> torch.Tensor:
         logits, row_max = self.logits(x, want_row_max=True)
-        lp, _ = sampled_forward(logits, targets, leaves(), row_max=row_max)
-        return lp
+        got = sampled_forward(logits, targets, leaves(), row_max=row_max)
+        if got is None:
+            raise RuntimeError(f"[isoexec-amd] the log-softmax kernel declined vocab {logits.shape[1]} with "
+                               f"{leaves()} leaves (the vocabulary must divide into the leaves)")
+        return got[0]
 
 
 def bound_implementations(cfg: HybridConfig) -> dict:
@@ -279,6 +290,7 @@ class TrainerModel:
     def hidden_states(self, tokens: torch.Tensor, lens: list) -> torch.Tensor:
         """``tokens`` int64 [sum(lens)] packed; returns the final-normed hidden states [sum(lens), H]."""
         b, c = self.blocks, self.cfg
+        check_lengths(c, lens, "trainer pass")
         dev = tokens.device
         offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
         cu = torch.from_numpy(offs).to(dev)
@@ -323,6 +335,9 @@ class RolloutEngine:
     """Prefill, then one token per step per sequence, out of per-layer state."""
 
     def __init__(self, cfg: HybridConfig, weights: HybridWeights, max_num_seqs: int, max_len: int):
+        if max_len > cfg.max_positions:
+            raise ValueError(f"[isoexec-amd] engine max_len = {max_len} exceeds max_positions = {cfg.max_positions} "
+                             "(the rotary tables hold that many positions)")
         self.cfg, self.blocks = cfg, _Blocks(cfg, weights)
         dev = weights.embed.device
         self.max_len = max_len
@@ -363,6 +378,9 @@ class RolloutEngine:
         """Prompts packed in ``tokens``; returns the final-normed hidden state of each prompt's LAST
         token ``[N, H]`` (the row the first response token is sampled from)."""
         b, c = self.blocks, self.cfg
+        check_lengths(c, lens, "prefill")
+        if int(max(lens)) > self.max_len:
+            raise ValueError(f"[isoexec-amd] prefill: a prompt of {int(max(lens))} tokens exceeds the cache length {self.max_len}")
         dev = tokens.device
         offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
         cu = torch.from_numpy(offs).to(dev)

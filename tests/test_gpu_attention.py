@@ -247,3 +247,20 @@ def test_rope_bit_exact_in_place_on_a_strided_slice():
     whole = apply_rope_(x.clone(), cos_f, sin_f, p)
     one = apply_rope_(x[4:5].clone(), cos_f, sin_f, p[4:5])
     assert same_bits(one, whole[4:5]) and same_bits(whole[0], x[0])
+
+
+def test_rope_positions_outside_the_tables_read_nothing_and_give_nan():
+    """The kernel bounds every position by the tables' row count: a position past the end (or negative) makes that
+    token's rotated lanes NaN instead of reading beyond the tables; its neighbours are rotated as usual."""
+    from isoexec_amd.ops.rope.rope_hip import apply_rope_, rope_tables
+    from oracle import attention as o_attn
+
+    g = cpu_gen(77)
+    x = torch.randn(4, 3, 128, generator=g).to(torch.bfloat16)
+    cos, sin = rope_tables(64, 128, 1e6, device=DEV)
+    pos = torch.tensor([0, 63, 64, -1], dtype=torch.int32)
+    got = apply_rope_(x.clone().to(DEV), cos, sin, pos.to(DEV)).float().cpu().numpy()
+    co, so = o_attn.rope_tables(64, 128, 1e6)
+    want = o_attn.rope(x[:2].float().numpy(), co, so, pos[:2].numpy())
+    assert np.array_equal(got[:2], want)
+    assert np.isnan(got[2:]).all()
