@@ -31,11 +31,12 @@ PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch of the dominant kernels, NOT measured in this run: from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE of the same workload (scaled by what the same counters read for a 1 GiB copy, x2.0 / x1.0), recorded in
 # the named file under profiles/.
-MEASURED_TRAFFIC_BYTES = {"dense_head_M4096_gemm": 9.08e9, "gdn_decode_B256": 1.1016e9,
-                          "moe_T16384_grouped_gemms": 3.80e9}
+MEASURED_TRAFFIC_BYTES = {"dense_head_M4096_gemm": 13.83e9, "gdn_decode_B256": 1.080e9,
+                          "moe_T16384_grouped_gemms": 3.87e9, "moe_T163840_grouped_gemms": 36.9e9}
 TRAFFIC_SOURCE = {"dense_head_M4096_gemm": "profiles/gemm_bf16_nt__dense_head_M4096.txt",
                   "gdn_decode_B256": "profiles/gdn_scan__decode_B256.txt",
-                  "moe_T16384_grouped_gemms": "profiles/moe_ffn__T16384.txt"}
+                  "moe_T16384_grouped_gemms": "profiles/moe_ffn__T16384.txt",
+                  "moe_T163840_grouped_gemms": "profiles/hybrid_trainer_pass__64x2560.txt"}
 
 
 def host_gen(seed: int):
@@ -394,7 +395,8 @@ def north_star_kernels(w, dev, steps):
     by = M * Vv * 2
     out["logprob_blocksums_M4096"] = {
         "bound": "hbm", "kernel": "k_lp_blocksums (+ finalize)", "kernel_ms": ms, "achieved": by / ms / 1e6,
-        "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": by / ms / 1e6 / PEAK_HBM_GBS, "traffic": None}
+        "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": by / ms / 1e6 / PEAK_HBM_GBS, "traffic": 1.245e9,
+        "traffic_source": "profiles/logprob_blocksums__dense_head_M4096.txt (not measured in this run)"}
     return out
 
 
@@ -495,7 +497,9 @@ def hybrid(args):
                       "tokens_per_step": total, "rng": "host torch.Generator (weights seed 0, tokens seed 4)"},
            "decode_tokens_per_s": n / t_graph,
            "roofline": {"bound": "mfma", "achieved": exp_fl / exp_ms / 1e9, "peak": PEAK_MFMA_BF16_TFLOPS,
-                        "unit": "TFLOP/s", "frac": exp_fl / exp_ms / 1e9 / PEAK_MFMA_BF16_TFLOPS, "traffic": None,
+                        "unit": "TFLOP/s", "frac": exp_fl / exp_ms / 1e9 / PEAK_MFMA_BF16_TFLOPS,
+                        "traffic": MEASURED_TRAFFIC_BYTES["moe_T163840_grouped_gemms"] if total == 163840 else None,
+                        "traffic_source": TRAFFIC_SOURCE["moe_T163840_grouped_gemms"] + " (not measured in this run)",
                         "kernel": f"k_moe_fc1_glu + k_moe_fc2 (grouped expert GEMMs, {total} tokens x top-8 per launch "
                                   f"pair, {cfg.layers} pairs per pass)", "kernel_ms": exp_ms,
                         "share_of_step": cfg.layers * exp_ms / (dt * 1e3)},
