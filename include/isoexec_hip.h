@@ -109,9 +109,13 @@ int ix_add_rmsnorm_gamma(const void* x, const void* residual, const void* weight
 /* C[M,N] = A[M,K] . W[N,K]^T (+ bias[N]), bf16 operands, fp32 accumulate in a fixed K order, no
  * split-K. C is bf16 (one round of the accumulator) or, with c_dtype = IX_DT_F32, the fp32
  * accumulator itself (the router's fp32 gating product when its fp32 weight is bf16-exact).
- * lda/ldw/ldc are row pitches in elements. bias (bf16 [N]) may be NULL. tile: 0 auto.
- * row_max_parts: NULL, or fp32 [M, parts_ld] receiving per column tile the max of the stored
- * values, parts_ld >= ix_gemm_bf16_n_tiles(M, N, K, tile). */
+ * lda/ldw/ldc are row pitches in elements. bias (bf16 [N]) may be NULL. tile: 0 auto; 1..6 name a tile shape
+ * (32x256, 128x128, 256x256 on eight waves, 256x256 on four waves, 128x256, 64x32); 4 takes the streaming form of its
+ * tile (one workgroup per CU walks many tiles) when the product has at least 512 tiles and the form serves it (bf16 C,
+ * no bias, K a multiple of 64 and >= 704, N and ldc multiples of 8, C 16-byte aligned), 7 never does, 8 always does
+ * and declines what the form does not serve. Every choice gives the same bits.
+ * row_max_parts: NULL, or fp32 [M, parts_ld] receiving per part the max of the stored values (one part per column
+ * tile; two for tiles 4, 7, 8), parts_ld >= ix_gemm_bf16_n_tiles(M, N, K, tile). */
 int ix_gemm_bf16_nt(const void* A, long lda, const void* W, long ldw, const void* bias, void* C, int c_dtype,
                     long ldc, long M, long N, long K, int tile, float* row_max_parts, long parts_ld,
                     void* stream);

@@ -417,6 +417,54 @@ __global__ __launch_bounds__(256) void k_rope(bf16_t* __restrict__ x, long x_pit
   row[d + half] = ix_f2bf(hi);
 }
 
+// The same rotation, eight pairs per thread: 16-byte accesses (two of x, four of the tables, two stores) instead of
+// 2-byte ones, 32-bit index arithmetic. Every output is the expression of k_rope above, so which kernel runs cannot
+// move a bit. Needs R / 2, D and the pitch to be multiples of 8 and 16-byte aligned operands.
+__global__ __launch_bounds__(256) void k_rope8(bf16_t* __restrict__ x, long x_pitch, const bf16_t* __restrict__ cs,
+                                               const bf16_t* __restrict__ sn, const int* __restrict__ pos,
+                                               unsigned total, int heads, int D, int R, int table_rows) {
+  const unsigned i = blockIdx.x * 256u + threadIdx.x;
+  if (i >= total) return;
+  const unsigned chunks = (unsigned)R >> 4;  // 8-pair chunks per head
+  const unsigned c = i % chunks;
+  const unsigned th = i / chunks;
+  const unsigned hd = th % (unsigned)heads;
+  const unsigned t = th / (unsigned)heads;
+  const int half = R >> 1;
+  bf16_t* row = x + (long)t * x_pitch + (long)hd * D + c * 8;
+  const int p = pos[t];
+  uint4 lo4, hi4;
+  if (p < 0 || p >= table_rows) {
+    lo4 = hi4 = make_uint4(0x7fc07fc0u, 0x7fc07fc0u, 0x7fc07fc0u, 0x7fc07fc0u);
+  } else {
+    const bf16_t* ct = cs + (long)p * R + c * 8;
+    const bf16_t* st = sn + (long)p * R + c * 8;
+    const uint4 a4 = *reinterpret_cast<const uint4*>(row), b4 = *reinterpret_cast<const uint4*>(row + half);
+    const uint4 c0 = *reinterpret_cast<const uint4*>(ct), c1 = *reinterpret_cast<const uint4*>(ct + half);
+    const uint4 s0 = *reinterpret_cast<const uint4*>(st), s1 = *reinterpret_cast<const uint4*>(st + half);
+    const uint32_t* aw = &a4.x; const uint32_t* bw = &b4.x;
+    const uint32_t* c0w = &c0.x; const uint32_t* c1w = &c1.x; const uint32_t* s0w = &s0.x; const uint32_t* s1w = &s1.x;
+    uint32_t* low = &lo4.x; uint32_t* hiw = &hi4.x;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      uint32_t lo_pair = 0, hi_pair = 0;
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        auto pick = [&](uint32_t u) { return e == 0 ? __uint_as_float(u << 16) : __uint_as_float(u & 0xffff0000u); };
+        const float a = pick(aw[w]), b = pick(bw[w]);
+        const float lo = ix_rbf(a * pick(c0w[w])) + ix_rbf((b * -1.0f) * pick(s0w[w]));
+        const float hi = ix_rbf(b * pick(c1w[w])) + ix_rbf(a * pick(s1w[w]));
+        lo_pair |= (uint32_t)ix_f2bf(lo) << (16 * e);
+        hi_pair |= (uint32_t)ix_f2bf(hi) << (16 * e);
+      }
+      low[w] = lo_pair;
+      hiw[w] = hi_pair;
+    }
+  }
+  *reinterpret_cast<uint4*>(row) = lo4;
+  *reinterpret_cast<uint4*>(row + half) = hi4;
+}
+
 extern "C" int ix_rope_inplace(void* x, long x_pitch, const void* cos_table, const void* sin_table, long table_rows,
                                const int* positions, long tokens, long heads, long D, long R, void* stream) {
   if (!x || !cos_table || !sin_table || !positions || tokens < 0 || heads <= 0 || D <= 0) return IX_ERR_ARG;
@@ -424,6 +472,14 @@ extern "C" int ix_rope_inplace(void* x, long x_pitch, const void* cos_table, con
   if (R <= 0 || R % 2 != 0 || R > D) return IX_ERR_ARG;
   const long total = tokens * heads * (R / 2);
   if (total == 0) return IX_OK;
+  if (R % 16 == 0 && D % 8 == 0 && x_pitch % 8 == 0 && ix_aligned(x, 16) && ix_aligned(cos_table, 16) &&
+      ix_aligned(sin_table, 16) && total / 8 < 0x7fffffffL) {
+    const unsigned total8 = (unsigned)(total / 8);
+    hipLaunchKernelGGL(k_rope8, dim3((total8 + 255u) / 256u), dim3(256), 0, (hipStream_t)stream, (bf16_t*)x, x_pitch,
+                       (const bf16_t*)cos_table, (const bf16_t*)sin_table, positions, total8, (int)heads, (int)D, (int)R,
+                       (int)table_rows);
+    return ix_launch_status();
+  }
   const long grid = (total + 255) / 256;
   if (grid > (1L << 24)) return IX_DECLINED;
   hipLaunchKernelGGL(k_rope, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, (bf16_t*)x, x_pitch,

@@ -3,6 +3,7 @@
 // override (ops/moe/moe_batch_invariant.py:422-473, ops/mm/mm_tiles.py:127-158) and of its
 // pinned non-split-K provider (ops/mm/csrc/cublaslt_pinned.cpp:1-36).
 #include "ix_gemm_core.h"
+#include "ix_gemm_stream.h"
 #include "../../include/isoexec_hip.h"
 
 // Workgroup -> tile map. Hardware hands consecutive workgroup ids to the 8 XCDs round-robin, and each XCD has
@@ -17,11 +18,10 @@
 #ifndef IX_GEMM_GN
 #define IX_GEMM_GN 4  // weight tiles of a group
 #endif
-__device__ __forceinline__ bool ix_tile_of_block(unsigned bid, int nb_m, int nb_n, int* tm, int* tn) {
+// Tile number idx of XCD xcd's run of that order.
+__device__ __forceinline__ bool ix_tile_of_run(unsigned xcd, unsigned idx, int nb_m, int nb_n, int* tm, int* tn) {
   // 32-bit arithmetic throughout (the launch refuses more than 2^31 tiles): a 64-bit division costs a workgroup
   // about a microsecond before its first fetch.
-  const unsigned xcd = bid & 7u;
-  const unsigned idx = bid >> 3;
   const unsigned tiles = (unsigned)nb_m * (unsigned)nb_n;
   // this XCD's run of the tile order: [tiles * xcd / 8, tiles * (xcd + 1) / 8)
   const unsigned q = tiles >> 3, r = tiles & 7u;
@@ -53,6 +53,16 @@ __device__ __forceinline__ void ix_store4(float* p, int valid, bool vec, const f
     for (int e = 0; e < 4; ++e)
       if (e < valid) p[e] = v[e];
   }
+}
+
+// Row-max parts a tile writes per row: one, except the four-wave 256 x 256 tile, which writes one per wave column.
+template <int BM, int BN, int WM, int WN, int PW>
+__host__ __device__ constexpr int ix_gemm_parts_per_tile() {
+  return (BM == 256 && BN == 256 && WM == 2 && WN == 2 && PW == 0) ? WN : 1;
+}
+
+__device__ __forceinline__ bool ix_tile_of_block(unsigned bid, int nb_m, int nb_n, int* tm, int* tn) {
+  return ix_tile_of_run(bid & 7u, bid >> 3, nb_m, nb_n, tm, tn);
 }
 
 // TC = bf16_t: C is the bf16 round of the fp32 accumulator; TC = float: the accumulator itself.
@@ -186,12 +196,99 @@ __global__ __launch_bounds__((WM * WN + PW) * 64) void k_gemm_bf16_nt(const bf16
     }
     __syncthreads();
     for (int r = threadIdx.x; r < m_valid; r += Cfg::NTT) {
-      float v = s_max[r];
+      if constexpr (ix_gemm_parts_per_tile<BM, BN, WM, WN, PW>() == WN) {
+        // one part per wave column: the layout the streaming form of this tile writes without passing through LDS
 #pragma unroll
-      for (int w = 1; w < WN; ++w) v = fmaxf(v, s_max[w * BM + r]);
-      row_max_parts[(m0 + r) * parts_ld + tn] = v;
+        for (int w = 0; w < WN; ++w) row_max_parts[(m0 + r) * parts_ld + tn * WN + w] = s_max[w * BM + r];
+      } else {
+        float v = s_max[r];
+#pragma unroll
+        for (int w = 1; w < WN; ++w) v = fmaxf(v, s_max[w * BM + r]);
+        row_max_parts[(m0 + r) * parts_ld + tn] = v;
+      }
     }
   }
+}
+
+// ---- the streaming form of the four-wave 256 x 256 tile (pipeline F) -----------------------------------------------
+// bf16 output without bias, K a multiple of 64 with at least IX_STREAM_MIN_KT k-tiles, N a multiple of 8, rows of C
+// 16-byte aligned. A workgroup takes every (gridDim.x / 8)-th tile of its XCD's run of the tile order.
+// Tile sequence of the dense product: position idx of XCD xcd's run of the tile order above.
+struct IxDenseStreamSeq {
+  const bf16_t* A;
+  const bf16_t* W;
+  bf16_t* C;
+  float* parts;
+  long lda, ldw, ldc, parts_ld;
+  int M, N, K, nb_m, nb_n;
+  __device__ __forceinline__ bool locate(unsigned xcd, unsigned idx, IxStreamTile& t) const {
+    int tm, tn;
+    if (!ix_tile_of_run(xcd, idx, nb_m, nb_n, &tm, &tn)) return false;
+    const long m0 = (long)tm * 256, n0 = (long)tn * 256;
+    t.x = A + m0 * lda;
+    t.w = W + n0 * ldw;
+    t.c = C + m0 * ldc + n0;
+    t.part = parts + m0 * parts_ld + tn * 2;
+    t.mv = (int)min(256L, (long)M - m0);
+    t.nv = (int)min(256L, (long)N - n0);
+    return true;
+  }
+};
+
+template <bool PARTS>
+__global__ __launch_bounds__(256) void k_gemm_bf16_nt_stream(const bf16_t* __restrict__ A, long lda,
+                                                             const bf16_t* __restrict__ W, long ldw,
+                                                             bf16_t* __restrict__ C, long ldc, int M, int N, int K,
+                                                             int nb_m, int nb_n, float* __restrict__ row_max_parts,
+                                                             long parts_ld) {
+  using Cfg = IxGemmCfg<256, 256, 2, 2>;
+  extern __shared__ __align__(16) char ix_lds[];
+  IxPlainStreamJob<Cfg, IxDenseStreamSeq, PARTS> job;
+  job.seq.A = A;
+  job.seq.lda = lda;
+  job.seq.W = W;
+  job.seq.ldw = ldw;
+  job.seq.C = C;
+  job.seq.ldc = ldc;
+  job.seq.M = M;
+  job.seq.N = N;
+  job.seq.K = K;
+  job.seq.nb_m = nb_m;
+  job.seq.nb_n = nb_n;
+  job.seq.parts = row_max_parts;
+  job.seq.parts_ld = parts_ld;
+  ix_gemm_stream4<Cfg>(job, K / IX_BK, ix_lds);
+}
+
+static bool ix_gemm_stream_fits(const void* C, long ldc, long M, long N, long K, const void* bias, long batch,
+                                long min_tiles) {
+  const long tiles = ((M + 255) / 256) * ((N + 255) / 256);
+  return !bias && batch == 1 && (K % IX_BK == 0) && K / IX_BK >= IX_STREAM_MIN_KT && (N % 8 == 0) && (ldc % 8 == 0) &&
+         ix_aligned(C, 16) && ldc * 512 < 0x40000000L && tiles >= min_tiles;
+}
+
+static int ix_gemm_bf16_stream_launch(const bf16_t* A, long lda, const bf16_t* W, long ldw, bf16_t* C, long ldc, long M,
+                                      long N, long K, float* parts, long parts_ld, hipStream_t st) {
+  using Cfg = IxGemmCfg<256, 256, 2, 2>;
+  const long nb_m = (M + 255) / 256, nb_n = (N + 255) / 256;
+  if (nb_m * nb_n > 0x7fffffffL) return IX_DECLINED;
+  if (parts && parts_ld < nb_n * 2) return IX_ERR_ARG;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)k_gemm_bf16_nt_stream<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            Cfg::LDS_BYTES) != hipSuccess ||
+        hipFuncSetAttribute((const void*)k_gemm_bf16_nt_stream<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            Cfg::LDS_BYTES) != hipSuccess)
+      return IX_ERR_LAUNCH;
+    attr_set = true;
+  }
+  if (parts)
+    hipLaunchKernelGGL(k_gemm_bf16_nt_stream<true>, dim3(IX_STREAM_WORKGROUPS), dim3(256), Cfg::LDS_BYTES, st, A, lda, W,
+                       ldw, C, ldc, (int)M, (int)N, (int)K, (int)nb_m, (int)nb_n, parts, parts_ld);
+  else
+    hipLaunchKernelGGL(k_gemm_bf16_nt_stream<false>, dim3(IX_STREAM_WORKGROUPS), dim3(256), Cfg::LDS_BYTES, st, A, lda, W,
+                       ldw, C, ldc, (int)M, (int)N, (int)K, (int)nb_m, (int)nb_n, parts, parts_ld);
+  return ix_launch_status();
 }
 
 template <int BM, int BN, int WM, int WN, typename TC, int PW = 0>
@@ -202,7 +299,7 @@ static int ix_gemm_bf16_launch(const bf16_t* A, long lda, const bf16_t* W, long 
   const long nb_m = (M + BM - 1) / BM, nb_n = (N + BN - 1) / BN;
   const long grid = 8 * ((nb_m * nb_n + 7) / 8);  // 8 XCD runs of the tile order, the longest one sets the count
   if (grid > 0x7fffffffL) return IX_DECLINED;
-  if (parts && parts_ld < nb_n) return IX_ERR_ARG;
+  if (parts && parts_ld < nb_n * ix_gemm_parts_per_tile<BM, BN, WM, WN, PW>()) return IX_ERR_ARG;
   auto kern = k_gemm_bf16_nt<BM, BN, WM, WN, TC, PW>;
   static bool attr_set = false;  // per instantiation
   if (!attr_set) {
@@ -259,8 +356,9 @@ static int ix_gemm_tile_for(long M, long N, long K, int tile) {
 // Row-max parts per row of C: one per column tile of the shape that runs.
 extern "C" long ix_gemm_bf16_n_tiles(long M, long N, long K, int tile) {
   const int t = ix_gemm_tile_for(M, N, K, tile);
-  const long bn = (t == 2) ? 128 : (t == 6) ? 32 : 256;  // ids 1, 3, 4, 5 are 256 wide
-  return N <= 0 ? 0 : (N + bn - 1) / bn;
+  const long bn = (t == 2) ? 128 : (t == 6) ? 32 : 256;  // ids 1, 3, 4, 5, 7, 8 are 256 wide
+  const long per_tile = (t == 4 || t == 7 || t == 8) ? 2 : 1;      // the four-wave tile writes one part per wave column
+  return N <= 0 ? 0 : per_tile * ((N + bn - 1) / bn);
 }
 
 template <typename TC>
@@ -273,9 +371,23 @@ static int ix_gemm_bf16_dispatch(const bf16_t* a, long lda, const bf16_t* w, lon
     case 1: return ix_gemm_bf16_launch<32, 256, 1, 4, TC, 4>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st IX_BATCH_ARGS);
     case 2: return ix_gemm_bf16_launch<128, 128, 2, 2, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st IX_BATCH_ARGS);
     case 3: return ix_gemm_bf16_launch<256, 256, 2, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st IX_BATCH_ARGS);
-    case 4: return ix_gemm_bf16_launch<256, 256, 2, 2, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st IX_BATCH_ARGS);
+    case 4:
+      if constexpr (sizeof(TC) == 2) {
+        // worth it from two tiles per workgroup up
+        if (ix_gemm_stream_fits(c, ldc, M, N, K, b, batch, 2 * IX_STREAM_WORKGROUPS))
+          return ix_gemm_bf16_stream_launch(a, lda, w, ldw, (bf16_t*)c, ldc, M, N, K, parts, parts_ld, st);
+      }
+      [[fallthrough]];
+    case 7:  // the same tile, one tile per workgroup
+      return ix_gemm_bf16_launch<256, 256, 2, 2, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st IX_BATCH_ARGS);
     case 5: return ix_gemm_bf16_launch<128, 256, 2, 4, TC>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st IX_BATCH_ARGS);
     case 6: return ix_gemm_bf16_launch<64, 32, 2, 1, TC, 2>(a, lda, w, ldw, b, c, ldc, M, N, K, parts, parts_ld, st IX_BATCH_ARGS);
+    case 8:  // the streaming form whatever the number of tiles (declines what it does not serve)
+      if constexpr (sizeof(TC) == 2) {
+        if (ix_gemm_stream_fits(c, ldc, M, N, K, b, batch, 1))
+          return ix_gemm_bf16_stream_launch(a, lda, w, ldw, (bf16_t*)c, ldc, M, N, K, parts, parts_ld, st);
+      }
+      return IX_DECLINED;
     default: return IX_ERR_ARG;
   }
 #undef IX_BATCH_ARGS

@@ -115,6 +115,28 @@ __device__ __forceinline__ void ix_dma16(ix_rsrc_t rsrc, uint32_t lds_addr, uint
                : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
                : "memory", "m0");
 }
+// Stores through a descriptor: an offset outside its range (IX_OOB, or a row past the tile) is dropped by the hardware,
+// so a predicated store needs no branch.
+typedef __attribute__((ext_vector_type(4))) uint32_t ix_u32x4;
+__device__ __forceinline__ ix_rsrc_t ix_rsrc_scalar(ix_rsrc_t r) {  // a descriptor operand must sit in scalar registers
+  r.x = __builtin_amdgcn_readfirstlane(r.x);
+  r.y = __builtin_amdgcn_readfirstlane(r.y);
+  r.z = __builtin_amdgcn_readfirstlane(r.z);
+  r.w = __builtin_amdgcn_readfirstlane(r.w);
+  return r;
+}
+__device__ __forceinline__ void ix_buffer_store16(uint4 v, ix_rsrc_t rsrc, uint32_t voff) {
+  const ix_u32x4 d = {v.x, v.y, v.z, v.w};
+  // the two idle states keep the next instruction from overwriting the data registers while the store still reads them
+  // (the compiler would place them itself for a store it knows; it does not look into this one)
+  asm volatile("buffer_store_dwordx4 %0, %1, %2, 0 offen\n\ts_nop 1"
+               :
+               : "v"(d), "v"(voff), "s"(ix_rsrc_scalar(rsrc))
+               : "memory");
+}
+__device__ __forceinline__ void ix_buffer_store4(uint32_t v, ix_rsrc_t rsrc, uint32_t voff) {
+  asm volatile("buffer_store_dword %0, %1, %2, 0 offen" : : "v"(v), "v"(voff), "s"(ix_rsrc_scalar(rsrc)) : "memory");
+}
 __device__ __forceinline__ uint32_t ix_lds_addr(const char* p) {
   return (uint32_t)reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) char*)p);
 }

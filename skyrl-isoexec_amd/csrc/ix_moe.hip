@@ -15,6 +15,7 @@
 // map are integer-only and only decide which workgroup computes a row; the GEMM core's K order
 // is fixed (ix_gemm_core.h).
 #include "ix_gemm_core.h"
+#include "ix_gemm_stream.h"
 #include "../../include/isoexec_hip.h"
 
 #define IX_MOE_KMAX 16
@@ -890,6 +891,51 @@ __global__ __launch_bounds__(WM* WN * 64) void k_moe_fc2(const bf16_t* __restric
   });
 }
 
+// ---- streaming form of the second expert GEMM (pipeline F): the four-wave 256 x 256 tile, Hd a multiple of 256, F a
+// multiple of 64 with at least IX_STREAM_MIN_KT k-tiles. A workgroup takes every (gridDim.x / 8)-th tile of its XCD's run
+// of the (row tile, column tile) order of ix_moe_tile_of_block.
+struct IxMoeFc2Seq {
+  const bf16_t* inter;
+  const bf16_t* W2;
+  bf16_t* out;
+  const int* meta;
+  int max_tiles, Hd, nb_n, K;  // K = F
+  long lda, ldw, ldc, parts_ld;  // F, F, Hd, unused
+  __device__ __forceinline__ bool locate(unsigned xcd, unsigned idx, IxStreamTile& t) const {
+    int mt, nt;
+    if (!ix_moe_tile_of_block(xcd + 8u * idx, meta[0], nb_n, &mt, &nt)) return false;
+    const long e = meta[1 + mt], row0 = meta[1 + max_tiles + mt];
+    t.x = inter + row0 * K;
+    t.w = W2 + (e * Hd + (long)nt * 256) * K;
+    t.c = out + row0 * Hd + (long)nt * 256;
+    t.part = nullptr;
+    t.mv = meta[1 + 2 * max_tiles + mt];
+    t.nv = 256;
+    return true;
+  }
+};
+
+__global__ __launch_bounds__(256) void k_moe_fc2_stream(const bf16_t* __restrict__ inter, const bf16_t* __restrict__ W2,
+                                                        const int* __restrict__ meta, int max_tiles,
+                                                        bf16_t* __restrict__ out, int Hd, int F, int nb_n) {
+  using Cfg = IxGemmCfg<256, 256, 2, 2>;
+  extern __shared__ __align__(16) char ix_lds[];
+  IxPlainStreamJob<Cfg, IxMoeFc2Seq, false> job;
+  job.seq.inter = inter;
+  job.seq.W2 = W2;
+  job.seq.out = out;
+  job.seq.meta = meta;
+  job.seq.max_tiles = max_tiles;
+  job.seq.Hd = Hd;
+  job.seq.nb_n = nb_n;
+  job.seq.K = F;
+  job.seq.lda = F;
+  job.seq.ldw = F;
+  job.seq.ldc = Hd;
+  job.seq.parts_ld = 0;
+  ix_gemm_stream4<Cfg>(job, F / IX_BK, ix_lds);
+}
+
 template <int BM, int BN, int WM, int WN>
 static int ix_moe_experts_launch(const bf16_t* x, long ldx, int T, const int* sorted_token,
                                  const float* permuted_prob,
@@ -913,6 +959,22 @@ static int ix_moe_experts_launch(const bf16_t* x, long ldx, int T, const int* so
   // 8 XCD runs of the tile order; the longest run sets the count
   hipLaunchKernelGGL(k1, dim3((unsigned)(8 * ((max_tiles * nb1 + 7) / 8))), dim3(Cfg::NT), Cfg::LDS_BYTES, st, x, ldx, T,
                      sorted_token, permuted_prob, W1, meta, (int)max_tiles, inter, Hd, F, (int)nb1);
+  if constexpr (BM == 256 && BN == 256 && WM == 2 && WN == 2) {
+    // worth it from two tiles per workgroup up (max_tiles bounds the row tiles from above by at most one per expert)
+    if (F % IX_BK == 0 && F / IX_BK >= IX_STREAM_MIN_KT && Hd % 256 == 0 && (long)Hd * 512 < 0x40000000L &&
+        max_tiles * nb2 >= 2 * IX_STREAM_WORKGROUPS) {
+      static bool attr2_set = false;
+      if (!attr2_set) {
+        if (hipFuncSetAttribute((const void*)k_moe_fc2_stream, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                Cfg::LDS_BYTES) != hipSuccess)
+          return IX_ERR_LAUNCH;
+        attr2_set = true;
+      }
+      hipLaunchKernelGGL(k_moe_fc2_stream, dim3(IX_STREAM_WORKGROUPS), dim3(256), Cfg::LDS_BYTES, st, inter, W2, meta,
+                         (int)max_tiles, out, Hd, F, (int)nb2);
+      return ix_launch_status();
+    }
+  }
   hipLaunchKernelGGL(k2, dim3((unsigned)(8 * ((max_tiles * nb2 + 7) / 8))), dim3(Cfg::NT), Cfg::LDS_BYTES, st, inter, W2, meta,
                      (int)max_tiles, out, Hd, F, (int)nb2);
   return ix_launch_status();

@@ -39,18 +39,19 @@ def test_host_only_entry_points():
 
 def test_gemm_tile_choice_is_a_host_decision_with_sane_answers():
     """ix_gemm_bf16_n_tiles reports the row-max parts of the tile shape that would run: forced shapes give
-    ceil(N / width); the automatic choice takes the big square tile for a large product, a 128-wide tile for the
-    router's 128-column product, and a narrow tile when there are few rows and few columns."""
+    ceil(N / width), twice that for the four-wave 256 x 256 tile in any of its forms (one part per wave column); the
+    automatic choice takes the big square tile for a large product, a 128-wide tile for the router's 128-column
+    product, and a narrow tile when there are few rows and few columns."""
     h = _lib.lib()
-    widths = {1: 256, 2: 128, 3: 256, 4: 256, 5: 256, 6: 32}
-    for tile, bn in widths.items():
+    widths = {1: (256, 1), 2: (128, 1), 3: (256, 1), 4: (256, 2), 5: (256, 1), 6: (32, 1), 7: (256, 2), 8: (256, 2)}
+    for tile, (bn, per_tile) in widths.items():
         for n in (1, 32, 128, 129, 2048, 151936):
-            assert h.ix_gemm_bf16_n_tiles(4096, n, 4096, tile) == -(-n // bn), (tile, n)
-    assert h.ix_gemm_bf16_n_tiles(4096, 151936, 4096, 0) == -(-151936 // 256)     # LM head: 256-wide tiles
+            assert h.ix_gemm_bf16_n_tiles(4096, n, 4096, tile) == per_tile * -(-n // bn), (tile, n)
+    assert h.ix_gemm_bf16_n_tiles(4096, 151936, 4096, 0) == 2 * -(-151936 // 256)  # LM head: the four-wave 256-wide tile
     assert h.ix_gemm_bf16_n_tiles(163840, 128, 2048, 0) == 1                       # gating product: one 128-wide column
     assert h.ix_gemm_bf16_n_tiles(64, 2048, 2048, 0) == 2048 // 32                 # decode projection: 64 x 32 tiles
     assert h.ix_gemm_bf16_n_tiles(64, 12352, 2048, 0) == 12352 // 32               # wide decode projection: the same
-    assert h.ix_gemm_bf16_n_tiles(256, 12352, 2048, 0) in (-(-12352 // 128), -(-12352 // 256))  # 256 rows: wider tiles
+    assert h.ix_gemm_bf16_n_tiles(256, 12352, 2048, 0) in (-(-12352 // 128), -(-12352 // 256), 2 * -(-12352 // 256))  # 256 rows: wider tiles
     assert h.ix_gemm_bf16_n_tiles(0, 0, 4096, 0) == 0
 
 

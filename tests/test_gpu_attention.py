@@ -249,6 +249,22 @@ def test_rope_bit_exact_in_place_on_a_strided_slice():
     assert same_bits(one, whole[4:5]) and same_bits(whole[0], x[0])
 
 
+@pytest.mark.parametrize("R", [8, 40, 48, 128])
+def test_rope_scalar_and_vector_kernels_give_the_oracle_bits(R):
+    """R / 2 a multiple of 8 takes the kernel with 16-byte accesses (48, 128), any other even width the element kernel
+    (8, 40): both are the oracle's expression element by element."""
+    from isoexec_amd.ops.rope.rope_hip import apply_rope_, rope_tables
+
+    g = cpu_gen(R)
+    x = torch.randn(37, 5, 128, generator=g).to(torch.bfloat16)
+    pos = torch.randint(0, 300, (37,), generator=g, dtype=torch.int32)
+    cos, sin = rope_tables(300, R, 1e6, device=DEV)
+    co, so = o_attn.rope_tables(300, R, 1e6)
+    got = apply_rope_(x.clone().to(DEV), cos, sin, pos.to(DEV))
+    want = o_attn.rope(bf16_to_np(x), co, so, pos.numpy())
+    assert np.array_equal(np_bits(bf16_to_np(got)), np_bits(want))
+
+
 def test_rope_positions_outside_the_tables_read_nothing_and_give_nan():
     """The kernel bounds every position by the tables' row count: a position past the end (or negative) makes that
     token's rotated lanes NaN instead of reading beyond the tables; its neighbours are rotated as usual."""
