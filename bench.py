@@ -31,8 +31,8 @@ PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch of the dominant kernels, NOT measured in this run: from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE of the same workload (scaled by what the same counters read for a 1 GiB copy, x2.0 / x1.0), recorded in
 # the named file under profiles/.
-MEASURED_TRAFFIC_BYTES = {"dense_head_M4096_gemm": 13.83e9, "gdn_decode_B256": 1.080e9,
-                          "moe_T16384_grouped_gemms": 3.87e9, "moe_T163840_grouped_gemms": 36.9e9}
+MEASURED_TRAFFIC_BYTES = {"dense_head_M4096_gemm": 15.5e9, "gdn_decode_B256": 1.080e9,
+                          "moe_T16384_grouped_gemms": 3.91e9, "moe_T163840_grouped_gemms": 34.4e9}
 TRAFFIC_SOURCE = {"dense_head_M4096_gemm": "profiles/gemm_bf16_nt__dense_head_M4096.txt",
                   "gdn_decode_B256": "profiles/gdn_scan__decode_B256.txt",
                   "moe_T16384_grouped_gemms": "profiles/moe_ffn__T16384.txt",
@@ -138,7 +138,7 @@ def dense_head(args):
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_MFMA_BF16_TFLOPS,
                      "traffic": MEASURED_TRAFFIC_BYTES["dense_head_M4096_gemm"] if M == 4096 else None,
-                     "kernel": "k_gemm_bf16_nt (+ 7 us row-max reduce)", "kernel_ms": gemm_ms},
+                     "kernel": "k_gemm_bf16_nt_stream (+ 12 us row-max reduce)", "kernel_ms": gemm_ms},
         "kernels_ms": {"rmsnorm": t_norm.mean_ms(), "gemm": gemm_ms, "logprob": lp_ms},
         "logprob_hbm": {"bound": "hbm", "achieved": M * V * 2 / (lp_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
                         "unit": "GB/s", "frac": M * V * 2 / (lp_ms * 1e-3) / 1e9 / PEAK_HBM_GBS},
@@ -256,7 +256,7 @@ def moe(args):
             "roofline": {"bound": "mfma", "achieved": exp_fl / (exp_ms * 1e-3) / 1e12, "peak": PEAK_MFMA_BF16_TFLOPS,
                          "unit": "TFLOP/s", "frac": exp_fl / (exp_ms * 1e-3) / 1e12 / PEAK_MFMA_BF16_TFLOPS,
                          "traffic": MEASURED_TRAFFIC_BYTES["moe_T16384_grouped_gemms"] if T == 16384 else None,
-                         "kernel": "k_moe_fc1_glu + k_moe_fc2 (grouped GEMMs)", "kernel_ms": exp_ms},
+                         "kernel": "k_moe_fc1_glu + k_moe_fc2_stream (grouped GEMMs)", "kernel_ms": exp_ms},
             "whole_ffn": {"kernel_ms": ms, "achieved": fl / (ms * 1e-3) / 1e12, "unit": "TFLOP/s",
                           "frac": fl / (ms * 1e-3) / 1e12 / PEAK_MFMA_BF16_TFLOPS,
                           "kernels": "router product + router + permutation + grouped GEMMs + combine"}}
@@ -351,7 +351,7 @@ def north_star_kernels(w, dev, steps):
     ms = _events_ms(lambda: experts_forward(x, lw["w1"], lw["w2"], perm), 3, steps)
     fl = 2.0 * T * k * H * (2 * F) + 2.0 * T * k * F * H
     out["moe_grouped_gemms_T16384"] = {
-        "bound": "mfma", "kernel": "k_moe_fc1_glu + k_moe_fc2", "kernel_ms": ms, "achieved": fl / ms / 1e9,
+        "bound": "mfma", "kernel": "k_moe_fc1_glu + k_moe_fc2_stream", "kernel_ms": ms, "achieved": fl / ms / 1e9,
         "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s", "frac": fl / ms / 1e9 / PEAK_MFMA_BF16_TFLOPS,
         "traffic": MEASURED_TRAFFIC_BYTES["moe_T16384_grouped_gemms"],
         "traffic_source": TRAFFIC_SOURCE["moe_T16384_grouped_gemms"] + " (not measured in this run)"}
@@ -386,7 +386,7 @@ def north_star_kernels(w, dev, steps):
     ms = _events_ms(gemm, 2, steps)
     fl = 2.0 * M * Vv * Kd
     out["lm_head_gemm_M4096_K4096"] = {
-        "bound": "mfma", "kernel": "k_gemm_bf16_nt (+ row-max reduce)", "kernel_ms": ms, "achieved": fl / ms / 1e9,
+        "bound": "mfma", "kernel": "k_gemm_bf16_nt_stream (+ row-max reduce)", "kernel_ms": ms, "achieved": fl / ms / 1e9,
         "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s", "frac": fl / ms / 1e9 / PEAK_MFMA_BF16_TFLOPS,
         "traffic": MEASURED_TRAFFIC_BYTES["dense_head_M4096_gemm"],
         "traffic_source": TRAFFIC_SOURCE["dense_head_M4096_gemm"] + " (not measured in this run)"}
@@ -500,7 +500,7 @@ def hybrid(args):
                         "unit": "TFLOP/s", "frac": exp_fl / exp_ms / 1e9 / PEAK_MFMA_BF16_TFLOPS,
                         "traffic": MEASURED_TRAFFIC_BYTES["moe_T163840_grouped_gemms"] if total == 163840 else None,
                         "traffic_source": TRAFFIC_SOURCE["moe_T163840_grouped_gemms"] + " (not measured in this run)",
-                        "kernel": f"k_moe_fc1_glu + k_moe_fc2 (grouped expert GEMMs, {total} tokens x top-8 per launch "
+                        "kernel": f"k_moe_fc1_glu + k_moe_fc2_stream (grouped expert GEMMs, {total} tokens x top-8 per launch "
                                   f"pair, {cfg.layers} pairs per pass)", "kernel_ms": exp_ms,
                         "share_of_step": cfg.layers * exp_ms / (dt * 1e3)},
            "rollout": {"prefill_tokens_per_s": n * prompt / t_prefill, "decode_ms_per_step": t_dec * 1e3,
