@@ -109,11 +109,26 @@ __device__ __forceinline__ ix_rsrc_t ix_make_rsrc(const void* base, uint32_t byt
 // that the compiler does not count these loads: it would otherwise force "all loads done" before
 // every LDS read, and the ring of stages below relies on waiting only for the oldest group
 // (explicit s_waitcnt vmcnt(N); vector loads retire in order).
+//
+// Wait states the compiler does not place for an instruction it cannot see into (asm_hazards.py checks the generated
+// code for both): M0 written by a scalar instruction needs one before the load reads it, and a scalar register written
+// by a VECTOR instruction (v_readfirstlane, or v_readlane: the reload of a spilled scalar register) needs five before a
+// vector-memory instruction reads it as descriptor word or scalar offset -- the load would otherwise go to the address
+// the old value gives, and the scalar offset is not even range-checked. IDLE = 0 gives the one state for M0 and is right
+// where every scalar operand comes from scalar arithmetic; a kernel short of scalar registers takes IDLE = 3.
+template <int IDLE = 0>
 __device__ __forceinline__ void ix_dma16(ix_rsrc_t rsrc, uint32_t lds_addr, uint32_t voff, int soff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-               :
-               : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
-               : "memory", "m0");
+  static_assert(IDLE == 0 || IDLE == 3, "one wait state for M0, or five for scalar operands a vector instruction wrote");
+  if constexpr (IDLE == 0)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+                 : "memory", "m0");
+  else
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+                 : "memory", "m0");
 }
 // Stores through a descriptor: an offset outside its range (IX_OOB, or a row past the tile) is dropped by the hardware,
 // so a predicated store needs no branch.
@@ -127,15 +142,22 @@ __device__ __forceinline__ ix_rsrc_t ix_rsrc_scalar(ix_rsrc_t r) {  // a descrip
 }
 __device__ __forceinline__ void ix_buffer_store16(uint4 v, ix_rsrc_t rsrc, uint32_t voff) {
   const ix_u32x4 d = {v.x, v.y, v.z, v.w};
-  // the two idle states keep the next instruction from overwriting the data registers while the store still reads them
-  // (the compiler would place them itself for a store it knows; it does not look into this one)
-  asm volatile("buffer_store_dwordx4 %0, %1, %2, 0 offen\n\ts_nop 1"
+  // the two idle states after it keep the next instruction from overwriting the data registers while the store still
+  // reads them (the compiler would place them itself for a store it knows; it does not look into this one); the five
+  // before it let the descriptor words, which a vector instruction has just moved into scalar registers, arrive
+  asm volatile("s_nop 4\n\tbuffer_store_dwordx4 %0, %1, %2, 0 offen\n\ts_nop 1"
                :
                : "v"(d), "v"(voff), "s"(ix_rsrc_scalar(rsrc))
                : "memory");
 }
 __device__ __forceinline__ void ix_buffer_store4(uint32_t v, ix_rsrc_t rsrc, uint32_t voff) {
-  asm volatile("buffer_store_dword %0, %1, %2, 0 offen" : : "v"(v), "v"(voff), "s"(ix_rsrc_scalar(rsrc)) : "memory");
+  asm volatile("s_nop 4\n\tbuffer_store_dword %0, %1, %2, 0 offen" : : "v"(v), "v"(voff), "s"(ix_rsrc_scalar(rsrc)) : "memory");
+}
+// A point the eight values must have been computed by, and that volatile assembly after it cannot pass: keeps the
+// compiler from issuing a long run of accumulator reads first and the arithmetic on them afterwards (hundreds of live
+// registers).
+__device__ __forceinline__ void ix_pin8(const uint32_t (&v)[8]) {
+  asm volatile("" : : "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]), "v"(v[4]), "v"(v[5]), "v"(v[6]), "v"(v[7]));
 }
 __device__ __forceinline__ uint32_t ix_lds_addr(const char* p) {
   return (uint32_t)reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) char*)p);

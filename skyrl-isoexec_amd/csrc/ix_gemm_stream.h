@@ -23,6 +23,10 @@
 //                                     the descriptors are tile-local)
 //   template <int J> uint32_t x_voff() / w_voff()   offset of chunk J; the ring asks for an operand's chunks in the
 //                                     cyclic order 0, 1, .. 7, 0, .., so a job may keep one running register
+//   void turn_offsets()               called in the second-last k-tile after the last fetch through the current tile's
+//                                     offsets: a job whose offsets depend on the tile (gathered rows) turns them to the
+//                                     next tile here; nothing in it may make the compiler wait for the operand stream
+//   static constexpr int DMA_IDLE     0, or 3 for a job that is short of scalar registers (ix_dma16)
 //   void drain(acc)                   accumulators -> pending registers; current tile becomes the pending one
 //   void advance()                    next tile becomes the current one
 //   template <int I> void micro()     micro-step I of the pending tile's epilogue, I in [0, 64 * NSK)
@@ -102,7 +106,7 @@ __device__ __forceinline__ void ix_gemm_stream4(Job& job, int KT, char* lds) {
 
   // chunk j of k-tile t of the tile that `rsrc` describes into ring slot `slot` (K is a multiple of 64 here: no tail)
   auto fetch = [&](const ix_rsrc_t& rsrc, uint32_t voff, int t, int slot, int j) {
-    ix_dma16(rsrc, lds_base + slot * UNIT + j * NT * 16, voff, t * (IX_BK * 2));
+    ix_dma16<Job::DMA_IDLE>(rsrc, lds_base + slot * UNIT + j * NT * 16, voff, t * (IX_BK * 2));
   };
   const int frow = lane & 31, fg = lane >> 5;
   int x_foff[4], w_foff[4];
@@ -194,6 +198,7 @@ __device__ __forceinline__ void ix_gemm_stream4(Job& job, int KT, char* lds) {
     const int t1 = TAIL == 1 ? 0 : kt + 1;                       // k-tile of the X half fetched in the first phase
     const int t2 = TAIL == 2 ? 0 : (TAIL == 1 ? 1 : kt + 2);     // k-tile of the W unit and the X half after it
     IXS_PHASE(fa, fb, xs, ws, 1, (TAIL == 1 ? xr_n : xr_c), x_voff, t1, slot_x, 4, 0, ZERO, SLICE);
+    if constexpr (TAIL == 2) job.turn_offsets();  // the current tile has made its last fetch through them
     IXS_PHASE(fb, fa, xs, ws, 2, ((TAIL == 1 || TAIL == 2) ? wr_n : wr_c), w_voff, t2, slot_w, 0, 1, false, SLICE);
     IXS_PHASE(fa, fb, xs, ws, 3, ((TAIL == 1 || TAIL == 2) ? wr_n : wr_c), w_voff, t2, slot_w, 4, 2, false, SLICE);
     // Every fragment of this k-tile is in registers, and everything older than the W unit just requested (and the
@@ -313,6 +318,8 @@ struct IxPlainStreamJob {
     asm volatile("v_add_u32 %0, %1, %0" : "+v"(wv) : "s"(J == 7 ? -7 * w_step : w_step));
     return v;
   }
+  __device__ __forceinline__ void turn_offsets() const {}  // tile-local descriptors: the offsets never change
+  static constexpr int DMA_IDLE = 0;  // every scalar operand of the loads comes from scalar arithmetic
   static constexpr int NSK = IX_STREAM_NSK;
   // (rows sit at the same offsets in every tile: the descriptors carry the tile)
   __device__ __forceinline__ void advance() { cur = nx; }

@@ -936,8 +936,291 @@ __global__ __launch_bounds__(256) void k_moe_fc2_stream(const bf16_t* __restrict
   ix_gemm_stream4<Cfg>(job, F / IX_BK, ix_lds);
 }
 
+// ---- streaming form of the first expert GEMM (pipeline F) ------------------------------------------------------------
+// The four-wave 256 x 256 tile (128 gate + 128 up columns -> 128 output columns), F a multiple of 128, Hd a multiple of
+// 64 with at least NSK + 3 k-tiles. What the one-tile kernel does after its main loop -- the SwiGLU chain of 128 outputs
+// per lane, two transcendentals each -- rides here on the NEXT tile's matrix instructions: when the accumulators move
+// out they are kept as bf16 pairs (the chain's first rounding: gate and up, 128 registers) and each pair's chain is cut
+// into eight steps of two to five instructions, one per matrix instruction of the next tile's first eight k-tiles; then,
+// in four more k-tiles, the quad transposes and the stores of the plain job. (NOW > 0 sends the first NOW of the wave's four
+// 32-token blocks through the chain at once instead: fewer registers, less hidden.) Same operations in the same order on
+// every element as chain2() of the one-tile kernel.
+// Column layout: row rho = 8 g + 4 h + i of gate block cb and of up block 2 + cb is output column 32 h + 16 cb + 4 g + i
+// of the wave's 64, so a lane ends up with 32 consecutive columns of its token. The permutation is applied where the
+// weight rows are fetched (the tile's LDS rows are in matrix-instruction order).
+// Token ids and routing weights of a tile are read with scalar loads, eight consecutive values each (the group's start
+// clamped so that the eight stay inside the arrays; the lane selector makes up for the shift), written into the lanes of
+// one register and dealt out through one lane-permute per group: a vector load inside the loop would make the compiler
+// wait for the whole operand stream before its first use.
+// Scalar registers are short here (six pointers, five descriptors, the ring's bookkeeping): every address part that can
+// be a running vector register is one, and the loads keep the five wait states for scalar operands that the compiler
+// had to reload (DMA_IDLE).
+typedef int ix_i32x8u __attribute__((ext_vector_type(8), aligned(4)));
+template <int LANE>
+__device__ __forceinline__ int ix_writelane(int v, int u) {  // v with lane LANE replaced by the wave-uniform u
+  asm volatile("v_writelane_b32 %0, %1, %2" : "+v"(v) : "s"(u), "n"(LANE));
+  return v;
+}
+
+struct IxMoeFc1StreamJob {
+  const bf16_t* x;
+  long ldx;
+  int T;
+  int rows;  // permuted rows in all (T * k)
+  const int* sorted_token;
+  const float* permuted_prob;
+  const bf16_t* W1;
+  const int* meta;
+  int max_tiles;
+  bf16_t* inter;
+  int Hd, F, nb_n;
+  unsigned xcd, idx, stride;
+  static constexpr int NOW = 0;                    // 32-token blocks chained while the accumulators move out (0: all deferred)
+  static constexpr int NCH = 2 * (4 - NOW);        // k-tiles of deferred chains
+  static constexpr int NSK = NCH + 4;              // + one k-tile of transposes and stores per 32-token block
+
+  ix_rsrc_t nx_xr, nx_wr;
+  bool has_next;
+  int nx_row0, c_row0, nx_nrows, nx_n0h, c_nrows, c_n0h;
+  static constexpr int DMA_IDLE = 3;
+  uint32_t xvo[8];  // this thread's eight activation chunks (gathered token rows)
+  uint32_t wv;      // its next weight chunk: the ring asks for chunks 0, 1, .. 7, 0, .. and w_voff() steps it on
+  int w_st16, w_stA, w_stB, w_stC;  // the four steps of that walk (bytes)
+  float prob[4];    // routing weights of this lane's four tokens: set for the current tile in its second-last k-tile, read
+                    // when its accumulators move out and by its deferred chains during the next tile
+  ix_rsrc_t p_ir;   // pending tile: descriptor of its part of inter
+  uint32_t p_voff;
+  uint32_t pg[4][2][8], pu[4][2][8];  // pending gate / up values of the deferred blocks, two bf16 per register
+  uint32_t res[4][2][8];              // chain results, accumulator layout
+  uint32_t ta[4][4], tb[4][4];
+  float g0, g1, a0, a1;               // a chain in flight
+
+  __device__ __forceinline__ void locate() {
+    int mt = 0, nt = 0;
+    has_next = ix_moe_tile_of_block(xcd + 8u * idx, meta[0], nb_n, &mt, &nt);
+    if (!has_next) {  // no tile: no rows, and a weight descriptor without bytes (its fetches touch no memory)
+      nx_row0 = nx_nrows = nx_n0h = 0;
+      nx_wr = ix_make_rsrc(W1, 0u);
+      return;
+    }
+    const long e = meta[1 + mt];
+    nx_row0 = meta[1 + max_tiles + mt];
+    nx_nrows = meta[1 + 2 * max_tiles + mt];
+    nx_n0h = nt * 128;
+    // weights: the expert's gate rows n0h .. n0h + 127 and, F rows further on, its up rows
+    nx_wr = ix_make_rsrc(W1 + (e * 2 * F + nx_n0h) * Hd, (uint32_t)(((long)F + 128) * Hd * 2));
+  }
+  __device__ __forceinline__ uint32_t kb() const {
+    return (uint32_t)(((threadIdx.x & 7) ^ ix_swz8(threadIdx.x >> 3)) * 16);  // rows 32 apart share the swizzle
+  }
+  // lanes lane0 .. lane0 + 7 of v <- the eight 32-bit values at p (wave-uniform address: one scalar load)
+  template <int LANE0>
+  __device__ __forceinline__ int put8(int v, const int* p) const {
+    const ix_i32x8u w = *reinterpret_cast<const ix_i32x8u*>(p);
+    ix_static_for<0, 8>([&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      v = ix_writelane<LANE0 + i>(v, __builtin_amdgcn_readfirstlane(w[i]));
+    });
+    return v;
+  }
+  // offsets of the gathered rows of the tile (row0, nrows): tile row r0 + 32 j of chunk j, r0 = thread / 8
+  __device__ __forceinline__ void gather_rows(int row0, int nrows) {
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int q = (threadIdx.x >> 3) & 7;
+    ix_static_for<0, 8>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+      const int base = 8 * wave + 32 * j;                // the wave's eight rows of chunk j, tile-relative
+      const int start = min(row0 + base, rows - 8);      // a permuted row past the last one is never a row of the tile
+      const int v = put8<0>(0, sorted_token + start);
+      // lane select: row base + q sits (row0 + base - start) lanes further on; rows the tile does not have read any lane
+      const uint32_t tok = (uint32_t)__builtin_amdgcn_ds_bpermute((q + (row0 + base - start)) * 4, v);
+      xvo[j] = (base + q < nrows) ? tok * (uint32_t)(ldx * 2) + kb() : IX_OOB;
+    });
+  }
+  __device__ __forceinline__ void gather_probs(int row0) {
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    ix_static_for<0, 4>([&](auto mc) {
+      constexpr int mi = decltype(mc)::value;
+      const int base = (wave >> 1) * 128 + 32 * mi;      // the 32 tokens of accumulator block row mi
+      const int start = min(row0 + base, rows - 32);
+      const int* p = reinterpret_cast<const int*>(permuted_prob) + start;
+      int v = put8<0>(0, p);
+      v = put8<8>(v, p + 8);
+      v = put8<16>(v, p + 16);
+      v = put8<24>(v, p + 24);
+      // rows past the tile's last get some lane's value: their products are dropped by the store's range check
+      prob[mi] = __int_as_float(__builtin_amdgcn_ds_bpermute(((int)(threadIdx.x & 31) + (row0 + base - start)) * 4, v));
+    });
+  }
+  __device__ __forceinline__ bool open_first() {
+    xcd = blockIdx.x & 7u;
+    idx = blockIdx.x >> 3;
+    stride = gridDim.x >> 3;
+    nx_xr = ix_make_rsrc(x, (uint32_t)(((long)(T - 1) * ldx + Hd) * 2));  // the same for every tile
+    locate();
+    p_ir = ix_make_rsrc(nullptr, 0u);  // the empty pending tile
+    p_voff = IX_OOB;
+#pragma unroll
+    for (int i = 0; i < 64; ++i) pg[i >> 4][(i >> 3) & 1][i & 7] = pu[i >> 4][(i >> 3) & 1][i & 7] = res[i >> 4][(i >> 3) & 1][i & 7] = 0u;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) prob[i] = 0.0f;
+    g0 = g1 = a0 = a1 = 0.0f;
+    return has_next;
+  }
+  __device__ __forceinline__ void open_next() {
+    idx += stride;
+    locate();
+  }
+  __device__ __forceinline__ void first_voffs() {
+    gather_rows(nx_row0, nx_nrows);
+    // Weight tile row r0 + 32 j (chunk j of thread row r0) = wave column j / 4, block j % 4 (gate 0, gate 1, up 0, up 1),
+    // matrix-instruction row r0: weight row [up: F] + 64 (j / 4) + 16 (j % 2) + lane_col(r0) of the descriptor.
+    // In rows, chunk 0..7 = 0, 16, F, F + 16, 64, 80, F + 64, F + 80 (+ lane_col); the walk's steps are the differences.
+    const int r0 = threadIdx.x >> 3;
+    const int lane_col = 32 * ((r0 >> 2) & 1) + 4 * (r0 >> 3) + (r0 & 3);
+    wv = (uint32_t)((long)lane_col * Hd * 2) + kb();
+    const int row_bytes = Hd * 2;
+    w_st16 = __builtin_amdgcn_readfirstlane(16 * row_bytes);
+    w_stA = __builtin_amdgcn_readfirstlane((F - 16) * row_bytes);
+    w_stB = __builtin_amdgcn_readfirstlane((48 - F) * row_bytes);
+    w_stC = __builtin_amdgcn_readfirstlane(-(F + 80) * row_bytes);
+  }
+  template <int J>
+  __device__ __forceinline__ uint32_t x_voff() const { return xvo[J]; }
+  // The step is added by an instruction the compiler cannot hoist, or it would keep every sum of every k-tile in a
+  // register of its own.
+  template <int J>
+  __device__ __forceinline__ uint32_t w_voff() {
+    const uint32_t v = wv;
+    asm volatile("v_add_u32 %0, %1, %0" : "+v"(wv) : "s"(J == 7 ? w_stC : (J == 3 ? w_stB : ((J & 1) ? w_stA : w_st16))));
+    return v;
+  }
+  __device__ __forceinline__ void turn_offsets() {
+    gather_probs(c_row0);                // the current tile's weights, before its accumulators move out
+    gather_rows(nx_row0, nx_nrows);      // a missing next tile has no rows: every offset out of range
+  }
+  __device__ __forceinline__ void advance() {
+    c_row0 = nx_row0;
+    c_nrows = nx_nrows;
+    c_n0h = nx_n0h;
+  }
+  // bf16(gate), bf16(up) -> s = bf16(silu(gate)) -> h = bf16(s * up) -> bf16(h * prob), two columns at a time
+  static __device__ __forceinline__ uint32_t chain2(float g0_, float g1_, float u0_, float u1_, float p) {
+    float gate0, gate1, up0, up1, s0, s1, h0, h1;
+    ix_rbf2_hw(g0_, g1_, gate0, gate1);
+    ix_rbf2_hw(u0_, u1_, up0, up1);
+    ix_rbf2_hw(ix_silu_div(gate0), ix_silu_div(gate1), s0, s1);
+    ix_rbf2_hw(s0 * up0, s1 * up1, h0, h1);
+    return ix_pack_bf2_hw(h0 * p, h1 * p);
+  }
+  template <typename Acc>
+  __device__ __forceinline__ void drain(Acc& acc) {
+    ix_static_for<0, 8>([&](auto bc) {
+      constexpr int mi = decltype(bc)::value >> 1, cb = decltype(bc)::value & 1;
+      float g16[16], u16[16];
+      ix_acc_read16<true>(acc[mi][cb], g16);
+      ix_acc_read16<true>(acc[mi][2 + cb], u16);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if constexpr (mi < NOW) {
+          res[mi][cb][i] = chain2(g16[2 * i], g16[2 * i + 1], u16[2 * i], u16[2 * i + 1], prob[mi]);
+        } else {
+          pg[mi][cb][i] = ix_pack_bf2_hw(g16[2 * i], g16[2 * i + 1]);
+          pu[mi][cb][i] = ix_pack_bf2_hw(u16[2 * i], u16[2 * i + 1]);
+        }
+      }
+      if constexpr (mi < NOW) {
+        ix_pin8(res[mi][cb]);
+      } else {
+        ix_pin8(pg[mi][cb]);
+        ix_pin8(pu[mi][cb]);
+      }
+    });
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // after the quad transposes a lane holds piece (lane % 4) of the four tokens of its quad
+    const int r = (wave >> 1) * 128 + (lane & 28), c = (wave & 1) * 64 + 32 * (lane >> 5) + 8 * (lane & 3);
+    p_ir = ix_make_rsrc(inter + (long)c_row0 * F + c_n0h, (uint32_t)(((long)(c_nrows - 1) * F + 128) * 2));
+    p_voff = (uint32_t)(((long)r * F + c) * 2);
+  }
+  static constexpr int stores_after_p1(int s) { return s >= NCH ? 4 : 0; }
+  static __device__ __forceinline__ int w_frag_row(int ni, int rho) { return ni * 32 + rho; }
+  // k-tile s < NCH: the eight chains of (mi = NOW + s / 2, cb = s % 2), chain c in slots 8 c .. 8 c + 7.
+  // k-tile s = NCH + mi: the 32 tokens mi: exchange stage 1 in slots 0..15, stage 2 in 16..31, stores 32..35.
+  template <int I>
+  __device__ __forceinline__ void micro() {
+    constexpr int s = I / 64, q = I % 64;
+    if constexpr (s < NCH) {
+      constexpr int mi = NOW + (s >> 1), cb = s & 1, c = q >> 3, st = q & 7;
+      if constexpr (st == 0) {
+        g0 = __uint_as_float(pg[mi][cb][c] << 16);
+        g1 = __uint_as_float(pg[mi][cb][c] & 0xffff0000u);
+        a0 = (-g0) * IX_LOG2E;
+        a1 = (-g1) * IX_LOG2E;
+      } else if constexpr (st == 1) {
+        a0 = ix_exp2(a0);
+      } else if constexpr (st == 2) {
+        a1 = ix_exp2(a1);
+      } else if constexpr (st == 3) {
+        a0 = 1.0f + a0;
+        a1 = 1.0f + a1;
+        a0 = __builtin_amdgcn_rcpf(a0);
+      } else if constexpr (st == 4) {
+        a1 = __builtin_amdgcn_rcpf(a1);
+        a0 = g0 * a0;
+      } else if constexpr (st == 5) {
+        a1 = g1 * a1;
+        ix_rbf2_hw(a0, a1, a0, a1);
+      } else if constexpr (st == 6) {
+        const float u0 = __uint_as_float(pu[mi][cb][c] << 16), u1 = __uint_as_float(pu[mi][cb][c] & 0xffff0000u);
+        ix_rbf2_hw(a0 * u0, a1 * u1, a0, a1);
+      } else {
+        res[mi][cb][c] = ix_pack_bf2_hw(a0 * prob[mi], a1 * prob[mi]);
+      }
+    } else {
+      constexpr int mi = s - NCH;
+      if constexpr (q < 16) {
+        // piece pi, dword d of the lane's 64 bytes: res[mi][pi / 2][4 (pi % 2) + d]; stage 1 pairs pieces (0, 1), (2, 3)
+        constexpr int d = q >> 2, t = q & 3, a = t & 2;
+        ta[t][d] = ix_quad_exchange<1, (t & 1) != 0>(res[mi][a >> 1][d], res[mi][a >> 1][4 + d]);
+      } else if constexpr (q < 32) {
+        constexpr int o = q - 16, d = o >> 2, t = o & 3, a = t & 1;
+        tb[t][d] = ix_quad_exchange<2, (t & 2) != 0>(ta[a][d], ta[a + 2][d]);
+      } else if constexpr (q < 36) {
+        constexpr int t = q - 32;  // token t of the quad
+        ix_buffer_store16(make_uint4(tb[t][0], tb[t][1], tb[t][2], tb[t][3]), p_ir,
+                          p_voff == IX_OOB ? IX_OOB : p_voff + (uint32_t)((long)(mi * 32 + t) * F * 2));
+      }
+    }
+  }
+};
+
+__global__ __launch_bounds__(256) void k_moe_fc1_glu_stream(const bf16_t* __restrict__ x, long ldx, int T, int rows,
+                                                            const int* __restrict__ sorted_token,
+                                                            const float* __restrict__ permuted_prob,
+                                                            const bf16_t* __restrict__ W1, const int* __restrict__ meta,
+                                                            int max_tiles, bf16_t* __restrict__ inter, int Hd, int F,
+                                                            int nb_n) {
+  using Cfg = IxGemmCfg<256, 256, 2, 2>;
+  extern __shared__ __align__(16) char ix_lds[];
+  IxMoeFc1StreamJob job;
+  job.x = x;
+  job.ldx = ldx;
+  job.T = T;
+  job.rows = rows;
+  job.sorted_token = sorted_token;
+  job.permuted_prob = permuted_prob;
+  job.W1 = W1;
+  job.meta = meta;
+  job.max_tiles = max_tiles;
+  job.inter = inter;
+  job.Hd = Hd;
+  job.F = F;
+  job.nb_n = nb_n;
+  ix_gemm_stream4<Cfg>(job, Hd / IX_BK, ix_lds);
+}
+
 template <int BM, int BN, int WM, int WN>
-static int ix_moe_experts_launch(const bf16_t* x, long ldx, int T, const int* sorted_token,
+static int ix_moe_experts_launch(const bf16_t* x, long ldx, int T, long rows, const int* sorted_token,
                                  const float* permuted_prob,
                                  const bf16_t* W1, const bf16_t* W2, const int* meta, long max_tiles,
                                  bf16_t* inter, bf16_t* out, int Hd, int F, hipStream_t st) {
@@ -957,8 +1240,27 @@ static int ix_moe_experts_launch(const bf16_t* x, long ldx, int T, const int* so
   const long nb2 = (Hd + BN - 1) / BN;
   if (max_tiles * nb1 > 0x7fffffffL || max_tiles * nb2 > 0x7fffffffL) return IX_DECLINED;
   // 8 XCD runs of the tile order; the longest run sets the count
-  hipLaunchKernelGGL(k1, dim3((unsigned)(8 * ((max_tiles * nb1 + 7) / 8))), dim3(Cfg::NT), Cfg::LDS_BYTES, st, x, ldx, T,
-                     sorted_token, permuted_prob, W1, meta, (int)max_tiles, inter, Hd, F, (int)nb1);
+  bool fc1_streamed = false;
+  if constexpr (BM == 256 && BN == 256 && WM == 2 && WN == 2) {
+    // worth it from two tiles per workgroup up (max_tiles bounds the row tiles from above by at most one per expert)
+    // (the scalar gathers read 32 consecutive permuted rows; the walk over an expert's weight rows is 32-bit)
+    if (Hd % IX_BK == 0 && Hd / IX_BK >= IxMoeFc1StreamJob::NSK + 3 && F % 128 == 0 && rows >= 32 && rows < 0x7fffffffL &&
+        ((long)F + 128) * Hd * 2 < 0x40000000L && max_tiles * nb1 >= 2 * IX_STREAM_WORKGROUPS) {
+      static bool attr1_set = false;
+      if (!attr1_set) {
+        if (hipFuncSetAttribute((const void*)k_moe_fc1_glu_stream, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                Cfg::LDS_BYTES) != hipSuccess)
+          return IX_ERR_LAUNCH;
+        attr1_set = true;
+      }
+      hipLaunchKernelGGL(k_moe_fc1_glu_stream, dim3(IX_STREAM_WORKGROUPS), dim3(256), Cfg::LDS_BYTES, st, x, ldx, T,
+                         (int)rows, sorted_token, permuted_prob, W1, meta, (int)max_tiles, inter, Hd, F, (int)nb1);
+      fc1_streamed = true;
+    }
+  }
+  if (!fc1_streamed)
+    hipLaunchKernelGGL(k1, dim3((unsigned)(8 * ((max_tiles * nb1 + 7) / 8))), dim3(Cfg::NT), Cfg::LDS_BYTES, st, x, ldx, T,
+                       sorted_token, permuted_prob, W1, meta, (int)max_tiles, inter, Hd, F, (int)nb1);
   if constexpr (BM == 256 && BN == 256 && WM == 2 && WN == 2) {
     // worth it from two tiles per workgroup up (max_tiles bounds the row tiles from above by at most one per expert)
     if (F % IX_BK == 0 && F / IX_BK >= IX_STREAM_MIN_KT && Hd % 256 == 0 && (long)Hd * 512 < 0x40000000L &&
@@ -998,17 +1300,17 @@ extern "C" int ix_moe_experts_tile(const void* x, long ldx, const int* sorted_to
   bf16_t *it = (bf16_t*)inter, *eo = (bf16_t*)expert_out;
   if (BN != 256 && !(BN == 128 && BM == 128)) return IX_ERR_ARG;
   if (BN == 128)
-    return ix_moe_experts_launch<128, 128, 2, 2>(xx, ldx, (int)T, sorted_token, permuted_prob, w1, w2, tile_meta,
+    return ix_moe_experts_launch<128, 128, 2, 2>(xx, ldx, (int)T, rows, sorted_token, permuted_prob, w1, w2, tile_meta,
                                                  max_tiles, it, eo, (int)Hd, (int)F, st);
   switch (BM) {
     case 32:
-      return ix_moe_experts_launch<32, 256, 1, 4>(xx, ldx, (int)T, sorted_token, permuted_prob, w1, w2, tile_meta,
+      return ix_moe_experts_launch<32, 256, 1, 4>(xx, ldx, (int)T, rows, sorted_token, permuted_prob, w1, w2, tile_meta,
                                                   max_tiles, it, eo, (int)Hd, (int)F, st);
     case 128:
-      return ix_moe_experts_launch<128, 256, 2, 4>(xx, ldx, (int)T, sorted_token, permuted_prob, w1, w2, tile_meta,
+      return ix_moe_experts_launch<128, 256, 2, 4>(xx, ldx, (int)T, rows, sorted_token, permuted_prob, w1, w2, tile_meta,
                                                    max_tiles, it, eo, (int)Hd, (int)F, st);
     case 256:
-      return ix_moe_experts_launch<256, 256, 2, 2>(xx, ldx, (int)T, sorted_token, permuted_prob, w1, w2, tile_meta,
+      return ix_moe_experts_launch<256, 256, 2, 2>(xx, ldx, (int)T, rows, sorted_token, permuted_prob, w1, w2, tile_meta,
                                                    max_tiles, it, eo, (int)Hd, (int)F, st);
     default: return IX_ERR_ARG;
   }

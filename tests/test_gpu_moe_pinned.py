@@ -32,7 +32,7 @@ def make(T, H, E, F, seed):
                                           (33, 2048, 128, 768, 8, None), (600, 2048, 8, 768, 2, 256),
                                           # enough tiles for the streaming form of the grouped kernels (one workgroup walks
                                           # many tiles): the smallest K it takes with ragged experts, and the full MoE shape
-                                          (9000, 1024, 8, 704, 4, 256), (16384, 2048, 128, 768, 8, None)])
+                                          (9000, 1024, 8, 704, 4, 256), (9000, 1024, 8, 768, 4, 256), (16384, 2048, 128, 768, 8, None)])
 def test_grouped_kernels_equal_the_dense_kernel_per_expert(T, H, E, F, k, BM):
     from isoexec_amd.ops.mm.mm_hip import linear_nt, router_gemm
     from isoexec_amd.ops.moe.moe_hip import experts_forward, permute, router_topk
