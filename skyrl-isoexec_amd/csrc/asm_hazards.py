@@ -12,10 +12,16 @@ on the source to keep:
   address the range check never saw;
 * M0 written by a scalar instruction must not be read by a load-to-LDS in the next wait state.
 
+A third rule is this library's own. ``ix_load4_uncounted`` issues ``global_load_dword vN`` from inline assembly, so the
+compiler believes vN holds the value at once; the value is taken into use through ``ix_landed`` (which leaves the
+comment ``; ix_landed vN`` in the assembly). Between the two
+* no instruction may mention vN (a copy or a spill would move a value that has not arrived), and
+* there must be an ``s_waitcnt vmcnt(n)`` with at least n vector-memory instructions issued after the load (they
+  retire in order, so that wait has retired the load).
+
 Usage: ``asm_hazards.py file.s [file.s ...]`` on the output of ``hipcc -S --offload-device-only`` (``make check``
-drives it). Exit status 1 and one line per finding if a rule is broken. The scan walks each function's lines upwards
-from every inline-assembly memory instruction; a branch target closer than the five wait states is a finding of its own,
-because the instructions that jump there are not on the lines above it.
+drives it). Exit status 1 and one line per finding if a rule is broken. The scan walks upwards from every
+inline-assembly memory instruction, at a branch target along the lines above it and along every jump to it.
 """
 import re
 import sys
@@ -65,13 +71,77 @@ def wait_states(ins):
     return int(m.group(1)) + 1 if m else 1
 
 
+def vregs(text):
+    out = set()
+    for m in re.finditer(r"\bv\[(\d+):(\d+)\]", text):
+        out.update(range(int(m.group(1)), int(m.group(2)) + 1))
+    for m in re.finditer(r"\bv(\d+)\b", text):
+        out.add(int(m.group(1)))
+    return out
+
+
 def scan(path):
     findings = []
     func = "?"
     in_asm = False
     hist = []  # (instruction, from inline asm, source line number), oldest first, of the current function
+    flying = {}  # vector register -> [line of its uncounted load, vector-memory instructions issued since, retired]
+
+    pending_checks = []  # indices into hist of the inline-assembly memory instructions of the current function
+
+    def check_operands():
+        """Walks upwards from every inline-assembly memory instruction, through the function's jumps as well."""
+        jumps = {}
+        for i, (pins, _, _) in enumerate(hist):
+            m = re.match(r"^s_c?branch\w*\s+(\.LBB\w+)", pins)
+            if m:
+                jumps.setdefault(m.group(1), []).append(i)
+        for at in pending_checks:
+            ins, _, ln = hist[at]
+            ops = ins.split(None, 1)[1] if " " in ins else ""
+            used = sregs(ops)
+            lds_dma = bool(re.search(r"\blds\b", ops))
+            seen = set()
+            stack = [(at - 1, 0)]
+            while stack:
+                i, dist = stack.pop()
+                while i >= 0 and dist < VMEM_SGPR_WAIT and (i, dist) not in seen:
+                    seen.add((i, dist))
+                    pins, _, pln = hist[i]
+                    if pins.startswith("<label> "):
+                        for j in jumps.get(pins[8:], []):
+                            stack.append((j, dist))  # the jump itself is one wait state: counted when it is visited
+                        i -= 1  # and the line above the label (walking up past an unconditional jump only adds checks)
+                        continue
+                    hit = valu_sgpr_defs(pins) & used
+                    if hit:
+                        findings.append(f"{path}:{ln}: {func}: '{ins}' reads s{sorted(hit)} {dist} wait states after "
+                                        f"'{pins}' (line {pln}); {VMEM_SGPR_WAIT} needed")
+                    if lds_dma and dist < M0_LDS_WAIT and re.match(r"^s_\w+\s+m0\b", pins):
+                        findings.append(f"{path}:{ln}: {func}: '{ins}' reads m0 {dist} wait states after '{pins}'")
+                    dist += wait_states(pins)
+                    i -= 1
+        pending_checks.clear()
+
+    def close_function():
+        check_operands()
+        for reg, (lln, _, _) in flying.items():
+            findings.append(f"{path}:{lln}: {func}: uncounted load into v{reg} is never taken into use (ix_landed)")
+        flying.clear()
+
     for ln, raw in enumerate(open(path), 1):
         s = raw.strip()
+        m = re.match(r"^;\s*ix_landed\s+v(\d+)", s)
+        if in_asm and m:
+            reg = int(m.group(1))
+            if reg not in flying:
+                findings.append(f"{path}:{ln}: {func}: ix_landed v{reg} without an uncounted load into it on the lines above")
+            else:
+                if not flying[reg][2]:
+                    findings.append(f"{path}:{ln}: {func}: v{reg} taken into use, but no wait since its load (line "
+                                    f"{flying[reg][0]}) has retired it")
+                del flying[reg]
+            continue
         if s.startswith(";;#ASMSTART"):
             in_asm = True
             continue
@@ -80,40 +150,40 @@ def scan(path):
             continue
         m = re.match(r"^([A-Za-z_][\w$.]*):\s*(;.*)?$", raw)
         if m and not raw.startswith(".L"):
+            close_function()
             func = m.group(1)
             hist = []
             continue
-        if re.match(r"^\.LBB\w+:", raw):
-            hist.append(("<label>", False, ln))  # a branch target: what ran before it is not on the lines above
+        m = re.match(r"^(\.LBB\w+):", raw)
+        if m:
+            hist.append(("<label> " + m.group(1), False, ln))
             continue
         if not raw.startswith("\t") or s.startswith(";") or s.startswith("."):
             continue
         ins = s.split(";")[0].strip()
         if not ins:
             continue
+        # uncounted loads in flight: nobody touches the register, and a wait has to retire it
+        touched = vregs(ins)
+        for reg in list(flying):
+            if reg in touched:
+                findings.append(f"{path}:{ln}: {func}: '{ins}' touches v{reg} while the uncounted load of line "
+                                f"{flying[reg][0]} is in flight")
+        m = re.match(r"^s_waitcnt\b.*\bvmcnt\((\d+)\)", ins)
+        if m:
+            for st in flying.values():
+                if int(m.group(1)) <= st[1]:
+                    st[2] = True
+        if VMEM.match(ins):
+            for st in flying.values():
+                st[1] += 1
+            m = re.match(r"^global_load_dword\s+v(\d+),", ins)
+            if in_asm and m:
+                flying[int(m.group(1))] = [ln, 0, False]
         if in_asm and VMEM.match(ins):
-            ops = ins.split(None, 1)[1] if " " in ins else ""
-            used = sregs(ops)
-            lds_dma = bool(re.search(r"\blds\b", ops))
-            dist = 0
-            for pins, _, pln in reversed(hist):
-                if dist >= VMEM_SGPR_WAIT:
-                    break
-                if pins == "<label>":
-                    if used - {124}:
-                        findings.append(f"{path}:{ln}: {func}: '{ins}' sits {dist} wait states after the branch target of "
-                                        f"line {pln}: the code that jumps there is not checked")
-                    continue
-                hit = valu_sgpr_defs(pins) & used
-                if hit:
-                    findings.append(f"{path}:{ln}: {func}: '{ins}' reads s{sorted(hit)} {dist} wait states after "
-                                    f"'{pins}' (line {pln}); {VMEM_SGPR_WAIT} needed")
-                if lds_dma and dist < M0_LDS_WAIT and re.match(r"^s_\w+\s+m0\b", pins):
-                    findings.append(f"{path}:{ln}: {func}: '{ins}' reads m0 {dist} wait states after '{pins}'")
-                dist += wait_states(pins)
+            pending_checks.append(len(hist))  # checked when the function is complete (its jumps are known then)
         hist.append((ins, in_asm, ln))
-        if len(hist) > 16:
-            hist.pop(0)
+    close_function()
     return findings
 
 

@@ -153,6 +153,19 @@ __device__ __forceinline__ void ix_buffer_store16(uint4 v, ix_rsrc_t rsrc, uint3
 __device__ __forceinline__ void ix_buffer_store4(uint32_t v, ix_rsrc_t rsrc, uint32_t voff) {
   asm volatile("s_nop 4\n\tbuffer_store_dword %0, %1, %2, 0 offen" : : "v"(v), "v"(voff), "s"(ix_rsrc_scalar(rsrc)) : "memory");
 }
+// A 4-byte load the compiler does not count (see ix_dma16 for why): the value is NOT there when the statement ends.
+// The caller's own wait retires it (vector-memory operations retire in order: any later s_waitcnt vmcnt(n) with at least
+// n of them issued after this load), and the value is taken into use through ix_landed() after that wait; until then
+// nothing may read or move the register. asm_hazards.py checks all three in the generated code of every build.
+__device__ __forceinline__ uint32_t ix_load4_uncounted(const void* base, uint32_t byte_off) {
+  uint32_t v;
+  asm volatile("global_load_dword %0, %1, %2" : "=&v"(v) : "v"(byte_off), "s"(base));
+  return v;
+}
+__device__ __forceinline__ uint32_t ix_landed(uint32_t v) {
+  asm volatile("; ix_landed %0" : "+v"(v));
+  return v;
+}
 // A point the eight values must have been computed by, and that volatile assembly after it cannot pass: keeps the
 // compiler from issuing a long run of accumulator reads first and the arithmetic on them afterwards (hundreds of live
 // registers).

@@ -948,20 +948,14 @@ __global__ __launch_bounds__(256) void k_moe_fc2_stream(const bf16_t* __restrict
 // Column layout: row rho = 8 g + 4 h + i of gate block cb and of up block 2 + cb is output column 32 h + 16 cb + 4 g + i
 // of the wave's 64, so a lane ends up with 32 consecutive columns of its token. The permutation is applied where the
 // weight rows are fetched (the tile's LDS rows are in matrix-instruction order).
-// Token ids and routing weights of a tile are read with scalar loads, eight consecutive values each (the group's start
-// clamped so that the eight stay inside the arrays; the lane selector makes up for the shift), written into the lanes of
-// one register and dealt out through one lane-permute per group: a vector load inside the loop would make the compiler
-// wait for the whole operand stream before its first use.
-// Scalar registers are short here (six pointers, five descriptors, the ring's bookkeeping): every address part that can
-// be a running vector register is one, and the loads keep the five wait states for scalar operands that the compiler
-// had to reload (DMA_IDLE).
-typedef int ix_i32x8u __attribute__((ext_vector_type(8), aligned(4)));
-template <int LANE>
-__device__ __forceinline__ int ix_writelane(int v, int u) {  // v with lane LANE replaced by the wave-uniform u
-  asm volatile("v_writelane_b32 %0, %1, %2" : "+v"(v) : "s"(u), "n"(LANE));
-  return v;
-}
-
+// Token ids and routing weights: every thread loads its own (eight rows' ids, four tokens' weights; the index clamped to
+// the last permuted row) with loads the compiler does not count (ix_load4_uncounted), issued in the third-last k-tile
+// -- ids of the NEXT tile, weights of the current one -- and taken into use in the second-last: the closing wait of the
+// k-tile in between has retired them. A load the compiler knows about would make it wait for the whole operand stream
+// at the first use; scalar loads cost their full latency one after the other (3.6 us per tile, measured).
+// Scalar registers are short here (six pointers, five descriptors, the ring's bookkeeping): the walk over the weight
+// rows is one running vector register, not eight scalar offsets, which the compiler would multiply by the k-tiles of
+// the unrolled loop, spill, and reload right in front of the loads that use them.
 struct IxMoeFc1StreamJob {
   const bf16_t* x;
   long ldx;
@@ -982,7 +976,7 @@ struct IxMoeFc1StreamJob {
   ix_rsrc_t nx_xr, nx_wr;
   bool has_next;
   int nx_row0, c_row0, nx_nrows, nx_n0h, c_nrows, c_n0h;
-  static constexpr int DMA_IDLE = 3;
+  static constexpr int DMA_IDLE = 0;  // no reloaded scalar operand in front of a load (checked in every build)
   uint32_t xvo[8];  // this thread's eight activation chunks (gathered token rows)
   uint32_t wv;      // its next weight chunk: the ring asks for chunks 0, 1, .. 7, 0, .. and w_voff() steps it on
   int w_st16, w_stA, w_stB, w_stC;  // the four steps of that walk (bytes)
@@ -1013,44 +1007,31 @@ struct IxMoeFc1StreamJob {
   __device__ __forceinline__ uint32_t kb() const {
     return (uint32_t)(((threadIdx.x & 7) ^ ix_swz8(threadIdx.x >> 3)) * 16);  // rows 32 apart share the swizzle
   }
-  // lanes lane0 .. lane0 + 7 of v <- the eight 32-bit values at p (wave-uniform address: one scalar load)
-  template <int LANE0>
-  __device__ __forceinline__ int put8(int v, const int* p) const {
-    const ix_i32x8u w = *reinterpret_cast<const ix_i32x8u*>(p);
-    ix_static_for<0, 8>([&](auto ic) {
-      constexpr int i = decltype(ic)::value;
-      v = ix_writelane<LANE0 + i>(v, __builtin_amdgcn_readfirstlane(w[i]));
-    });
-    return v;
-  }
-  // offsets of the gathered rows of the tile (row0, nrows): tile row r0 + 32 j of chunk j, r0 = thread / 8
-  __device__ __forceinline__ void gather_rows(int row0, int nrows) {
-    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const int q = (threadIdx.x >> 3) & 7;
+  // Loads for the tile after the current one (token ids of this thread's eight rows: tile row r0 + 32 j of chunk j,
+  // r0 = thread / 8) and for the current one (routing weights of this lane's four tokens). In flight until take_gathers().
+  uint32_t g_tok[8], g_prob[4];
+  __device__ __forceinline__ void issue_gathers() {
+    const int r0 = threadIdx.x >> 3, last = rows - 1;
+    const int trow = (int)(threadIdx.x >> 7) * 128 + (int)(threadIdx.x & 31);  // token of accumulator block row 0
     ix_static_for<0, 8>([&](auto jc) {
       constexpr int j = decltype(jc)::value;
-      const int base = 8 * wave + 32 * j;                // the wave's eight rows of chunk j, tile-relative
-      const int start = min(row0 + base, rows - 8);      // a permuted row past the last one is never a row of the tile
-      const int v = put8<0>(0, sorted_token + start);
-      // lane select: row base + q sits (row0 + base - start) lanes further on; rows the tile does not have read any lane
-      const uint32_t tok = (uint32_t)__builtin_amdgcn_ds_bpermute((q + (row0 + base - start)) * 4, v);
-      xvo[j] = (base + q < nrows) ? tok * (uint32_t)(ldx * 2) + kb() : IX_OOB;
+      g_tok[j] = ix_load4_uncounted(sorted_token, (uint32_t)min(nx_row0 + r0 + 32 * j, last) * 4u);
     });
-  }
-  __device__ __forceinline__ void gather_probs(int row0) {
-    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     ix_static_for<0, 4>([&](auto mc) {
       constexpr int mi = decltype(mc)::value;
-      const int base = (wave >> 1) * 128 + 32 * mi;      // the 32 tokens of accumulator block row mi
-      const int start = min(row0 + base, rows - 32);
-      const int* p = reinterpret_cast<const int*>(permuted_prob) + start;
-      int v = put8<0>(0, p);
-      v = put8<8>(v, p + 8);
-      v = put8<16>(v, p + 16);
-      v = put8<24>(v, p + 24);
-      // rows past the tile's last get some lane's value: their products are dropped by the store's range check
-      prob[mi] = __int_as_float(__builtin_amdgcn_ds_bpermute(((int)(threadIdx.x & 31) + (row0 + base - start)) * 4, v));
+      g_prob[mi] = ix_load4_uncounted(permuted_prob, (uint32_t)min(c_row0 + trow + 32 * mi, last) * 4u);
     });
+  }
+  __device__ __forceinline__ void take_gathers() {
+    const int r0 = threadIdx.x >> 3;
+    ix_static_for<0, 8>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+      const uint32_t tok = ix_landed(g_tok[j]);
+      // a row the tile does not have (a missing next tile has none) gets an offset outside the descriptor
+      xvo[j] = (r0 + 32 * j < nx_nrows) ? tok * (uint32_t)(ldx * 2) + kb() : IX_OOB;
+    });
+    // rows past the tile's last got some row's weight: their products are dropped by the store's range check
+    ix_static_for<0, 4>([&](auto mc) { prob[decltype(mc)::value] = __uint_as_float(ix_landed(g_prob[decltype(mc)::value])); });
   }
   __device__ __forceinline__ bool open_first() {
     xcd = blockIdx.x & 7u;
@@ -1067,12 +1048,20 @@ struct IxMoeFc1StreamJob {
     g0 = g1 = a0 = a1 = 0.0f;
     return has_next;
   }
-  __device__ __forceinline__ void open_next() {
+  __device__ __forceinline__ void open_next() {  // start of the third-last k-tile
     idx += stride;
     locate();
+    issue_gathers();
   }
   __device__ __forceinline__ void first_voffs() {
-    gather_rows(nx_row0, nx_nrows);
+    {  // the first tile's rows: nothing is in flight yet, ordinary loads
+      const int r0 = threadIdx.x >> 3;
+      uint32_t tok[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) tok[j] = (uint32_t)sorted_token[min(nx_row0 + r0 + 32 * j, rows - 1)];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) xvo[j] = (r0 + 32 * j < nx_nrows) ? tok[j] * (uint32_t)(ldx * 2) + kb() : IX_OOB;
+    }
     // Weight tile row r0 + 32 j (chunk j of thread row r0) = wave column j / 4, block j % 4 (gate 0, gate 1, up 0, up 1),
     // matrix-instruction row r0: weight row [up: F] + 64 (j / 4) + 16 (j % 2) + lane_col(r0) of the descriptor.
     // In rows, chunk 0..7 = 0, 16, F, F + 16, 64, 80, F + 64, F + 80 (+ lane_col); the walk's steps are the differences.
@@ -1095,10 +1084,8 @@ struct IxMoeFc1StreamJob {
     asm volatile("v_add_u32 %0, %1, %0" : "+v"(wv) : "s"(J == 7 ? w_stC : (J == 3 ? w_stB : ((J & 1) ? w_stA : w_st16))));
     return v;
   }
-  __device__ __forceinline__ void turn_offsets() {
-    gather_probs(c_row0);                // the current tile's weights, before its accumulators move out
-    gather_rows(nx_row0, nx_nrows);      // a missing next tile has no rows: every offset out of range
-  }
+  // second-last k-tile, after the current tile's last fetch through xvo: the loads of the k-tile before have retired
+  __device__ __forceinline__ void turn_offsets() { take_gathers(); }
   __device__ __forceinline__ void advance() {
     c_row0 = nx_row0;
     c_nrows = nx_nrows;
@@ -1243,8 +1230,8 @@ static int ix_moe_experts_launch(const bf16_t* x, long ldx, int T, long rows, co
   bool fc1_streamed = false;
   if constexpr (BM == 256 && BN == 256 && WM == 2 && WN == 2) {
     // worth it from two tiles per workgroup up (max_tiles bounds the row tiles from above by at most one per expert)
-    // (the scalar gathers read 32 consecutive permuted rows; the walk over an expert's weight rows is 32-bit)
-    if (Hd % IX_BK == 0 && Hd / IX_BK >= IxMoeFc1StreamJob::NSK + 3 && F % 128 == 0 && rows >= 32 && rows < 0x7fffffffL &&
+    // (32-bit byte offsets into the permutation's arrays and into an expert's weight rows)
+    if (Hd % IX_BK == 0 && Hd / IX_BK >= IxMoeFc1StreamJob::NSK + 3 && F % 128 == 0 && rows > 0 && rows < 0x20000000L &&
         ((long)F + 128) * Hd * 2 < 0x40000000L && max_tiles * nb1 >= 2 * IX_STREAM_WORKGROUPS) {
       static bool attr1_set = false;
       if (!attr1_set) {
