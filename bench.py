@@ -256,7 +256,7 @@ def moe(args):
             "roofline": {"bound": "mfma", "achieved": exp_fl / (exp_ms * 1e-3) / 1e12, "peak": PEAK_MFMA_BF16_TFLOPS,
                          "unit": "TFLOP/s", "frac": exp_fl / (exp_ms * 1e-3) / 1e12 / PEAK_MFMA_BF16_TFLOPS,
                          "traffic": MEASURED_TRAFFIC_BYTES["moe_T16384_grouped_gemms"] if T == 16384 else None,
-                         "kernel": "k_moe_fc1_glu + k_moe_fc2_stream (grouped GEMMs)", "kernel_ms": exp_ms},
+                         "kernel": "k_moe_fc1_glu_stream + k_moe_fc2_stream (grouped GEMMs)", "kernel_ms": exp_ms},
             "whole_ffn": {"kernel_ms": ms, "achieved": fl / (ms * 1e-3) / 1e12, "unit": "TFLOP/s",
                           "frac": fl / (ms * 1e-3) / 1e12 / PEAK_MFMA_BF16_TFLOPS,
                           "kernels": "router product + router + permutation + grouped GEMMs + combine"}}
@@ -351,7 +351,7 @@ def north_star_kernels(w, dev, steps):
     ms = _events_ms(lambda: experts_forward(x, lw["w1"], lw["w2"], perm), 3, steps)
     fl = 2.0 * T * k * H * (2 * F) + 2.0 * T * k * F * H
     out["moe_grouped_gemms_T16384"] = {
-        "bound": "mfma", "kernel": "k_moe_fc1_glu + k_moe_fc2_stream", "kernel_ms": ms, "achieved": fl / ms / 1e9,
+        "bound": "mfma", "kernel": "k_moe_fc1_glu_stream + k_moe_fc2_stream", "kernel_ms": ms, "achieved": fl / ms / 1e9,
         "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s", "frac": fl / ms / 1e9 / PEAK_MFMA_BF16_TFLOPS,
         "traffic": MEASURED_TRAFFIC_BYTES["moe_T16384_grouped_gemms"],
         "traffic_source": TRAFFIC_SOURCE["moe_T16384_grouped_gemms"] + " (not measured in this run)"}
@@ -500,7 +500,7 @@ def hybrid(args):
                         "unit": "TFLOP/s", "frac": exp_fl / exp_ms / 1e9 / PEAK_MFMA_BF16_TFLOPS,
                         "traffic": MEASURED_TRAFFIC_BYTES["moe_T163840_grouped_gemms"] if total == 163840 else None,
                         "traffic_source": TRAFFIC_SOURCE["moe_T163840_grouped_gemms"] + " (not measured in this run)",
-                        "kernel": f"k_moe_fc1_glu + k_moe_fc2_stream (grouped expert GEMMs, {total} tokens x top-8 per launch "
+                        "kernel": f"k_moe_fc1_glu_stream + k_moe_fc2_stream (grouped expert GEMMs, {total} tokens x top-8 per launch "
                                   f"pair, {cfg.layers} pairs per pass)", "kernel_ms": exp_ms,
                         "share_of_step": cfg.layers * exp_ms / (dt * 1e3)},
            "rollout": {"prefill_tokens_per_s": n * prompt / t_prefill, "decode_ms_per_step": t_dec * 1e3,

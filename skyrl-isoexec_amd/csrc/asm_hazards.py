@@ -105,13 +105,17 @@ def scan(path):
             stack = [(at - 1, 0)]
             while stack:
                 i, dist = stack.pop()
+                arrived_by_jump = i != at - 1
                 while i >= 0 and dist < VMEM_SGPR_WAIT and (i, dist) not in seen:
                     seen.add((i, dist))
                     pins, _, pln = hist[i]
+                    if re.match(r"^s_branch\b", pins) and not arrived_by_jump:
+                        break  # nothing falls through an unconditional jump
+                    arrived_by_jump = False
                     if pins.startswith("<label> "):
                         for j in jumps.get(pins[8:], []):
                             stack.append((j, dist))  # the jump itself is one wait state: counted when it is visited
-                        i -= 1  # and the line above the label (walking up past an unconditional jump only adds checks)
+                        i -= 1  # and the line above the label
                         continue
                     hit = valu_sgpr_defs(pins) & used
                     if hit:

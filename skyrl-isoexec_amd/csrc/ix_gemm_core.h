@@ -140,15 +140,24 @@ __device__ __forceinline__ ix_rsrc_t ix_rsrc_scalar(ix_rsrc_t r) {  // a descrip
   r.w = __builtin_amdgcn_readfirstlane(r.w);
   return r;
 }
+// NT: the non-temporal hint -- the line is not kept for a reader that comes soon (for outputs far larger than the
+// caches, written once while the same caches feed the operand stream).
+template <bool NT = false>
 __device__ __forceinline__ void ix_buffer_store16(uint4 v, ix_rsrc_t rsrc, uint32_t voff) {
   const ix_u32x4 d = {v.x, v.y, v.z, v.w};
   // the two idle states after it keep the next instruction from overwriting the data registers while the store still
   // reads them (the compiler would place them itself for a store it knows; it does not look into this one); the five
   // before it let the descriptor words, which a vector instruction has just moved into scalar registers, arrive
-  asm volatile("s_nop 4\n\tbuffer_store_dwordx4 %0, %1, %2, 0 offen\n\ts_nop 1"
-               :
-               : "v"(d), "v"(voff), "s"(ix_rsrc_scalar(rsrc))
-               : "memory");
+  if constexpr (NT)
+    asm volatile("s_nop 4\n\tbuffer_store_dwordx4 %0, %1, %2, 0 offen nt\n\ts_nop 1"
+                 :
+                 : "v"(d), "v"(voff), "s"(ix_rsrc_scalar(rsrc))
+                 : "memory");
+  else
+    asm volatile("s_nop 4\n\tbuffer_store_dwordx4 %0, %1, %2, 0 offen\n\ts_nop 1"
+                 :
+                 : "v"(d), "v"(voff), "s"(ix_rsrc_scalar(rsrc))
+                 : "memory");
 }
 __device__ __forceinline__ void ix_buffer_store4(uint32_t v, ix_rsrc_t rsrc, uint32_t voff) {
   asm volatile("s_nop 4\n\tbuffer_store_dword %0, %1, %2, 0 offen" : : "v"(v), "v"(voff), "s"(ix_rsrc_scalar(rsrc)) : "memory");

@@ -48,6 +48,16 @@
 // Workgroups a streaming kernel launches: one per CU (the ring fills a CU's LDS), a multiple of 8 so that every XCD's run
 // of the tile order is shared by the same number of them.
 #define IX_STREAM_WORKGROUPS 256
+// Non-temporal stores of the output tiles: of the plain job (dense GEMM, the experts' second GEMM: outputs of 64 MB and
+// up, written once while the caches feed the operand stream -- 131072 x 768 x 2048: 0.395 -> 0.34 ms, nothing lost at
+// large K or in the kernels that read the output next) and of the experts' first GEMM (whose output the second one
+// reads back at once: no gain, left off).
+#ifndef IX_STREAM_STORE_NT_PLAIN
+#define IX_STREAM_STORE_NT_PLAIN true
+#endif
+#ifndef IX_STREAM_STORE_NT_FC1
+#define IX_STREAM_STORE_NT_FC1 false
+#endif
 
 // Output layout of the streaming kernels. A lane of a 32 x 32 accumulator block holds result rows 8 g + 4 h + i (g < 4,
 // i < 4; h = lane / 32) for the token lane % 32. With the wave's weight rows dealt to (block, row) by
@@ -376,7 +386,7 @@ struct IxPlainStreamJob {
       constexpr int t = q - 40;  // token t of the quad
       const uint32_t off =
           (64 * L < p_cols) ? p_voff + (uint32_t)(((long)(mi * 32 + t) * seq.ldc + 64 * L) * 2) : IX_OOB;
-      ix_buffer_store16(make_uint4(tb[t][0], tb[t][1], tb[t][2], tb[t][3]), p_cr, off);
+      ix_buffer_store16<IX_STREAM_STORE_NT_PLAIN>(make_uint4(tb[t][0], tb[t][1], tb[t][2], tb[t][3]), p_cr, off);
     } else if constexpr (PARTS && L == 1 && q == 44) {
       const float v = fmaxf(rmax, __shfl_xor(rmax, 32, IX_WAVE));
       ix_buffer_store4(__float_as_uint(v), p_pr,

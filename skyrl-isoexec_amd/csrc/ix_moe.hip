@@ -1174,7 +1174,7 @@ struct IxMoeFc1StreamJob {
         tb[t][d] = ix_quad_exchange<2, (t & 2) != 0>(ta[a][d], ta[a + 2][d]);
       } else if constexpr (q < 36) {
         constexpr int t = q - 32;  // token t of the quad
-        ix_buffer_store16(make_uint4(tb[t][0], tb[t][1], tb[t][2], tb[t][3]), p_ir,
+        ix_buffer_store16<IX_STREAM_STORE_NT_FC1>(make_uint4(tb[t][0], tb[t][1], tb[t][2], tb[t][3]), p_ir,
                           p_voff == IX_OOB ? IX_OOB : p_voff + (uint32_t)((long)(mi * 32 + t) * F * 2));
       }
     }
