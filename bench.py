@@ -32,7 +32,7 @@ PEAK_HBM_GBS = 8000.0
 # WRITE_SIZE of the same workload (scaled by what the same counters read for a 1 GiB copy, x2.0 / x1.0), recorded in
 # the named file under profiles/.
 MEASURED_TRAFFIC_BYTES = {"dense_head_M4096_gemm": 15.5e9, "gdn_decode_B256": 1.080e9,
-                          "moe_T16384_grouped_gemms": 3.91e9, "moe_T163840_grouped_gemms": 34.4e9}
+                          "moe_T16384_grouped_gemms": 3.61e9, "moe_T163840_grouped_gemms": 32.3e9}
 TRAFFIC_SOURCE = {"dense_head_M4096_gemm": "profiles/gemm_bf16_nt__dense_head_M4096.txt",
                   "gdn_decode_B256": "profiles/gdn_scan__decode_B256.txt",
                   "moe_T16384_grouped_gemms": "profiles/moe_ffn__T16384.txt",
