@@ -32,7 +32,8 @@ def make(T, H, E, F, seed):
                                           (33, 2048, 128, 768, 8, None), (600, 2048, 8, 768, 2, 256),
                                           # enough tiles for the streaming form of the grouped kernels (one workgroup walks
                                           # many tiles): the smallest K it takes with ragged experts, and the full MoE shape
-                                          (9000, 1024, 8, 704, 4, 256), (9000, 1024, 8, 768, 4, 256), (16384, 2048, 128, 768, 8, None)])
+                                          (9000, 1024, 8, 704, 4, 256), (9000, 1024, 8, 768, 4, 256), (7000, 960, 8, 640, 4, 256),
+                                          (16384, 2048, 128, 768, 8, None)])
 def test_grouped_kernels_equal_the_dense_kernel_per_expert(T, H, E, F, k, BM):
     from isoexec_amd.ops.mm.mm_hip import linear_nt, router_gemm
     from isoexec_amd.ops.moe.moe_hip import experts_forward, permute, router_topk
@@ -62,6 +63,25 @@ def test_grouped_kernels_equal_the_dense_kernel_per_expert(T, H, E, F, k, BM):
         assert same_bits(eo[lo:hi], linear_nt(inter[lo:hi].contiguous(), w2[e])), f"fc2, expert {e}"
         checked += hi - lo
     assert checked == T * k
+
+
+def test_streamed_experts_with_a_pitched_activation_matrix():
+    """The streaming kernels gather token rows through the caller's row pitch: a column slice of a wider matrix gives
+    the bits of its contiguous copy (sizes that take the streaming form of both grouped GEMMs)."""
+    from isoexec_amd.ops.mm.mm_hip import router_gemm
+    from isoexec_amd.ops.moe.moe_hip import experts_forward, permute, router_topk
+
+    T, H, E, F, k = 9000, 1024, 8, 768, 4
+    x, wr, w1, w2 = make(T, H, E, F, seed=5)
+    wide = torch.zeros(T, H + 192, dtype=torch.bfloat16, device=DEV)
+    wide[:, 64:64 + H] = x
+    xs = wide[:, 64:64 + H]
+    assert xs.stride(0) == H + 192 and xs.data_ptr() % 16 == 0
+    idx, prob, _, _ = router_topk(router_gemm(x, wr), k, pre_softmax=True)
+    p = permute(idx, prob, E, BM=256)
+    eo, inter = experts_forward(x, w1, w2, p, return_inter=True)
+    eo2, inter2 = experts_forward(xs, w1, w2, p, return_inter=True)
+    assert same_bits(inter, inter2) and same_bits(eo, eo2)
 
 
 def fake_sequential_mlp(w1, w2, stacked=True):
