@@ -272,7 +272,9 @@ int ix_moe_permute_static(const int* topk_idx, const float* topk_prob, long T, l
  * moe_fused_experts.py:292-503): grouped fc1 + SwiGLU + prob epilogue, then grouped fc2.
  * x bf16 [T, Hd] (pitch ldx) gathered through sorted_token; W1 bf16 [E, 2F, Hd] (gate rows
  * then up rows); W2 bf16 [E, Hd, F]; inter bf16 [rows, F]; expert_out bf16 [rows, Hd];
- * rows = T*k. BM must be the value given to ix_moe_permute. */
+ * rows = T*k = the length of sorted_token and permuted_prob (the kernels clamp their reads of both to rows - 1, so it
+ * must not exceed what the arrays hold). BM must be the value given to ix_moe_permute. With 256-row tiles and at
+ * least 512 tiles of work both GEMMs run as streaming kernels (one workgroup per CU walking many tiles); same bits. */
 int ix_moe_experts(const void* x, long ldx, const int* sorted_token, const float* permuted_prob,
                    const void* W1, const void* W2, const int* tile_meta, long max_tiles, long BM, void* inter,
                    void* expert_out, long T, long rows, long Hd, long F, void* stream);
