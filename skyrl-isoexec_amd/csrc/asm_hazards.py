@@ -12,7 +12,11 @@ on the source to keep:
   address the range check never saw;
 * M0 written by a scalar instruction must not be read by a load-to-LDS in the next wait state.
 
-A third rule is this library's own. ``ix_load4_uncounted`` issues ``global_load_dword vN`` from inline assembly, so the
+* an accumulation register written by a matrix instruction must not be read by an inline-assembly
+  ``v_accvgpr_read_b32`` before the matrix pipeline has delivered it: 19 wait states cover the longest instruction
+  (the kernels place ``s_nop 15`` twice in front of the first read).
+
+A last rule is this library's own. ``ix_load4_uncounted`` issues ``global_load_dword vN`` from inline assembly, so the
 compiler believes vN holds the value at once; the value is taken into use through ``ix_landed`` (which leaves the
 comment ``; ix_landed vN`` in the assembly). Between the two
 * no instruction may mention vN (a copy or a spill would move a value that has not arrived), and
@@ -33,6 +37,9 @@ VCMP_E32 = re.compile(r"^v_cmpx?_\w+_e32\s")
 VALU_CARRY = re.compile(r"^v_(add_co|sub_co|subrev_co|addc_co|subb_co|subbrev_co|div_scale|mad_u64_u32|mad_i64_i32)\w*\s+\S+,\s*(s\[\d+:\d+\]|vcc)")
 VMEM_SGPR_WAIT = 5
 M0_LDS_WAIT = 1
+MFMA_AGPR_WAIT = 19
+ACC_READ = re.compile(r"^v_accvgpr_read_b32\s+v\d+,\s*a(\d+)")
+MFMA_DEF = re.compile(r"^v_mfma_\w+\s+a\[(\d+):(\d+)\]")
 
 
 def sregs(text):
@@ -88,6 +95,7 @@ def scan(path):
     flying = {}  # vector register -> [line of its uncounted load, vector-memory instructions issued since, retired]
 
     pending_checks = []  # indices into hist of the inline-assembly memory instructions of the current function
+    acc_checks = []      # and of its inline-assembly accumulator reads
 
     def check_operands():
         """Walks upwards from every inline-assembly memory instruction, through the function's jumps as well."""
@@ -126,6 +134,22 @@ def scan(path):
                     dist += wait_states(pins)
                     i -= 1
         pending_checks.clear()
+        # accumulator reads from inline assembly: straight up the lines (these sit in straight-line epilogue code)
+        for at in acc_checks:
+            ins, _, ln = hist[at]
+            reg = int(ACC_READ.match(ins).group(1))
+            dist, i = 0, at - 1
+            while i >= 0 and dist < MFMA_AGPR_WAIT:
+                pins, _, pln = hist[i]
+                m = MFMA_DEF.match(pins)
+                if m and int(m.group(1)) <= reg <= int(m.group(2)):
+                    findings.append(f"{path}:{ln}: {func}: '{ins}' {dist} wait states after '{pins[:60]}' (line {pln}); "
+                                    f"{MFMA_AGPR_WAIT} needed")
+                    break
+                if not pins.startswith("<label> "):
+                    dist += wait_states(pins)
+                i -= 1
+        acc_checks.clear()
 
     def close_function():
         check_operands()
@@ -184,6 +208,8 @@ def scan(path):
             m = re.match(r"^global_load_dword\s+v(\d+),", ins)
             if in_asm and m:
                 flying[int(m.group(1))] = [ln, 0, False]
+        if in_asm and ACC_READ.match(ins):
+            acc_checks.append(len(hist))
         if in_asm and VMEM.match(ins):
             pending_checks.append(len(hist))  # checked when the function is complete (its jumps are known then)
         hist.append((ins, in_asm, ln))

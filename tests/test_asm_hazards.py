@@ -92,6 +92,19 @@ def test_uncounted_load_must_be_retired_and_untouched(tmp_path):
     assert any("without an uncounted load" in f for f in scan(tmp_path, take))
 
 
+def test_accumulator_read_waits_for_the_matrix_pipeline(tmp_path):
+    mfma = "\tv_mfma_f32_32x32x16_bf16 a[240:255], v[64:67], v[12:15], a[240:255]\n"
+    read = asm("v_accvgpr_read_b32 v5, a241")
+    assert len(scan(tmp_path, mfma + read)) == 1
+    assert scan(tmp_path, mfma + asm("s_nop 15", "s_nop 15") + read) == []
+    # fifteen other matrix instructions and their companions in between (the streaming kernels' distance): legal
+    others = "".join(f"\tv_mfma_f32_32x32x16_bf16 a[{16 * i}:{16 * i + 15}], v[64:67], v[12:15], a[{16 * i}:{16 * i + 15}]\n"
+                     "\tds_read_b128 v[0:3], v9\n" for i in range(14))
+    assert scan(tmp_path, mfma + others + read) == []
+    # a read of another block right behind it is no hazard of this instruction
+    assert scan(tmp_path, mfma + asm("v_accvgpr_read_b32 v5, a17")) == []
+
+
 def test_built_assembly_is_clean_when_present():
     files = [os.path.join(CSRC, f) for f in ("ix_gemm.dev.s", "ix_moe.dev.s", "ix_attn.dev.s")]
     if not all(os.path.exists(f) for f in files):
