@@ -1311,6 +1311,9 @@ extern "C" int ix_moe_experts(const void* x, long ldx, const int* sorted_token, 
 }
 
 // ---------------------------------------------------------------------------------------------
+// KC > 0: k known at compile time -- the k row numbers and the k rows are requested before the first add, so a thread has
+// k loads in flight instead of one (the sum is the same left-to-right sum). KC = 0: any k.
+template <int KC>
 __global__ __launch_bounds__(256) void k_moe_combine(const bf16_t* __restrict__ expert_out,
                                                      const int* __restrict__ combine_rows,
                                                      bf16_t* __restrict__ out, long T, int Hd, int k, int fp32_acc,
@@ -1321,18 +1324,37 @@ __global__ __launch_bounds__(256) void k_moe_combine(const bf16_t* __restrict__ 
   const long t = i / groups;
   const int c0 = (int)(i % groups) * 8;
   float acc[8];
-  for (int r = 0; r < k; ++r) {
-    const long row = combine_rows[t * k + r];
-    float xv[8];
-    ix_load8(expert_out + row * Hd + c0, Hd - c0, vec != 0, 0.0f, xv);
-    if (r == 0) {
+  if constexpr (KC > 0) {
+    long row[KC];
+    float xv[KC][8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) acc[j] = xv[j];
-    } else {
+    for (int r = 0; r < KC; ++r) row[r] = combine_rows[t * KC + r];
+#pragma unroll
+    for (int r = 0; r < KC; ++r) ix_load8(expert_out + row[r] * Hd + c0, Hd - c0, vec != 0, 0.0f, xv[r]);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = xv[0][j];
+#pragma unroll
+    for (int r = 1; r < KC; ++r) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float sum = acc[j] + xv[j];
+        const float sum = acc[j] + xv[r][j];
         acc[j] = fp32_acc ? sum : ix_rbf(sum);
+      }
+    }
+  } else {
+    for (int r = 0; r < k; ++r) {
+      const long row = combine_rows[t * k + r];
+      float xv[8];
+      ix_load8(expert_out + row * Hd + c0, Hd - c0, vec != 0, 0.0f, xv);
+      if (r == 0) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[j] = xv[j];
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float sum = acc[j] + xv[j];
+          acc[j] = fp32_acc ? sum : ix_rbf(sum);
+        }
       }
     }
   }
@@ -1347,7 +1369,15 @@ extern "C" int ix_moe_combine(const void* expert_out, const int* combine_rows, v
   const long grid = (T * groups + 255) / 256;
   if (grid > 0x7fffffffL) return IX_DECLINED;
   const int vec = (Hd % 8 == 0) && ix_aligned(expert_out, 16) && ix_aligned(out, 16);
-  hipLaunchKernelGGL(k_moe_combine, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream,
-                     (const bf16_t*)expert_out, combine_rows, (bf16_t*)out, T, (int)Hd, (int)k, fp32_acc, vec);
+#define IX_COMBINE(KC_)                                                                                        \
+  hipLaunchKernelGGL(k_moe_combine<KC_>, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream,             \
+                     (const bf16_t*)expert_out, combine_rows, (bf16_t*)out, T, (int)Hd, (int)k, fp32_acc, vec)
+  switch (k) {
+    case 2: IX_COMBINE(2); break;
+    case 4: IX_COMBINE(4); break;
+    case 8: IX_COMBINE(8); break;
+    default: IX_COMBINE(0); break;
+  }
+#undef IX_COMBINE
   return ix_launch_status();
 }
