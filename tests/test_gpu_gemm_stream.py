@@ -28,6 +28,7 @@ def operands(M, K, N, seed):
                                    (2500, 1024, 1304),     # 60 tiles, most workgroups idle
                                    (4096, 2048, 4096),     # one tile per workgroup
                                    (70000, 768, 256),      # 274 tiles: some workgroups walk two
+                                   (20100, 768, 4360),     # 79 x 18 tiles: the wide group shape, partial groups both ways
                                    (16384, 1536, 8192)])   # 2048 tiles: eight per workgroup
 def test_streaming_tile_equals_the_other_tiles_bit_for_bit(M, K, N):
     from isoexec_amd.ops.mm.mm_hip import linear_nt
