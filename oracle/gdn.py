@@ -8,6 +8,18 @@ as the reference's fp32 ``_torch_chunk_gdr_one``, gdn_ops.py:261-315, in float64
 recall ``o_t = v_t`` for q = k * sqrt(K)); prefix / split / cross-sequence invariance of the bits
 (the reference's gates T1-T4 of gdn_native_kernel_parity_test_gpu.py and
 gdn_batch_invariant.py:141-215); conv against a brute-force loop.
+
+``cpr_forward`` restates the boundary form (reference ops/gdn/gdn_cpr.py:104-186 ``chunk_boundary_states``:
+"the bf16 snapshot entering chunk c", "final_state is the fp32 accumulator ... the chaining dtype";
+:222-319 ``_state_pool`` + one segmented recurrent scan in which every chunk starts from its snapshot).
+Pinned by (tests/test_oracle_gdn_moe.py): every snapshot against the float64 state entering that chunk
+computed by the chunk-parallel WY pass ``chunk_states_fp64`` (a different algorithm: a triangular solve per
+chunk, no token loop) to within one wire-dtype rounding, over enough chunks that a chain restarted from the
+rounded snapshots fails; the final states against the same pass; every chunk's outputs against the float64
+recurrence started from that chunk's snapshot, far closer than to the one started from the unrounded state;
+and bit for bit against ``scan`` where the structure fixes the answer (one chunk per sequence; fp32 wire).
+What stays unpinned: bit parity with the third-party chunk kernels the reference calls for the boundary states
+(vLLM's FLA ops, not in the reference tree; the reference's tests hold no vectors for them).
 """
 
 from __future__ import annotations
@@ -102,9 +114,13 @@ def scan_fp64(q, k, v, g, beta, state0=None, scale=None):
     return o, S
 
 
-def chunk_fp64(q, k, v, g, beta, chunk=64, scale=None):
-    """Chunk-parallel WY form in float64 for one sequence from a zero state: the algorithm of the
-    reference's fp32 ``_torch_chunk_gdr_one`` (gdn_ops.py:261-315). ``H == HV`` expected."""
+def chunk_fp64(q, k, v, g, beta, chunk=64, scale=None, state0=None, return_states=False):
+    """Chunk-parallel WY form in float64 for one sequence: the algorithm of the reference's fp32
+    ``_torch_chunk_gdr_one`` (gdn_ops.py:261-315). ``H == HV`` expected. ``state0 [H, V, K]`` is the entry
+    state (zero when absent). With ``return_states``: ``(o, entering [NT, H, V, K], final [H, V, K])`` where
+    ``entering[c]`` is the state before the first token of chunk ``c`` (the chunk pass never walks tokens:
+    one triangular solve and three products per chunk). A ragged last chunk is padded with g = 0, beta = 0,
+    k = 0 tokens, which leave the state untouched."""
     T, H, K = q.shape
     V = v.shape[2]
     scale = K ** -0.5 if scale is None else scale
@@ -113,9 +129,12 @@ def chunk_fp64(q, k, v, g, beta, chunk=64, scale=None):
     q, k, v, g, beta = f(q) * scale, f(k), f(v), f(g), f(beta)
     Tp = T + pad
     o = np.zeros((Tp, H, V))
+    entering = np.zeros((Tp // chunk, H, V, K))
+    final = np.zeros((H, V, K))
     for h in range(H):
-        S = np.zeros((K, V))
+        S = np.zeros((K, V)) if state0 is None else state0[h].astype(np.float64).T.copy()
         for c0 in range(0, Tp, chunk):
+            entering[c0 // chunk, h] = S.T
             sl = slice(c0, c0 + chunk)
             qc, kc, vc, bc = q[sl, h], k[sl, h], v[sl, h], beta[sl, h]
             gc = np.cumsum(g[sl, h])
@@ -128,4 +147,49 @@ def chunk_fp64(q, k, v, g, beta, chunk=64, scale=None):
             v_new = u - kcd @ S
             o[sl, h] = (qc * np.exp(gc)[:, None]) @ S + attn @ v_new
             S = S * np.exp(gc[-1]) + (kc * np.exp(gc[-1] - gc)[:, None]).T @ v_new
-    return o[:T]
+        final[h] = S.T
+    return (o[:T], entering, final) if return_states else o[:T]
+
+
+def chunk_states_fp64(k, v, g, beta, chunk, state0=None):
+    """Float64 state entering every chunk of ONE sequence, and the final state, by the chunk-parallel pass
+    above (GQA-expanded here). ``k [T, H, K]``, ``v [T, HV, V]``, ``g, beta [T, HV]``.
+    Returns ``(entering [ceil(T/chunk), HV, V, K], final [HV, V, K])``."""
+    rep = v.shape[1] // k.shape[1]
+    kx = np.repeat(k, rep, axis=1)
+    _, entering, final = chunk_fp64(kx, kx, v, g, beta, chunk, state0=state0, return_states=True)
+    return entering, final
+
+
+def cpr_forward(q, k, v, g, beta, lens, chunk, init=None, wire="bf16", prims: Prims = DEFAULT):
+    """Boundary form of the forward over a packed batch (reference ops/gdn/gdn_cpr.py:104-186, :288-319).
+
+    Per sequence an UNROUNDED fp32 state chain runs over the tokens (the reference's ``final_state`` "is the fp32
+    accumulator ... the chaining dtype"); the state ENTERING chunk ``c`` is snapshotted in the wire dtype
+    (``h [N, NT, HV, V, K]`` "the bf16 snapshot entering chunk c"), widened back to fp32 (``_state_pool``:
+    ``copy_`` does the widening cast) and chunk ``c`` is then scanned as its own sequence from that snapshot
+    (``chunked_cu_seqlens_and_indices``: one pool row per chunk). The chain's arithmetic is this library's token
+    recurrence (``scan``); the reference's comes from third-party chunk kernels.
+
+    ``q, k [T, H, K]``, ``v [T, HV, V]``, ``g, beta [T, HV]`` packed over ``sum(lens)`` tokens (values already
+    in the wire dtype's grid), ``init [N, HV, V, K]`` fp32 entry states or None, ``wire`` "bf16" | "fp32".
+    Returns ``(o [T, HV, V]`` in the wire dtype's grid, ``snapshots`` list of ``[HV, V, K]`` in (sequence, chunk)
+    order, ``finals`` list of fp32 ``[HV, V, K]`` per sequence``)``."""
+    assert wire in ("bf16", "fp32")
+    HV, V, K = v.shape[1], v.shape[2], k.shape[2]
+    to_wire = round_bf16 if wire == "bf16" else (lambda a: a.astype(F32))
+    outs, snaps, finals = [], [], []
+    pos = 0
+    for n, length in enumerate(lens):
+        chain = np.zeros((HV, V, K), F32) if init is None else np.ascontiguousarray(init[n], dtype=F32).copy()
+        for c0 in range(0, length, chunk):
+            sl = slice(pos + c0, pos + min(c0 + chunk, length))
+            snap = to_wire(chain)                      # the state entering the chunk, in the wire dtype
+            snaps.append(snap.copy())
+            start = np.ascontiguousarray(snap, dtype=F32).copy()
+            outs.append(scan(q[sl], k[sl], v[sl], g[sl], beta[sl], start, io_bf16=wire == "bf16", prims=prims))
+            scan(q[sl], k[sl], v[sl], g[sl], beta[sl], chain, prims=prims)   # the chain advances unrounded
+        finals.append(chain)
+        pos += length
+    o = np.concatenate(outs, 0) if outs else np.zeros((0, HV, V), F32)
+    return o, snaps, finals

@@ -1,11 +1,11 @@
 """GPU parity of the chunk-boundary GatedDeltaNet forward (``ops/gdn/gdn_cpr.py``; reference gdn_cpr.py:104-319).
 
-The oracle composes the CPU recurrence the way the reference's contract states it: an unrounded fp32 state chain
-gives the state entering every chunk, that state is snapshotted in the wire dtype, and every chunk is then scanned
-as its own sequence from its snapshot. The reference's own boundary arithmetic (third-party chunk kernels, absent
-here) is not reproduced: parity with it is unpinned; what is pinned is this library's definition, bit for bit,
-and the special cases the structure fixes (one chunk per sequence = the recurrent forward; fp32 wire = no rounding
-at the boundaries = the recurrent forward for every chunk size)."""
+The checker is ``oracle.gdn.cpr_forward``: an unrounded fp32 state chain gives the state entering every chunk, that
+state is snapshotted in the wire dtype, and every chunk is then scanned as its own sequence from its snapshot. Its
+structure is pinned on the CPU against a float64 chunk-state pass (tests/test_oracle_gdn_moe.py). The reference's own
+boundary arithmetic (third-party chunk kernels, absent here) cannot be reproduced bit for bit: that one parity is
+unpinned. Also checked here: the special cases the structure fixes (one chunk per sequence = the recurrent forward;
+fp32 wire = no rounding at the boundaries = the recurrent forward for every chunk size)."""
 
 import numpy as np
 import pytest
@@ -36,24 +36,11 @@ def make_inputs(lens, seed):
 
 
 def oracle_cpr(q, k, v, gate, beta, lens, chunk, dprims, init=None):
-    """Per sequence: fp32 chain -> snapshot (bf16) entering each chunk -> scan of the chunk from the snapshot."""
+    """``oracle.gdn.cpr_forward`` (pinned on the CPU against the float64 chunk-state pass, tests/test_oracle_gdn_moe.py)
+    on the bf16 images of the inputs, with the device's transcendentals plugged in."""
     r = lambda t: bf16_to_np(t.to(torch.bfloat16))
-    qn, kn, vn, bn = r(q[0]), r(k[0]), r(v[0]), r(beta[0])
-    gn = gate[0].numpy().astype(np.float32)
-    outs, snaps, finals = [], [], []
-    pos = 0
-    for n, length in enumerate(lens):
-        chain = np.zeros((HV, V, K), np.float32) if init is None else init[n].numpy().copy()
-        for c0 in range(0, length, chunk):
-            sl = slice(pos + c0, pos + min(c0 + chunk, length))
-            snap = bf16_to_np(np_to_bf16(chain))            # the state entering the chunk, in the wire dtype
-            snaps.append(snap.copy())
-            start = snap.astype(np.float32).copy()
-            outs.append(o_gdn.scan(qn[sl], kn[sl], vn[sl], gn[sl], bn[sl], start, io_bf16=True, prims=dprims))
-            o_gdn.scan(qn[sl], kn[sl], vn[sl], gn[sl], bn[sl], chain, io_bf16=True, prims=dprims)  # the chain itself
-        finals.append(chain)
-        pos += length
-    return np.concatenate(outs, 0) if outs else np.zeros((0, HV, V), np.float32), snaps, finals
+    return o_gdn.cpr_forward(r(q[0]), r(k[0]), r(v[0]), gate[0].numpy().astype(np.float32), r(beta[0]), lens, chunk,
+                             init=None if init is None else init.numpy(), prims=dprims)
 
 
 @pytest.mark.parametrize("chunk", [16, 64])

@@ -166,3 +166,133 @@ def test_expert_chain_against_brute_force():
         assert np.abs(out[t] - acc).max() <= 0.03 * np.abs(acc).max() + 1e-3
     one = o_moe.moe_ffn(x[3:4], wr, w1, w2, k)
     assert np.array_equal(one[0], out[3])
+
+
+# ---- the boundary (cpr) form: reference ops/gdn/gdn_cpr.py:104-186, :288-319 ------------------------------------
+
+def _cpr_inputs(lens, seed, H=2, HV=4, K=32, V=16, slow_decay=True):
+    """Packed inputs on the bf16 grid. ``slow_decay`` keeps the state alive over many chunks (|g| ~ 0.02 per token),
+    so that an error made at one boundary is still there at the next ones."""
+    g = torch.Generator().manual_seed(seed)
+    T = sum(lens)
+    bf = lambda t: t.to(torch.bfloat16).float().numpy()
+    q = bf(torch.nn.functional.normalize(torch.randn(T, H, K, generator=g), dim=-1))
+    k = bf(torch.nn.functional.normalize(torch.randn(T, H, K, generator=g), dim=-1))
+    v = bf(torch.randn(T, HV, V, generator=g))
+    gate = -torch.nn.functional.softplus(torch.randn(T, HV, generator=g))
+    gate = (gate * (0.02 if slow_decay else 1.0)).numpy().astype(np.float32)
+    beta = bf(torch.sigmoid(torch.randn(T, HV, generator=g)))
+    return q, k, v, gate, beta
+
+
+def _bf16_half_ulp(x):
+    """Half a bf16 unit in the last place at the magnitude of (float64) x."""
+    e = np.floor(np.log2(np.maximum(np.abs(x), 2.0 ** -126)))
+    return 2.0 ** (e - 8)
+
+
+def _restarted_chain_snapshots(q, k, v, g, beta, length, chunk, HV, V, K):
+    """The mistake the snapshot test must catch: the chain continues from the ROUNDED snapshot."""
+    chain = np.zeros((HV, V, K), np.float32)
+    snaps = []
+    for c0 in range(0, length, chunk):
+        chain = o_prims.round_bf16(chain)
+        snaps.append(chain.copy())
+        sl = slice(c0, min(c0 + chunk, length))
+        o_gdn.scan(q[sl], k[sl], v[sl], g[sl], beta[sl], chain)
+    return snaps
+
+
+def test_cpr_snapshots_are_the_rounded_fp64_boundary_states():
+    lens, chunk = [200, 37, 0, 130], 16           # 13 + 3 + 0 + 9 chunks
+    q, k, v, g, beta = _cpr_inputs(lens, 31)
+    HV, V, K = v.shape[1], v.shape[2], k.shape[2]
+    _, snaps, finals = o_gdn.cpr_forward(q, k, v, g, beta, lens, chunk)
+    assert len(snaps) == sum(-(-n // chunk) for n in lens) and len(finals) == len(lens)
+    pos, at = 0, 0
+    for n, length in enumerate(lens):
+        sl = slice(pos, pos + length)
+        if length == 0:
+            assert not finals[n].any()
+            continue
+        entering, final = o_gdn.chunk_states_fp64(k[sl], v[sl], g[sl], beta[sl], chunk)
+        # the chunk pass itself against the token recurrence (two algorithms, one mathematics)
+        _, s_rec = o_gdn.scan_fp64(q[sl], k[sl], v[sl], g[sl], beta[sl])
+        assert np.abs(final - s_rec).max() <= 1e-11
+        nt = entering.shape[0]
+        got = np.stack(snaps[at:at + nt]).astype(np.float64)
+        # a correctly rounded value of a chain that is within ~1e-6 of the truth: half a unit + the chain's error
+        slack = np.abs(got - entering) - _bf16_half_ulp(entering)
+        assert slack.max() <= 2e-6, (n, slack.max())
+        assert np.array_equal(o_prims.round_bf16(got.astype(np.float32)), got.astype(np.float32))  # on the bf16 grid
+        assert np.abs(finals[n] - final).max() <= 2e-6                                     # fp32 chain, unrounded
+        assert not np.array_equal(o_prims.round_bf16(finals[n]), finals[n])
+        if nt >= 8:   # the same check refuses a chain restarted from its rounded snapshots
+            bad = np.stack(_restarted_chain_snapshots(q[sl], k[sl], v[sl], g[sl], beta[sl], length, chunk, HV, V, K))
+            bad_slack = np.abs(bad.astype(np.float64) - entering) - _bf16_half_ulp(entering)
+            assert bad_slack.max() > 1e-3 and (bad_slack > 2e-6).mean() > 0.05
+        at += nt
+        pos += length
+    assert at == len(snaps)
+
+
+def test_cpr_entry_states_and_snapshot_placement():
+    lens, chunk = [70, 5], 32
+    q, k, v, g, beta = _cpr_inputs(lens, 32)
+    HV, V, K = v.shape[1], v.shape[2], k.shape[2]
+    init = np.random.default_rng(3).standard_normal((2, HV, V, K)).astype(np.float32)
+    _, snaps, finals = o_gdn.cpr_forward(q, k, v, g, beta, lens, chunk, init=init)
+    assert np.array_equal(snaps[0], o_prims.round_bf16(init[0]))       # chunk 0 enters with the caller's state
+    assert np.array_equal(snaps[3], o_prims.round_bf16(init[1]))
+    entering, final = o_gdn.chunk_states_fp64(k[:70], v[:70], g[:70], beta[:70], chunk, state0=init[0])
+    for c in range(3):
+        assert (np.abs(snaps[c] - entering[c]) - _bf16_half_ulp(entering[c])).max() <= 2e-5
+    assert np.abs(finals[0] - final).max() <= 2e-5
+    # "entering", not "leaving": the state after chunk c is the state entering chunk c + 1, far from entering[c]
+    assert np.abs(entering[1] - entering[0]).max() > 0.1
+
+
+def test_cpr_outputs_start_from_the_snapshot_not_from_the_chain():
+    lens, chunk = [96], 32
+    q, k, v, g, beta = _cpr_inputs(lens, 33)
+    HV, V, K = v.shape[1], v.shape[2], k.shape[2]
+    base = o_prims.round_bf16(np.random.default_rng(4).standard_normal((1, HV, V, K)).astype(np.float32))
+    moved = (base * np.float32(1 + 0.4 * 2.0 ** -8)).astype(np.float32)   # same bf16 value, different fp32 chain
+    assert np.array_equal(o_prims.round_bf16(moved), base) and not np.array_equal(moved, base)
+    o_a, snaps_a, fin_a = o_gdn.cpr_forward(q, k, v, g, beta, lens, chunk, init=base)
+    o_b, snaps_b, fin_b = o_gdn.cpr_forward(q, k, v, g, beta, lens, chunk, init=moved)
+    assert np.array_equal(snaps_a[0], snaps_b[0])
+    assert np.array_equal(o_a[:chunk], o_b[:chunk])                       # chunk 0 sees only the snapshot
+    assert not np.array_equal(fin_a[0], fin_b[0])                        # the chain carries the difference on
+    st = moved[0].copy()                                                  # the mistake: chunk 0 scanned from the chain
+    from_chain = o_gdn.scan(q[:chunk], k[:chunk], v[:chunk], g[:chunk], beta[:chunk], st, io_bf16=True)
+    assert not np.array_equal(from_chain, o_b[:chunk])
+    # numerically: every chunk's outputs are the float64 recurrence started from that chunk's snapshot
+    for c in range(3):
+        sl = slice(c * chunk, (c + 1) * chunk)
+        want, _ = o_gdn.scan_fp64(q[sl], k[sl], v[sl], g[sl], beta[sl], state0=snaps_b[c])
+        assert (np.abs(o_b[sl] - want) - _bf16_half_ulp(want)).max() <= 2e-5
+
+
+def test_cpr_structural_identities_on_the_oracle():
+    lens = [5, 64, 33]
+    q, k, v, g, beta = _cpr_inputs(lens, 34, slow_decay=False)
+    HV, V, K = v.shape[1], v.shape[2], k.shape[2]
+
+    def recurrent(io_bf16):
+        outs, pos = [], 0
+        for length in lens:
+            sl = slice(pos, pos + length)
+            st = np.zeros((HV, V, K), np.float32)
+            outs.append(o_gdn.scan(q[sl], k[sl], v[sl], g[sl], beta[sl], st, io_bf16=io_bf16))
+            pos += length
+        return np.concatenate(outs)
+
+    same = lambda a, b: np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    one, snaps, _ = o_gdn.cpr_forward(q, k, v, g, beta, lens, 64)        # one chunk per sequence
+    assert len(snaps) == 3 and same(one, recurrent(True))
+    for chunk in (16, 32):                                               # fp32 wire: no rounding at the boundaries
+        got, _, _ = o_gdn.cpr_forward(q, k, v, g, beta, lens, chunk, wire="fp32")
+        assert same(got, recurrent(False)), chunk
+    small, _, _ = o_gdn.cpr_forward(q, k, v, g, beta, lens, 16)          # bf16 boundaries: a different function
+    assert not same(small, recurrent(True)) and np.abs(small - recurrent(True)).max() <= 2 ** -5
