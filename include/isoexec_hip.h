@@ -183,9 +183,12 @@ int ix_gdn_l2norm(const void* x, long x_pitch, void* y, int io_dtype, long token
 /* gdn_gate_and_beta (gdn_ops.py:1197-1210) in the fp32 form of the fused core (gdn/_register.py:33-55):
  * g = -exp(A_log[hv]) * softplus(a + dt_bias[hv]) fp32; beta = sigmoid(b) in io_dtype.
  * a, b [tokens, HV] with token pitches a_pitch, b_pitch (elements; column slices of a wider projection are read in
- * place); g, beta [tokens, HV] contiguous; A_log, dt_bias fp32 [HV]. */
+ * place); g, beta [tokens, HV] contiguous; A_log, dt_bias fp32 [HV]. exp_dtype = the dtype exp(A_log) is held in:
+ * IX_DT_F32 for the fused core's form (parameter widened first, gdn/_register.py:33-55), IX_DT_BF16 for the eager
+ * form on a bf16 parameter (gdn_ops.py:1197-1210: "A_log.exp() is taken in the parameter's own dtype"; A_log then
+ * holds the widened bf16 values and exp's result is rounded to bf16 before the product). */
 int ix_gdn_gate(const void* a, long a_pitch, const void* b, long b_pitch, const float* A_log, const float* dt_bias,
-                float* g, void* beta, int io_dtype, long tokens, long HV, void* stream);
+                float* g, void* beta, int io_dtype, long tokens, long HV, int exp_dtype, void* stream);
 
 /* cpr_resolve_rows (gdn_cpr_rows.py:29-80; eager chain gdn_recurrent_state.py:271-284): engine slot ids of a
  * decode batch -> state-pool rows, one launch, host-free. slots int32 or int64 [n] (slots_i64). With slot2row
@@ -250,10 +253,12 @@ int ix_moe_permute(const int* topk_idx, const float* topk_prob, long T, long E, 
 /* _block_map / fused_block_map (moe_fused_experts.py:156-205, moe_blockmap_kernel.py): the block map for rows that
  * are ALREADY grouped by expert (SequentialMLP.forward's tokens_per_expert, moe_batched_experts.py:301-330). counts
  * int32 or int64 [E] (counts_i64) in device memory; offsets int32 [E+1] (may be NULL) receives the exclusive scan;
- * tile_meta as in ix_moe_permute, max_tiles >= ix_moe_max_tiles(rows, 1, E, BM). Integer work only, one launch, nothing
- * read back by the host. */
-int ix_moe_block_map(const void* counts, int counts_i64, long E, long BM, int* offsets, int* tile_meta, long max_tiles,
-                     void* stream);
+ * tile_meta as in ix_moe_permute, max_tiles >= ix_moe_max_tiles(rows, 1, E, BM). rows = the number of rows the
+ * caller's buffers hold: the host cannot see the counts, so the kernel keeps every tile inside [0, rows) -- counts that
+ * add up to more lose their tail (offsets[E] = min(rows, sum)); counts that add up to less leave the last rows in no
+ * tile. Integer work only, one launch, nothing read back by the host. */
+int ix_moe_block_map(const void* counts, int counts_i64, long E, long BM, long rows, int* offsets, int* tile_meta,
+                     long max_tiles, void* stream);
 
 /* ix_moe_permute for callers that cannot allocate device memory or bring a workspace: code under HIP graph
  * capture, tight serving loops, harnesses that forbid allocation. No counterpart in the reference (its permutation
@@ -262,8 +267,11 @@ int ix_moe_block_map(const void* counts, int counts_i64, long E, long BM, int* o
  * process ends. The call allocates and frees nothing. Limit: ix_moe_permute_scratch_ints(T, E) <=
  * ix_moe_permute_static_max_ints() (262,144 ints: 262,144 tokens at E = 128), else IX_ERR_SIZE and nothing is
  * launched. All calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads) race;
- * calls in stream order do not, and no call depends on what an earlier one left in the array. */
+ * calls in stream order do not, and no call depends on what an earlier one left in the array. The first call on a
+ * device looks the array's address up in the runtime (no allocation, but a runtime call): ix_moe_permute_static_init()
+ * does that lookup for the current device ahead of time, for callers that then enter a stream capture. */
 size_t ix_moe_permute_static_max_ints(void);
+int ix_moe_permute_static_init(void);
 int ix_moe_permute_static(const int* topk_idx, const float* topk_prob, long T, long E, long k, long BM, int* counts,
                           int* offsets, int* sorted_token, float* permuted_prob, int* combine_rows, int* tile_meta,
                           long max_tiles, void* stream);
@@ -292,6 +300,15 @@ int ix_moe_experts_tile(const void* x, long ldx, const int* sorted_token, const 
  * ascending expert order; fp32_acc 0 = bf16 adds (a round per add), 1 = fp32 sum, one round. */
 int ix_moe_combine(const void* expert_out, const int* combine_rows, void* out, long T, long Hd, long k,
                    int fp32_acc, void* stream);
+
+/* The eager unpermute with routing weights and any of its dtypes (_deterministic_unpermute,
+ * moe_batch_invariant.py:338-385: `permuted_tokens * permuted_probs.unsqueeze(-1)` then _fixed_order_combine, :276-320):
+ * out[t] = the left-to-right sum over the token's k rows of expert_out[row] * row_weight[row] (row_weight NULL: no
+ * product). expert_out [rows, Hd] in in_dtype; row_weight fp32 values [rows]; arith_dtype = torch's promotion of the
+ * token and weight dtypes (IX_DT_BF16: the product and every partial sum are rounded to bf16; IX_DT_F32: nothing is
+ * rounded before the store); out [T, Hd] in out_dtype (one round when it is narrower). */
+int ix_moe_combine_weighted(const void* expert_out, int in_dtype, const float* row_weight, int arith_dtype,
+                            const int* combine_rows, void* out, int out_dtype, long T, long Hd, long k, void* stream);
 
 /* ---- order-invariant digests: debug/thash ------------------------------------------------- */
 

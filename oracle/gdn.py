@@ -64,10 +64,15 @@ def l2norm(x, io_bf16=True):
     return round_bf16(y) if io_bf16 else y
 
 
-def gate_and_beta(a, b, A_log, dt_bias, io_bf16=True, prims: Prims = DEFAULT):
-    """``g = -exp(A_log) * softplus(a + dt_bias)`` fp32; ``beta = sigmoid(b)`` (io dtype)."""
+def gate_and_beta(a, b, A_log, dt_bias, io_bf16=True, prims: Prims = DEFAULT, exp_bf16=False):
+    """``g = -exp(A_log) * softplus(a + dt_bias)`` fp32; ``beta = sigmoid(b)`` (io dtype). ``exp_bf16``: the eager
+    form on a bf16 parameter (gdn_ops.py:1197-1210), whose ``A_log.exp()`` is a bf16 value; otherwise the parameter
+    is widened first (the fused core's form, and ``native_matched_prep``, gdn_cpr.py:241-244)."""
     sp = prims.softplus((a.astype(F32) + dt_bias.astype(F32)[None, :]).astype(F32))
-    g = ((-prims.exp(A_log.astype(F32)))[None, :] * sp).astype(F32)
+    ea = prims.exp(A_log.astype(F32))
+    if exp_bf16:
+        ea = round_bf16(ea)
+    g = ((-ea)[None, :] * sp).astype(F32)
     beta = prims.sigmoid(b.astype(F32))
     return g, (round_bf16(beta) if io_bf16 else beta)
 

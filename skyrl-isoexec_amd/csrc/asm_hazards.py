@@ -21,7 +21,14 @@ compiler believes vN holds the value at once; the value is taken into use throug
 comment ``; ix_landed vN`` in the assembly). Between the two
 * no instruction may mention vN (a copy or a spill would move a value that has not arrived), and
 * there must be an ``s_waitcnt vmcnt(n)`` with at least n vector-memory instructions issued after the load (they
-  retire in order, so that wait has retired the load).
+  retire in order, so that wait has retired the load);
+* and no label, branch or jump may lie between the load and its ``ix_landed``: this rule is judged on the lines in
+  their order in the file, which is only the order of execution for straight-line code.
+
+The rules cover the instruction classes the inline assembly of this library uses today. A NEW class of inline-assembly
+instruction (an LDS instruction that reads M0, a scalar load whose result feeds a vector-memory instruction, a
+different matrix instruction with its own latency, ...) gets its own rule here and a case in tests/test_asm_hazards.py
+before the kernel that contains it runs on a GPU for the first time.
 
 Usage: ``asm_hazards.py file.s [file.s ...]`` on the output of ``hipcc -S --offload-device-only`` (``make check``
 drives it). Exit status 1 and one line per finding if a rule is broken. The scan walks upwards from every
@@ -184,6 +191,9 @@ def scan(path):
             continue
         m = re.match(r"^(\.LBB\w+):", raw)
         if m:
+            for reg, st in flying.items():
+                findings.append(f"{path}:{ln}: {func}: label {m.group(1)} between the uncounted load into v{reg} (line "
+                                f"{st[0]}) and its ix_landed: not straight-line code, the in-flight rule cannot be judged")
             hist.append(("<label> " + m.group(1), False, ln))
             continue
         if not raw.startswith("\t") or s.startswith(";") or s.startswith("."):
@@ -197,6 +207,10 @@ def scan(path):
             if reg in touched:
                 findings.append(f"{path}:{ln}: {func}: '{ins}' touches v{reg} while the uncounted load of line "
                                 f"{flying[reg][0]} is in flight")
+        if re.match(r"^s_c?branch|^s_setpc|^s_swappc|^s_call", ins):
+            for reg, st in flying.items():
+                findings.append(f"{path}:{ln}: {func}: '{ins}' between the uncounted load into v{reg} (line {st[0]}) and "
+                                f"its ix_landed: not straight-line code, the in-flight rule cannot be judged")
         m = re.match(r"^s_waitcnt\b.*\bvmcnt\((\d+)\)", ins)
         if m:
             for st in flying.values():

@@ -509,13 +509,15 @@ __global__ __launch_bounds__(256) void k_gdn_gate(const TIO* __restrict__ a, lon
                                                   const TIO* __restrict__ b, long b_pitch,
                                                   const float* __restrict__ A_log,
                                                   const float* __restrict__ dt_bias, float* __restrict__ g,
-                                                  TIO* __restrict__ beta, long n, int HV) {
+                                                  TIO* __restrict__ beta, long n, int HV, int exp_bf16) {
   const long i = (long)blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
   const long t = i / HV;
   const int hv = (int)(i - t * HV);
   const float sp = ix_softplus(ix_ld(a + t * a_pitch + hv) + dt_bias[hv]);
-  const float neg_ea = -ix_exp(A_log[hv]);
+  float ea = ix_exp(A_log[hv]);
+  if (exp_bf16) ea = ix_bf2f(ix_f2bf(ea));  // a bf16 parameter's exp() is a bf16 value (the eager form's rounding)
+  const float neg_ea = -ea;
   g[i] = neg_ea * sp;
   ix_st(beta + i, ix_sigmoid(ix_ld(b + t * b_pitch + hv)));
 }
@@ -549,10 +551,12 @@ extern "C" int ix_gdn_l2norm(const void* x, long x_pitch, void* y, int io_dtype,
 
 extern "C" int ix_gdn_gate(const void* a, long a_pitch, const void* b, long b_pitch, const float* A_log,
                            const float* dt_bias, float* g, void* beta, int io_dtype, long tokens, long HV,
-                           void* stream) {
+                           int exp_dtype, void* stream) {
   if (!a || !b || !A_log || !dt_bias || !g || !beta || tokens < 0 || HV <= 0 || a_pitch < HV || b_pitch < HV)
     return IX_ERR_ARG;
   if (io_dtype != IX_DT_F32 && io_dtype != IX_DT_BF16) return IX_DECLINED;
+  if (exp_dtype != IX_DT_F32 && exp_dtype != IX_DT_BF16) return IX_DECLINED;
+  const int exp_bf16 = exp_dtype == IX_DT_BF16;
   const long n = tokens * HV;
   if (n == 0) return IX_OK;
   const long grid = (n + 255) / 256;
@@ -560,10 +564,10 @@ extern "C" int ix_gdn_gate(const void* a, long a_pitch, const void* b, long b_pi
   hipStream_t st = (hipStream_t)stream;
   if (io_dtype == IX_DT_BF16)
     hipLaunchKernelGGL((k_gdn_gate<bf16_t>), dim3((unsigned)grid), dim3(256), 0, st, (const bf16_t*)a, a_pitch,
-                       (const bf16_t*)b, b_pitch, A_log, dt_bias, g, (bf16_t*)beta, n, (int)HV);
+                       (const bf16_t*)b, b_pitch, A_log, dt_bias, g, (bf16_t*)beta, n, (int)HV, exp_bf16);
   else
     hipLaunchKernelGGL((k_gdn_gate<float>), dim3((unsigned)grid), dim3(256), 0, st, (const float*)a, a_pitch,
-                       (const float*)b, b_pitch, A_log, dt_bias, g, (float*)beta, n, (int)HV);
+                       (const float*)b, b_pitch, A_log, dt_bias, g, (float*)beta, n, (int)HV, exp_bf16);
   return ix_launch_status();
 }
 

@@ -527,30 +527,44 @@ __global__ __launch_bounds__(256) void k_moe_permute_one_tile(const int* __restr
 
 // Block map for rows that are ALREADY grouped by expert (the caller holds tokens_per_expert, e.g. a dispatcher's
 // output): exclusive scan of the counts, then every expert writes its own row tiles. One workgroup, integer only.
+// The counts live on the device, so the host cannot check them against the size of the row buffers: the kernel
+// itself keeps every tile inside [0, rows) -- an expert's count is cut to what is left of `rows` after the experts
+// before it (counts that add up to more than `rows` lose their tail instead of reaching past the buffers).
 template <typename TI>
 __global__ __launch_bounds__(256) void k_moe_block_map(const TI* __restrict__ counts_in, int E, int BM, int max_tiles,
-                                                       int* __restrict__ offsets, int* __restrict__ meta) {
+                                                       int rows, int* __restrict__ offsets, int* __restrict__ meta) {
   __shared__ int s_rows[256], s_tiles[256];
   const int tid = threadIdx.x;
   int c[2], tl[2];  // lane owns experts 2 tid and 2 tid + 1 (E <= 512)
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
     const int e = 2 * tid + h;
-    c[h] = e < E ? max(0, (int)counts_in[e]) : 0;
-    tl[h] = (c[h] + BM - 1) / BM;
+    const long want = e < E ? (long)counts_in[e] : 0;
+    c[h] = (int)(want < 0 ? 0 : (want > rows ? rows : want));
   }
-  s_rows[tid] = c[0] + c[1];
-  s_tiles[tid] = tl[0] + tl[1];
+  s_rows[tid] = min(c[0] + c[1], rows);  // a partial sum never needs to exceed `rows`: no overflow for any counts
   __syncthreads();
   for (int d = 1; d < 256; d <<= 1) {
     const int a = tid >= d ? s_rows[tid - d] : 0;
+    __syncthreads();
+    s_rows[tid] = min(s_rows[tid] + a, rows);
+    __syncthreads();
+  }
+  // Saturating adds are associative for non-negative terms: s_rows[tid] = min(rows, sum of the counts up to this lane).
+  const int before = tid > 0 ? s_rows[tid - 1] : 0;
+  c[0] = min(c[0], rows - before);
+  c[1] = min(c[1], rows - before - c[0]);
+#pragma unroll
+  for (int h = 0; h < 2; ++h) tl[h] = (c[h] + BM - 1) / BM;
+  s_tiles[tid] = tl[0] + tl[1];
+  __syncthreads();
+  for (int d = 1; d < 256; d <<= 1) {
     const int b = tid >= d ? s_tiles[tid - d] : 0;
     __syncthreads();
-    s_rows[tid] += a;
     s_tiles[tid] += b;
     __syncthreads();
   }
-  int row0 = s_rows[tid] - (c[0] + c[1]);
+  int row0 = before;
   int tile0 = s_tiles[tid] - (tl[0] + tl[1]);
   int* tile_expert = meta + 1;
   int* tile_row0 = tile_expert + max_tiles;
@@ -576,17 +590,17 @@ __global__ __launch_bounds__(256) void k_moe_block_map(const TI* __restrict__ co
   }
 }
 
-extern "C" int ix_moe_block_map(const void* counts, int counts_i64, long E, long BM, int* offsets, int* tile_meta,
-                                long max_tiles, void* stream) {
-  if (!counts || !tile_meta || E <= 0 || BM <= 0 || max_tiles <= 0) return IX_ERR_ARG;
-  if (E > IX_MOE_EMAX) return IX_DECLINED;
+extern "C" int ix_moe_block_map(const void* counts, int counts_i64, long E, long BM, long rows, int* offsets,
+                                int* tile_meta, long max_tiles, void* stream) {
+  if (!counts || !tile_meta || E <= 0 || BM <= 0 || max_tiles <= 0 || rows < 0) return IX_ERR_ARG;
+  if (E > IX_MOE_EMAX || rows > 0x3fffffffL) return IX_DECLINED;  // two clamped counts are added in an int
   hipStream_t st = (hipStream_t)stream;
   if (counts_i64)
     hipLaunchKernelGGL(k_moe_block_map<long>, dim3(1), dim3(256), 0, st, (const long*)counts, (int)E, (int)BM,
-                       (int)max_tiles, offsets, tile_meta);
+                       (int)max_tiles, (int)rows, offsets, tile_meta);
   else
     hipLaunchKernelGGL(k_moe_block_map<int>, dim3(1), dim3(256), 0, st, (const int*)counts, (int)E, (int)BM,
-                       (int)max_tiles, offsets, tile_meta);
+                       (int)max_tiles, (int)rows, offsets, tile_meta);
   return ix_launch_status();
 }
 
@@ -665,6 +679,13 @@ static int ix_moe_static_scratch_for_current_device(int** out) {
 }
 
 extern "C" size_t ix_moe_permute_static_max_ints(void) { return (size_t)IX_MOE_STATIC_SCRATCH_INTS; }
+
+// Set-up call: resolves the array's address on the current device, so that a caller can take the one runtime lookup
+// out of the region where it may make no such call (a stream capture). Launches nothing; may be called again.
+extern "C" int ix_moe_permute_static_init(void) {
+  int* scratch = nullptr;
+  return ix_moe_static_scratch_for_current_device(&scratch);
+}
 
 extern "C" int ix_moe_permute_static(const int* topk_idx, const float* topk_prob, long T, long E, long k, long BM,
                                      int* counts, int* offsets, int* sorted_token, float* permuted_prob,
@@ -1379,5 +1400,77 @@ extern "C" int ix_moe_combine(const void* expert_out, const int* combine_rows, v
     default: IX_COMBINE(0); break;
   }
 #undef IX_COMBINE
+  return ix_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// The combine with a weight per expert row and any of the eager form's dtypes (moe_batch_invariant.py:276-320 after
+// :366-369 `permuted_tokens * permuted_probs.unsqueeze(-1)`): value_r = x[row_r] * w[row_r], summed left to right
+// over a token's k rows. The arithmetic dtype is torch's promotion of (token dtype, weight dtype): in bf16 the
+// product and every partial sum are rounded to bf16, in fp32 nothing is rounded before the store.
+template <typename TIN>
+__global__ __launch_bounds__(256) void k_moe_combine_weighted(const TIN* __restrict__ expert_out,
+                                                              const float* __restrict__ row_weight,
+                                                              const int* __restrict__ combine_rows, void* __restrict__ out,
+                                                              long T, int Hd, int k, int arith_bf16, int out_bf16,
+                                                              int vec) {
+  const int groups = (Hd + 7) / 8;
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= T * groups) return;
+  const long t = i / groups;
+  const int c0 = (int)(i % groups) * 8;
+  float acc[8];
+  for (int r = 0; r < k; ++r) {
+    const long row = combine_rows[t * k + r];
+    float xv[8];
+    ix_load8(expert_out + row * Hd + c0, Hd - c0, vec != 0, 0.0f, xv);
+    if (row_weight) {
+      const float w = row_weight[row];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float prod = xv[j] * w;
+        xv[j] = arith_bf16 ? ix_rbf(prod) : prod;
+      }
+    }
+    if (r == 0) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] = xv[j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float sum = acc[j] + xv[j];
+        acc[j] = arith_bf16 ? ix_rbf(sum) : sum;
+      }
+    }
+  }
+  if (out_bf16) {
+    ix_store8_bf16((bf16_t*)out + t * Hd + c0, Hd - c0, vec != 0, acc);
+  } else {
+    float* o = (float*)out + t * Hd + c0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (c0 + j < Hd) o[j] = acc[j];
+  }
+}
+
+extern "C" int ix_moe_combine_weighted(const void* expert_out, int in_dtype, const float* row_weight, int arith_dtype,
+                                       const int* combine_rows, void* out, int out_dtype, long T, long Hd, long k,
+                                       void* stream) {
+  if (!expert_out || !combine_rows || !out || T < 0 || Hd <= 0 || k <= 0) return IX_ERR_ARG;
+  const auto known = [](int d) { return d == IX_DT_F32 || d == IX_DT_BF16; };
+  if (!known(in_dtype) || !known(arith_dtype) || !known(out_dtype)) return IX_DECLINED;
+  if (in_dtype == IX_DT_F32 && arith_dtype == IX_DT_BF16) return IX_ERR_ARG;  // promotion never narrows
+  if (T == 0) return IX_OK;
+  const long groups = (Hd + 7) / 8;
+  const long grid = (T * groups + 255) / 256;
+  if (grid > 0x7fffffffL) return IX_DECLINED;
+  const int vec = (Hd % 8 == 0) && ix_aligned(expert_out, 16) && ix_aligned(out, 16);
+  const int ab = arith_dtype == IX_DT_BF16, ob = out_dtype == IX_DT_BF16;
+  if (in_dtype == IX_DT_BF16)
+    hipLaunchKernelGGL(k_moe_combine_weighted<bf16_t>, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream,
+                       (const bf16_t*)expert_out, row_weight, combine_rows, out, T, (int)Hd, (int)k, ab, ob, vec);
+  else
+    hipLaunchKernelGGL(k_moe_combine_weighted<float>, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream,
+                       (const float*)expert_out, row_weight, combine_rows, out, T, (int)Hd, (int)k, ab, ob, vec);
   return ix_launch_status();
 }

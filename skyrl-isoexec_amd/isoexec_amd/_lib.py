@@ -70,7 +70,7 @@ SIGNATURES = {
     "ix_gdn_cpr_scatter": (c_int, [P, c_long, P, c_long, P, P, P, P, P, P, P, P, P, c_int, c_long, c_long, c_long, c_long, c_long, c_long, P]),
     "ix_gdn_cpr_handoff": (c_int, [P, P, P, c_long, c_long, c_int, P]),
     "ix_gdn_resolve_rows": (c_int, [P, c_int, c_long, P, c_long, c_long, P, P, P, P, P]),
-    "ix_gdn_gate": (c_int, [P, c_long, P, c_long, P, P, P, P, c_int, c_long, c_long, P]),
+    "ix_gdn_gate": (c_int, [P, c_long, P, c_long, P, P, P, P, c_int, c_long, c_long, c_int, P]),
     "ix_gdn_conv": (c_int, [P, c_long, P, P, P, P, P, P, P, c_long, c_long, c_long, c_long, c_int, P]),
     "ix_attn_varlen": (c_int, [P, c_long, P, P, c_long, P, P, P, P, c_long, c_long, c_long, c_long, c_long, c_float, P]),
     "ix_rope_inplace": (c_int, [P, c_long, P, P, c_long, P, c_long, c_long, c_long, c_long, P]),
@@ -82,8 +82,9 @@ SIGNATURES = {
         c_int,
         [P, P, c_long, c_long, c_long, c_long, P, P, P, P, P, P, c_long, P, P],
     ),
-    "ix_moe_block_map": (c_int, [P, c_int, c_long, c_long, P, P, c_long, P]),
+    "ix_moe_block_map": (c_int, [P, c_int, c_long, c_long, c_long, P, P, c_long, P]),
     "ix_moe_permute_static_max_ints": (c_size_t, []),
+    "ix_moe_permute_static_init": (c_int, []),
     "ix_moe_permute_static": (
         c_int,
         [P, P, c_long, c_long, c_long, c_long, P, P, P, P, P, P, c_long, P],
@@ -97,6 +98,7 @@ SIGNATURES = {
         [P, c_long, P, P, P, P, P, c_long, c_long, c_long, P, P, c_long, c_long, c_long, c_long, P],
     ),
     "ix_moe_combine": (c_int, [P, P, P, c_long, c_long, c_long, c_int, P]),
+    "ix_moe_combine_weighted": (c_int, [P, c_int, P, c_int, P, P, c_int, c_long, c_long, c_long, P]),
     "ix_digest_sums": (c_int, [P, c_int, c_long, c_uint64, P, c_int, P, c_size_t, P, P]),
     "ix_digest_segment_sums": (c_int, [P, c_int, c_long, c_long, c_long, c_uint64, c_uint64, P, c_size_t, P, P]),
     "ix_digest_workspace_words": (c_size_t, [c_long, c_long, c_int]),

@@ -20,7 +20,7 @@ from collections import OrderedDict
 import numpy as np
 import torch
 
-from .gdn_ops import gdn_gate_and_beta, gdn_l2norm, gdn_native_core_kernel, gdn_recurrent_kernel
+from .gdn_ops import gate_and_beta_fp32, gdn_l2norm, gdn_native_core_kernel, gdn_recurrent_kernel
 
 # Host-built chunk metadata (gdn_cpr.py:15-51): pure integers, so identical tensors however they are built.
 _META_CACHE: OrderedDict = OrderedDict()
@@ -199,7 +199,7 @@ def native_matched_prep(k_raw, a, b, A_log, dt_bias):
     """``(kn, g, beta)`` from raw inputs for the boundary pass (gdn_cpr.py:225-254), by the same kernels as the
     scan's own preparation, so the boundary pass and the segmented scan see identical operands."""
     HV = a.shape[-1]
-    g, beta = gdn_gate_and_beta(a.reshape(-1, HV), b.reshape(-1, HV), A_log, dt_bias)
+    g, beta = gate_and_beta_fp32(a.reshape(-1, HV), b.reshape(-1, HV), A_log, dt_bias)
     return gdn_l2norm(k_raw), g, beta.to(k_raw.dtype)
 
 

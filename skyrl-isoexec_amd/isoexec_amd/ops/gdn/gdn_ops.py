@@ -142,7 +142,26 @@ def gdn_l2norm(x: torch.Tensor) -> torch.Tensor:
 
 
 def gdn_gate_and_beta(a: torch.Tensor, b: torch.Tensor, A_log: torch.Tensor, dt_bias: torch.Tensor):
-    """``g = -exp(A_log) * softplus(a + dt_bias)`` in fp32; ``beta = sigmoid(b)``. Elementwise."""
+    """``g = -exp(A_log) * softplus(a + dt_bias)`` in fp32; ``beta = sigmoid(b)``. Elementwise.
+
+    The eager form of gdn_ops.py:1197-1210: ``A_log.exp()`` is taken in the parameter's own dtype, so a bf16
+    parameter's exponential is rounded to bf16 before the fp32 product ("exp(bf16(x)).float() is not exp(float(x))").
+    The fused core's form, which widens the parameter first, is ``gate_and_beta_fp32``."""
+    if A_log.dtype is torch.bfloat16:
+        return _gate_and_beta(a, b, A_log, dt_bias, _lib.DT_BF16)
+    if A_log.dtype is not torch.float32:
+        raise RuntimeError(f"[isoexec-amd] gdn_gate_and_beta serves fp32 and bf16 A_log, got {A_log.dtype}")
+    return _gate_and_beta(a, b, A_log, dt_bias, _lib.DT_F32)
+
+
+def gate_and_beta_fp32(a: torch.Tensor, b: torch.Tensor, A_log: torch.Tensor, dt_bias: torch.Tensor):
+    """The gating of the fused core (``fused_sigmoid_gating_delta_rule_update``, gdn/_register.py:33-55) and of
+    ``native_matched_prep`` (gdn_cpr.py:241-244: ``-torch.exp(A_log.float())``): every parameter widened to fp32
+    before any arithmetic, whatever its storage dtype."""
+    return _gate_and_beta(a, b, A_log, dt_bias, _lib.DT_F32)
+
+
+def _gate_and_beta(a, b, A_log, dt_bias, exp_dtype):
     _lib.require_device(a, b, A_log, dt_bias)
     HV = a.shape[-1]
 
@@ -159,7 +178,7 @@ def gdn_gate_and_beta(a: torch.Tensor, b: torch.Tensor, A_log: torch.Tensor, dt_
     dt32 = dt_bias if dt_bias.dtype is torch.float32 and dt_bias.is_contiguous() else dt_bias.float().contiguous()
     _lib.check(
         _lib.lib().ix_gdn_gate(ac.data_ptr(), ap, bc.data_ptr(), bp, A32.data_ptr(), dt32.data_ptr(), g.data_ptr(),
-                               beta.data_ptr(), _lib.dtype_code(a.dtype), a.numel() // HV, HV,
+                               beta.data_ptr(), _lib.dtype_code(a.dtype), a.numel() // HV, HV, exp_dtype,
                                _lib.current_stream(a.device)),
         "ix_gdn_gate")
     return g, beta
@@ -318,7 +337,7 @@ def gdn_native_core_kernel(q, k, v, a, b, A_log, dt_bias, *, ssm_state, state_in
     calls bitwise."""
     qn, kn = gdn_l2norm(q), gdn_l2norm(k)
     HV = v.shape[-2]
-    g, beta = gdn_gate_and_beta(a.reshape(-1, HV), b.reshape(-1, HV), A_log, dt_bias)
+    g, beta = gate_and_beta_fp32(a.reshape(-1, HV), b.reshape(-1, HV), A_log, dt_bias)
     lead = v.shape[:2]
     return gdn_recurrent_kernel(qn, kn, v, g.view(*lead, HV), beta.view(*lead, HV), ssm_state=ssm_state,
                                 state_indices=state_indices, cu_seqlens=cu_seqlens)

@@ -26,7 +26,7 @@ from typing import Callable, Iterable, Sequence
 import numpy as np
 import torch
 
-from .gdn_ops import conv_packed, gdn_gate_and_beta, gdn_l2norm, gdn_recurrent_kernel
+from .gdn_ops import conv_packed, gate_and_beta_fp32, gdn_l2norm, gdn_recurrent_kernel
 
 _SLOT_MAP_ENV = "SKYRL_ISOEXEC_GDN_SLOT_MAP_SIZE"
 _CHUNKED_PREFILL_ENV = "SKYRL_ISOEXEC_GDN_CHUNKED_PREFILL"
@@ -440,7 +440,7 @@ class RecurrentGDN:
         return gdn_l2norm(q), gdn_l2norm(k), v
 
     def _gate_and_beta(self, a: torch.Tensor, b: torch.Tensor):
-        return gdn_gate_and_beta(a, b, self.A_log, self.dt_bias)
+        return gate_and_beta_fp32(a, b, self.A_log, self.dt_bias)
 
     def _continuation_mask(self, slots_cpu, has_initial_state) -> list[bool]:
         """Which prefill rows resume carried state. Table membership and the scheduler's

@@ -156,8 +156,11 @@ def bmm_batch_invariant(a: torch.Tensor, b: torch.Tensor):
 # aten::mm / addmm / bmm on the device dispatch key are replaced, so every F.linear / torch.matmul of the process
 # lands on the fixed-order kernels (matmul and linear are composite: only these three primitives need replacing).
 # A signature the kernels do not serve (other dtypes, K or a row pitch that is not a multiple of 8, alpha/beta forms)
-# is handed to the kernel that was registered before, counted under "declined" and named once on stderr: the process
-# keeps working, and the count says whether anything on the hot path escaped. ``strict=True`` raises instead.
+# raises by default (``strict=True``): a product that silently took the stock kernel is not batch-invariant, and the
+# reference's own notes record that partial coverage of the override broke bitwise parity live. With the explicit
+# opt-in ``strict=False`` (a process that also runs products outside the contract, e.g. a backward pass) such a
+# signature is handed to the kernel that was registered before, counted under "declined" and named once on stderr;
+# ``assert_none_declined()`` then turns the count into a refusal at a point of the caller's choosing.
 _STOCK = {}
 _STRICT = False
 _NAMED = set()
@@ -201,8 +204,19 @@ def _bmm_impl(keyset, a, b):
     return out
 
 
-def install_mm_override(strict: bool = False) -> bool:
-    """Route ``aten::mm/addmm/bmm`` on device tensors to the kernels (moe_batch_invariant.py:453-464)."""
+def assert_none_declined(since: int = 0) -> None:
+    """Raise if any product was handed to the stock kernel since the count stood at ``since`` (``stats()["declined"]``
+    read before the forward): the check a fall-through install owes after every forward under the contract."""
+    n = _COUNTS["declined"] - since
+    if n > 0:
+        raise RuntimeError(f"[isoexec-amd] {n} matrix product(s) ran on the stock kernel, which is not batch-invariant: "
+                           f"{sorted(_NAMED)[:8]}")
+
+
+def install_mm_override(strict: bool = True) -> bool:
+    """Route ``aten::mm/addmm/bmm`` on device tensors to the kernels (moe_batch_invariant.py:453-464). ``strict``
+    (the default): a signature the kernels do not serve raises; ``strict=False``: it falls through to the stock kernel
+    and is counted."""
     global _LIBRARY, _STRICT
     _STRICT = bool(strict)
     if _LIBRARY is not None:

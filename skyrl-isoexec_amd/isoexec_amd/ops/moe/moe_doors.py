@@ -17,6 +17,9 @@ from ... import _lib
 from . import moe_hip
 
 _STACKED = {}   # id(module) -> (key, w1 [E, 2F, H], w2 [E, H, F])
+_VALIDATE_FIRST_N_CALLS = 8     # moe_batch_invariant.py:24
+_validated_calls = 0            # layouts checked by the combine
+_validated_counts = 0           # per-expert counts checked by the experts' door
 
 
 def _stacked_weights(module):
@@ -80,12 +83,21 @@ def _batched_experts_forward(self, permuted_local_hidden_states, tokens_per_expe
     if counts.dtype not in (torch.int32, torch.int64):
         counts = counts.to(torch.int64)
     counts = counts.contiguous()
+    global _validated_counts
+    if _validated_counts < _VALIDATE_FIRST_N_CALLS:
+        # The kernels keep every tile inside the R rows whatever the counts say, but rows that no expert claims
+        # would be left unwritten: on the first calls the counts are read back and checked, like the combine's layout.
+        _validated_counts += 1
+        total = int(counts.sum().item())
+        if total != R or counts.numel() != E:
+            raise RuntimeError(f"[isoexec-amd] SequentialMLP.forward: tokens_per_expert has {counts.numel()} entries "
+                               f"adding up to {total} for {R} permuted rows and {E} local experts")
     BM = int(L.ix_moe_pick_bm(R, 1, E))
     max_tiles = int(L.ix_moe_max_tiles(R, 1, E, BM))
     meta = torch.empty(1 + 3 * max_tiles, dtype=torch.int32, device=dev)
     stream = _lib.current_stream(dev)
-    rc = _lib.check(L.ix_moe_block_map(counts.data_ptr(), int(counts.dtype is torch.int64), E, BM, None, meta.data_ptr(),
-                                       max_tiles, stream), "ix_moe_block_map")
+    rc = _lib.check(L.ix_moe_block_map(counts.data_ptr(), int(counts.dtype is torch.int64), E, BM, R, None,
+                                       meta.data_ptr(), max_tiles, stream), "ix_moe_block_map")
     if rc != _lib.IX_OK:
         raise RuntimeError(f"[isoexec-amd] ix_moe_block_map declined E={E}")
     rows = torch.arange(R, dtype=torch.int32, device=dev)      # the rows are already in expert order
@@ -101,19 +113,69 @@ def _batched_experts_forward(self, permuted_local_hidden_states, tokens_per_expe
     return out, None
 
 
+def reset_combine_validation() -> None:
+    """Start the first-calls layout validations over (the reference resets its counter on install, :556)."""
+    global _validated_calls, _validated_counts
+    _validated_calls = 0
+    _validated_counts = 0
+
+
+def _combine_rows(sorted_indices, num_tokens: int, k: int):
+    """``[T, k]`` int32 row numbers: a token's rows in ascending expert order. Rows are expert-major, so a stable sort
+    by token groups them. On the first calls the layout is checked, as the reference does (:307-316): every token must
+    own exactly k rows; token dropping or capacity padding would otherwise sum the wrong rows without a sign."""
+    global _validated_calls
+    rows = torch.argsort(sorted_indices, stable=True)
+    if _validated_calls < _VALIDATE_FIRST_N_CALLS:
+        _validated_calls += 1
+        expected = torch.arange(num_tokens, device=sorted_indices.device).repeat_interleave(k)
+        if not torch.equal(sorted_indices[rows].to(expected.dtype), expected):
+            raise RuntimeError(
+                "[isoexec-amd] MoE combine: tokens do not each route to exactly topk experts "
+                f"(num_tokens={num_tokens}, permuted_rows={int(sorted_indices.numel())}). Token dropping / capacity "
+                "padding must be disabled for bitwise IsoExec.")
+    return rows.to(torch.int32).view(num_tokens, k).contiguous()
+
+
+def _weighted_combine(permuted_tokens, permuted_probs, sorted_indices, restore_shape, out_dtype):
+    """The eager chain of moe_batch_invariant.py:366-385 in one launch: ``(tokens * probs[:, None])`` in torch's
+    promoted dtype, a token's k rows summed left to right in that dtype, one cast to ``out_dtype``. ``None`` when the
+    layout is not "n rows = k per token" (the reference's decline)."""
+    num_tokens = int(restore_shape[0])
+    n = int(sorted_indices.numel())
+    if num_tokens == 0 or n == 0 or n % num_tokens != 0:
+        return None
+    _lib.require_device(permuted_tokens, sorted_indices, permuted_probs)
+    k = n // num_tokens
+    arith = permuted_tokens.dtype if permuted_probs is None else torch.promote_types(permuted_tokens.dtype,
+                                                                                       permuted_probs.dtype)
+    for what, dt in (("token", permuted_tokens.dtype), ("arithmetic", arith), ("output", out_dtype)):
+        if dt not in (torch.bfloat16, torch.float32):
+            raise RuntimeError(f"[isoexec-amd] unpermute: {what} dtype {dt} is not served (bf16 and fp32 are)")
+    rows = _combine_rows(sorted_indices, num_tokens, k)
+    pt = permuted_tokens.contiguous()
+    w = None if permuted_probs is None else permuted_probs.to(torch.float32).contiguous()
+    out = torch.empty(num_tokens, pt.shape[1], dtype=out_dtype, device=pt.device)
+    _lib.check(_lib.lib().ix_moe_combine_weighted(pt.data_ptr(), _lib.dtype_code(pt.dtype), _lib.ptr(w),
+                                                  _lib.dtype_code(arith), rows.data_ptr(), out.data_ptr(),
+                                                  _lib.dtype_code(out_dtype), num_tokens, pt.shape[1], k,
+                                                  _lib.current_stream(pt.device)), "ix_moe_combine_weighted")
+    return out
+
+
 def _fixed_order_combine(permuted_tokens, sorted_indices, restore_shape):
-    """Each token's k expert rows summed in ascending expert order, a bf16 round per add (moe_batch_invariant.py:
-    276-320). ``None`` when the layout is not "every token routes to exactly k experts" (the reference's decline)."""
+    """Each token's k expert rows summed in ascending expert order in the rows' own dtype: a bf16 round per add for
+    bf16 rows, plain fp32 adds for fp32 rows (moe_batch_invariant.py:276-320). ``None`` when the layout is not
+    "every token routes to exactly k experts" (the reference's decline)."""
     num_tokens = int(restore_shape[0])
     n = int(sorted_indices.numel())
     if num_tokens == 0 or n == 0 or n % num_tokens != 0:
         return None
     _lib.require_device(permuted_tokens, sorted_indices)
     if permuted_tokens.dtype is not torch.bfloat16:
-        return None
+        return _weighted_combine(permuted_tokens, None, sorted_indices, restore_shape, permuted_tokens.dtype)
     k = n // num_tokens
-    # rows are expert-major, so a stable sort by token groups a token's rows in ascending expert order
-    rows = torch.argsort(sorted_indices, stable=True).to(torch.int32).view(num_tokens, k).contiguous()
+    rows = _combine_rows(sorted_indices, num_tokens, k)
     pt = permuted_tokens.contiguous()
     out = torch.empty(num_tokens, pt.shape[1], dtype=torch.bfloat16, device=pt.device)
     _lib.check(_lib.lib().ix_moe_combine(pt.data_ptr(), rows.data_ptr(), out.data_ptr(), num_tokens, pt.shape[1], k, 0,
@@ -123,19 +185,23 @@ def _fixed_order_combine(permuted_tokens, sorted_indices, restore_shape):
 
 def _deterministic_unpermute(permuted_tokens, sorted_indices, restore_shape, probs=None, routing_map=None, fused=False,
                              drop_and_pad=False, isoexec_out_dtype=None, **kwargs):
-    """Drop-in ``moe_utils.unpermute`` (moe_batch_invariant.py:338-385). There is no incumbent to fall back to here:
-    the fused / drop-and-pad forms, and a layout the combine declines, raise."""
+    """Drop-in ``moe_utils.unpermute`` (moe_batch_invariant.py:338-385). With ``probs`` the rows are weighted in torch's
+    promoted dtype (bf16 rows x fp32 probs: an fp32 product and an fp32 fixed-order sum, then the trailing cast), as the
+    eager expression there. There is no incumbent to fall back to here: the fused / drop-and-pad forms, and a layout
+    the combine declines, raise."""
     if fused or drop_and_pad:
         raise RuntimeError("[isoexec-amd] unpermute: the fused and drop-and-pad forms are not batch-invariant; not served")
     out_dtype = permuted_tokens.dtype if isoexec_out_dtype is None else isoexec_out_dtype
     if probs is not None:
         assert routing_map is not None, "Mask must be provided to permute the probs."
         permuted_probs = probs.T.contiguous().masked_select(routing_map.T.contiguous())
-        permuted_tokens = permuted_tokens * permuted_probs.unsqueeze(-1)
-    out = _fixed_order_combine(permuted_tokens, sorted_indices, restore_shape)
+        out = _weighted_combine(permuted_tokens, permuted_probs, sorted_indices, restore_shape, out_dtype)
+    else:
+        out = _fixed_order_combine(permuted_tokens, sorted_indices, restore_shape)
     if out is None:
-        raise RuntimeError("[isoexec-amd] unpermute: tokens do not each route to exactly topk experts "
-                           f"(tokens {int(restore_shape[0])}, rows {int(sorted_indices.numel())})")
+        raise RuntimeError("[isoexec-amd] unpermute: the row count is not a multiple of the token count "
+                           f"(tokens {int(restore_shape[0])}, rows {int(sorted_indices.numel())}); token dropping / "
+                           "capacity padding is not served")
     return out.to(dtype=out_dtype)
 
 

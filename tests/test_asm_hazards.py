@@ -90,6 +90,13 @@ def test_uncounted_load_must_be_retired_and_untouched(tmp_path):
     assert any("never taken into use" in f for f in scan(tmp_path, load + dmas + wait))
     # a marker without a load
     assert any("without an uncounted load" in f for f in scan(tmp_path, take))
+    # control flow between the load and its use: the file order is not the execution order, the rule says so
+    found = scan(tmp_path, load + dmas + ".LBB0_3:\n" + wait + take)
+    assert len(found) == 1 and "label .LBB0_3" in found[0] and "not straight-line" in found[0]
+    found = scan(tmp_path, load + dmas + "\ts_cbranch_scc1 .LBB0_9\n" + wait + take)
+    assert len(found) == 1 and "s_cbranch_scc1" in found[0]
+    # the same label or branch outside the window is nobody's business
+    assert scan(tmp_path, ".LBB0_3:\n" + load + dmas + wait + take + "\ts_cbranch_scc1 .LBB0_3\n") == []
 
 
 def test_accumulator_read_waits_for_the_matrix_pipeline(tmp_path):

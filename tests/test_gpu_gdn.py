@@ -196,6 +196,15 @@ def test_l2norm_and_gate_bit_exact(dprims):
         # softplus is evaluated as one device primitive; exp(A_log) and the product are IEEE
         assert np.array_equal(np_bits(gg.cpu().numpy()), np_bits(wg))
         assert np.array_equal(np_bits(bb.float().cpu().numpy()), np_bits(wb))
+        # a bf16 parameter under the eager name: exp() is rounded to bf16 before the product (gdn_ops.py:1197-1210)
+        A16 = A_log.to(torch.bfloat16)
+        wg16, _ = o_gdn.gate_and_beta(a.float().numpy(), b.float().numpy(), A16.float().numpy(), dt_bias.numpy(),
+                                      io_bf16=dtype is torch.bfloat16, prims=dprims, exp_bf16=True)
+        gg16, _ = gdn_gate_and_beta(a.to(DEV), b.to(DEV), A16.to(DEV), dt_bias.to(DEV))
+        assert np.array_equal(np_bits(gg16.cpu().numpy()), np_bits(wg16))
+        assert not np.array_equal(np_bits(gg16.cpu().numpy()), np_bits(wg))
+        with pytest.raises(RuntimeError, match="fp32 and bf16 A_log"):
+            gdn_gate_and_beta(a.to(DEV), b.to(DEV), A_log.half().to(DEV), dt_bias.to(DEV))
 
 
 def test_conv_bit_exact_prefill_decode_and_state(dprims):

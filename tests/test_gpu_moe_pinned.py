@@ -139,6 +139,111 @@ def test_doors_with_the_reference_call_shapes(stacked):
         moe_doors._batched_experts_forward(mlp, hidden, tpe, pprobs)
 
 
+def test_unpermute_with_probs_and_layout_validation():
+    """``moe_utils.unpermute(..., probs=, routing_map=)`` (moe_batch_invariant.py:366-385): bf16 rows times fp32 probs is
+    an fp32 product, summed per token in ascending expert order in fp32, then cast. Expected values by the same eager
+    torch expressions (elementwise IEEE products and sums: no reduction order of torch's own is involved)."""
+    from isoexec_amd.ops.mm.mm_hip import router_gemm
+    from isoexec_amd.ops.moe import moe_doors
+    from isoexec_amd.ops.moe.moe_hip import fused_router_dense
+
+    T, H, E, F, k = 70, 200, 16, 64, 4              # H not a multiple of 8: the element-wise load path too
+    x, wr, w1, w2 = make(T, 256, E, F, seed=12)
+    rprobs, rmap = fused_router_dense(router_gemm(x, wr), k)
+    disp = SimpleNamespace(routing_map=rmap, local_expert_indices=list(range(E)), config=SimpleNamespace(moe_router_topk=k))
+    _, _, _ = moe_doors._dispatch_postprocess_fixed_shape(disp, x, rprobs)
+    sorted_indices = disp.reversed_local_input_permutation_mapping
+    g = cpu_gen(13)
+    moe_doors.reset_combine_validation()
+
+    def eager(tokens, probs, out_dtype):
+        pt = tokens
+        if probs is not None:
+            pp = probs.T.contiguous().masked_select(rmap.T.contiguous())
+            pt = tokens * pp.unsqueeze(-1)
+        rows = torch.argsort(sorted_indices, stable=True).view(T, k)
+        acc = pt.index_select(0, rows[:, 0].contiguous())
+        for j in range(1, k):
+            acc = acc + pt.index_select(0, rows[:, j].contiguous())
+        return acc.to(out_dtype)
+
+    for width in (H, 256):
+        tok16 = torch.randn(T * k, width, generator=g).to(torch.bfloat16).to(DEV)
+        for tokens, probs, out_dtype in ((tok16, rprobs, None), (tok16, rprobs, torch.float32),
+                                         (tok16, rprobs.to(torch.bfloat16), None), (tok16.float(), None, None),
+                                         (tok16.float(), rprobs, torch.bfloat16), (tok16, None, None)):
+            got = moe_doors._deterministic_unpermute(tokens, sorted_indices, (T, width), probs=probs,
+                                                     routing_map=None if probs is None else rmap,
+                                                     isoexec_out_dtype=out_dtype)
+            want = eager(tokens, probs, tokens.dtype if out_dtype is None else out_dtype)
+            assert got.dtype is want.dtype and same_bits(got, want), (width, tokens.dtype, probs is None, out_dtype)
+    # a layout where the row count is a multiple of the token count but a token owns the wrong number of rows
+    # (token dropping / padding) is refused on the first calls instead of summing the wrong rows
+    moe_doors.reset_combine_validation()
+    uneven = sorted_indices.clone()
+    uneven[uneven == 3] = 4
+    with pytest.raises(RuntimeError, match="do not each route to exactly topk"):
+        moe_doors._deterministic_unpermute(tok16, uneven, (T, 256))
+    with pytest.raises(RuntimeError, match="not a multiple"):
+        moe_doors._deterministic_unpermute(tok16[:-1], sorted_indices[:-1], (T, 256))
+    with pytest.raises(RuntimeError, match="not served"):
+        moe_doors._deterministic_unpermute(tok16.half(), sorted_indices, (T, 256), probs=rprobs, routing_map=rmap)
+    moe_doors.reset_combine_validation()
+
+
+def test_block_map_keeps_every_tile_inside_the_row_buffers():
+    """Per-expert counts live on the device; counts that add up to more rows than the buffers hold lose their tail,
+    counts that add up to fewer leave the last rows in no tile; the experts' door refuses both on its first calls."""
+    from isoexec_amd import _lib
+    from isoexec_amd.ops.moe import moe_doors
+
+    L = _lib.lib()
+    E, BM, R = 6, 32, 100
+    max_tiles = int(L.ix_moe_max_tiles(R, 1, E, BM))
+
+    def block_map(counts, dtype):
+        c = torch.tensor(counts, dtype=dtype, device=DEV)
+        meta = torch.full((1 + 3 * max_tiles,), -7, dtype=torch.int32, device=DEV)
+        off = torch.full((E + 1,), -7, dtype=torch.int32, device=DEV)
+        assert L.ix_moe_block_map(c.data_ptr(), int(dtype is torch.int64), E, BM, R, off.data_ptr(), meta.data_ptr(),
+                                  max_tiles, _lib.current_stream(torch.device(DEV))) == 0
+        m = meta.cpu().tolist()
+        n = m[0]
+        tiles = [(m[1 + i], m[1 + max_tiles + i], m[1 + 2 * max_tiles + i]) for i in range(n)]
+        return tiles, off.cpu().tolist()
+
+    def expected(counts):
+        tiles, off, row = [], [], 0
+        for e, c in enumerate(counts):
+            c = max(0, min(c, R - row))
+            off.append(row)
+            tiles += [(e, row + r0, min(BM, c - r0)) for r0 in range(0, c, BM)]
+            row += c
+        return tiles, off + [row]
+
+    for counts in ([10, 0, 33, 7, 50, 0], [10, 0, 33, 7, 80, 5], [70, 70, 1, 0, 0, 9], [2 ** 31 - 1] * 6, [0] * 6,
+                   [10, -4, 20, 0, 0, 3], [5, 5, 5, 5, 5, 5]):
+        for dtype in (torch.int32, torch.int64):
+            tiles, off = block_map(counts, dtype)
+            assert (tiles, off) == expected(counts), counts
+            assert all(0 <= r0 and n > 0 and r0 + n <= R for _, r0, n in tiles)
+    tiles, _ = block_map([2 ** 40, 1, 1, 1, 1, 1], torch.int64)             # a count beyond 32 bits is still only "too many"
+    assert tiles == [(0, 0, 32), (0, 32, 32), (0, 64, 32), (0, 96, 4)]
+    # the door: a batch whose counts do not add up to its rows is refused while the first calls are being checked
+    T, H, F = 72, 256, 128
+    hidden, _, w1, w2 = make(T, H, E, F, seed=14)
+    mlp = fake_sequential_mlp(w1, w2)
+    pprobs = torch.ones(hidden.shape[0], device=DEV)
+    moe_doors.reset_combine_validation()
+    good = torch.tensor([12] * 6, device=DEV)
+    out, _ = moe_doors._batched_experts_forward(mlp, hidden, good, pprobs)
+    assert out.shape == hidden.shape
+    for bad in ([12, 12, 12, 12, 12, 40], [12, 12, 12, 12, 12, 2]):
+        with pytest.raises(RuntimeError, match="adding up to"):
+            moe_doors._batched_experts_forward(mlp, hidden, torch.tensor(bad, device=DEV), pprobs)
+    moe_doors.reset_combine_validation()
+
+
 def test_operator_override_door():
     """aten::mm / addmm / bmm on the device key land on the fixed-order kernels: F.linear, torch.mm, torch.addmm,
     torch.bmm, 2-D and 3-D, with and without bias, forward and backward; what the kernels do not serve goes to the
@@ -155,7 +260,7 @@ def test_operator_override_door():
     want_b = mm_hip.linear_nt(x, w, b)
     stock = Fn.linear(x, w)
     mm_hip.reset_stats()
-    assert mm_hip.install_mm_override() and mm_hip.mm_override_installed()
+    assert mm_hip.install_mm_override(strict=False) and mm_hip.mm_override_installed()
     try:
         assert same_bits(Fn.linear(x, w), want) and mm_hip.stats()["mm"] == 1
         assert same_bits(torch.mm(x, w.t()), want) and same_bits(x @ w.t(), want) and mm_hip.stats()["mm"] == 3
@@ -188,8 +293,12 @@ def test_operator_override_door():
         f = torch.randn(9, 64, generator=g).to(DEV)
         served = mm_hip.stats()["mm"]
         assert same_bits(f @ f.t(), mm_hip.linear_f32_nt(f, f)) and mm_hip.stats()["mm"] == served + 1
-        # strict mode refuses instead of falling through
-        mm_hip.install_mm_override(strict=True)
+        # what fell through can be turned into a refusal after the fact
+        mm_hip.assert_none_declined(since=mm_hip.stats()["declined"])
+        with pytest.raises(RuntimeError, match="stock kernel"):
+            mm_hip.assert_none_declined(since=before)
+        # strict mode (the default) refuses instead of falling through
+        mm_hip.install_mm_override()
         with pytest.raises(RuntimeError):
             h @ h.t()
         mm_hip.install_mm_override(strict=False)

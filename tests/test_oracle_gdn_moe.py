@@ -86,6 +86,15 @@ def test_l2norm_gate_and_conv_against_eager_expressions():
     want_g = -A_log.exp() * torch.nn.functional.softplus(a + dt_bias)  # gdn_ops.py:1208
     assert np.abs(gg - want_g.numpy()).max() <= 1e-6 * np.abs(want_g.numpy()).max()
     assert np.abs(bb - torch.sigmoid(b).numpy()).max() <= 2e-7
+    # a bf16 parameter: the eager expression takes exp() in bf16 (torch on the CPU is the library routine here)
+    A16 = A_log.to(torch.bfloat16)
+    gg16, _ = o_gdn.gate_and_beta(a.numpy(), b.numpy(), A16.float().numpy(), dt_bias.numpy(), io_bf16=False,
+                                  exp_bf16=True)
+    want16 = -A16.exp() * torch.nn.functional.softplus(a.float() + dt_bias.float())
+    assert want16.dtype is torch.float32
+    assert np.abs(gg16 - want16.numpy()).max() <= 1e-6 * np.abs(want16.numpy()).max()
+    widened = -A16.float().exp() * torch.nn.functional.softplus(a + dt_bias)     # NOT the same function
+    assert np.abs(gg16 - widened.numpy()).max() > 1e-4 * np.abs(widened.numpy()).max()
     # conv: brute-force loop over (t, d, tap) in float64, and the split-anywhere property
     T, D, W = 19, 6, 4
     xx = torch.randn(T, D, generator=g).to(torch.bfloat16).float().numpy()

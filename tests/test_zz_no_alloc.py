@@ -69,6 +69,32 @@ def test_static_scratch_permutation_equals_workspace_permutation(sizes):
             assert np.array_equal(got[name].view(np.uint32), want[name].view(np.uint32)), (name, T, E, k, BM)
 
 
+def test_static_scratch_permutation_allocates_nothing():
+    """What the entry point exists for: after set-up, calls move neither the device's free memory (the runtime's own
+    figure, hipMemGetInfo) nor torch's allocator; the workspace form needs its scratch tensor for the same input."""
+    from isoexec_amd import _lib
+
+    L = _lib.lib()
+    assert L.ix_moe_permute_static_init() == 0 and L.ix_moe_permute_static_init() == 0
+    T, E, k, BM = 5000, 128, 8, 256
+    idx, prob = _routing(T, E, k, seed=77)
+    max_tiles, b = _buffers(L, T, E, k, BM)
+    stream = torch.cuda.current_stream().cuda_stream
+    args = [idx.data_ptr(), prob.data_ptr(), T, E, k, BM, b["counts"].data_ptr(), b["offsets"].data_ptr(),
+            b["sorted_token"].data_ptr(), b["permuted_prob"].data_ptr(), b["combine_rows"].data_ptr(),
+            b["tile_meta"].data_ptr(), max_tiles, stream]
+    assert L.ix_moe_permute_static(*args) == 0
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    alloc0, reserved0 = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    for _ in range(20):
+        assert L.ix_moe_permute_static(*args) == 0
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0 and torch.cuda.memory_allocated() == alloc0 and torch.cuda.memory_reserved() == reserved0
+    assert int(b["counts"].sum()) == T * k
+
+
 def test_static_scratch_permutation_refuses_what_does_not_fit():
     """Host-side check only: nothing is launched for an input beyond the array."""
     from isoexec_amd import _lib
