@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define IX_ABI_VERSION 2
+#define IX_ABI_VERSION 3
 
 #ifndef IX_OK
 #define IX_OK 0
@@ -57,6 +57,25 @@ const char* ix_arch_tag(void); /* "gfx950"; counterpart of core/arch.py:27-51 de
  * these into the CPU restatement so that order-of-operations parity is bit-exact. No
  * counterpart in the reference (its probes compare kernels against eager torch on device). */
 int ix_prim_unary(int op, const float* x, float* y, long n, void* stream);
+
+/* ---- device self-check: ops/collectives/pik_bootstrap.py:82-93 ----------------------------- */
+
+/* pik_arch_selfcheck (pik_bootstrap.py:82-93 -> pik/arch.py:90-168 _verify: "check on this GPU that no GEMM tiling
+ * knob moves the bits of a non-split-K K-reduction"; a failure disables the provider for good). Runs on the device,
+ * through this library's own entry points: a seeded 512 x 1024 x 1024 product whose operands span 2^24 in magnitude
+ * through every tile shape and launch form of ix_gemm_bf16_nt (ids 1..8), compared bit for bit on the device; the same
+ * with small-integer operands against an independently computed integer product; and both launch shapes of
+ * ix_logprob_rowinv_sampled on seeded logits. workspace: caller-owned device memory, 256-byte aligned, at
+ * least ix_arch_selfcheck_workspace_bytes() (about 6 MiB); nothing is allocated. failed_checks (host memory, may be
+ * NULL) receives a mask: bit 0 seeded product, bit 1 integer product, bit 2 log-softmax shapes, bit 3 an id declined
+ * the shape. Returns IX_OK (every check passed), IX_DECLINED (a check failed: do not serve from this device), < 0
+ * (the checks could not run). Ends with a stream synchronisation: a set-up call, not a hot-path one. */
+size_t ix_arch_selfcheck_workspace_bytes(void);
+int ix_arch_selfcheck(void* workspace, size_t workspace_bytes, unsigned* failed_checks, void* stream);
+/* The same call with one bit of the reference side of every check named in `inject` (bits 0..2) flipped first: it must
+ * then report exactly those checks. No counterpart in the reference; it shows that each comparison sees a single bit. */
+int ix_arch_selfcheck_probe(void* workspace, size_t workspace_bytes, unsigned inject, unsigned* failed_checks,
+                            void* stream);
 
 /* ---- log-softmax + target gather: ops/logprobs/rowinv.py ---------------------------------- */
 

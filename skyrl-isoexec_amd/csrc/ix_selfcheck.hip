@@ -7,7 +7,7 @@
 //          (ids 1..8) stores the same bits as id 1;
 //   bit 1  small-integer operands (every partial sum exact in fp32, so the result does not depend on any order): every
 //          id stores bf16(the integer product), computed independently by a plain integer kernel;
-//   bit 2  the row-invariant log-softmax + gather gives the same bits in both of its launch shapes;
+//   bit 2  the row-invariant log-softmax + gather gives the same bits in both of its launch shapes (seeded logits);
 //   bit 3  an id declined a shape it documents as served (nothing compared for it).
 // The caller owns the scratch memory; nothing is allocated. The call ends with a stream synchronisation and a 16-byte
 // copy to the host: it is a set-up call, not a hot-path one.
@@ -28,7 +28,8 @@ __device__ __forceinline__ uint64_t ix_sc_mix(uint64_t z) {
 }
 
 // mode 0: sign * 2^e * (1 + m / 128), e in [-12, 12]: a spread of 2^24 between operands, so that a changed
-// summation order shows in the rounding of almost every partial sum. mode 1: integers in [-3, 3].
+// summation order shows in the rounding of almost every partial sum. mode 1: integers in [-3, 3]. mode 2: the same
+// form as mode 0 with e in [-3, 2] (logit-sized values, so that many columns of a row contribute to its sum).
 __global__ __launch_bounds__(256) void k_sc_fill(bf16_t* __restrict__ p, long n, uint64_t seed, int mode) {
   const long i = (long)blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
@@ -38,8 +39,13 @@ __global__ __launch_bounds__(256) void k_sc_fill(bf16_t* __restrict__ p, long n,
     const uint32_t e = 127u - 12u + (uint32_t)((h >> 1) % 25u);
     const uint32_t m = (uint32_t)(h >> 8) & 0x7fu;
     p[i] = (bf16_t)(sign | (e << 7) | m);
-  } else {
+  } else if (mode == 1) {
     p[i] = ix_f2bf((float)((int)((h >> 3) % 7u) - 3));
+  } else {
+    const uint32_t sign = (uint32_t)(h & 1u) << 15;
+    const uint32_t e = 127u - 3u + (uint32_t)((h >> 1) % 6u);
+    const uint32_t m = (uint32_t)(h >> 8) & 0x7fu;
+    p[i] = (bf16_t)(sign | (e << 7) | m);
   }
 }
 
@@ -64,6 +70,11 @@ __global__ __launch_bounds__(256) void k_sc_compare(const uint32_t* __restrict__
                                                     long words, int* __restrict__ flags, int which) {
   const long i = (long)blockIdx.x * 256 + threadIdx.x;
   if (i < words && a[i] != b[i]) flags[which] = 1;
+}
+
+// Flips the lowest bit of one 32-bit word: how ix_arch_selfcheck_probe shows that a comparison sees a single bit.
+__global__ void k_sc_flip(uint32_t* __restrict__ words, long at) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) words[at] ^= 1u;
 }
 
 __global__ void k_sc_clear(int* __restrict__ flags) {
@@ -97,6 +108,14 @@ static IxScLayout ix_sc_layout() {
 extern "C" size_t ix_arch_selfcheck_workspace_bytes(void) { return ix_sc_layout().total; }
 
 extern "C" int ix_arch_selfcheck(void* workspace, size_t workspace_bytes, unsigned* failed_checks, void* stream) {
+  return ix_arch_selfcheck_probe(workspace, workspace_bytes, 0u, failed_checks, stream);
+}
+
+// The self-check with one bit of a comparison's reference side flipped first, for every check named in `inject` (bits
+// 0..2 as in failed_checks): the call must then report exactly those checks. It is how a test (or a suspicious
+// operator) shows that the comparisons have teeth; inject = 0 is the self-check itself.
+extern "C" int ix_arch_selfcheck_probe(void* workspace, size_t workspace_bytes, unsigned inject, unsigned* failed_checks,
+                                       void* stream) {
   if (failed_checks) *failed_checks = 0;
   const IxScLayout L = ix_sc_layout();
   if (!workspace || !ix_aligned(workspace, 256)) return IX_ERR_ARG;
@@ -127,6 +146,7 @@ extern "C" int ix_arch_selfcheck(void* workspace, size_t workspace_bytes, unsign
     } else {
       hipLaunchKernelGGL(k_sc_int_product, grid(nC), dim3(256), 0, st, A, W, Cref, M, N, K);
     }
+    if (inject >> mode & 1u) hipLaunchKernelGGL(k_sc_flip, dim3(1), dim3(64), 0, st, (uint32_t*)Cref, nC / 4 + 17);
     for (int tile = mode == 0 ? 2 : 1; tile <= 8; ++tile) {
       const int rc = ix_gemm_bf16_nt(A, K, W, K, nullptr, Cgot, IX_DT_BF16, N, M, N, K, tile, nullptr, 0, stream);
       if (rc < 0) return rc;
@@ -138,15 +158,17 @@ extern "C" int ix_arch_selfcheck(void* workspace, size_t workspace_bytes, unsign
                          nC / 2, flags, mode);
     }
     if (mode == 0) {
-      // the seeded product's logits through both launch shapes of the log-softmax
+      // seeded logits (the product buffer is free again) through both launch shapes of the log-softmax
+      hipLaunchKernelGGL(k_sc_fill, grid(nC), dim3(256), 0, st, Cgot, nC, 0x4242ull, 2);
       hipLaunchKernelGGL(k_sc_targets, grid(M), dim3(256), 0, st, targets, (long)M, (long)N, 0x5555ull);
       float* outs[2] = {lp1, lp2};
       for (int shape = 1; shape <= 2; ++shape) {
-        const int rc = ix_logprob_rowinv_sampled(Cref, IX_DT_BF16, M, N, N, targets, IX_SC_G, outs[shape - 1], nullptr,
+        const int rc = ix_logprob_rowinv_sampled(Cgot, IX_DT_BF16, M, N, N, targets, IX_SC_G, outs[shape - 1], nullptr,
                                                  base + L.lp_ws, L.lp_ws_bytes, shape, nullptr, stream);
         if (rc < 0) return rc;
         if (rc != IX_OK) declined |= 1u << (8 + shape);
       }
+      if (inject >> 2 & 1u) hipLaunchKernelGGL(k_sc_flip, dim3(1), dim3(64), 0, st, (uint32_t*)lp1, (long)(M / 2));
       hipLaunchKernelGGL(k_sc_compare, grid(M), dim3(256), 0, st, (const uint32_t*)lp1, (const uint32_t*)lp2, (long)M,
                          flags, 2);
     }

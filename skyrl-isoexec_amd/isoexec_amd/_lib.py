@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_float, c_int, c_long, c_size_t, c_uint64, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_long, c_size_t, c_uint, c_uint64, c_void_p
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC_DIR = os.path.normpath(os.path.join(_PKG_DIR, "..", "csrc"))
@@ -38,6 +38,9 @@ SIGNATURES = {
     "ix_abi_version": (c_int, []),
     "ix_arch_tag": (c_char_p, []),
     "ix_prim_unary": (c_int, [c_int, P, P, c_long, P]),
+    "ix_arch_selfcheck_workspace_bytes": (c_size_t, []),
+    "ix_arch_selfcheck": (c_int, [P, c_size_t, P, P]),
+    "ix_arch_selfcheck_probe": (c_int, [P, c_size_t, c_uint, P, P]),
     "ix_logprob_workspace_bytes": (c_size_t, [c_long, c_long, c_int]),
     "ix_logprob_rowinv_sampled": (
         c_int,
@@ -105,6 +108,7 @@ SIGNATURES = {
 }
 
 _LIB = None
+_DISABLED = None   # the reason, once the device self-check has failed: the library then serves nothing in this process
 
 
 class IsoExecLibraryError(RuntimeError):
@@ -114,6 +118,8 @@ class IsoExecLibraryError(RuntimeError):
 def lib() -> ctypes.CDLL:
     """Load (once) and return the shared library; raise loudly if it is not built."""
     global _LIB
+    if _DISABLED is not None:
+        raise IsoExecLibraryError(f"[isoexec-amd] the library is switched off for this process: {_DISABLED}")
     if _LIB is not None:
         return _LIB
     if not os.path.exists(LIB_PATH):
@@ -128,6 +134,17 @@ def lib() -> ctypes.CDLL:
         fn.argtypes = argtypes
     _LIB = handle
     return handle
+
+
+def disable(reason: str) -> None:
+    """Switch the library off for the rest of the process (a failed device self-check): every later ``lib()`` raises.
+    There is no way back short of a new process, as for the reference's providers after a failed first-use check."""
+    global _DISABLED
+    _DISABLED = str(reason)
+
+
+def disabled_reason():
+    return _DISABLED
 
 
 def check(rc: int, what: str) -> int:

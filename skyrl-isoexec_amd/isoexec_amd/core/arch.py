@@ -79,3 +79,50 @@ class HardwareTarget:
 
     def assert_homogeneous(self, other_arch: str) -> None:
         assert_homogeneous(self.arch, other_arch)
+
+
+# ---- device self-check -------------------------------------------------------------------------------------------
+SELFCHECK_OBLIGATION = "domain_check:arch.selfcheck"
+SELFCHECK_BITS = ("seeded product differs between tile shapes", "integer product differs from the integer truth",
+                  "log-softmax launch shapes differ", "a tile id declined the check's shape")
+_SELFCHECK = None   # None = not run in this process, else (ok, evidence)
+
+
+def arch_selfcheck(verbose: bool = True, device=None) -> bool:
+    """Check on THIS device that no tile shape or launch form moves the bits (the reference's ``pik_arch_selfcheck``,
+    ops/collectives/pik_bootstrap.py:82-93: True on PASS; "the library's invariance guarantee does not hold if this
+    fails"). The check itself runs in the library (``ix_arch_selfcheck``) on caller-owned scratch memory. The verdict
+    is filed with the enforcement ledger at the install phase; a failure switches the library off for the rest of the
+    process, so nothing can be served from a device whose premise failed. Run once per process; later calls return
+    the first verdict."""
+    global _SELFCHECK
+    if _SELFCHECK is not None:
+        return _SELFCHECK[0]
+    import ctypes
+
+    import torch
+
+    from .. import _lib
+    from . import enforce
+
+    L = _lib.lib()
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    with torch.cuda.device(dev):
+        need = int(L.ix_arch_selfcheck_workspace_bytes())
+        ws = torch.empty(need, dtype=torch.uint8, device=dev)
+        mask = ctypes.c_uint(0)
+        rc = L.ix_arch_selfcheck(ws.data_ptr(), need, ctypes.byref(mask), _lib.current_stream(dev))
+    if rc == _lib.IX_OK:
+        ok, evidence = True, f"{ARCH}: tile ids 1-8 and both log-softmax shapes agree bit for bit"
+    elif rc == _lib.IX_DECLINED:
+        failed = [text for bit, text in enumerate(SELFCHECK_BITS) if mask.value >> bit & 1]
+        ok, evidence = False, f"{ARCH}: " + "; ".join(failed)
+    else:
+        ok, evidence = False, f"{ARCH}: the self-check could not run (code {rc})"
+    _SELFCHECK = (ok, evidence)
+    enforce.report(SELFCHECK_OBLIGATION, enforce.INSTALL, enforce.OK if ok else enforce.VIOLATION, evidence)
+    if verbose:
+        print(f"[ISOEXEC-AMD] arch self-check on {ARCH}: {'PASS' if ok else 'FAIL'} ({evidence})", flush=True)
+    if not ok:
+        _lib.disable(f"arch self-check failed: {evidence}")
+    return ok

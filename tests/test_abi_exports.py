@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_host_only_entry_points():
     h = _lib.lib()
-    assert h.ix_abi_version() == 2 and h.ix_arch_tag() == b"gfx950"
+    assert h.ix_abi_version() == 3 and h.ix_arch_tag() == b"gfx950"
     assert h.ix_moe_max_tiles(16384, 8, 128, 256) == 16384 * 8 // 256 + 128
     assert h.ix_moe_pick_bm(16384, 8, 128) == 256 and h.ix_moe_pick_bm(1, 8, 128) == 32
     assert h.ix_logprob_workspace_bytes(4, 151936, 8) == 4 * (19 + 40 + 2) * 4

@@ -54,3 +54,59 @@ def test_a_declined_logprob_kernel_is_not_ignored(monkeypatch):
     monkeypatch.setattr(hybrid, "sampled_forward", lambda *a, **k: None)
     with pytest.raises(RuntimeError, match="declined"):
         blocks.sampled_logprobs(torch.zeros(2, 4), torch.zeros(2, dtype=torch.int64))
+
+
+def test_failed_selfcheck_switches_the_library_off_and_is_a_ledger_violation(monkeypatch):
+    """The failure path of ``arch_selfcheck`` on a stand-in library (no device needed): the verdict is a violation at the
+    install phase, and every later ``lib()`` of the process raises."""
+    import ctypes
+    import sys
+    import types
+
+    import pytest
+
+    from isoexec_amd import _lib
+    from isoexec_amd.core import arch, enforce
+
+    class FakeLib:
+        def ix_arch_selfcheck_workspace_bytes(self):
+            return 1024
+
+        def ix_arch_selfcheck(self, ws, nbytes, mask, stream):
+            ctypes.cast(mask, ctypes.POINTER(ctypes.c_uint))[0] = 0b0101
+            return _lib.IX_DECLINED
+
+    class FakeTensor:
+        def data_ptr(self):
+            return 4096
+
+    class FakeCtx:
+        def __enter__(self):
+            return self
+
+        def __exit__(self, *a):
+            return False
+
+    fake_torch = types.SimpleNamespace(
+        device=lambda *a: "cuda:0", uint8="u8", empty=lambda *a, **k: FakeTensor(),
+        cuda=types.SimpleNamespace(current_device=lambda: 0, device=lambda d: FakeCtx()))
+    enforce._reset_for_tests()
+    monkeypatch.setattr(arch, "_SELFCHECK", None)
+    monkeypatch.setattr(_lib, "_DISABLED", None)
+    monkeypatch.setattr(_lib, "lib", lambda: FakeLib())
+    monkeypatch.setattr(_lib, "current_stream", lambda dev=None: 0)
+    monkeypatch.setitem(sys.modules, "torch", fake_torch)
+    assert arch.arch_selfcheck(verbose=False) is False
+    record, = enforce.ledger().by_id(arch.SELFCHECK_OBLIGATION)
+    assert (record.phase, record.result) == (enforce.INSTALL, enforce.VIOLATION)
+    assert "seeded product differs" in record.evidence and "log-softmax launch shapes differ" in record.evidence
+    assert "integer product" not in record.evidence
+    assert _lib.disabled_reason().startswith("arch self-check failed")
+    monkeypatch.undo()
+    # the real loader now refuses, until the process-wide latch is cleared again (here: by hand, for the other tests)
+    monkeypatch.setattr(_lib, "_DISABLED", "arch self-check failed: test")
+    with pytest.raises(_lib.IsoExecLibraryError, match="switched off"):
+        _lib.lib()
+    monkeypatch.undo()
+    assert _lib.disabled_reason() is None
+    enforce._reset_for_tests()
