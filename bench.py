@@ -9,8 +9,8 @@ kernels the target names, each timed in this run at its own configuration; ``cpu
 composition of the same model on a stated slice. Weights and inputs come from a host generator (seeded), so they do
 not depend on the GPU. Prints ONE JSON line.
 
-Other workloads (``--workload dense_head | gdn_decode | moe | attention | digest``) time configs[1], [2], [3] and
-parts of [4] alone with the same contract; they are for profiling one kernel family, not the headline.
+Other workloads (``--workload dense_head | gdn_decode | moe | attention | digest | decode``) time configs[1], [2], [3]
+and parts of [4] alone with the same contract; they are for profiling one kernel family, not the headline.
 """
 
 from __future__ import annotations
@@ -401,6 +401,122 @@ def north_star_kernels(w, dev, steps):
     return out
 
 
+def decode_bytes_per_step(cfg, n, context, distinct_experts):
+    """Bytes a decode step cannot avoid moving at batch ``n`` and mean context ``context``: every byte below is read
+    (or read and written) exactly once per step by the algorithm, whatever the kernels do.
+      experts   the fc1 + fc2 weights of the experts the step's tokens actually route to (``distinct_experts``: one count
+                per layer, read from the step's own routing), 3 * hidden * inter * 2 B each
+      gdn       the fp32 delta-rule state of every sequence, read and written: 2 * HV * V * K * 4 B per sequence and layer,
+                plus the convolution window (D * (W - 1) * 2 B, read and written)
+      kv        the cached keys and values of every sequence: 2 * context * HKV * D * 2 B per sequence and layer
+      dense     the projection, router and LM-head weights (read once) and the logits (written once, read once)"""
+    gdn_layers = sum(1 for i in range(cfg.layers) if not cfg.is_attention(i))
+    att_layers = cfg.layers - gdn_layers
+    H = cfg.hidden
+    experts = sum(distinct_experts) * 3 * H * cfg.expert_inter * 2
+    state = 2 * cfg.gdn_v_heads * cfg.gdn_head_dim * cfg.gdn_head_dim * 4 + 2 * cfg.gdn_qkv * (cfg.conv_width - 1) * 2
+    gdn = gdn_layers * n * state
+    kv = att_layers * n * 2 * context * cfg.kv_heads * cfg.head_dim * 2
+    gdn_proj = (cfg.gdn_qkv + cfg.gdn_z + 2 * cfg.gdn_v_heads) * H + H * cfg.gdn_z
+    att_proj = (cfg.q_heads + 2 * cfg.kv_heads) * cfg.head_dim * H + H * cfg.q_heads * cfg.head_dim
+    dense = (gdn_layers * gdn_proj + att_layers * att_proj + cfg.layers * cfg.experts * H + cfg.vocab * H) * 2
+    dense += 2 * n * cfg.vocab * 2
+    parts = {"expert_weights": experts, "gdn_state": gdn, "kv_cache": kv, "dense_weights_and_logits": dense}
+    return float(sum(parts.values())), {k: float(v) for k, v in parts.items()}
+
+
+def decode_roofline(cfg, engine, slots, tokens_step, ms_per_step):
+    """HBM roofline of one decode step: the step's own routing says how many experts' weights it has to read."""
+    import torch
+
+    log = []
+    engine.blocks.routing_log = log
+    try:
+        engine.decode(slots, tokens_step)
+    finally:
+        engine.blocks.routing_log = None
+    distinct = [int(torch.unique(ids).numel()) for ids in log]
+    context = sum(engine.context[s] for s in slots) / len(slots)
+    total, parts = decode_bytes_per_step(cfg, len(slots), context, distinct)
+    return {"bound": "hbm", "bytes_per_step": total, "bytes_by_part": parts, "distinct_experts_per_layer": distinct,
+            "mean_context": context, "ms_per_step": ms_per_step, "achieved": total / (ms_per_step * 1e-3) / 1e9,
+            "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": total / (ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBS}
+
+
+def rollout_leg(cfg, w, tokens, n, prompt, resp, graph_steps=36):
+    """The rollout side of configs[4]: prefill of ``n`` prompts (timed on its second run: the first pays for module
+    loads and allocator growth), then decode steps at batch ``n`` with the full-row logprobs the engine reports,
+    eager and replayed from a captured graph."""
+    import torch
+
+    from isoexec_amd.ops.logprobs.rowinv import full_forward, leaves
+    from isoexec_amd.runtimes.hybrid import RolloutEngine
+
+    plens = [prompt] * n
+    engine = RolloutEngine(cfg, w, max_num_seqs=n, max_len=prompt + resp)
+    slots = list(range(n))
+    prompts = tokens.view(n, -1)[:, :prompt].reshape(-1)
+    engine.prefill(slots, prompts, plens)
+    for s in slots:
+        engine.release(s)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    x = engine.prefill(slots, prompts, plens)
+    torch.cuda.synchronize()
+    t_prefill = time.perf_counter() - t0
+    dec_steps = min(resp - 1, 64)
+    nxt = tokens.view(n, -1)[:, prompt:prompt + dec_steps]
+    for sidx in range(4):
+        x = engine.decode(slots, nxt[:, sidx].contiguous())
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for sidx in range(4, dec_steps):
+        x = engine.decode(slots, nxt[:, sidx].contiguous())
+        full_forward(engine.blocks.logits(x), leaves())
+    torch.cuda.synchronize()
+    t_dec = (time.perf_counter() - t0) / (dec_steps - 4)
+    # the same steps replayed from a captured graph
+    graph = engine.capture_decode(slots)
+    more = tokens.view(n, -1)[:, prompt + dec_steps:prompt + dec_steps + 4 + graph_steps]
+    for sidx in range(4):
+        graph.step(more[:, sidx].contiguous())
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for sidx in range(4, 4 + graph_steps):
+        x = graph.step(more[:, sidx].contiguous())
+        full_forward(engine.blocks.logits(x), leaves())
+    torch.cuda.synchronize()
+    t_graph = (time.perf_counter() - t0) / graph_steps
+    roof = decode_roofline(cfg, engine, slots, more[:, 0].contiguous(), t_graph * 1e3)
+    del engine, graph
+    return {"prefill_tokens_per_s": n * prompt / t_prefill, "prefill_ms": t_prefill * 1e3,
+            "decode_ms_per_step": t_dec * 1e3, "eager_decode_tokens_per_s": n / t_dec,
+            "graph_decode_ms_per_step": t_graph * 1e3, "graph_decode_tokens_per_s": n / t_graph, "batch": n,
+            "decode_roofline": roof}
+
+
+def decode(args):
+    """The rollout leg of configs[4] alone (what the decode profiles run): ``value`` = decode tokens/s at batch
+    ``--seqs`` from the captured graph, ``roofline`` = the step against HBM."""
+    import torch
+
+    from isoexec_amd.runtimes.hybrid import HybridConfig, HybridWeights
+
+    dev = "cuda:0"
+    cfg = HybridConfig()
+    n, prompt, resp = args.seqs, args.prompt, args.response
+    w = HybridWeights.make(cfg, seed=0, device=dev, host_rng=True)
+    tokens = torch.randint(0, cfg.vocab, (n * (prompt + resp),), generator=host_gen(4)).to(dev)
+    leg = rollout_leg(cfg, w, tokens, n, prompt, resp, graph_steps=max(args.steps, 8))
+    roof = leg.pop("decode_roofline")
+    return {"metric": "decode tokens/s", "value": leg["graph_decode_tokens_per_s"], "unit": "tokens/s", "n_gpus": 1,
+            "steps": max(args.steps, 8), "warmup": 4, "ms_per_step": leg["graph_decode_ms_per_step"],
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": f"hybrid (BASELINE configs[4]) rollout: decode at batch {n} after {prompt}-token prompts, "
+                                   "full-row logprobs per step, replayed from a captured graph"},
+            "roofline": {**roof, "traffic": None}, "rollout": leg}
+
+
 def hybrid_cpu_baseline(cfg, w, tokens, seqs, prompt, resp):
     """The CPU oracle composition of the same model (same weights) scoring a slice of the same token stream: the first
     ``seqs`` sequences cut to ``prompt`` + ``resp`` tokens each, on this box's host cores."""
@@ -456,40 +572,8 @@ def hybrid(args):
     total = n * (prompt + resp)
     exp_ms = t_experts.mean_ms()
     exp_fl = 2.0 * total * cfg.topk * cfg.hidden * (2 * cfg.expert_inter) + 2.0 * total * cfg.topk * cfg.expert_inter * cfg.hidden
-    # rollout: prefill once, then timed decode steps at batch n
-    engine = RolloutEngine(cfg, w, max_num_seqs=n, max_len=prompt + resp)
-    slots = list(range(n))
-    prompts = tokens.view(n, -1)[:, :prompt].reshape(-1)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    x = engine.prefill(slots, prompts, plens)
-    torch.cuda.synchronize()
-    t_prefill = time.perf_counter() - t0
-    dec_steps = min(resp - 1, 64)
-    nxt = tokens.view(n, -1)[:, prompt:prompt + dec_steps]
-    from isoexec_amd.ops.logprobs.rowinv import full_forward, leaves
-    for sidx in range(4):
-        x = engine.decode(slots, nxt[:, sidx].contiguous())
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for sidx in range(4, dec_steps):
-        x = engine.decode(slots, nxt[:, sidx].contiguous())
-        full_forward(engine.blocks.logits(x), leaves())
-    torch.cuda.synchronize()
-    t_dec = (time.perf_counter() - t0) / (dec_steps - 4)
-    # the same steps replayed from a captured graph
-    graph = engine.capture_decode(slots)
-    more = tokens.view(n, -1)[:, prompt + dec_steps:prompt + dec_steps + 40]
-    for sidx in range(4):
-        graph.step(more[:, sidx].contiguous())
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for sidx in range(4, 40):
-        x = graph.step(more[:, sidx].contiguous())
-        full_forward(engine.blocks.logits(x), leaves())
-    torch.cuda.synchronize()
-    t_graph = (time.perf_counter() - t0) / 36
-    del engine, graph
+    leg = rollout_leg(cfg, w, tokens, n, prompt, resp)
+    t_graph = leg["graph_decode_ms_per_step"] * 1e-3
     out = {"metric": "trainer-fwd & decode tokens/s at bitwise parity; % of HBM/MFMA roofline", "value": total / dt,
            "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt * 1e3,
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
@@ -504,9 +588,7 @@ def hybrid(args):
                         "kernel": f"k_moe_fc1_glu_stream + k_moe_fc2_stream (grouped expert GEMMs, {total} tokens x top-8 per launch "
                                   f"pair, {cfg.layers} pairs per pass)", "kernel_ms": exp_ms,
                         "share_of_step": cfg.layers * exp_ms / (dt * 1e3)},
-           "rollout": {"prefill_tokens_per_s": n * prompt / t_prefill, "decode_ms_per_step": t_dec * 1e3,
-                       "eager_decode_tokens_per_s": n / t_dec, "graph_decode_ms_per_step": t_graph * 1e3,
-                       "graph_decode_tokens_per_s": n / t_graph, "batch": n}}
+           "rollout": leg}
     out["kernels"] = north_star_kernels(w, dev, max(args.steps, 10))
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = hybrid_cpu_baseline(cfg, w, tokens, args.cpu_seqs, args.cpu_prompt, args.cpu_response)
@@ -579,7 +661,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="hybrid", choices=["dense_head", "gdn_decode", "moe", "hybrid", "attention", "digest"])
+    ap.add_argument("--workload", default="hybrid", choices=["dense_head", "gdn_decode", "moe", "hybrid", "attention", "digest", "decode"])
     ap.add_argument("--seqs", type=int, default=64)
     ap.add_argument("--prompt", type=int, default=2048)
     ap.add_argument("--response", type=int, default=512)
@@ -603,7 +685,8 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(3)
-    out = {"dense_head": dense_head, "gdn_decode": gdn_decode, "moe": moe, "hybrid": hybrid, "attention": attention, "digest": digest}[args.workload](args)
+    out = {"dense_head": dense_head, "gdn_decode": gdn_decode, "moe": moe, "hybrid": hybrid, "attention": attention, "digest": digest,
+           "decode": decode}[args.workload](args)
     print(json.dumps(out))
 
 

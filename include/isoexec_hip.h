@@ -209,6 +209,18 @@ int ix_gdn_l2norm(const void* x, long x_pitch, void* y, int io_dtype, long token
 int ix_gdn_gate(const void* a, long a_pitch, const void* b, long b_pitch, const float* A_log, const float* dt_bias,
                 float* g, void* beta, int io_dtype, long tokens, long HV, int exp_dtype, void* stream);
 
+/* Everything a decode step does in front of the scan, one launch (the engine's decode of gdn_recurrent_state.py:628-869:
+ * causal_conv1d_update, the two l2norms and the gating, which the reference's fused core folds into its own kernel,
+ * gdn_ops.py:513-558): for each of N sequences (one token each) the width-4 conv of x [N, D] (pitch x_pitch,
+ * D = 2 H K + HV V) on the W - 1 inputs stored in conv_pool row rows[n], with that window slid in place; q and k heads
+ * (channels < 2 H K) l2-normalised; g = -exp(A_log) * softplus(a + dt_bias) fp32 and beta = sigmoid(b) bf16. y [N, D]
+ * bf16 contiguous, g / beta [N, HV]. Bit for bit what ix_gdn_conv + ix_gdn_l2norm + ix_gdn_gate (exp_dtype fp32) give.
+ * rows[n] <= 0: zero window read, none written. Serves bf16, W = 4, K = 128, 16-byte aligned operands; else declined. */
+int ix_gdn_decode_prep(const void* x, long x_pitch, const void* a, long a_pitch, const void* b, long b_pitch,
+                       const void* conv_weight, const void* conv_bias, const float* A_log, const float* dt_bias,
+                       void* conv_pool, const int* rows, void* y, float* g, void* beta, long N, long H, long K, long HV,
+                       long V, long W, int silu, float eps, void* stream);
+
 /* cpr_resolve_rows (gdn_cpr_rows.py:29-80; eager chain gdn_recurrent_state.py:271-284): engine slot ids of a
  * decode batch -> state-pool rows, one launch, host-free. slots int32 or int64 [n] (slots_i64). With slot2row
  * (int64 [map_n]): row = slot2row[clamp(slot, 0, map_n - 1)]; with slot2row NULL: row = slot if 0 <= slot < blocks

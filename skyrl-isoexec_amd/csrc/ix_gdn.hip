@@ -929,3 +929,135 @@ extern "C" int ix_gdn_conv(const void* x, long x_pitch, const void* weight, cons
   }
   return ix_launch_status();
 }
+
+// ---------------------------------------------------------------------------------------------
+// Everything a decode step does in front of the scan, in ONE launch (one token per sequence): the width-4 conv on the
+// row's stored window with the window slid in place, the l2norm of the q and k heads, the gating. It replaces four
+// launches (k_gdn_conv8<4, 1>, k_gdn_conv_state, k_gdn_l2norm<16>, k_gdn_gate: 4 - 8 us each at batch 64, all of it
+// launch latency) and computes every value by the same statements:
+//   conv    ix_conv8_finish on [h0, h1, h2, x] -> eight packed bf16 (k_gdn_conv8's expression)
+//   window  [h1, h2, x] back to the same pool row (k_gdn_conv_state's values; a thread owns its eight channels' window,
+//           reads it before it writes it, and nobody else touches it: no second launch is needed when the row a
+//           sequence reads is the row it writes)
+//   l2norm  on the bf16 values the conv stored, ix_tree8 + ix_lane_tree<16> (k_gdn_l2norm<16>'s expression): a head of
+//           128 channels is 16 consecutive threads
+//   gate    k_gdn_gate's two expressions, by the first HV threads of the sequence's first workgroup
+// Layout: thread = eight consecutive channels of one sequence; workgroup = 2048 channels; grid = (D / 2048, N).
+// y [N, D] receives normalised q and k (channels < 2 H K) and the conv's v behind them. A row <= 0 (a padded lane)
+// reads a zero window and writes none.
+__global__ __launch_bounds__(256) void k_gdn_decode_prep(const bf16_t* __restrict__ x, long x_pitch,
+                                                         const bf16_t* __restrict__ a, long a_pitch,
+                                                         const bf16_t* __restrict__ b, long b_pitch,
+                                                         const bf16_t* __restrict__ w, const bf16_t* __restrict__ bias,
+                                                         const float* __restrict__ A_log,
+                                                         const float* __restrict__ dt_bias, bf16_t* __restrict__ pool,
+                                                         const int* __restrict__ rows, bf16_t* __restrict__ y,
+                                                         float* __restrict__ g, bf16_t* __restrict__ beta, long D,
+                                                         int qk_channels, int HV, int silu, float eps) {
+  constexpr int W = 4;
+  const int n = blockIdx.y;
+  const int d = (blockIdx.x * 256 + threadIdx.x) * 8;
+  const int row = rows[n];
+  if (blockIdx.x == 0) {
+    for (int hv = threadIdx.x; hv < HV; hv += 256) {
+      const float sp = ix_softplus(ix_ld(a + (long)n * a_pitch + hv) + dt_bias[hv]);
+      const float neg_ea = -ix_exp(A_log[hv]);
+      g[(long)n * HV + hv] = neg_ea * sp;
+      ix_st(beta + (long)n * HV + hv, ix_sigmoid(ix_ld(b + (long)n * b_pitch + hv)));
+    }
+  }
+  // whole 16-lane groups leave together (D is a multiple of 128): the lane tree below stays inside live groups
+  if (d >= D) return;
+  float wv[8][W], bv[8];
+  {
+    const uint4* wp = reinterpret_cast<const uint4*>(w + (long)d * W);
+#pragma unroll
+    for (int c2 = 0; c2 < 4; ++c2) {
+      float t8[8];
+      ix_unpack8(wp[c2], t8);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        wv[2 * c2][j] = t8[j];
+        wv[2 * c2 + 1][j] = t8[4 + j];
+      }
+    }
+    if (bias) {
+      ix_unpack8(*reinterpret_cast<const uint4*>(bias + d), bv);
+    } else {
+#pragma unroll
+      for (int c = 0; c < 8; ++c) bv[c] = 0.0f;
+    }
+  }
+  // the window of the thread's eight channels: 8 x 3 consecutive bf16 of the pool row
+  bf16_t hist[8 * (W - 1)];
+  bf16_t* hp = pool + ((long)(row > 0 ? row : 0) * D + d) * (W - 1);
+  if (row > 0) {
+    const uint4* h4 = reinterpret_cast<const uint4*>(hp);
+#pragma unroll
+    for (int i = 0; i < 3; ++i) reinterpret_cast<uint4*>(hist)[i] = h4[i];
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8 * (W - 1); ++i) hist[i] = 0;
+  }
+  const uint4 xin = *reinterpret_cast<const uint4*>(x + (long)n * x_pitch + d);
+  float xv[W][8];
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+#pragma unroll
+    for (int j = 0; j < W - 1; ++j) xv[j][c] = ix_bf2f(hist[c * (W - 1) + j]);
+  }
+  ix_unpack8(xin, xv[W - 1]);
+  __attribute__((aligned(16))) bf16_t yv[8];
+  ix_conv8_finish<W>(xv, wv, bias != nullptr, bv, silu, yv);
+  if (row > 0) {
+    // slide the window: slot j <- slot j + 1, last slot <- this step's input
+    __attribute__((aligned(16))) bf16_t nh[8 * (W - 1)];
+    const bf16_t* xb = reinterpret_cast<const bf16_t*>(&xin);
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+#pragma unroll
+      for (int j = 0; j < W - 2; ++j) nh[c * (W - 1) + j] = hist[c * (W - 1) + j + 1];
+      nh[c * (W - 1) + W - 2] = xb[c];
+    }
+    uint4* o4 = reinterpret_cast<uint4*>(hp);
+#pragma unroll
+    for (int i = 0; i < 3; ++i) o4[i] = reinterpret_cast<const uint4*>(nh)[i];
+  }
+  bf16_t* yo = y + (long)n * D + d;
+  if (d < qk_channels) {
+    float v8[8], sq[8];
+    ix_unpack8(*reinterpret_cast<const uint4*>(yv), v8);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sq[i] = v8[i] * v8[i];
+    const float ssum = ix_lane_tree<16>(ix_tree8(sq));
+    const float rn = ix_rsqrt_ieee(ssum + eps);
+    __attribute__((aligned(16))) bf16_t out[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = ix_f2bf(v8[i] * rn);
+    *reinterpret_cast<uint4*>(yo) = *reinterpret_cast<const uint4*>(out);
+  } else {
+    *reinterpret_cast<uint4*>(yo) = *reinterpret_cast<const uint4*>(yv);
+  }
+}
+
+extern "C" int ix_gdn_decode_prep(const void* x, long x_pitch, const void* a, long a_pitch, const void* b, long b_pitch,
+                                  const void* conv_weight, const void* conv_bias, const float* A_log,
+                                  const float* dt_bias, void* conv_pool, const int* rows, void* y, float* g, void* beta,
+                                  long N, long H, long K, long HV, long V, long W, int silu, float eps, void* stream) {
+  if (!x || !a || !b || !conv_weight || !A_log || !dt_bias || !conv_pool || !rows || !y || !g || !beta) return IX_ERR_ARG;
+  if (N < 0 || H <= 0 || K <= 0 || HV <= 0 || V <= 0) return IX_ERR_ARG;
+  const long D = 2 * H * K + HV * V;
+  if (x_pitch < D || a_pitch < HV || b_pitch < HV) return IX_ERR_ARG;
+  // one head = 16 threads of eight channels; 16-byte accesses everywhere
+  if (W != 4 || K != 128 || (D % 128) || (x_pitch % 8) || N > 65535) return IX_DECLINED;
+  if (!ix_aligned(x, 16) || !ix_aligned(y, 16) || !ix_aligned(conv_weight, 16) || !ix_aligned(conv_pool, 16) ||
+      (conv_bias && !ix_aligned(conv_bias, 16)))
+    return IX_DECLINED;
+  if (N == 0) return IX_OK;
+  const long gx = (D / 8 + 255) / 256;
+  hipLaunchKernelGGL(k_gdn_decode_prep, dim3((unsigned)gx, (unsigned)N), dim3(256), 0, (hipStream_t)stream,
+                     (const bf16_t*)x, x_pitch, (const bf16_t*)a, a_pitch, (const bf16_t*)b, b_pitch,
+                     (const bf16_t*)conv_weight, (const bf16_t*)conv_bias, A_log, dt_bias, (bf16_t*)conv_pool, rows,
+                     (bf16_t*)y, g, (bf16_t*)beta, D, (int)(2 * H * K), (int)HV, silu, eps);
+  return ix_launch_status();
+}

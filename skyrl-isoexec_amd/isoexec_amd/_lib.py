@@ -74,6 +74,8 @@ SIGNATURES = {
     "ix_gdn_cpr_handoff": (c_int, [P, P, P, c_long, c_long, c_int, P]),
     "ix_gdn_resolve_rows": (c_int, [P, c_int, c_long, P, c_long, c_long, P, P, P, P, P]),
     "ix_gdn_gate": (c_int, [P, c_long, P, c_long, P, P, P, P, c_int, c_long, c_long, c_int, P]),
+    "ix_gdn_decode_prep": (c_int, [P, c_long, P, c_long, P, c_long, P, P, P, P, P, P, P, P, P, c_long, c_long, c_long, c_long,
+                                   c_long, c_long, c_int, c_float, P]),
     "ix_gdn_conv": (c_int, [P, c_long, P, P, P, P, P, P, P, c_long, c_long, c_long, c_long, c_int, P]),
     "ix_attn_varlen": (c_int, [P, c_long, P, P, c_long, P, P, P, P, c_long, c_long, c_long, c_long, c_long, c_float, P]),
     "ix_rope_inplace": (c_int, [P, c_long, P, P, c_long, P, c_long, c_long, c_long, c_long, P]),

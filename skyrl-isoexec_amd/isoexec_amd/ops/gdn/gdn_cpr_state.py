@@ -112,10 +112,7 @@ class CprGDN(RecurrentGDN):
         cu = self._decode_cu.get(N)
         if cu is None:
             cu = self._decode_cu[N] = torch.arange(N + 1, dtype=torch.int32, device=x.device)
-        y = conv_packed(x, self.conv_weight, self.conv_bias, cu_seqlens=cu, conv_state=self.conv_state,
-                        rows_in=rows32, rows_out=rows32, activation=self.activation)
-        q, k, v = self._split_qkv(y)
-        g, beta = self._gate_and_beta(a, b)
+        q, k, v, g, beta = self._decode_prepare(x, a, b, rows32, cu)
         o = gdn_recurrent_kernel(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), g.unsqueeze(0), beta.unsqueeze(0),
                                  ssm_state=self.ssm_state, state_indices=rows32, cu_seqlens=cu, time_tile=1)
         H, K, HV, V = self.num_k_heads, self.head_k_dim, self.num_v_heads, self.head_v_dim

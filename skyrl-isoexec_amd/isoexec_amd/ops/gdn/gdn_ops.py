@@ -184,6 +184,37 @@ def _gate_and_beta(a, b, A_log, dt_bias, exp_dtype):
     return g, beta
 
 
+def decode_prep(x, a, b, conv_weight, conv_bias, A_log, dt_bias, conv_state, rows, *, H, K, HV, V, activation="silu"):
+    """One launch in front of a decode step's scan: conv on the stored window (slid in place), l2norm of the q and k
+    heads, gate and beta. ``x [N, D]`` pre-conv (rows may be a column slice of a wider buffer), ``a, b [N, HV]``,
+    ``rows`` int32 ``[N]`` pool rows (<= 0: a padded lane). Returns ``(y [N, D], g [N, HV] fp32, beta [N, HV])`` with
+    the bits of ``conv_packed`` + ``gdn_l2norm`` + ``gate_and_beta_fp32``, or ``None`` when the kernel does not serve
+    the shape (the caller then takes those three)."""
+    if x.dtype is not torch.bfloat16 or a.dtype is not torch.bfloat16 or b.dtype is not torch.bfloat16:
+        return None
+    if activation not in (None, "silu", "swish") or conv_weight.shape[-1] != 4 or K != 128:
+        return None
+    _lib.require_device(x, a, b, conv_weight, conv_bias, A_log, dt_bias, conv_state, rows)
+    N, D = x.shape
+    if D != 2 * H * K + HV * V or x.stride(1) != 1 or a.stride(-1) != 1 or b.stride(-1) != 1 or a.ndim != 2 or b.ndim != 2:
+        return None
+    if A_log.dtype is not torch.float32 or dt_bias.dtype is not torch.float32 or rows.dtype is not torch.int32:
+        return None
+    y = torch.empty(N, D, dtype=x.dtype, device=x.device)
+    g = torch.empty(N, HV, dtype=torch.float32, device=x.device)
+    beta = torch.empty(N, HV, dtype=x.dtype, device=x.device)
+    wc = conv_weight if conv_weight.is_contiguous() else conv_weight.contiguous()
+    bc = None if conv_bias is None else (conv_bias if conv_bias.is_contiguous() else conv_bias.contiguous())
+    rc = _lib.check(
+        _lib.lib().ix_gdn_decode_prep(x.data_ptr(), x.stride(0), a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0),
+                                      wc.data_ptr(), _lib.ptr(bc), A_log.contiguous().data_ptr(),
+                                      dt_bias.contiguous().data_ptr(), conv_state.data_ptr(), rows.data_ptr(),
+                                      y.data_ptr(), g.data_ptr(), beta.data_ptr(), N, H, K, HV, V, 4,
+                                      int(activation is not None), L2NORM_EPS, _lib.current_stream(x.device)),
+        "ix_gdn_decode_prep")
+    return (y, g, beta) if rc == _lib.IX_OK else None
+
+
 def conv_packed(x, weight, bias, *, cu_seqlens, conv_state=None, rows_in=None, rows_out=None, activation="silu"):
     """Packed varlen conv: ``x [T, D]`` -> ``y [T, D]``; optional pool rows for history in/out."""
     _lib.require_device(x, weight, bias, cu_seqlens, conv_state, rows_in, rows_out)

@@ -26,7 +26,7 @@ from typing import Callable, Iterable, Sequence
 import numpy as np
 import torch
 
-from .gdn_ops import conv_packed, gate_and_beta_fp32, gdn_l2norm, gdn_recurrent_kernel
+from .gdn_ops import conv_packed, decode_prep, gate_and_beta_fp32, gdn_l2norm, gdn_recurrent_kernel
 
 _SLOT_MAP_ENV = "SKYRL_ISOEXEC_GDN_SLOT_MAP_SIZE"
 _CHUNKED_PREFILL_ENV = "SKYRL_ISOEXEC_GDN_CHUNKED_PREFILL"
@@ -304,6 +304,7 @@ class RecurrentGDN:
         self.num_k_heads, self.head_k_dim = num_k_heads, head_k_dim
         self.num_v_heads, self.head_v_dim = num_v_heads, head_v_dim
         self.activation = activation
+        self.fused_decode_prep = True   # False: the decode step takes conv, l2norm and gating as separate launches
         self._decode_cu: dict[int, torch.Tensor] = {}
 
     # -- table passthroughs (the reference's method names)
@@ -527,6 +528,25 @@ class RecurrentGDN:
         """Rows that start a new request (device int64, 0 = none)."""
         self.ssm_state.index_fill_(0, fresh_rows, 0.0)
 
+    def _decode_prepare(self, x, a, b, rows32, cu):
+        """A decode step in front of its scan: the convolution on the row's W-1 stored inputs (the window slides in
+        the pool itself), q and k normalised, gate and beta. One launch where the library serves the shape
+        (``decode_prep``), else the three launches it stands for: the same bits either way."""
+        fused = None
+        if self.fused_decode_prep and a.ndim == 2 and b.ndim == 2:
+            fused = decode_prep(x, a, b, self.conv_weight, self.conv_bias, self.A_log, self.dt_bias, self.conv_state, rows32,
+                                H=self.num_k_heads, K=self.head_k_dim, HV=self.num_v_heads, V=self.head_v_dim,
+                                activation=self.activation)
+        if fused is not None:
+            y, g, beta = fused
+            q, k, v = self._split_qkv_raw(y)
+            return q, k, v, g, beta
+        y = conv_packed(x, self.conv_weight, self.conv_bias, cu_seqlens=cu, conv_state=self.conv_state,
+                        rows_in=rows32, rows_out=rows32, activation=self.activation)
+        q, k, v = self._split_qkv(y)
+        g, beta = self._gate_and_beta(a, b)
+        return q, k, v, g, beta
+
     @torch.no_grad()
     def decode(self, slots: torch.Tensor, x: torch.Tensor, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
         """One decode step for N requests: ``x [N, D]`` pre-conv, ``a, b [N, HV]``. Returns
@@ -537,11 +557,7 @@ class RecurrentGDN:
         cu = self._decode_cu.get(N)
         if cu is None:
             cu = self._decode_cu[N] = torch.arange(N + 1, dtype=torch.int32, device=x.device)
-        # The convolution reads the row's W-1 stored inputs and slides the window in the pool itself.
-        y = conv_packed(x, self.conv_weight, self.conv_bias, cu_seqlens=cu, conv_state=self.conv_state,
-                        rows_in=rows32, rows_out=rows32, activation=self.activation)
-        q, k, v = self._split_qkv(y)
-        g, beta = self._gate_and_beta(a, b)
+        q, k, v, g, beta = self._decode_prepare(x, a, b, rows32, cu)
         o = gdn_recurrent_kernel(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), g.unsqueeze(0), beta.unsqueeze(0),
                                  ssm_state=self.ssm_state, state_indices=rows32, cu_seqlens=cu, time_tile=1)
         return o[0]

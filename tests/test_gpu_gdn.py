@@ -271,3 +271,41 @@ def test_native_core_varlen_equals_decode_steps():
                                    dt_bias, ssm_state=pool2, state_indices=one, cu_seqlens=None)
             for t in range(T)]
     assert same_bits(torch.cat(outs, dim=1), o) and same_bits(pool2, pool)
+
+
+def test_fused_decode_prep_equals_the_three_launches_bit_for_bit():
+    """``decode_prep`` (one launch: conv on the stored window slid in place, l2norm of q and k, gating) against
+    ``conv_packed`` + ``gdn_l2norm`` + ``gate_and_beta_fp32``, each pinned against the oracle above: outputs AND the
+    pool, over several steps, with a padded lane and operands that are column slices of one projection buffer."""
+    from isoexec_amd.ops.gdn.gdn_ops import conv_packed, decode_prep, gate_and_beta_fp32, gdn_l2norm
+
+    g = cpu_gen(41)
+    N, H, K, HV, V, W = 5, 2, 128, 4, 128, 4
+    D = 2 * H * K + HV * V
+    rows = torch.tensor([3, 0, 1, 6, 2], dtype=torch.int32, device=DEV)       # lane 1 is padded
+    cw = (0.5 * torch.randn(D, W, generator=g)).to(torch.bfloat16).to(DEV)
+    cb = (0.1 * torch.randn(D, generator=g)).to(torch.bfloat16).to(DEV)
+    A_log, dt_bias = (0.3 * torch.randn(HV, generator=g)).to(DEV), (0.3 * torch.randn(HV, generator=g)).to(DEV)
+    pool0 = torch.randn(8, D, W - 1, generator=g).to(torch.bfloat16).to(DEV)
+    cu = torch.arange(N + 1, dtype=torch.int32, device=DEV)
+    for bias in (cb, None):
+        pool_a, pool_b = pool0.clone(), pool0.clone()
+        for step in range(4):
+            proj = torch.randn(N, D + 2 * HV + 24, generator=g).to(torch.bfloat16).to(DEV)
+            proj[0, :D] *= 30.0                                                # large activations, softplus branch
+            x, b_in, a_in = proj[:, :D], proj[:, D:D + HV], proj[:, D + HV:D + 2 * HV]
+            y = conv_packed(x, cw, bias, cu_seqlens=cu, conv_state=pool_a, rows_in=rows, rows_out=rows)
+            want_qk = gdn_l2norm(y[:, :2 * H * K].unflatten(1, (2 * H, K)))
+            want_g, want_beta = gate_and_beta_fp32(a_in, b_in, A_log, dt_bias)
+            got = decode_prep(x, a_in, b_in, cw, bias, A_log, dt_bias, pool_b, rows, H=H, K=K, HV=HV, V=V)
+            assert got is not None
+            yy, gg, bb = got
+            assert same_bits(yy[:, :2 * H * K].reshape(N, 2 * H, K), want_qk), step
+            assert same_bits(yy[:, 2 * H * K:].contiguous(), y[:, 2 * H * K:].contiguous())
+            assert same_bits(gg, want_g) and same_bits(bb, want_beta)
+            assert same_bits(pool_a, pool_b)
+        assert same_bits(pool_a[0], pool0[0]) and not same_bits(pool_a[3], pool0[3])
+    # what the kernel does not serve is declined, not approximated
+    assert decode_prep(x.float(), a_in, b_in, cw, cb, A_log, dt_bias, pool_b, rows, H=H, K=K, HV=HV, V=V) is None
+    assert decode_prep(x[:, :2 * 2 * 64 + HV * V], a_in, b_in, cw[:2 * 2 * 64 + HV * V], None, A_log, dt_bias, pool_b, rows,
+                       H=2, K=64, HV=HV, V=V) is None
