@@ -281,6 +281,14 @@ int ix_moe_permute(const int* topk_idx, const float* topk_prob, long T, long E, 
                    int* offsets, int* sorted_token, float* permuted_prob, int* combine_rows, int* tile_meta,
                    long max_tiles, int* scratch, void* stream);
 
+/* fused_router_dense + fused_permute_index back to back (moe_router_o2_kernel.py:272-351) for a batch of at most one
+ * token tile (T <= 256, a decode step) and E <= 128: ix_moe_router_topk and ix_moe_permute in ONE launch, the same
+ * integers and the same weights in every output (arguments as there; no dense outputs, no scratch). Declined beyond
+ * those sizes: the caller then makes the two calls. */
+int ix_moe_route_one_tile(const float* logits, long ld, long T, long E, long k, int mode, float scaling, long BM,
+                          int* topk_idx, float* topk_prob, int* counts, int* offsets, int* sorted_token,
+                          float* permuted_prob, int* combine_rows, int* tile_meta, long max_tiles, void* stream);
+
 /* _block_map / fused_block_map (moe_fused_experts.py:156-205, moe_blockmap_kernel.py): the block map for rows that
  * are ALREADY grouped by expert (SequentialMLP.forward's tokens_per_expert, moe_batched_experts.py:301-330). counts
  * int32 or int64 [E] (counts_i64) in device memory; offsets int32 [E+1] (may be NULL) receives the exclusive scan;

@@ -159,14 +159,13 @@ __global__ __launch_bounds__(256) void k_moe_router(const float* __restrict__ lo
 // bit for bit: the winner under ix_beats does not depend on the exchange network, and the softmax denominator is
 // built as there -- s[v] + s[v + 64] per v = e mod 64, then the adjacent-pairwise tree over v (two levels inside the
 // lane, four across the row).
-__global__ __launch_bounds__(256) void k_moe_router_row16(const float* __restrict__ logits, long ld, int T, int E,
-                                                          int k, int mode, float scaling, int* __restrict__ topk_idx,
-                                                          float* __restrict__ topk_prob,
-                                                          float* __restrict__ dense_probs,
-                                                          uint8_t* __restrict__ dense_map) {
-  const int li = threadIdx.x & 15;
-  const long t = (long)blockIdx.x * 16 + (threadIdx.x >> 4);
-  if (t >= T) return;  // whole rows leave together; the lane controls below stay inside a row
+// Token t by the 16 lanes of one row of a wave (li = lane within the row). Called with whole rows only (every lane of
+// a row has the same t), so the lane controls below stay inside live lanes.
+__device__ __forceinline__ void ix_moe_route_row16(const float* __restrict__ logits, long ld, long t, int li, int E,
+                                                   int k, int mode, float scaling, int* __restrict__ topk_idx,
+                                                   float* __restrict__ topk_prob, float* __restrict__ dense_probs,
+                                                   uint8_t* __restrict__ dense_map, int* __restrict__ lds_idx,
+                                                   float* __restrict__ lds_prob) {
   float s[8];
   int eid[8];
   bool live[8];
@@ -252,6 +251,10 @@ __global__ __launch_bounds__(256) void k_moe_router_row16(const float* __restric
     if (j < k && li == j) {
       topk_idx[t * k + j] = idxs[j];
       topk_prob[t * k + j] = p[j];
+      if (lds_idx) {  // a kernel that goes on to permute keeps the winners in LDS as well
+        lds_idx[t * k + j] = idxs[j];
+        lds_prob[t * k + j] = p[j];
+      }
     }
   }
   if (dense_probs || dense_map) {
@@ -269,6 +272,17 @@ __global__ __launch_bounds__(256) void k_moe_router_row16(const float* __restric
       }
     }
   }
+}
+
+__global__ __launch_bounds__(256) void k_moe_router_row16(const float* __restrict__ logits, long ld, int T, int E,
+                                                          int k, int mode, float scaling, int* __restrict__ topk_idx,
+                                                          float* __restrict__ topk_prob,
+                                                          float* __restrict__ dense_probs,
+                                                          uint8_t* __restrict__ dense_map) {
+  const long t = (long)blockIdx.x * 16 + (threadIdx.x >> 4);
+  if (t >= T) return;  // whole rows leave together
+  ix_moe_route_row16(logits, ld, t, threadIdx.x & 15, E, k, mode, scaling, topk_idx, topk_prob, dense_probs, dense_map,
+                     nullptr, nullptr);
 }
 
 extern "C" int ix_moe_router_topk(const float* logits, long ld, long T, long E, long k, int mode, float scaling,
@@ -448,6 +462,100 @@ __global__ __launch_bounds__(256) void k_moe_scatter(const int* __restrict__ top
 // The three steps above in one launch for a batch of at most one token tile (a decode step): the membership masks
 // stay in LDS, the expert offsets come from a workgroup-wide scan (two experts per lane), and every output is the
 // integer the general path writes.
+// Body of the one-tile permutation for the first 256 threads of a workgroup (`tid`; threads past 255 of a larger
+// workgroup pass through and only meet the barriers). s_idx [T * k] holds the winners already when `idx_in_lds`; the
+// routing weights come from `prob_src` (global or LDS). Every thread of the workgroup must call it.
+__device__ __forceinline__ void ix_moe_permute_tile_body(const int* __restrict__ topk_idx, const float* prob_src, int T,
+                                                         int E, int k, int BM, int max_tiles, int* __restrict__ counts,
+                                                         int* __restrict__ offsets, int* __restrict__ sorted_token,
+                                                         float* __restrict__ permuted_prob,
+                                                         int* __restrict__ combine_rows, int* __restrict__ meta,
+                                                         int* s_idx, uint32_t* s_mask, int* s_off, int* s_rows,
+                                                         int* s_tiles, bool idx_in_lds) {
+  const int tid = threadIdx.x;
+  const bool worker = tid < 256;
+  if (worker) {
+    for (int i = tid; i < E * 8; i += 256) s_mask[i] = 0u;
+    if (!idx_in_lds)
+      for (int i = tid; i < T * k; i += 256) s_idx[i] = topk_idx[i];
+  }
+  __syncthreads();
+  if (worker && tid < T) {
+    for (int j = 0; j < k; ++j) {
+      const int e = s_idx[tid * k + j];
+      atomicOr(&s_mask[e * 8 + (tid >> 5)], 1u << (tid & 31));
+    }
+  }
+  __syncthreads();
+  // lane owns experts 2 tid and 2 tid + 1
+  int c[2] = {0, 0}, tl[2] = {0, 0};
+  if (worker) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int e = 2 * tid + h;
+      if (e < E) {
+#pragma unroll
+        for (int w = 0; w < 8; ++w) c[h] += __popc(s_mask[e * 8 + w]);
+      }
+      tl[h] = (c[h] + BM - 1) / BM;
+    }
+    s_rows[tid] = c[0] + c[1];
+    s_tiles[tid] = tl[0] + tl[1];
+  }
+  __syncthreads();
+  for (int d = 1; d < 256; d <<= 1) {  // inclusive scan over the 256 lane sums
+    const int a = (worker && tid >= d) ? s_rows[tid - d] : 0;
+    const int b = (worker && tid >= d) ? s_tiles[tid - d] : 0;
+    __syncthreads();
+    if (worker) {
+      s_rows[tid] += a;
+      s_tiles[tid] += b;
+    }
+    __syncthreads();
+  }
+  if (worker) {
+    int row0 = s_rows[tid] - (c[0] + c[1]);   // rows before expert 2 tid
+    int tile0 = s_tiles[tid] - (tl[0] + tl[1]);
+    int* tile_expert = meta + 1;
+    int* tile_row0 = tile_expert + max_tiles;
+    int* tile_nrows = tile_row0 + max_tiles;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int e = 2 * tid + h;
+      if (e < E) {
+        s_off[e] = row0;
+        counts[e] = c[h];
+        offsets[e] = row0;
+        int nt = tile0;
+        for (int r0 = 0; r0 < c[h] && nt < max_tiles; r0 += BM, ++nt) {
+          tile_expert[nt] = e;
+          tile_row0[nt] = row0 + r0;
+          tile_nrows[nt] = min(BM, c[h] - r0);
+        }
+      }
+      row0 += c[h];
+      tile0 += tl[h];
+    }
+    if (tid == 255) {
+      offsets[E] = s_rows[255];
+      meta[0] = min(s_tiles[255], max_tiles);
+    }
+  }
+  __syncthreads();
+  if (!worker || tid >= T) return;
+  for (int j = 0; j < k; ++j) {
+    const int e = s_idx[tid * k + j];
+    int local = __popc(s_mask[e * 8 + (tid >> 5)] & ((1u << (tid & 31)) - 1u));
+    for (int w = 0; w < (tid >> 5); ++w) local += __popc(s_mask[e * 8 + w]);
+    int rank = 0;
+    for (int j2 = 0; j2 < k; ++j2) rank += (s_idx[tid * k + j2] < e);
+    const int pos = s_off[e] + local;
+    sorted_token[pos] = tid;
+    permuted_prob[pos] = prob_src[(long)tid * k + j];
+    combine_rows[(long)tid * k + rank] = pos;
+  }
+}
+
 __global__ __launch_bounds__(256) void k_moe_permute_one_tile(const int* __restrict__ topk_idx,
                                                               const float* __restrict__ topk_prob, int T, int E,
                                                               int k, int BM, int max_tiles, int* __restrict__ counts,
@@ -459,70 +567,35 @@ __global__ __launch_bounds__(256) void k_moe_permute_one_tile(const int* __restr
   __shared__ uint32_t s_mask[IX_MOE_EMAX * 8];
   __shared__ int s_off[IX_MOE_EMAX + 1];
   __shared__ int s_rows[256], s_tiles[256];
-  ix_moe_build_masks(topk_idx, 0, T, E, k, s_mask, s_idx);
-  const int tid = threadIdx.x;
-  // lane owns experts 2 tid and 2 tid + 1
-  int c[2], tl[2];
-#pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const int e = 2 * tid + h;
-    c[h] = 0;
-    if (e < E) {
-#pragma unroll
-      for (int w = 0; w < 8; ++w) c[h] += __popc(s_mask[e * 8 + w]);
-    }
-    tl[h] = (c[h] + BM - 1) / BM;
+  ix_moe_permute_tile_body(topk_idx, topk_prob, T, E, k, BM, max_tiles, counts, offsets, sorted_token, permuted_prob,
+                           combine_rows, meta, s_idx, s_mask, s_off, s_rows, s_tiles, false);
+}
+
+// Router and permutation of a batch of at most one token tile (a decode step) in ONE launch: a workgroup of 1024
+// threads routes 64 tokens at a time (16 lanes each, ix_moe_route_row16: the function of k_moe_router_row16), keeps the
+// winners in LDS, and goes straight on to the one-tile permutation above. Same integers and same weights as
+// ix_moe_router_topk followed by ix_moe_permute; two launches and about ten microseconds of launch latency less.
+__global__ __launch_bounds__(1024) void k_moe_route_one_tile(const float* __restrict__ logits, long ld, int T, int E,
+                                                             int k, int mode, float scaling, int BM, int max_tiles,
+                                                             int* __restrict__ topk_idx, float* __restrict__ topk_prob,
+                                                             int* __restrict__ counts, int* __restrict__ offsets,
+                                                             int* __restrict__ sorted_token,
+                                                             float* __restrict__ permuted_prob,
+                                                             int* __restrict__ combine_rows, int* __restrict__ meta) {
+  __shared__ int s_idx[IX_MOE_TILE_T * IX_MOE_KMAX];
+  __shared__ float s_prob[IX_MOE_TILE_T * IX_MOE_KMAX];
+  __shared__ uint32_t s_mask[128 * 8];
+  __shared__ int s_off[128 + 1];
+  __shared__ int s_rows[256], s_tiles[256];
+  for (int t0 = 0; t0 < T; t0 += 64) {
+    const int t = t0 + (int)(threadIdx.x >> 4);
+    if (t < T)
+      ix_moe_route_row16(logits, ld, t, threadIdx.x & 15, E, k, mode, scaling, topk_idx, topk_prob, nullptr, nullptr,
+                         s_idx, s_prob);
   }
-  s_rows[tid] = c[0] + c[1];
-  s_tiles[tid] = tl[0] + tl[1];
-  __syncthreads();
-  for (int d = 1; d < 256; d <<= 1) {  // inclusive scan over the 256 lane sums
-    const int a = tid >= d ? s_rows[tid - d] : 0;
-    const int b = tid >= d ? s_tiles[tid - d] : 0;
-    __syncthreads();
-    s_rows[tid] += a;
-    s_tiles[tid] += b;
-    __syncthreads();
-  }
-  int row0 = s_rows[tid] - (c[0] + c[1]);   // rows before expert 2 tid
-  int tile0 = s_tiles[tid] - (tl[0] + tl[1]);
-  int* tile_expert = meta + 1;
-  int* tile_row0 = tile_expert + max_tiles;
-  int* tile_nrows = tile_row0 + max_tiles;
-#pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const int e = 2 * tid + h;
-    if (e < E) {
-      s_off[e] = row0;
-      counts[e] = c[h];
-      offsets[e] = row0;
-      int nt = tile0;
-      for (int r0 = 0; r0 < c[h] && nt < max_tiles; r0 += BM, ++nt) {
-        tile_expert[nt] = e;
-        tile_row0[nt] = row0 + r0;
-        tile_nrows[nt] = min(BM, c[h] - r0);
-      }
-    }
-    row0 += c[h];
-    tile0 += tl[h];
-  }
-  if (tid == 255) {
-    offsets[E] = s_rows[255];
-    meta[0] = min(s_tiles[255], max_tiles);
-  }
-  __syncthreads();
-  if (tid >= T) return;
-  for (int j = 0; j < k; ++j) {
-    const int e = s_idx[tid * k + j];
-    int local = __popc(s_mask[e * 8 + (tid >> 5)] & ((1u << (tid & 31)) - 1u));
-    for (int w = 0; w < (tid >> 5); ++w) local += __popc(s_mask[e * 8 + w]);
-    int rank = 0;
-    for (int j2 = 0; j2 < k; ++j2) rank += (s_idx[tid * k + j2] < e);
-    const int pos = s_off[e] + local;
-    sorted_token[pos] = tid;
-    permuted_prob[pos] = topk_prob[(long)tid * k + j];
-    combine_rows[(long)tid * k + rank] = pos;
-  }
+  // (the body's first barrier publishes s_idx and s_prob)
+  ix_moe_permute_tile_body(topk_idx, s_prob, T, E, k, BM, max_tiles, counts, offsets, sorted_token, permuted_prob,
+                           combine_rows, meta, s_idx, s_mask, s_off, s_rows, s_tiles, true);
 }
 
 // Block map for rows that are ALREADY grouped by expert (the caller holds tokens_per_expert, e.g. a dispatcher's
@@ -647,6 +720,25 @@ extern "C" int ix_moe_permute(const int* topk_idx, const float* topk_prob, long 
   if (ntiles > 0)
     hipLaunchKernelGGL(k_moe_scatter, dim3((unsigned)ntiles), dim3(256), 0, st, topk_idx, topk_prob, (int)T, (int)E,
                        (int)k, tile_base, offsets, sorted_token, permuted_prob, combine_rows);
+  return ix_launch_status();
+}
+
+// ix_moe_router_topk + ix_moe_permute for a batch of at most one token tile (T <= 256) and E <= 128, in one launch.
+extern "C" int ix_moe_route_one_tile(const float* logits, long ld, long T, long E, long k, int mode, float scaling,
+                                     long BM, int* topk_idx, float* topk_prob, int* counts, int* offsets,
+                                     int* sorted_token, float* permuted_prob, int* combine_rows, int* tile_meta,
+                                     long max_tiles, void* stream) {
+  if (!logits || !topk_idx || !topk_prob || !counts || !offsets || !sorted_token || !permuted_prob || !combine_rows ||
+      !tile_meta)
+    return IX_ERR_ARG;
+  if (T < 0 || E <= 0 || k <= 0 || BM <= 0 || ld < E) return IX_ERR_ARG;
+  if (mode != 0 && mode != 1) return IX_ERR_ARG;
+  if (k > E || k > IX_MOE_KMAX || (k & (k - 1)) != 0) return IX_DECLINED;  // as the router
+  if (T > IX_MOE_TILE_T || E > 128) return IX_DECLINED;                    // one token tile, 16 lanes per token
+  if (max_tiles < ix_moe_max_tiles(T, k, E, BM)) return IX_ERR_ARG;
+  hipLaunchKernelGGL(k_moe_route_one_tile, dim3(1), dim3(1024), 0, (hipStream_t)stream, logits, ld, (int)T, (int)E, (int)k,
+                     mode, scaling, (int)BM, (int)max_tiles, topk_idx, topk_prob, counts, offsets, sorted_token,
+                     permuted_prob, combine_rows, tile_meta);
   return ix_launch_status();
 }
 

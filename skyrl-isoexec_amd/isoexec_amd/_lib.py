@@ -87,6 +87,8 @@ SIGNATURES = {
         c_int,
         [P, P, c_long, c_long, c_long, c_long, P, P, P, P, P, P, c_long, P, P],
     ),
+    "ix_moe_route_one_tile": (c_int, [P, c_long, c_long, c_long, c_long, c_int, c_float, c_long, P, P, P, P, P, P, P, P,
+                                      c_long, P]),
     "ix_moe_block_map": (c_int, [P, c_int, c_long, c_long, c_long, P, P, c_long, P]),
     "ix_moe_permute_static_max_ints": (c_size_t, []),
     "ix_moe_permute_static_init": (c_int, []),

@@ -93,6 +93,45 @@ def permute(topk_idx: torch.Tensor, topk_prob: torch.Tensor, E: int, *, BM: int 
     return p
 
 
+def route_and_permute(logits: torch.Tensor, k: int, *, pre_softmax: bool = False, scaling_factor: float | None = None,
+                      BM: int | None = None):
+    """``router_topk`` then ``permute`` -> ``(topk_idx, topk_prob, Permutation)``. A batch of at most one token tile
+    (T <= 256, E <= 128: a decode step) takes ONE launch for both (``ix_moe_route_one_tile``); the integers and the
+    weights are the same either way."""
+    _lib.require_device(logits)
+    if logits.dtype is not torch.float32 or logits.ndim != 2:
+        raise RuntimeError("[isoexec-amd] router logits must be fp32 [T, E]")
+    T, E = logits.shape
+    if T > 256 or E > 128 or T == 0:
+        idx, prob, _, _ = router_topk(logits, k, pre_softmax=pre_softmax, scaling_factor=scaling_factor)
+        return idx, prob, permute(idx, prob, E, BM=BM)
+    lg = logits if logits.stride(1) == 1 else logits.contiguous()
+    dev = lg.device
+    L = _lib.lib()
+    p = Permutation()
+    p.T, p.E, p.k = T, E, k
+    p.BM = int(BM or L.ix_moe_pick_bm(T, k, E))
+    p.BN = 256
+    p.max_tiles = int(L.ix_moe_max_tiles(T, k, E, p.BM))
+    i32 = dict(dtype=torch.int32, device=dev)
+    idx = torch.empty(T, k, **i32)
+    prob = torch.empty(T, k, dtype=torch.float32, device=dev)
+    p.counts = torch.empty(E, **i32)
+    p.offsets = torch.empty(E + 1, **i32)
+    p.sorted_token = torch.empty(T * k, **i32)
+    p.permuted_prob = torch.empty(T * k, dtype=torch.float32, device=dev)
+    p.combine_rows = torch.empty(T, k, **i32)
+    p.tile_meta = torch.empty(1 + 3 * p.max_tiles, **i32)
+    rc = _lib.check(
+        L.ix_moe_route_one_tile(lg.data_ptr(), lg.stride(0), T, E, k, int(pre_softmax), float(scaling_factor or 0.0), p.BM,
+                                idx.data_ptr(), prob.data_ptr(), p.counts.data_ptr(), p.offsets.data_ptr(),
+                                p.sorted_token.data_ptr(), p.permuted_prob.data_ptr(), p.combine_rows.data_ptr(),
+                                p.tile_meta.data_ptr(), p.max_tiles, _lib.current_stream(dev)), "ix_moe_route_one_tile")
+    if rc != _lib.IX_OK:
+        raise RuntimeError(f"[isoexec-amd] router declined E={E} k={k} (k must be a power of two <= 16)")
+    return idx, prob, p
+
+
 def fused_permute_index(routing_map: torch.Tensor, routing_probs: torch.Tensor, topk: int):
     """``(sorted_indices [T*k] int64, permuted_probs [T*k], tokens_per_expert [E] int64)`` from the
     dense routing tensors (moe_router_o2_kernel.py:313-351)."""
@@ -152,8 +191,7 @@ def moe_ffn_forward(x: torch.Tensor, router_weight: torch.Tensor, w1: torch.Tens
         raise RuntimeError("[isoexec-amd] router GEMM declined")
     if logit_bias is not None:
         logits = logits + logit_bias  # elementwise, per token
-    idx, prob, _, _ = router_topk(logits, k, pre_softmax=pre_softmax, scaling_factor=scaling_factor)
+    idx, prob, p = route_and_permute(logits, k, pre_softmax=pre_softmax, scaling_factor=scaling_factor, BM=BM)
     if routing_out is not None:
         routing_out.append(idx)
-    p = permute(idx, prob, router_weight.shape[0], BM=BM)
     return combine(experts_forward(x, w1, w2, p), p, fp32_acc=fp32_combine)

@@ -164,3 +164,40 @@ def test_config3_shapes_small_T():
         acc += a @ w2[ej].double().T
     err = (ref[0].double().cpu() - acc).abs().max().item()
     assert err <= 0.03 * acc.abs().max().item() + 1e-3, err
+
+
+@pytest.mark.parametrize("T,E,k,mode", [(1, 128, 8, 1), (16, 128, 8, 1), (64, 128, 8, 1), (64, 128, 8, 0), (255, 128, 8, 1),
+                                         (256, 128, 8, 0), (33, 64, 4, 1), (100, 16, 2, 0), (70, 60, 4, 1)])
+def test_one_launch_route_and_permute_equals_the_two_calls(T, E, k, mode):
+    """``ix_moe_route_one_tile`` (router + permutation of a decode-size batch in one launch) against ``router_topk`` +
+    ``permute``, both pinned against the oracle in this file: every integer and every weight, on poisoned outputs, with
+    ties and a NaN in the logits and a skewed routing."""
+    from isoexec_amd.ops.moe.moe_hip import permute, route_and_permute, router_topk
+
+    g = cpu_gen(1000 * T + E)
+    logits = torch.randn(T, E, generator=g)
+    logits[:, :4] += 3.0
+    logits[0, : min(E, 12)] = 0.25          # ties: lowest index wins
+    if T > 2:
+        logits[2, 5] = float("nan")
+    lg = logits.to(DEV)
+    pre = bool(mode)
+    for scaling in (None, 2.5):
+        idx, prob, _, _ = router_topk(lg, k, pre_softmax=pre, scaling_factor=scaling)
+        want = permute(idx, prob, E)
+        gi, gp, got = route_and_permute(lg, k, pre_softmax=pre, scaling_factor=scaling)
+        assert torch.equal(gi, idx) and same_bits(gp, prob)
+        assert (got.BM, got.max_tiles) == (want.BM, want.max_tiles)
+        n = int(want.tile_meta[0])
+        assert int(got.tile_meta[0]) == n
+        for name in ("counts", "offsets", "sorted_token", "combine_rows"):
+            assert torch.equal(getattr(got, name), getattr(want, name)), name
+        assert same_bits(got.permuted_prob, want.permuted_prob)
+        mt = want.max_tiles
+        for part in range(3):
+            assert torch.equal(got.tile_meta[1 + part * mt: 1 + part * mt + n], want.tile_meta[1 + part * mt: 1 + part * mt + n])
+    # a strided logits view (the gating product's output inside a wider buffer)
+    wide = torch.zeros(T, E + 8, device=DEV)
+    wide[:, :E] = lg
+    gi2, gp2, got2 = route_and_permute(wide[:, :E], k, pre_softmax=pre, scaling_factor=2.5)
+    assert torch.equal(gi2, gi) and same_bits(gp2, gp) and torch.equal(got2.sorted_token, got.sorted_token)
