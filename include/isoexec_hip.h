@@ -122,6 +122,16 @@ int ix_gated_out_norm(const void* x, const void* gate, long gate_stride_t, const
 int ix_add_rmsnorm_gamma(const void* x, const void* residual, const void* weight, void* out, void* h_out,
                          long M, long N, float eps, int zero_centered, void* stream);
 
+/* The tail of a mixture layer in one launch: _fixed_order_combine (moe_batch_invariant.py:276-320, kernel
+ * moe_combine_kernel.py:36-76) followed by the residual add + norm (fused_add_rmsnorm.py:1-25). expert_out bf16
+ * [rows, N], combine_rows int32 [T, k] (a token's rows in ascending expert order), fp32_acc as in ix_moe_combine;
+ * h_out [T, N] = bf16(combine + residual), out [T, N] = the norm chain of ix_rmsnorm_gamma on h_out. Bit for bit
+ * ix_moe_combine then ix_add_rmsnorm_gamma, without the [T, N] round trip of the combine's output. Serves N in
+ * {512, 1024, 2048, 4096} with k in {2, 4, 8} as instantiated, 16-byte aligned operands; else declined. */
+int ix_moe_combine_add_rmsnorm(const void* expert_out, const int* combine_rows, long k, int fp32_acc, const void* residual,
+                               const void* weight, void* out, void* h_out, long T, long N, float eps, int zero_centered,
+                               void* stream);
+
 /* ---- dense matmuls: ops/moe/moe_batch_invariant.py:422-473 (aten mm/addmm/bmm override),
  *      ops/mm/mm_tiles.py:127-158, ops/mm/csrc/cublaslt_pinned.cpp:319-327 mm(x, w, out, slot) - */
 

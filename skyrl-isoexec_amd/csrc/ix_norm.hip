@@ -236,3 +236,105 @@ extern "C" int ix_add_rmsnorm_gamma(const void* x, const void* residual, const v
   return ix_norm_launch<2>((const bf16_t*)x, (const bf16_t*)weight, (bf16_t*)out, M, (int)N, eps, zero_centered,
                            (const bf16_t*)residual, 0, 1, (bf16_t*)h_out, (hipStream_t)stream);
 }
+
+// ---------------------------------------------------------------------------------------------
+// The experts' combine, the residual add and the norm in one launch (the tail of every layer: moe_batch_invariant.py:
+// 276-320 / moe_combine_kernel.py:36-76, then fused_add_rmsnorm.py:1-25): the token's k expert rows are summed in
+// ascending expert order exactly as k_moe_combine sums them (left to right; bf16 adds, or fp32 adds and one round), the
+// bf16 result takes the place of x in the residual-add form above. The [T, N] combine output is never written or read
+// back. Row layout and reduction order are those of k_rmsnorm_reg<64, 2, NG>, so the results are the two launches'.
+template <int NG, int KC>
+__global__ __launch_bounds__(256) void k_combine_add_rmsnorm_reg(const bf16_t* __restrict__ expert_out,
+                                                                 const int* __restrict__ combine_rows,
+                                                                 const bf16_t* __restrict__ residual,
+                                                                 const bf16_t* __restrict__ w, bf16_t* __restrict__ out,
+                                                                 bf16_t* __restrict__ h_out, long M, float eps,
+                                                                 int zero_centered, int fp32_acc) {
+  constexpr int LPR = 64, RPB = 256 / LPR, N = LPR * 8 * NG;
+  const int tid = threadIdx.x;
+  const int sub = tid % LPR;
+  const long row = (long)blockIdx.x * RPB + tid / LPR;
+  const bool live = row < M;
+  const long rrow = live ? row : (M - 1);
+  long src[KC];
+#pragma unroll
+  for (int r = 0; r < KC; ++r) src[r] = combine_rows[rrow * KC + r];
+  uint4 ap[NG], wp[NG];
+  const bf16_t* rr = residual + rrow * N + sub * 8;
+#pragma unroll
+  for (int c = 0; c < NG; ++c) ap[c] = *reinterpret_cast<const uint4*>(rr + c * LPR * 8);
+#pragma unroll
+  for (int c = 0; c < NG; ++c) wp[c] = *reinterpret_cast<const uint4*>(w + sub * 8 + c * LPR * 8);
+  float xv[NG][8];
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int c = 0; c < NG; ++c) {
+    uint4 ep[KC];
+#pragma unroll
+    for (int r = 0; r < KC; ++r)
+      ep[r] = *reinterpret_cast<const uint4*>(expert_out + src[r] * N + sub * 8 + c * LPR * 8);
+    float sum[8];
+    ix_unpack8(ep[0], sum);
+#pragma unroll
+    for (int r = 1; r < KC; ++r) {
+      float e[8];
+      ix_unpack8(ep[r], e);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float t = sum[i] + e[i];
+        sum[i] = fp32_acc ? t : ix_rbf(t);
+      }
+    }
+    float r8[8];
+    ix_unpack8(ap[c], r8);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float delta = ix_rbf(sum[i]);         // what k_moe_combine stores
+      xv[c][i] = ix_rbf(delta + r8[i]);           // h = bf16(x + residual)
+      const float sq = xv[c][i] * xv[c][i];
+      acc[i] = acc[i] + sq;
+    }
+  }
+  const float s = ix_lane_tree<LPR>(ix_tree8(acc));
+  const float ms = s / (float)N;
+  const float rstd = ix_rsqrt_ieee(ms + eps);
+  if (!live) return;
+  bf16_t* orow = out + row * N + sub * 8;
+#pragma unroll
+  for (int c = 0; c < NG; ++c) {
+    float wv[8], o[8];
+    ix_unpack8(wp[c], wv);
+    ix_store8_bf16(h_out + row * N + sub * 8 + c * LPR * 8, 8, true, xv[c]);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float nb = ix_rbf(xv[c][i] * rstd);
+      const float gam = zero_centered ? ix_rbf(1.0f + wv[i]) : wv[i];
+      o[i] = ix_rbf(nb * gam);
+    }
+    ix_store8_bf16(orow + c * LPR * 8, 8, true, o);
+  }
+}
+
+extern "C" int ix_moe_combine_add_rmsnorm(const void* expert_out, const int* combine_rows, long k, int fp32_acc,
+                                          const void* residual, const void* weight, void* out, void* h_out, long T,
+                                          long N, float eps, int zero_centered, void* stream) {
+  if (!expert_out || !combine_rows || !residual || !weight || !out || !h_out || T < 0 || N <= 0 || k <= 0)
+    return IX_ERR_ARG;
+  if (!ix_aligned(expert_out, 16) || !ix_aligned(residual, 16) || !ix_aligned(weight, 16) || !ix_aligned(out, 16) ||
+      !ix_aligned(h_out, 16))
+    return IX_DECLINED;
+  if (T == 0) return IX_OK;
+  const long grid = (T + 3) / 4;
+  if (grid > 0x7fffffffL) return IX_DECLINED;
+  hipStream_t st = (hipStream_t)stream;
+#define IX_CAN(NG_, KC_)                                                                                              \
+  if (N == 512 * NG_ && k == KC_) {                                                                                   \
+    hipLaunchKernelGGL((k_combine_add_rmsnorm_reg<NG_, KC_>), dim3((unsigned)grid), dim3(256), 0, st,                 \
+                       (const bf16_t*)expert_out, combine_rows, (const bf16_t*)residual, (const bf16_t*)weight,       \
+                       (bf16_t*)out, (bf16_t*)h_out, T, eps, zero_centered, fp32_acc);                                \
+    return ix_launch_status();                                                                                        \
+  }
+  IX_CAN(2, 8) IX_CAN(4, 8) IX_CAN(8, 8) IX_CAN(2, 4) IX_CAN(4, 4) IX_CAN(8, 4) IX_CAN(4, 2) IX_CAN(1, 8) IX_CAN(1, 4)
+#undef IX_CAN
+  return IX_DECLINED;
+}

@@ -54,6 +54,7 @@ SIGNATURES = {
     "ix_rmsnorm_gamma": (c_int, [P, P, P, c_long, c_long, c_float, c_int, P]),
     "ix_gated_out_norm": (c_int, [P, P, c_long, P, P, c_long, c_long, c_long, c_float, c_int, P]),
     "ix_add_rmsnorm_gamma": (c_int, [P, P, P, P, P, c_long, c_long, c_float, c_int, P]),
+    "ix_moe_combine_add_rmsnorm": (c_int, [P, P, c_long, c_int, P, P, P, P, c_long, c_long, c_float, c_int, P]),
     "ix_gemm_bf16_nt": (
         c_int,
         [P, c_long, P, c_long, P, P, c_int, c_long, c_long, c_long, c_long, c_int, P, c_long, P],

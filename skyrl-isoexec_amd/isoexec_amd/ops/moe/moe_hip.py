@@ -179,13 +179,35 @@ def combine(expert_out: torch.Tensor, p: Permutation, *, fp32_acc: bool = False)
     return out
 
 
+def combine_add_rms_norm(expert_out: torch.Tensor, p: Permutation, residual: torch.Tensor, weight: torch.Tensor,
+                         eps: float, *, fp32_acc: bool = False, zero_centered: bool = True):
+    """``combine`` followed by ``fused_add_rms_norm_gamma`` in one launch -> ``(y, h)``: ``h = bf16(combine + residual)``,
+    ``y = norm(h)``, the bits of the two calls without the round trip of the combine's output. ``None`` when the kernel
+    does not serve the width or k (the caller then makes the two calls)."""
+    H = expert_out.shape[1]
+    if (residual.shape != (p.T, H) or not residual.is_contiguous() or residual.dtype is not torch.bfloat16
+            or weight.dtype is not torch.bfloat16 or not weight.is_contiguous() or not expert_out.is_contiguous()):
+        return None
+    _lib.require_device(expert_out, residual, weight)
+    out = torch.empty(p.T, H, dtype=torch.bfloat16, device=expert_out.device)
+    h = torch.empty_like(out)
+    rc = _lib.check(
+        _lib.lib().ix_moe_combine_add_rmsnorm(expert_out.data_ptr(), p.combine_rows.data_ptr(), p.k, int(fp32_acc),
+                                              residual.data_ptr(), weight.data_ptr(), out.data_ptr(), h.data_ptr(), p.T,
+                                              H, float(eps), int(zero_centered),
+                                              _lib.current_stream(expert_out.device)), "ix_moe_combine_add_rmsnorm")
+    return (out, h) if rc == _lib.IX_OK else None
+
+
 def moe_ffn_forward(x: torch.Tensor, router_weight: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, k: int, *,
                     pre_softmax: bool = False, logit_bias: torch.Tensor | None = None,
                     scaling_factor: float | None = None, fp32_combine: bool = False, BM: int | None = None,
-                    routing_out: list | None = None):
+                    routing_out: list | None = None, add_norm: tuple | None = None):
     """Router GEMM (fp32) -> top-k -> permutation -> grouped experts -> combine. ``x [T, H]`` bf16.
     ``routing_out``: a list that receives this call's ``topk_idx [T, k]`` (for comparing composed models whose
-    discrete choices must be like for like)."""
+    discrete choices must be like for like). ``add_norm = (residual, weight, eps)``: the layer's residual add and the
+    next norm are folded into the combine's launch and ``(normed, h)`` is returned instead of the FFN output (the same
+    bits as ``fused_add_rms_norm_gamma`` on it)."""
     logits = router_gemm(x, router_weight)
     if logits is None:
         raise RuntimeError("[isoexec-amd] router GEMM declined")
@@ -194,4 +216,13 @@ def moe_ffn_forward(x: torch.Tensor, router_weight: torch.Tensor, w1: torch.Tens
     idx, prob, p = route_and_permute(logits, k, pre_softmax=pre_softmax, scaling_factor=scaling_factor, BM=BM)
     if routing_out is not None:
         routing_out.append(idx)
-    return combine(experts_forward(x, w1, w2, p), p, fp32_acc=fp32_combine)
+    expert_out = experts_forward(x, w1, w2, p)
+    if add_norm is None:
+        return combine(expert_out, p, fp32_acc=fp32_combine)
+    residual, norm_weight, eps = add_norm
+    fused = combine_add_rms_norm(expert_out, p, residual, norm_weight, eps, fp32_acc=fp32_combine)
+    if fused is not None:
+        return fused
+    from ..norms.fused_outnorm import fused_add_rms_norm_gamma
+
+    return fused_add_rms_norm_gamma(combine(expert_out, p, fp32_acc=fp32_combine), residual, norm_weight, eps)

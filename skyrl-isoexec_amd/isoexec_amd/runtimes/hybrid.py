@@ -205,10 +205,13 @@ class _Blocks:
     def attn_out(self, layer: int, o: torch.Tensor) -> torch.Tensor:
         return _linear(o.view(o.shape[0], -1), self.w.layers[layer]["o_proj"])
 
-    def moe(self, layer: int, x: torch.Tensor) -> torch.Tensor:
+    def moe(self, layer: int, x: torch.Tensor, add_norm=None):
+        """The layer's mixture of experts; with ``add_norm = (residual, weight, eps)`` also the residual add and the next
+        norm, folded into the combine's launch: returns ``(normed, h)`` then."""
         lw = self.w.layers[layer]
         return moe_ffn_forward(x, lw["router"], lw["w1"], lw["w2"], self.cfg.topk, pre_softmax=True,
-                               fp32_combine=self.cfg.moe_combine_dtype == "fp32", routing_out=self.routing_log)
+                               fp32_combine=self.cfg.moe_combine_dtype == "fp32", routing_out=self.routing_log,
+                               add_norm=add_norm)
 
     def run_layers(self, h: torch.Tensor, mixer) -> torch.Tensor:
         """The residual stream over all layers; ``mixer(layer, x)`` is the runtime's own part."""
@@ -219,10 +222,13 @@ class _Blocks:
             mixed = mixer(i, x)
             self._note("attention.varlen" if c.is_attention(i) else "gdn.core", i, mixed)
             x, h = fused_add_rms_norm_gamma(mixed, h, lw["post_norm"], c.eps)
-            delta = self.moe(i, x)
-            self._note("moe.combine", i, delta)
             nxt = self.w.layers[i + 1]["pre_norm"] if i + 1 < c.layers else self.w.final_norm
-            x, h = fused_add_rms_norm_gamma(delta, h, nxt, c.eps)
+            if self.region_log is None:
+                x, h = self.moe(i, x, add_norm=(h, nxt, c.eps))
+            else:  # the mixture's own output is a region of the comparison: keep it as a tensor
+                delta = self.moe(i, x)
+                self._note("moe.combine", i, delta)
+                x, h = fused_add_rms_norm_gamma(delta, h, nxt, c.eps)
             self._note("norms.rms", i, (x, h))
         return x  # final-normed hidden states
 

@@ -201,3 +201,25 @@ def test_one_launch_route_and_permute_equals_the_two_calls(T, E, k, mode):
     wide[:, :E] = lg
     gi2, gp2, got2 = route_and_permute(wide[:, :E], k, pre_softmax=pre, scaling_factor=2.5)
     assert torch.equal(gi2, gi) and same_bits(gp2, gp) and torch.equal(got2.sorted_token, got.sorted_token)
+
+
+@pytest.mark.parametrize("T,H,k", [(1, 2048, 8), (67, 2048, 8), (300, 1024, 4), (9, 4096, 8), (130, 512, 4), (5, 2048, 2)])
+def test_combine_add_norm_in_one_launch_equals_the_two_calls(T, H, k):
+    """``combine_add_rms_norm`` against ``combine`` + ``fused_add_rms_norm_gamma`` (both pinned against the oracle):
+    the normed rows and the new residual stream, both combine arithmetics, bit for bit."""
+    from isoexec_amd.ops.moe.moe_hip import combine, combine_add_rms_norm, permute, router_topk
+    from isoexec_amd.ops.norms.fused_outnorm import fused_add_rms_norm_gamma
+
+    g = cpu_gen(77 * T + H)
+    E = 16
+    idx, prob, _, _ = router_topk(torch.randn(T, E, generator=g).to(DEV), k)
+    p = permute(idx, prob, E)
+    eo = torch.randn(T * k, H, generator=g).to(torch.bfloat16).to(DEV)
+    res = torch.randn(T, H, generator=g).to(torch.bfloat16).to(DEV)
+    w = (0.1 * torch.randn(H, generator=g)).to(torch.bfloat16).to(DEV)
+    for fp32_acc in (False, True):
+        want_y, want_h = fused_add_rms_norm_gamma(combine(eo, p, fp32_acc=fp32_acc), res, w, 1e-6)
+        got = combine_add_rms_norm(eo, p, res, w, 1e-6, fp32_acc=fp32_acc)
+        assert got is not None
+        assert same_bits(got[0], want_y) and same_bits(got[1], want_h), fp32_acc
+    assert combine_add_rms_norm(eo[:, :384].contiguous(), p, res[:, :384].contiguous(), w[:384].contiguous(), 1e-6) is None
