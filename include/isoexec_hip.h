@@ -344,6 +344,25 @@ int ix_moe_experts_tile(const void* x, long ldx, const int* sorted_token, const 
                         const void* W1, const void* W2, const int* tile_meta, long max_tiles, long BM, long BN,
                         void* inter, void* expert_out, long T, long rows, long Hd, long F, void* stream);
 
+/* Fragment-packed copies of the experts' two matrices, and the grouped GEMMs of a decode step reading them. No
+ * counterpart in the reference (its engine reads the checkpoint layout through vLLM's fused-MoE kernel,
+ * moe_fused_experts.py:292-503); the arithmetic is ix_moe_experts' at BM = 32, bit for bit -- only where the weight
+ * bytes are fetched from, and through what, differs. A decode step is bound by streaming every touched expert's weights
+ * once. Staged in LDS a CU never has more than ~100 KiB of them in flight, and read in place a k-tile of a weight tile is
+ * 128 bytes out of each of 256 rows K * 2 bytes apart (a 4 KiB stride for K = 2048: about 4.6 TB/s on this memory system,
+ * against 6.3 TB/s for the same bytes laid out contiguously). Packed, every load instruction of the decode kernels is
+ * 1 KiB of contiguous memory, taken straight into the registers the matrix instruction reads, four k-tiles ahead.
+ * W1f / W2f have the sizes of W1 [E, 2F, Hd] / W2 [E, Hd, F]; 16-byte chunk layouts (chunk = W[row][64 kt + 32 (lane / 32)
+ * + 8 s .. + 7], r = lane % 32):
+ *   W1f [E][F / 128][wave 4][Hd / 64][b 2][s 4][lane 64]   row = b F + 128 nt + 32 wave + r   (b: gate, up)
+ *   W2f [E][Hd / 256][wave 4][F / 64][b 2][s 4][lane 64]   row = 256 nt + 64 wave + 32 b + r
+ * Serves Hd % 256 == 0, F % 128 == 0 with Hd / 64 and F / 64 in {8, 12, 16, 24, 32, 48, 64}; else declined. Pack once per
+ * weight version (one pass over each matrix), not per step. ix_moe_experts_decode takes a block map of BM = 32. */
+int ix_moe_pack_decode(const void* W1, const void* W2, void* W1f, void* W2f, long E, long Hd, long F, void* stream);
+int ix_moe_experts_decode(const void* x, long ldx, const int* sorted_token, const float* permuted_prob, const void* W1f,
+                          const void* W2f, const int* tile_meta, long max_tiles, void* inter, void* expert_out, long T,
+                          long rows, long Hd, long F, void* stream);
+
 /* _fixed_order_combine / _combine_topk_kernel (moe_batch_invariant.py:276-320,
  * moe_combine_kernel.py:36-76): out bf16 [T, Hd] = the token's k rows of expert_out summed in
  * ascending expert order; fp32_acc 0 = bf16 adds (a round per add), 1 = fp32 sum, one round. */

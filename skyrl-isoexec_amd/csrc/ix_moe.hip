@@ -1424,6 +1424,227 @@ extern "C" int ix_moe_experts(const void* x, long ldx, const int* sorted_token, 
 }
 
 // ---------------------------------------------------------------------------------------------
+// The grouped GEMMs of a decode step: weights streamed through registers.
+//
+// At decode sizes an expert has a handful of rows, the matrix pipes idle and the step is the time memory needs to
+// deliver every touched expert's weights once. The ring kernels above stage weights in LDS, so a CU never has more
+// than its 160 KiB in flight (one workgroup, ~100 KiB of weight bytes): about 5.1 TB/s. Here no LDS is used at all:
+//   * weights are stored FRAGMENT-PACKED (ix_moe_pack_decode): per (expert, column tile, wave, k-tile) the 8 KiB a wave's
+//     eight matrix instructions of that k-tile take as their A operands, in (block, step, lane) order, so that a load
+//     instruction is 1 KiB of contiguous memory and a wave walks one contiguous stream;
+//   * a lane keeps the fragments of the next D k-tiles in registers (D x 8 loads of 16 bytes in flight per lane, two
+//     workgroups per CU: up to 256 KiB of weight bytes in flight per CU);
+//   * activations (at most 32 token rows per tile, typically four live ones) come straight from memory as B operands,
+//     a lane loading the 16 bytes of its own token, as far ahead as the weights; a dead token's lanes load a live row
+//     and multiply zeros instead. No barrier, no shared state: the four waves of a workgroup only share the tile.
+// Arithmetic is that of every other tile shape: v_mfma_f32_32x32x16_bf16, weights the A operand, K in tiles of 64, step
+// s consuming k = 8 s .. 8 s + 7 (lane group 0) and 32 + 8 s .. (lane group 1), one fp32 accumulator per element, the
+// epilogues of k_moe_fc1_glu / k_moe_fc2 statement for statement.
+// Packed layouts (16-byte chunk index; r = lane % 32, g = lane / 32; chunk = W[row][64 kt + 32 g + 8 s .. + 7]):
+//   W1f [E][F / 128][wave 4][Hd / 64][b 2][s 4][lane 64]   row = b F + 128 nt + 32 wave + r      (b: gate, up)
+//   W2f [E][Hd / 256][wave 4][F / 64][b 2][s 4][lane 64]   row = 256 nt + 64 wave + 32 b + r
+#define IX_DEC_D 4  // k-tiles of weight fragments a lane holds ahead of the matrix instructions
+
+__global__ __launch_bounds__(256) void k_moe_pack_frag(const bf16_t* __restrict__ W, bf16_t* __restrict__ Wf,
+                                                       int rows_per_expert, int K, int nb, int is_fc1, long chunks) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= chunks) return;
+  const int KT = K / 64;
+  const int lane = (int)(i & 63), st = (int)((i >> 6) & 3), b = (int)((i >> 8) & 1);
+  long rest = i >> 9;
+  const int kt = (int)(rest % KT);
+  rest /= KT;
+  const int w = (int)(rest & 3);
+  rest >>= 2;
+  const int nt = (int)(rest % nb);
+  const long e = rest / nb;
+  const int r = lane & 31, g = lane >> 5;
+  const int row = is_fc1 ? b * (rows_per_expert / 2) + 128 * nt + 32 * w + r : 256 * nt + 64 * w + 32 * b + r;
+  const uint4 v = *reinterpret_cast<const uint4*>(W + (e * rows_per_expert + row) * (long)K + 64 * kt + 32 * g + 8 * st);
+  *reinterpret_cast<uint4*>(Wf + i * 8) = v;
+}
+
+template <int D>
+struct IxDecStream {
+  const uint4* wp;   // this lane's first chunk of the wave's stream: k-tile kt, chunk c at wp[kt * 512 + c * 64]
+  const bf16_t* xp;  // this lane's token row + 32 g (a dead token's lanes point at a live row and discard what they load)
+  bool live;
+  uint4 wreg[D][8];
+  uint4 xreg[D][4];
+  __device__ __forceinline__ void load_w(uint4 (&dst)[8], int kt) {
+#pragma unroll
+    for (int c = 0; c < 8; ++c) dst[c] = wp[(long)kt * 512 + c * 64];
+  }
+  __device__ __forceinline__ void load_x(uint4 (&dst)[4], int kt) {
+#pragma unroll
+    for (int st = 0; st < 4; ++st) dst[st] = *reinterpret_cast<const uint4*>(xp + 64 * kt + 8 * st);
+  }
+  template <int d>
+  __device__ __forceinline__ void multiply(const uint4 (&xc)[4], ix_f32x16& a0, ix_f32x16& a1) {
+#pragma unroll
+    for (int st = 0; st < 4; ++st) {
+      uint4 xv = xc[st];
+      if (!live) xv = make_uint4(0u, 0u, 0u, 0u);  // a select, not a branch
+      const ix_bf16x8 xf = *reinterpret_cast<const ix_bf16x8*>(&xv);
+      a0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const ix_bf16x8*>(&wreg[d][st]), xf, a0, 0, 0, 0);
+      a1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const ix_bf16x8*>(&wreg[d][4 + st]), xf, a1, 0, 0, 0);
+    }
+  }
+  // The whole product of a wave: two 32 x 32 blocks (weight chunks 0..3 -> a0, 4..7 -> a1) over KT_ k-tiles. KT_ is a
+  // compile-time constant and the walk is straight-line code: with a loop (or any branch) the compiler's wait
+  // bookkeeping falls back to "wait for every load" at the join, which would drain the D k-tiles in flight at every
+  // step; in straight-line code it waits for exactly the loads a matrix instruction reads.
+  template <int KT_>
+  __device__ __forceinline__ void run(ix_f32x16& a0, ix_f32x16& a1) {
+    static_assert(KT_ >= D, "the ring is filled before the first multiply");
+    // sched_barrier(0): the compiler's scheduler may not move a load across it -- left alone it sinks every load down
+    // to its first use (fewest live registers), which is a ring of depth zero. Loads retire in order, so the
+    // activation fragments of a k-tile are requested together with its weight fragments, D k-tiles ahead: a wait for
+    // k-tile kt then leaves the (D - 1) x 12 younger loads in flight.
+    ix_static_for<0, D>([&](auto dc) {
+      load_x(xreg[decltype(dc)::value], decltype(dc)::value);
+      load_w(wreg[decltype(dc)::value], decltype(dc)::value);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+    ix_static_for<0, KT_>([&](auto kc) {
+      constexpr int kt = decltype(kc)::value, d = kt % D;
+      multiply<d>(xreg[d], a0, a1);
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (kt + D < KT_) {
+        load_x(xreg[d], kt + D);
+        load_w(wreg[d], kt + D);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  }
+};
+
+template <int D, int KT>
+__global__ __launch_bounds__(256, 2) void k_moe_fc1_dec(const bf16_t* __restrict__ x, long ldx,
+                                                        const int* __restrict__ sorted_token,
+                                                        const float* __restrict__ permuted_prob,
+                                                        const bf16_t* __restrict__ W1f, const int* __restrict__ meta,
+                                                        int max_tiles, bf16_t* __restrict__ inter, int Hd, int F,
+                                                        int nb_n) {
+  int mt, nt;
+  if (!ix_moe_tile_of_block(blockIdx.x, meta[0], nb_n, &mt, &nt)) return;
+  const long e = meta[1 + mt];
+  const long row0 = meta[1 + max_tiles + mt];
+  const int nrows = meta[1 + 2 * max_tiles + mt];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int r = lane & 31, g = lane >> 5;
+  const bool live = r < nrows;
+  IxDecStream<D> st;
+  st.wp = reinterpret_cast<const uint4*>(W1f) + (((e * nb_n + nt) * 4 + w) * (long)KT) * 512 + lane;
+  st.live = live;
+  st.xp = x + (long)sorted_token[row0 + (live ? r : 0)] * ldx + 32 * g;  // a tile has at least one row
+  ix_f32x16 ag, au;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) ag[i] = au[i] = 0.0f;
+  st.template run<KT>(ag, au);
+  if (!live) return;
+  const long m = row0 + r;
+  const float prob = permuted_prob[m];
+  const int c0 = nt * 128 + w * 32;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int col = c0 + ix_acc_row(q * 4, lane);
+    const uint32_t lo = IxMoeFc1StreamJob::chain2(ag[q * 4], ag[q * 4 + 1], au[q * 4], au[q * 4 + 1], prob);
+    const uint32_t hi = IxMoeFc1StreamJob::chain2(ag[q * 4 + 2], ag[q * 4 + 3], au[q * 4 + 2], au[q * 4 + 3], prob);
+    *reinterpret_cast<uint2*>(inter + m * F + col) = make_uint2(lo, hi);  // col % 4 == 0, F % 8 == 0, inter 16-byte aligned
+  }
+}
+
+template <int D, int KT>
+__global__ __launch_bounds__(256, 2) void k_moe_fc2_dec(const bf16_t* __restrict__ inter, const bf16_t* __restrict__ W2f,
+                                                        const int* __restrict__ meta, int max_tiles,
+                                                        bf16_t* __restrict__ out, int Hd, int F, int nb_n) {
+  int mt, nt;
+  if (!ix_moe_tile_of_block(blockIdx.x, meta[0], nb_n, &mt, &nt)) return;
+  const long e = meta[1 + mt];
+  const long row0 = meta[1 + max_tiles + mt];
+  const int nrows = meta[1 + 2 * max_tiles + mt];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int r = lane & 31, g = lane >> 5;
+  const bool live = r < nrows;
+  IxDecStream<D> st;
+  st.wp = reinterpret_cast<const uint4*>(W2f) + (((e * nb_n + nt) * 4 + w) * (long)KT) * 512 + lane;
+  st.live = live;
+  st.xp = inter + (row0 + (live ? r : 0)) * (long)F + 32 * g;  // a tile has at least one row
+  ix_f32x16 a0, a1;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) a0[i] = a1[i] = 0.0f;
+  st.template run<KT>(a0, a1);
+  if (!live) return;
+  const long m = row0 + r;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const long n = (long)nt * 256 + w * 64 + ix_acc_row(q * 4, lane);
+    ix_store4_bf16(out + m * Hd + n, 4, true, a0[q * 4], a0[q * 4 + 1], a0[q * 4 + 2], a0[q * 4 + 3]);
+    ix_store4_bf16(out + m * Hd + n + 32, 4, true, a1[q * 4], a1[q * 4 + 1], a1[q * 4 + 2], a1[q * 4 + 3]);
+  }
+}
+
+// The k-tile counts the straight-line kernels are instantiated for (K = 64 KT).
+#define IX_DEC_KTS(M) M(8) M(12) M(16) M(24) M(32) M(48) M(64)
+static bool ix_moe_decode_kt_served(long kt) {
+#define IX_DEC_IS(KT_) if (kt == KT_) return true;
+  IX_DEC_KTS(IX_DEC_IS)
+#undef IX_DEC_IS
+  return false;
+}
+static bool ix_moe_decode_serves(long Hd, long F) {
+  return Hd % 256 == 0 && F % 128 == 0 && ix_moe_decode_kt_served(Hd / 64) && ix_moe_decode_kt_served(F / 64);
+}
+
+// Fragment-packed copies of both expert matrices for the decode kernels (each the size of its source).
+extern "C" int ix_moe_pack_decode(const void* W1, const void* W2, void* W1f, void* W2f, long E, long Hd, long F,
+                                  void* stream) {
+  if (!W1 || !W2 || !W1f || !W2f || E <= 0 || Hd <= 0 || F <= 0) return IX_ERR_ARG;
+  if (!ix_moe_decode_serves(Hd, F) || !ix_aligned(W1, 16) || !ix_aligned(W2, 16) || !ix_aligned(W1f, 16) ||
+      !ix_aligned(W2f, 16))
+    return IX_DECLINED;
+  const long c1 = E * 2 * F * Hd / 8, c2 = E * Hd * F / 8;
+  if ((c1 + 255) / 256 > 0x7fffffffL) return IX_DECLINED;
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(k_moe_pack_frag, dim3((unsigned)((c1 + 255) / 256)), dim3(256), 0, st, (const bf16_t*)W1, (bf16_t*)W1f,
+                     (int)(2 * F), (int)Hd, (int)(F / 128), 1, c1);
+  hipLaunchKernelGGL(k_moe_pack_frag, dim3((unsigned)((c2 + 255) / 256)), dim3(256), 0, st, (const bf16_t*)W2, (bf16_t*)W2f,
+                     (int)Hd, (int)F, (int)(Hd / 256), 0, c2);
+  return ix_launch_status();
+}
+
+// ix_moe_experts for a block map of 32-row tiles (BM = 32), reading the fragment-packed matrices.
+extern "C" int ix_moe_experts_decode(const void* x, long ldx, const int* sorted_token, const float* permuted_prob,
+                                     const void* W1f, const void* W2f, const int* tile_meta, long max_tiles, void* inter,
+                                     void* expert_out, long T, long rows, long Hd, long F, void* stream) {
+  if (!x || !sorted_token || !permuted_prob || !W1f || !W2f || !tile_meta || !inter || !expert_out) return IX_ERR_ARG;
+  if (T < 0 || rows < 0 || Hd <= 0 || F <= 0 || max_tiles < 0 || ldx < Hd) return IX_ERR_ARG;
+  if (!ix_moe_decode_serves(Hd, F) || (ldx % 8) || !ix_aligned(x, 16) || !ix_aligned(W1f, 16) || !ix_aligned(W2f, 16) ||
+      !ix_aligned(inter, 16) || !ix_aligned(expert_out, 16))
+    return IX_DECLINED;
+  if (rows == 0 || max_tiles == 0) return IX_OK;
+  const long nb1 = F / 128, nb2 = Hd / 256;
+  if (max_tiles * nb1 > 0x7fffffffL || max_tiles * nb2 > 0x7fffffffL) return IX_DECLINED;
+  hipStream_t st = (hipStream_t)stream;
+#define IX_DEC_FC1(KT_)                                                                                               \
+  if (Hd / 64 == KT_)                                                                                                 \
+    hipLaunchKernelGGL((k_moe_fc1_dec<IX_DEC_D, KT_>), dim3((unsigned)(8 * ((max_tiles * nb1 + 7) / 8))), dim3(256), 0, st, \
+                       (const bf16_t*)x, ldx, sorted_token, permuted_prob, (const bf16_t*)W1f, tile_meta, (int)max_tiles, \
+                       (bf16_t*)inter, (int)Hd, (int)F, (int)nb1);
+#define IX_DEC_FC2(KT_)                                                                                               \
+  if (F / 64 == KT_)                                                                                                  \
+    hipLaunchKernelGGL((k_moe_fc2_dec<IX_DEC_D, KT_>), dim3((unsigned)(8 * ((max_tiles * nb2 + 7) / 8))), dim3(256), 0, st, \
+                       (const bf16_t*)inter, (const bf16_t*)W2f, tile_meta, (int)max_tiles, (bf16_t*)expert_out, (int)Hd, \
+                       (int)F, (int)nb2);
+  IX_DEC_KTS(IX_DEC_FC1)
+  IX_DEC_KTS(IX_DEC_FC2)
+#undef IX_DEC_FC1
+#undef IX_DEC_FC2
+  return ix_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
 // KC > 0: k known at compile time -- the k row numbers and the k rows are requested before the first add, so a thread has
 // k loads in flight instead of one (the sum is the same left-to-right sum). KC = 0: any k.
 template <int KC>

@@ -105,6 +105,11 @@ SIGNATURES = {
         c_int,
         [P, c_long, P, P, P, P, P, c_long, c_long, c_long, P, P, c_long, c_long, c_long, c_long, P],
     ),
+    "ix_moe_pack_decode": (c_int, [P, P, P, P, c_long, c_long, c_long, P]),
+    "ix_moe_experts_decode": (
+        c_int,
+        [P, c_long, P, P, P, P, P, c_long, P, P, c_long, c_long, c_long, c_long, P],
+    ),
     "ix_moe_combine": (c_int, [P, P, P, c_long, c_long, c_long, c_int, P]),
     "ix_moe_combine_weighted": (c_int, [P, c_int, P, c_int, P, P, c_int, c_long, c_long, c_long, P]),
     "ix_digest_sums": (c_int, [P, c_int, c_long, c_uint64, P, c_int, P, c_size_t, P, P]),

@@ -142,10 +142,31 @@ def fused_permute_index(routing_map: torch.Tensor, routing_probs: torch.Tensor, 
     return p.sorted_token.long(), p.permuted_prob, p.counts.long()
 
 
-def experts_forward(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, p: Permutation, *, return_inter: bool = False):
+def pack_decode(w1: torch.Tensor, w2: torch.Tensor):
+    """Fragment-packed copies ``(w1f, w2f)`` of ``w1 [E, 2F, H]`` and ``w2 [E, H, F]`` for the decode-size expert kernels
+    (``ix_moe_pack_decode``): the same values, laid out in the order the kernels' matrix instructions take them, so that a
+    decode step streams them as contiguous memory. ``None`` when the kernels do not serve the shape. Make them once per
+    weight version and hand them to ``experts_forward`` / ``moe_ffn_forward`` as ``packed``."""
+    _lib.require_device(w1, w2)
+    if w1.dtype is not torch.bfloat16 or w2.dtype is not torch.bfloat16 or w1.ndim != 3 or w2.ndim != 3:
+        return None
+    if not w1.is_contiguous() or not w2.is_contiguous():
+        return None
+    E, F2, H = w1.shape
+    if w2.shape != (E, H, F2 // 2):
+        raise RuntimeError(f"[isoexec-amd] expert matrices disagree: w1 {tuple(w1.shape)}, w2 {tuple(w2.shape)}")
+    w1f, w2f = torch.empty_like(w1), torch.empty_like(w2)
+    rc = _lib.check(_lib.lib().ix_moe_pack_decode(w1.data_ptr(), w2.data_ptr(), w1f.data_ptr(), w2f.data_ptr(), E, H, F2 // 2,
+                                                  _lib.current_stream(w1.device)), "ix_moe_pack_decode")
+    return (w1f, w2f) if rc == _lib.IX_OK else None
+
+
+def experts_forward(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, p: Permutation, *, return_inter: bool = False,
+                    packed: tuple | None = None):
     """Grouped fc1 + SwiGLU + prob epilogue + fc2 over the permuted rows. ``x [T, H]`` bf16,
     ``w1 [E, 2F, H]``, ``w2 [E, H, F]``. Returns ``expert_out [T*k, H]`` in permuted order; with ``return_inter`` also
-    the activation that enters fc2, ``inter [T*k, F]`` = bf16(bf16(bf16(silu(gate)) * up) * prob)."""
+    the activation that enters fc2, ``inter [T*k, F]`` = bf16(bf16(bf16(silu(gate)) * up) * prob). ``packed``
+    (``pack_decode(w1, w2)``): read by the decode-size tile (BM = 32) instead of ``w1`` / ``w2``; same bits."""
     _lib.require_device(x, w1, w2)
     if x.dtype is not torch.bfloat16 or w1.dtype is not torch.bfloat16 or w2.dtype is not torch.bfloat16:
         raise RuntimeError("[isoexec-amd] experts serve bf16 only")
@@ -157,6 +178,17 @@ def experts_forward(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, p: Perm
     inter = torch.empty(rows, F, dtype=torch.bfloat16, device=dev)
     out = torch.empty(rows, H, dtype=torch.bfloat16, device=dev)
     xc = x if x.stride(1) == 1 else x.contiguous()
+    if packed is not None and p.BM == 32 and p.BN == 256:
+        w1f, w2f = packed
+        if w1f.shape != w1.shape or w2f.shape != w2.shape or w1f.dtype is not torch.bfloat16 or w2f.dtype is not torch.bfloat16:
+            raise RuntimeError("[isoexec-amd] packed must come from pack_decode(w1, w2)")
+        rc = _lib.check(
+            _lib.lib().ix_moe_experts_decode(xc.data_ptr(), xc.stride(0), p.sorted_token.data_ptr(),
+                                             p.permuted_prob.data_ptr(), w1f.data_ptr(), w2f.data_ptr(),
+                                             p.tile_meta.data_ptr(), p.max_tiles, inter.data_ptr(), out.data_ptr(), T, rows,
+                                             H, F, _lib.current_stream(dev)), "ix_moe_experts_decode")
+        if rc == _lib.IX_OK:
+            return (out, inter) if return_inter else out
     rc = _lib.check(
         _lib.lib().ix_moe_experts_tile(xc.data_ptr(), xc.stride(0), p.sorted_token.data_ptr(),
                                        p.permuted_prob.data_ptr(), w1.contiguous().data_ptr(),
@@ -202,7 +234,8 @@ def combine_add_rms_norm(expert_out: torch.Tensor, p: Permutation, residual: tor
 def moe_ffn_forward(x: torch.Tensor, router_weight: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, k: int, *,
                     pre_softmax: bool = False, logit_bias: torch.Tensor | None = None,
                     scaling_factor: float | None = None, fp32_combine: bool = False, BM: int | None = None,
-                    routing_out: list | None = None, add_norm: tuple | None = None):
+                    routing_out: list | None = None, add_norm: tuple | None = None,
+                    packed: tuple | None = None):
     """Router GEMM (fp32) -> top-k -> permutation -> grouped experts -> combine. ``x [T, H]`` bf16.
     ``routing_out``: a list that receives this call's ``topk_idx [T, k]`` (for comparing composed models whose
     discrete choices must be like for like). ``add_norm = (residual, weight, eps)``: the layer's residual add and the
@@ -216,7 +249,7 @@ def moe_ffn_forward(x: torch.Tensor, router_weight: torch.Tensor, w1: torch.Tens
     idx, prob, p = route_and_permute(logits, k, pre_softmax=pre_softmax, scaling_factor=scaling_factor, BM=BM)
     if routing_out is not None:
         routing_out.append(idx)
-    expert_out = experts_forward(x, w1, w2, p)
+    expert_out = experts_forward(x, w1, w2, p, packed=packed)
     if add_norm is None:
         return combine(expert_out, p, fp32_acc=fp32_combine)
     residual, norm_weight, eps = add_norm

@@ -167,6 +167,21 @@ class _Blocks:
         self.region_log = None
         # a list, or None: when set, every mixture call appends its top-k expert ids [T, k] (layer order)
         self.routing_log = None
+        # layer -> fragment-packed copies of the experts' matrices (pack_expert_weights): read by decode-size batches only
+        self.packed_experts = {}
+
+    def pack_expert_weights(self) -> int:
+        """Make the packed copies of the experts' matrices that decode-size batches stream (one pass over each matrix; a
+        second copy of them in memory). To be called again after a weight sync. Returns the bytes they take."""
+        from ..ops.moe.moe_hip import pack_decode
+
+        total = 0
+        for i, lw in enumerate(self.w.layers):
+            packed = pack_decode(lw["w1"], lw["w2"])
+            if packed is not None:
+                self.packed_experts[i] = packed
+                total += sum(t.numel() * t.element_size() for t in packed)
+        return total
 
     def _note(self, region: str, layer, out) -> None:
         if self.region_log is not None:
@@ -211,7 +226,7 @@ class _Blocks:
         lw = self.w.layers[layer]
         return moe_ffn_forward(x, lw["router"], lw["w1"], lw["w2"], self.cfg.topk, pre_softmax=True,
                                fp32_combine=self.cfg.moe_combine_dtype == "fp32", routing_out=self.routing_log,
-                               add_norm=add_norm)
+                               add_norm=add_norm, packed=self.packed_experts.get(layer))
 
     def run_layers(self, h: torch.Tensor, mixer) -> torch.Tensor:
         """The residual stream over all layers; ``mixer(layer, x)`` is the runtime's own part."""
@@ -340,11 +355,15 @@ class TrainerModel:
 class RolloutEngine:
     """Prefill, then one token per step per sequence, out of per-layer state."""
 
-    def __init__(self, cfg: HybridConfig, weights: HybridWeights, max_num_seqs: int, max_len: int):
+    def __init__(self, cfg: HybridConfig, weights: HybridWeights, max_num_seqs: int, max_len: int,
+                 pack_expert_weights: bool = True):
         if max_len > cfg.max_positions:
             raise ValueError(f"[isoexec-amd] engine max_len = {max_len} exceeds max_positions = {cfg.max_positions} "
                              "(the rotary tables hold that many positions)")
         self.cfg, self.blocks = cfg, _Blocks(cfg, weights)
+        if pack_expert_weights:
+            # the engine's decode steps stream every touched expert's weights: from a contiguous packed copy
+            self.blocks.pack_expert_weights()
         dev = weights.embed.device
         self.max_len = max_len
         self.gdn, self.kv = {}, {}

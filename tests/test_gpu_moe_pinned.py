@@ -307,3 +307,37 @@ def test_operator_override_door():
     assert not mm_hip.mm_override_installed()
     served = dict(mm_hip.stats())
     assert same_bits(Fn.linear(x, w), stock) and mm_hip.stats() == served          # the stock kernel is back
+
+
+@pytest.mark.parametrize("T,H,E,F,k", [(64, 2048, 128, 768, 8), (1, 2048, 128, 768, 8), (33, 512, 16, 1024, 4), (256, 1024, 8, 512, 2),
+                                       (200, 768, 4, 1536, 2)])
+def test_decode_kernels_read_fragment_packed_matrices_with_the_same_bits(T, H, E, F, k):
+    """``pack_decode`` + ``ix_moe_experts_decode`` (weights streamed through registers from fragment-packed copies) against
+    the 32-row ring tile reading the matrices in place: the packed copies hold exactly the values of the layout formula
+    (checked on the host), and both grouped GEMMs give the same bits from them -- ragged tiles, tiles of 32 full rows,
+    dead token lanes."""
+    from isoexec_amd.ops.mm.mm_hip import router_gemm
+    from isoexec_amd.ops.moe.moe_hip import experts_forward, pack_decode, permute, router_topk
+
+    x, wr, w1, w2 = make(T, H, E, F, seed=50 + T)
+    packed = pack_decode(w1, w2)
+    assert packed is not None
+    w1f, w2f = packed
+    assert w1f.shape == w1.shape and w2f.shape == w2.shape
+    # W1f [E][F/128][wave 4][H/64][b 2][s 4][g 2][r 32][8]: row b F + 128 nt + 32 wave + r, k = 64 kt + 32 g + 8 s + c
+    got1 = w1f.view(E, F // 128, 4, H // 64, 2, 4, 2, 32, 8)                  # [e, nt, w, kt, b, s, g, r, c]
+    src1 = w1.view(E, 2, F // 128, 4, 32, H // 64, 2, 4, 8)                    # [e, b, nt, w, r, kt, g, s, c]
+    assert torch.equal(got1, src1.permute(0, 2, 3, 5, 1, 7, 6, 4, 8))
+    # W2f [E][H/256][wave 4][F/64][b 2][s 4][g 2][r 32][8]: row 256 nt + 64 wave + 32 b + r
+    got2 = w2f.view(E, H // 256, 4, F // 64, 2, 4, 2, 32, 8)                  # [e, nt, w, kt, b, s, g, r, c]
+    src2 = w2.view(E, H // 256, 4, 2, 32, F // 64, 2, 4, 8)                    # [e, nt, w, b, r, kt, g, s, c]
+    assert torch.equal(got2, src2.permute(0, 1, 2, 5, 3, 7, 6, 4, 8))
+    idx, prob, _, _ = router_topk(router_gemm(x, wr), k, pre_softmax=True)
+    p = permute(idx, prob, E, BM=32)
+    want, want_inter = experts_forward(x, w1, w2, p, return_inter=True)
+    got, got_inter = experts_forward(x, w1, w2, p, return_inter=True, packed=packed)
+    assert same_bits(got_inter, want_inter) and same_bits(got, want)
+    # a larger tile ignores the packed copies
+    p256 = permute(idx, prob, E, BM=256)
+    assert same_bits(experts_forward(x, w1, w2, p256, packed=packed), experts_forward(x, w1, w2, p256))
+    assert pack_decode(w1[:, :, : H - 64].contiguous(), w2[:, : H - 64].contiguous()) is None   # H not a multiple of 256
