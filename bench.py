@@ -9,7 +9,7 @@ kernels the target names, each timed in this run at its own configuration; ``cpu
 composition of the same model on a stated slice. Weights and inputs come from a host generator (seeded), so they do
 not depend on the GPU. Prints ONE JSON line.
 
-Other workloads (``--workload dense_head | gdn_decode | moe | attention | digest | decode``) time configs[1], [2], [3]
+Other workloads (``--workload dense_head | gdn_decode | moe | attention | digest | decode | gemm``) time configs[1], [2], [3]
 and parts of [4] alone with the same contract; they are for profiling one kernel family, not the headline.
 """
 
@@ -495,6 +495,31 @@ def rollout_leg(cfg, w, tokens, n, prompt, resp, graph_steps=36):
             "decode_roofline": roof}
 
 
+def gemm(args):
+    """One dense product ``[m, k] x [n, k]^T`` of the batch-invariant GEMM at a shape of the trainer pass (what the traffic
+    profiles of the large products run): ``value`` = TFLOP/s, HIP events around each call."""
+    import torch
+
+    from isoexec_amd.ops.mm.mm_hip import linear_nt
+
+    dev = "cuda:0"
+    g = host_gen(21)
+    M, K, N = args.m, args.k, args.n
+    a = hrandn((M, K), g, dev)
+    w = hrandn((N, K), g, dev, std=0.02)
+    fn = lambda: linear_nt(a, w, tile=args.tile, want_row_max=args.row_max)
+    ms = _events_ms(fn, args.warmup, args.steps)
+    fl = 2.0 * M * N * K
+    algo = 2.0 * (M * K + N * K + M * N)
+    return {"metric": "dense GEMM TFLOP/s", "value": fl / ms / 1e9, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": f"gemm_bf16_nt {M} x {K} x {N} (tile {args.tile}, row max {bool(args.row_max)})"},
+            "roofline": {"bound": "mfma", "achieved": fl / ms / 1e9, "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s",
+                         "frac": fl / ms / 1e9 / PEAK_MFMA_BF16_TFLOPS, "traffic": None,
+                         "algorithmic_bytes": algo}}
+
+
 def decode(args):
     """The rollout leg of configs[4] alone (what the decode profiles run): ``value`` = decode tokens/s at batch
     ``--seqs`` from the captured graph, ``roofline`` = the step against HBM."""
@@ -661,13 +686,17 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="hybrid", choices=["dense_head", "gdn_decode", "moe", "hybrid", "attention", "digest", "decode"])
+    ap.add_argument("--workload", default="hybrid", choices=["dense_head", "gdn_decode", "moe", "hybrid", "attention", "digest", "decode", "gemm"])
     ap.add_argument("--seqs", type=int, default=64)
     ap.add_argument("--prompt", type=int, default=2048)
     ap.add_argument("--response", type=int, default=512)
     ap.add_argument("--tokens", type=int, default=None)
     ap.add_argument("--batch", type=int, default=256)
     ap.add_argument("--tile", type=int, default=0)
+    ap.add_argument("--m", type=int, default=32768)
+    ap.add_argument("--k", type=int, default=2048)
+    ap.add_argument("--n", type=int, default=151936)
+    ap.add_argument("--row-max", type=int, default=0)
     ap.add_argument("--cpu-tokens", type=int, default=2048)
     ap.add_argument("--cpu-seqs", type=int, default=4)
     ap.add_argument("--cpu-prompt", type=int, default=160)
@@ -686,7 +715,7 @@ def main():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(3)
     out = {"dense_head": dense_head, "gdn_decode": gdn_decode, "moe": moe, "hybrid": hybrid, "attention": attention, "digest": digest,
-           "decode": decode}[args.workload](args)
+           "decode": decode, "gemm": gemm}[args.workload](args)
     print(json.dumps(out))
 
 
