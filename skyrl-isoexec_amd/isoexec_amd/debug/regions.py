@@ -9,8 +9,8 @@ the difference and what the slabs say about where it is.
 
 This is the in-process core of the reference's debug mode: its capture layer writes the same kind of record to JSONL
 files per process (isoexec/debug/trace.py:200-262) and an offline tool compares them (isoexec/debug/compare.py:123-181,
-291-470). The record fields, the ladder verdict and the slab note keep the reference's meaning; the file trace, the
-env switches and the door installation are not part of this package.
+291-470). The record fields, the ladder verdict and the slab note keep the reference's meaning. ``debug.trace`` puts
+the environment switches and the per-process files on top of this log, ``debug.compare`` is the offline tool.
 """
 
 from __future__ import annotations
@@ -21,6 +21,7 @@ from typing import Callable, Dict, List, Optional, Tuple
 import torch
 
 from . import thash
+from .compare import ladder_verdict, segment_note  # noqa: F401 -- the verdicts are shared with the offline tool
 
 FORMAT_VERSION = 3
 
@@ -85,6 +86,17 @@ class RegionLog:
             rec["seq"] = len(self.records) + 1
             self.records.append(rec)
 
+    def next_call(self, region: str, layer: Optional[int] = None) -> int:
+        """The number the next call of ``region`` at ``layer`` will carry."""
+        return self._calls.get((region, layer), 0) + 1
+
+    def skip(self, region: str, layer: Optional[int] = None) -> int:
+        """Count a call of ``region`` without digesting it (a caller that records only some calls keeps the call
+        numbers of the others honest this way). Returns the call's number."""
+        call = self._calls.get((region, layer), 0) + 1
+        self._calls[(region, layer)] = call
+        return call
+
     # -- persistence (one JSON object per line)
     def dump(self, path: str) -> None:
         with open(path, "w") as fh:
@@ -114,40 +126,6 @@ def wrap_region(log: Optional[RegionLog], region: str, fn: Callable, *, layer: O
 
     recorded.__wrapped__ = fn
     return recorded
-
-
-def ladder_verdict(a: dict, b: dict) -> Tuple[Optional[int], str]:
-    """(the finest rung at which two records agree, what that says about the size of the difference). The bound is
-    a maximum over elements, relative; a ladder that differs at every rung bounds nothing and is not called large."""
-    la, lb = a.get("ladder") or {}, b.get("ladder") or {}
-    shared = sorted((int(name[1:]) for name in set(la) & set(lb) if name.startswith("k")), reverse=True)
-    if not shared:
-        return None, "unknown (no ladder recorded on both sides)"
-    agree = next((k for k in shared if la[f"k{k}"] == lb[f"k{k}"]), None)
-    if agree is None:
-        return None, ("not bounded by the ladder: differs at every rung down to k=0 (a sign or exponent difference, or "
-                      "small differences in enough elements that some straddle every truncation boundary)")
-    finer = [k for k in shared if k > agree]
-    if not finer:
-        return agree, f"< 2^-{agree} relative, max over elements (agrees at the finest rung recorded)"
-    return agree, (f"between ~2^-{min(finer)} and 2^-{agree} relative, max over elements (the upper end is a bound, the "
-                   f"lower end holds if no element straddles the k={min(finer)} boundary)")
-
-
-def segment_note(a: dict, b: dict) -> Optional[str]:
-    """Which slabs of rows differ, when both records carry slab digests of the same count."""
-    sa, sb = a.get("segments"), b.get("segments")
-    if not sa or not sb or len(sa) != len(sb):
-        return None
-    differing = thash.first_divergent_segments(sa, sb)
-    if not differing:
-        return f"all {len(sa)} row segments match (the difference is below segment resolution)"
-    if len(differing) == len(sa):
-        return f"all {len(sa)} row segments differ: a whole-tensor difference, not one confined to some rows"
-    rows = a.get("seg_rows") or 0
-    first = differing[0]
-    span = f", rows {first * rows}..{(first + 1) * rows - 1}" if rows else ""
-    return f"{len(differing)} of {len(sa)} row segments differ (first: segment {first}{span})"
 
 
 def _pairing_key(rec: dict) -> tuple:

@@ -22,6 +22,7 @@ from dataclasses import dataclass, field
 import numpy as np
 import torch
 
+from ..debug.trace import get_tracer
 from ..ops.attention.varlen_attn import KVCache, varlen_attention
 from ..ops.gdn.gdn_ops import conv_packed, gdn_native_core
 from ..ops.gdn.gdn_cpr import gdn_native_cpr_fwd
@@ -162,9 +163,10 @@ class _Blocks:
         self.cfg, self.w = cfg, weights
         dev = weights.embed.device
         self.cos, self.sin = rope_tables(cfg.max_positions, cfg.head_dim, cfg.rope_theta, device=dev)
-        # a debug.regions.RegionLog, or None: when set, the residual stream's per-layer outputs are digested on the
-        # device as they are produced, so that two runtimes' passes over the same tokens can be compared region by region
-        self.region_log = None
+        # a debug.regions.RegionLog or the process's debug.trace.Tracer (there is one when SKYRL_ISOEXEC_DEBUG_TRACE names
+        # a directory), else None: when set, the residual stream's per-layer outputs are digested on the device as they
+        # are produced, so that two runtimes' passes over the same tokens can be compared region by region
+        self.region_log = get_tracer()
         # a list, or None: when set, every mixture call appends its top-k expert ids [T, k] (layer order)
         self.routing_log = None
         # layer -> fragment-packed copies of the experts' matrices (pack_expert_weights): read by decode-size batches only

@@ -110,3 +110,65 @@ def test_wrap_region_records_the_return_value():
     from isoexec_amd.debug import thash
 
     assert log.records[0]["digest"] == f"{thash.tensor_digest(x * 2):016x}"
+
+
+def test_file_traces_of_both_runtimes_compare_offline(tmp_path):
+    """The same comparison through files: each runtime writes its trace directory, the offline tool reads both."""
+    from isoexec_amd.debug import compare as offline
+    from isoexec_amd.debug.trace import Tracer
+
+    cfg, w, prompts, lens, TrainerModel, RolloutEngine, HybridWeights = setup()
+    other = HybridWeights.make(cfg, seed=0, device=DEV)
+    other.layers[2]["w2"].view(torch.int16)[:, 0, :] ^= 0x40
+
+    def trace_trainer(name):
+        tracer = Tracer(str(tmp_path / name), side="trainer", ladder=True, segment_rows=16, ring=7)
+        trainer = TrainerModel(cfg, w)
+        trainer.blocks.region_log = tracer
+        tracer.set_step(0)
+        trainer.hidden_states(prompts, lens)
+        tracer.flush()
+        return tracer
+
+    def trace_engine(name, weights):
+        tracer = Tracer(str(tmp_path / name), side="engine", ladder=True, segment_rows=16)
+        engine = RolloutEngine(cfg, weights, max_num_seqs=len(lens) + 2, max_len=max(lens) + 8)
+        engine.blocks.region_log = tracer
+        tracer.set_step(0)
+        engine.prefill([11 + 3 * i for i in range(len(lens))], prompts, lens)
+        tracer.flush()
+        return tracer
+
+    a, b, c = trace_trainer("trainer"), trace_engine("engine", w), trace_engine("engine_changed", other)
+    assert a.written == cfg.layers * 4 and a.manifest()["digest_backend"]
+    assert offline.main([a.dir, b.dir]) == 0
+    report = offline.compare_dirs(a.dir, c.dir)
+    first = report["first_divergence"]
+    assert report["status"] == "divergent" and (first["region"], first["layer"], first["kind"]) == ("moe.combine", 2, "value")
+    assert report["regions"]["gdn.core"]["aligned_on"] == ["step"] and not first["inherited"]
+    assert all(d["layer"] >= 2 for d in report["divergences"]) and offline.main([a.dir, c.dir]) == 2
+
+
+def test_the_environment_switch_reaches_the_runtime(tmp_path, monkeypatch):
+    from isoexec_amd.debug import trace
+
+    cfg, w, prompts, lens, TrainerModel, _, _ = setup(prompt_lens=(9, 4))
+    trace._forget_for_tests()
+    monkeypatch.delenv(trace.ENV_TRACE, raising=False)
+    assert TrainerModel(cfg, w).blocks.region_log is None
+    trace._forget_for_tests()
+    monkeypatch.setenv(trace.ENV_TRACE, str(tmp_path / "t"))
+    monkeypatch.setenv(trace.ENV_SIDE, "trainer")
+    monkeypatch.setenv(trace.ENV_REGIONS, "gdn.core,attention.varlen")
+    try:
+        trainer = TrainerModel(cfg, w)
+        assert trainer.blocks.region_log is trace.get_tracer()
+        trainer.hidden_states(prompts, lens)
+        trace.flush()
+        from isoexec_amd.debug.compare import load_dir
+
+        records = load_dir(str(tmp_path / "t"))
+        assert len(records) == cfg.layers and {r["region"] for r in records} == {"gdn.core", "attention.varlen"}
+        assert all(r["side"] == "trainer" and r["layer_src"] == "caller" for r in records)
+    finally:
+        trace._forget_for_tests()
