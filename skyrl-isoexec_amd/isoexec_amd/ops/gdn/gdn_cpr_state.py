@@ -15,9 +15,30 @@ snapshotted in the wire dtype, inside a chunk it advances token by token. That m
   at every boundary, then one segmented scan of the new tokens (first segment from the running state, the others
   from the boundary snapshots), then the tail of the open chunk goes to the buffers.
 
-Not carried over from the reference: its sleep arenas and prefix-cache store (engine plumbing around the same state).
+Around that state, as in the reference:
+
+* the boundary store (``CprBoundaryStore``, gdn_cpr_state.py:96-196): at a multiple of C a request's whole state is
+  (fp32 entry state, convolution window), so a prefix that ends on a boundary can be resumed from a stored pair and
+  the continuation is the ordinary chunked-prefill one -- bit for bit what a cold prefill of the whole prompt gives.
+  Prefill stashes the pairs of the last boundaries it closes (``_apc_pending``), ``cpr_apc_publish`` stacks them over
+  the layers and stores them under the driver's prefix key, ``cpr_apc_adopt_many`` installs stored pairs for a
+  scheduler step. A miss is never a correctness event: the prompt is prefilled cold.
+* sleep (gdn_cpr_sleep.py:45-282): every layer's seven state tensors are views into one flat allocation, which
+  ``cpr_sleep`` gives back to the device with no host copy and ``cpr_wake`` makes anew, zeroed, with every row released.
+  The store is dropped first, so nothing advertises a checkpoint no layer could continue from. The new allocation has a
+  new address: a decode graph captured before the sleep must be captured again (the reference's arena keeps its
+  virtual address through the engine's allocator; there is no such allocator in this package).
+
+The reference's lazy boundary resync (``host_resync`` / ``layer_batched_resync``, gdn_cpr_state.py:295-358, 581-648)
+has no counterpart: it exists to keep a host-side position read out of the captured decode step, and here the boundary
+pass runs inside the step from device-side marks.
 """
 from __future__ import annotations
+
+import os
+import sys
+from collections import OrderedDict
+from typing import Callable, Optional
 
 import numpy as np
 import torch
@@ -28,6 +49,258 @@ from .gdn_ops import gdn_recurrent_kernel
 from .gdn_recurrent_state import RecurrentGDN
 
 CPR_LAYERS: list = []
+
+_CPR_APC_ENV = "SKYRL_ISOEXEC_GDN_CPR_APC"
+_CPR_APC_MB_ENV = "SKYRL_ISOEXEC_GDN_CPR_APC_MB"
+_OFF = ("", "0", "false", "no")
+# rows of one prefill call that may stash checkpoints: each stash is a cloned fp32 state held until it is published
+_APC_PENDING_MAX = 16
+_APC_ADOPT_WRITE_BATCH = 64
+
+
+def cpr_apc_enabled() -> bool:
+    """True when prefill stashes boundary checkpoints for the store (default off; gdn_cpr_state.py:71-73)."""
+    return os.environ.get(_CPR_APC_ENV, "0").strip().lower() not in _OFF
+
+
+def cpr_apc_shared_mode() -> bool:
+    """True for ``SKYRL_ISOEXEC_GDN_CPR_APC`` in {2, shm, shared}: the store's membership is mirrored to a scheduler
+    in another process, so within an epoch it only grows (a published key must stay servable; :76-83)."""
+    return os.environ.get(_CPR_APC_ENV, "0").strip().lower() in ("2", "shm", "shared")
+
+
+def cpr_apc_budget_bytes() -> int:
+    """Device-memory ceiling of the store, ``SKYRL_ISOEXEC_GDN_CPR_APC_MB`` MiB (default 1024; :86-88)."""
+    return int(float(os.environ.get(_CPR_APC_MB_ENV, "1024") or 1024) * 2**20)
+
+
+# Called by ``CprBoundaryStore.clear()`` after the local drop, so that a published index is retracted before anyone can
+# be admitted against it. An exception propagates: an index that still advertises dropped entries must not pass silently.
+CPR_APC_ON_CLEAR: list = []
+
+
+def _nbytes(*tensors) -> int:
+    return sum(t.numel() * t.element_size() for t in tensors)
+
+
+class CprBoundaryStore:
+    """Checkpoints of requests at chunk boundaries, keyed by a digest of the token prefix, least recently used first
+    out. A value is ``(position, entry [L, HV, V, K] fp32, conv [L, D, W-1])``: one pair per GDN layer, stacked.
+
+    The store must not outlive the engine's own prefix cache (it would resume a prefix computed under older
+    weights): whoever resets that cache calls ``cpr_apc_reset``."""
+
+    def __init__(self, budget_bytes: int, evict: bool = True, say: Optional[Callable[[str], None]] = None):
+        self.budget = int(budget_bytes)
+        self.evict = bool(evict)  # False: append-only (shared-index mode), a full store refuses instead of evicting
+        self._items: "OrderedDict[bytes, tuple]" = OrderedDict()
+        self._bytes = 0
+        self.hits = self.misses = self.stores = self.evictions = self.full_refusals = self.oversize_refusals = 0
+        self._say = say or (lambda msg: print(msg, file=sys.stderr, flush=True))
+
+    def __contains__(self, key: bytes) -> bool:
+        return key in self._items
+
+    def __len__(self) -> int:
+        return len(self._items)
+
+    @property
+    def nbytes(self) -> int:
+        return self._bytes
+
+    def get(self, key: bytes):
+        item = self._items.get(key)
+        if item is None:
+            self.misses += 1
+            return None
+        self._items.move_to_end(key)
+        self.hits += 1
+        return item
+
+    def put(self, key: bytes, pos: int, entry: torch.Tensor, conv: torch.Tensor) -> bool:
+        """True when a NEW checkpoint was stored (the cue to publish its key); a known key is only refreshed."""
+        if key in self._items:
+            self._items.move_to_end(key)
+            return False
+        size = _nbytes(entry, conv)
+        if size > self.budget:
+            self.oversize_refusals += 1
+            if self.oversize_refusals == 1:
+                self._say(f"[isoexec-cpr-apc] one boundary checkpoint takes {size / 2**20:.1f} MiB, the whole store "
+                          f"{self.budget / 2**20:.1f} MiB: nothing can be stored, no prefix will ever hit. Raise "
+                          f"{_CPR_APC_MB_ENV} or set {_CPR_APC_ENV}=0.")
+            return False
+        if self._bytes + size > self.budget and not self.evict:
+            self.full_refusals += 1
+            if self.full_refusals == 1:
+                self._say(f"[isoexec-cpr-apc] store full at {self._bytes / 2**20:.1f} of {self.budget / 2**20:.1f} MiB "
+                          f"({len(self._items)} checkpoints) and append-only: new checkpoints are refused until the "
+                          f"next reset. Raise {_CPR_APC_MB_ENV} if this repeats.")
+            return False
+        while self._bytes + size > self.budget and self._items:
+            _, (_, old_entry, old_conv) = self._items.popitem(last=False)
+            self._bytes -= _nbytes(old_entry, old_conv)
+            self.evictions += 1
+        self._items[key] = (int(pos), entry, conv)
+        self._bytes += size
+        self.stores += 1
+        return True
+
+    def clear(self) -> None:
+        self._items.clear()
+        self._bytes = 0
+        for hook in list(CPR_APC_ON_CLEAR):
+            hook()
+
+    def stats(self) -> dict:
+        return {"entries": len(self._items), "MiB": round(self._bytes / 2**20, 1), "hits": self.hits,
+                "misses": self.misses, "stores": self.stores, "evictions": self.evictions,
+                "full_refusals": self.full_refusals, "oversize_refusals": self.oversize_refusals}
+
+
+CPR_APC_STORE: Optional[CprBoundaryStore] = None
+
+
+def cpr_apc_store() -> CprBoundaryStore:
+    """The process's store, made on first use with the budget and mode the environment names."""
+    global CPR_APC_STORE
+    if CPR_APC_STORE is None:
+        CPR_APC_STORE = CprBoundaryStore(cpr_apc_budget_bytes(), evict=not cpr_apc_shared_mode())
+    return CPR_APC_STORE
+
+
+def cpr_apc_reset() -> None:
+    """Drop every checkpoint. To be called wherever the engine resets its own prefix cache (a weight sync)."""
+    if CPR_APC_STORE is not None:
+        CPR_APC_STORE.clear()
+
+
+def cpr_apc_store_invalidate() -> None:
+    """Drop the store because its tensors are about to become unreadable (a sleep). Runs BEFORE the release."""
+    cpr_apc_reset()
+
+
+def cpr_apc_publish(layers: list, items: list) -> list:
+    """Move the checkpoints that the layers' last prefill stashed into the store.
+
+    ``items`` are ``(slot, position, prefix_key)`` as the driver knows them (it alone can name a prefix). A checkpoint
+    is stored when EVERY layer stashed one for that slot's row at that position; the per-layer pairs are stacked on a
+    new first axis. Returns the keys newly stored (what a shared index would advertise). Whatever was stashed and not
+    asked for is dropped: a stash lives for one step."""
+    if not layers:
+        return []
+    store = cpr_apc_store()
+    fresh = []
+    for slot, pos, key in items:
+        row = layers[0]._slot2row.get(int(slot))
+        if row is None or key in store:
+            continue
+        found = []
+        for ly in layers:
+            pair = next(((e, c) for p, e, c in ly._apc_pending.get(ly._slot2row.get(int(slot), -1), ()) if p == int(pos)), None)
+            if pair is None:
+                break
+            found.append(pair)
+        if len(found) != len(layers):
+            continue
+        if store.put(key, int(pos), torch.stack([e for e, _ in found]), torch.stack([c for _, c in found])):
+            fresh.append(key)
+    for ly in layers:
+        ly._apc_pending.clear()
+    return fresh
+
+
+def cpr_apc_adopt_many(layers: list, items: list):
+    """Install stored boundary states for one scheduler step: ``items`` are ``(slot, position, prefix_key)`` in
+    scheduler order; returns the pool row given to each, or ``None`` when any of them cannot be served (then nothing
+    was touched: every condition is checked before the first row changes hands; gdn_cpr_state.py:222-278). After a
+    successful call the requests' prefills are ordinary continuations (``has_initial_state`` true)."""
+    if not items:
+        return []
+    if not layers:
+        return None
+    first = layers[0]
+    C = first.chunk_size
+    store = cpr_apc_store()
+    checkpoints = []
+    for _slot, pos, key in items:
+        if pos <= 0 or pos % C:
+            return None
+        got = store.get(key)
+        if got is None:
+            return None
+        at, entry, conv = got
+        if at != pos or entry.shape[0] != len(layers) or conv.shape[0] != len(layers):
+            return None
+        checkpoints.append((entry, conv))
+    slots = [int(slot) for slot, _pos, _key in items]
+    rows_by_layer = [ly._assign_many(slots) for ly in layers]
+    rows = rows_by_layer[0]
+    if any(other != rows for other in rows_by_layer[1:]):
+        raise RuntimeError("[isoexec-gdn] adoption found the layers' state pools out of step: the same request would "
+                           "sit in different rows of different layers")
+    dev = first.ssm_state.device
+    positions = [int(pos) for _slot, pos, _key in items]
+    for j, ly in enumerate(layers):
+        wire = ly.k_buf.dtype if getattr(ly, "k_buf", None) is not None else torch.bfloat16
+        for lo in range(0, len(items), _APC_ADOPT_WRITE_BATCH):
+            hi = min(lo + _APC_ADOPT_WRITE_BATCH, len(items))
+            r = torch.tensor(rows[lo:hi], dtype=torch.long, device=dev)
+            entry = torch.stack([checkpoints[i][0][j] for i in range(lo, hi)])
+            conv = torch.stack([checkpoints[i][1][j] for i in range(lo, hi)])
+            ly.entry_state[r] = entry
+            ly.ssm_state[r] = entry.to(wire).to(torch.float32)   # the running state at a boundary is the snapshot
+            ly.conv_state[r] = conv.to(ly.conv_state.dtype)
+        ly.pos[torch.tensor(rows, dtype=torch.long, device=dev)] = torch.tensor(positions, dtype=torch.long, device=dev)
+        for row in rows:
+            ly._apc_pending.pop(row, None)
+    return rows
+
+
+def cpr_apc_adopt(layers: list, slot: int, pos: int, key: bytes) -> bool:
+    """One request's adoption; False means a cold prefill (gdn_cpr_state.py:281-287)."""
+    return cpr_apc_adopt_many(layers, [(int(slot), int(pos), key)]) is not None
+
+
+def cpr_arena_specs(*, rows, C, HV, K, V, Hk, dt, gdt, conv_shape) -> list:
+    """``[(attribute, shape, dtype), ...]`` of a layer's device state in allocation order (gdn_cpr_state.py:360-371)."""
+    return [("ssm_state", (rows, HV, V, K), torch.float32), ("conv_state", tuple(conv_shape), dt),
+            ("entry_state", (rows, HV, V, K), torch.float32), ("k_buf", (rows, C, Hk, K), dt),
+            ("v_buf", (rows, C, HV, V), dt), ("g_buf", (rows, C, HV), gdt), ("b_buf", (rows, C, HV), dt)]
+
+
+def _carve(specs, device):
+    """One zeroed flat allocation and the views the specs name, each on a 256-byte boundary."""
+    offsets, at = [], 0
+    for _name, shape, dtype in specs:
+        offsets.append(at)
+        at += (int(np.prod(shape)) * torch.empty((), dtype=dtype).element_size() + 255) // 256 * 256
+    flat = torch.zeros(at, dtype=torch.uint8, device=device)
+    views = {}
+    for (name, shape, dtype), off in zip(specs, offsets):
+        n = int(np.prod(shape)) * torch.empty((), dtype=dtype).element_size()
+        views[name] = flat[off:off + n].view(dtype).view(shape)
+    return flat, views
+
+
+def cpr_arena_bytes(layers=None) -> int:
+    return sum(ly._flat_arena.numel() for ly in (CPR_LAYERS if layers is None else layers) if ly._flat_arena is not None)
+
+
+def cpr_sleep(layers=None, *, empty_cache: bool = True) -> int:
+    """Give every layer's state back to the device (no host copy: the state of a sleeping engine is not kept) after
+    dropping the boundary store. Returns the bytes released."""
+    layers = list(CPR_LAYERS if layers is None else layers)
+    cpr_apc_store_invalidate()
+    released = sum(ly._release_arena() for ly in layers)
+    if empty_cache and released and torch.cuda.is_available():
+        torch.cuda.empty_cache()
+    return released
+
+
+def cpr_wake(layers=None) -> int:
+    """Make the state of every sleeping layer anew: zeroed, every row released. Returns the bytes allocated."""
+    return sum(ly._restore_arena() for ly in (CPR_LAYERS if layers is None else layers))
 
 
 def build_cpr_gdn(*, max_num_seqs: int, chunk_size: int, **kw) -> "CprGDN":
@@ -50,12 +323,16 @@ class CprGDN(RecurrentGDN):
         HV, K, V, H = self.num_v_heads, self.head_k_dim, self.head_v_dim, self.num_k_heads
         dev, dt = self.ssm_state.device, self.conv_state.dtype
         self.chunk_size = C
-        self.entry_state = torch.zeros(rows, HV, V, K, dtype=torch.float32, device=dev)
-        # prepared values, as the boundary pass consumes them (k normalised, g fp32, beta in the wire dtype)
-        self.k_buf = torch.zeros(rows, C, H, K, dtype=dt, device=dev)
-        self.v_buf = torch.zeros(rows, C, HV, V, dtype=dt, device=dev)
-        self.g_buf = torch.zeros(rows, C, HV, dtype=torch.float32, device=dev)
-        self.b_buf = torch.zeros(rows, C, HV, dtype=dt, device=dev)
+        # the running and convolution states, the fp32 entry states and the open-chunk buffers (prepared values, as
+        # the boundary pass consumes them: k normalised, g fp32, beta in the wire dtype) are views into one allocation
+        self._arena_specs = cpr_arena_specs(rows=rows, C=C, HV=HV, K=K, V=V, Hk=H, dt=dt, gdt=torch.float32,
+                                            conv_shape=self.conv_state.shape)
+        self._arena_device = dev
+        self._flat_arena = None
+        self._restore_arena(release_rows=False)
+        # row -> [(boundary position, fp32 entry state, convolution window)] stashed by the last prefill
+        self._apc = cpr_apc_enabled()
+        self._apc_pending: dict = {}
         # absolute position (tokens consumed) per row; pos % C is how full the open chunk is
         self.pos = torch.zeros(rows, dtype=torch.int64, device=dev)
         # rows whose boundary pass is pending inside the current decode step (row id, or 0)
@@ -63,13 +340,50 @@ class CprGDN(RecurrentGDN):
         self._cu_pool = torch.arange(0, (rows + 1) * C, C, dtype=torch.int32, device=dev)
         CPR_LAYERS.append(self)
 
+    # -- sleep
+    @property
+    def asleep(self) -> bool:
+        return self._flat_arena is None
+
+    def _release_arena(self) -> int:
+        if self._flat_arena is None:
+            return 0
+        size = self._flat_arena.numel()
+        self._flat_arena = None
+        for name, _shape, _dtype in self._arena_specs:
+            setattr(self, name, None)
+        self._apc_pending.clear()
+        return size
+
+    def _restore_arena(self, release_rows: bool = True) -> int:
+        if self._flat_arena is not None:
+            return 0
+        self._flat_arena, views = _carve(self._arena_specs, self._arena_device)
+        for name, view in views.items():
+            setattr(self, name, view)
+        if release_rows:  # what the rows held is gone: nobody may resume from them
+            self.table.release_all()
+            self.flush_slot_map()
+            self.last_used.zero_()
+            self._clock.zero_()
+            self.pos.zero_()
+            self._due.zero_()
+        return self._flat_arena.numel()
+
+    def _awake(self) -> None:
+        if self._flat_arena is None:
+            raise RuntimeError("[isoexec-gdn] this layer's state was released by cpr_sleep; call cpr_wake first")
+
     # -- row lifecycle
     def _reset_rows(self, rows) -> None:
         if len(rows) == 0:
             return
         t = torch.tensor(list(rows), dtype=torch.long, device=self.pos.device)
         self.pos[t] = 0
-        self.entry_state[t] = 0.0
+        if self.entry_state is not None:
+            self.entry_state[t] = 0.0
+        for r in rows:
+            self._apc_pending.pop(int(r), None)
 
     def _on_row_released(self, row: int) -> None:
         self._reset_rows([row])
@@ -81,11 +395,37 @@ class CprGDN(RecurrentGDN):
         self.pos[0] = 0  # "none" is spelled row 0
 
     def reset(self) -> int:
+        self._awake()
         freed = super().reset()
         self.entry_state.zero_()
         self.pos.zero_()
         self._due.zero_()
+        self._apc_pending.clear()
         return freed
+
+    # -- boundary checkpoints of a prefill call
+    def _apc_capture(self, x, rows, qsl, pos0, lens, nb, snaps) -> None:
+        """Stash ``(position, fp32 entry state, convolution window)`` for the last two boundaries each sequence closed
+        in this call. A boundary is taken only when its whole window of W-1 inputs lies inside this call's ``x``;
+        one that does not is skipped, never pieced together (gdn_cpr_state.py:555-578)."""
+        W = self.conv_weight.shape[-1]
+        C = self.chunk_size
+        for i, m in enumerate(nb):
+            if not m:
+                continue
+            if len(self._apc_pending) >= _APC_PENDING_MAX:
+                break
+            first = (pos0[i] // C + 1) * C            # the first boundary this call closed
+            stash = []
+            for j in range(max(0, m - 2), m):
+                at = first + j * C
+                inside = at - pos0[i]                    # tokens of this call in front of the boundary
+                if inside < W - 1 or inside > lens[i]:
+                    continue
+                t = int(qsl[i]) + inside                 # row of x of the token after the boundary
+                stash.append((at, snaps[i][j].detach().clone(), x[t - (W - 1):t].transpose(0, 1).contiguous()))
+            if stash:
+                self._apc_pending[rows[i]] = stash
 
     # -- the boundary pass of a decode step (host-free)
     def _boundary_pass(self) -> None:
@@ -107,6 +447,7 @@ class CprGDN(RecurrentGDN):
         """One decode step for N requests, the buffer append, and the boundary pass where a chunk closed."""
         from .gdn_ops import conv_packed
 
+        self._awake()
         N = x.shape[0]
         rows32 = self._decode_rows(slots)
         cu = self._decode_cu.get(N)
@@ -129,6 +470,7 @@ class CprGDN(RecurrentGDN):
     def prefill(self, slots, slots_cpu, x, a, b, qsl, has_initial_state=None, prefill_query_start_loc=None):
         """Prefill a packed batch of N prompts or prompt chunks (a resumed row continues at its stored position,
         which may be inside an open chunk). Returns ``o [T, HV, V]``."""
+        self._awake()
         rows, is_cont, _rows_out, cu, q, k, v, g, beta = self._prefill_prepare(
             slots_cpu, x, a, b, qsl, has_initial_state, prefill_query_start_loc)
         C = self.chunk_size
@@ -171,6 +513,8 @@ class CprGDN(RecurrentGDN):
             crossed = [i for i, m in enumerate(nb) if m]
             ct = torch.tensor([rows[i] for i in crossed], dtype=torch.long, device=dev)
             self.entry_state[ct] = torch.stack([snaps[i][-1] for i in crossed])
+            if self._apc:
+                self._apc_capture(x, rows, qsl, pos0, lens, nb, snaps)
 
         # ---- the outputs: one segmented scan of the new tokens
         wire = k.dtype

@@ -243,3 +243,111 @@ def test_wide_heads_take_the_lane_pair_scan_in_the_boundary_pass():
             assert same_bits(od[row], want[i][have[i]]), (i, have[i])
             have[i] += 1
     assert not layer._due.any()
+
+
+def two_layers(monkeypatch, capacity=6):
+    """Two layers with their own parameters (as two GDN layers of a model), checkpointing on."""
+    from isoexec_amd.ops.gdn import gdn_cpr_state as cpr
+
+    monkeypatch.setenv("SKYRL_ISOEXEC_GDN_CHUNKED_PREFILL", "1")
+    monkeypatch.setenv("SKYRL_ISOEXEC_GDN_CPR_APC", "1")
+    monkeypatch.setattr(cpr, "CPR_APC_STORE", cpr.CprBoundaryStore(64 << 20))
+    layers = [make_layer(capacity), make_layer(capacity)]
+    layers[1].conv_weight = (layers[1].conv_weight.float() * 0.9).to(torch.bfloat16)
+    layers[1].A_log = layers[1].A_log * 0.8
+    assert all(ly._apc for ly in layers)
+    return cpr, layers
+
+
+def test_adopted_prefix_continues_bit_for_bit_as_a_cold_prefill(monkeypatch):
+    """A prompt of 75 tokens (C = 16) is prefilled cold by one request; its boundary checkpoints are published under
+    prefix keys; two later requests with the same prefix adopt the checkpoints at 64 and at 48 and prefill only the
+    rest -- outputs, states and the decode steps after are the cold request's, bit for bit, in both layers."""
+    cpr, layers = two_layers(monkeypatch)
+    n, total = 75, 84
+    req = request(7, total)
+    other = request(8, 40)                                         # a second sequence in the same packed call
+    want = [one_pass(ly, *(t[:n] for t in req)) for ly in layers]
+    st = torch.tensor([1, 2], device=DEV)
+    xs, as_, bs = (torch.cat([req[j][:n], other[j]]) for j in range(3))
+    for ly, w in zip(layers, want):
+        o = ly.prefill(st, [1, 2], xs, as_, bs, [0, n, n + 40])
+        assert same_bits(o[:n], w[0])
+        # the last two boundaries closed by each sequence were stashed: 48 and 64 of the first, 16 and 32 of the second
+        assert {row: [p for p, _, _ in v] for row, v in ly._apc_pending.items()} == \
+            {ly.require_row(1): [48, 64], ly.require_row(2): [16, 32]}
+    fresh = cpr.cpr_apc_publish(layers, [(1, 64, b"p64"), (1, 48, b"p48"), (2, 32, b"o32"), (1, 32, b"never-stashed")])
+    assert fresh == [b"p64", b"p48", b"o32"] and all(not ly._apc_pending for ly in layers)
+    pos, entry, conv = cpr.cpr_apc_store().get(b"p64")
+    assert pos == 64 and entry.shape == (2, HV, V, K) and entry.dtype is torch.float32 and conv.shape == (2, D, W - 1)
+    for j, ly in enumerate(layers):                                # the stored entry IS the chain at the boundary
+        assert same_bits(entry[j], one_pass(ly, *(t[:64] for t in req))[1])
+
+    rows = cpr.cpr_apc_adopt_many(layers, [(5, 64, b"p64"), (6, 48, b"p48")])
+    assert rows is not None and all(ly.require_row(5) == rows[0] and ly.require_row(6) == rows[1] for ly in layers)
+    st2 = torch.tensor([5, 6], device=DEV)
+    xs, as_, bs = (torch.cat([req[j][64:n], req[j][48:n]]) for j in range(3))
+    for ly, w in zip(layers, want):
+        o = ly.prefill(st2, [5, 6], xs, as_, bs, [0, n - 64, n - 64 + n - 48], has_initial_state=[True, True])
+        assert same_bits(o[:n - 64], w[0][64:]) and same_bits(o[n - 64:], w[0][48:])
+        for slot in (5, 6):
+            check_row(ly, slot, n, w)
+            assert same_bits(ly.conv_state[ly.require_row(slot)], ly.conv_state[ly.require_row(1)])
+    # and the three requests decode alike from here, across the boundary at 80
+    st3 = torch.tensor([1, 5, 6], device=DEV)
+    for t in range(n, total):
+        step = [req[j][t].expand(3, -1).contiguous() for j in range(3)]
+        for ly in layers:
+            od = ly.decode(st3, *step)
+            assert same_bits(od[0], od[1]) and same_bits(od[0], od[2]), t
+    for ly in layers:
+        full = one_pass(ly, *req)
+        for slot in (1, 5, 6):
+            check_row(ly, slot, total, full)
+    assert cpr.cpr_apc_store().stats()["hits"] == 3
+
+
+def test_boundaries_whose_window_is_not_inside_the_call_are_not_stashed(monkeypatch):
+    cpr, layers = two_layers(monkeypatch)
+    ly = layers[0]
+    req = request(9, 40)
+    st = torch.tensor([3], device=DEV)
+    ly.prefill(st, [3], *(t[:14] for t in req), [0, 14])
+    assert not ly._apc_pending                                     # no boundary closed
+    ly.prefill(st, [3], *(t[14:18] for t in req), [0, 4], has_initial_state=[True])
+    assert not ly._apc_pending                                     # 16 closed, but only 2 of its 3 window inputs are here
+    ly.prefill(st, [3], *(t[18:40] for t in req), [0, 22], has_initial_state=[True])
+    assert [p for p, _, _ in ly._apc_pending[ly.require_row(3)]] == [32]
+    ly.release_slot(3)
+    assert not ly._apc_pending                                     # a released row keeps no stash
+
+
+def test_sleep_gives_the_state_back_and_wake_starts_from_nothing(monkeypatch):
+    cpr, layers = two_layers(monkeypatch)
+    req = request(7, 40)
+    st = torch.tensor([1], device=DEV)
+    cold = [ly.prefill(st, [1], *req, [0, 40]) for ly in layers]
+    cpr.cpr_apc_publish(layers, [(1, 32, b"p32")])
+    assert len(cpr.cpr_apc_store()) == 1
+    size = cpr.cpr_arena_bytes(layers)
+    rows = 7
+    per_layer = 2 * rows * HV * V * K * 4 + rows * D * (W - 1) * 2 + rows * C * (KD + HV * V) * 2 + rows * C * HV * 6
+    assert per_layer <= size // 2 < per_layer + 7 * 256            # seven views, each on a 256-byte boundary
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    before = torch.cuda.memory_reserved()
+    assert cpr.cpr_sleep(layers) == size and all(ly.asleep and ly.ssm_state is None and ly.k_buf is None for ly in layers)
+    assert len(cpr.cpr_apc_store()) == 0                           # nothing advertises what no layer could continue
+    assert torch.cuda.memory_reserved() <= before - size + (4 << 20)
+    with pytest.raises(RuntimeError, match="cpr_wake"):
+        layers[0].prefill(st, [1], *req, [0, 40])
+    with pytest.raises(RuntimeError, match="cpr_wake"):
+        layers[0].decode(st, req[0][:1], req[1][:1], req[2][:1])
+    assert cpr.cpr_sleep(layers) == 0                              # asleep already
+    assert cpr.cpr_wake(layers) == size and cpr.cpr_wake(layers) == 0
+    for ly, o in zip(layers, cold):
+        assert not ly.asleep and len(ly.table) == 0 and not ly.ssm_state.any() and not ly.entry_state.any()
+        assert not ly.pos.any() and not ly.conv_state.any()
+        with pytest.raises(RuntimeError):
+            ly.prefill(st, [1], *(t[32:] for t in req), [0, 8], has_initial_state=[True])   # nobody resumes over a sleep
+        assert same_bits(ly.prefill(st, [1], *req, [0, 40]), o)    # the same request, cold, gives the same bits
