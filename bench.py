@@ -391,6 +391,19 @@ def north_star_kernels(w, dev, steps):
         "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s", "frac": fl / ms / 1e9 / PEAK_MFMA_BF16_TFLOPS,
         "traffic": MEASURED_TRAFFIC_BYTES["dense_head_M4096_gemm"],
         "traffic_source": TRAFFIC_SOURCE["dense_head_M4096_gemm"] + " (not measured in this run)"}
+    # configs[1] at M <= 64: the product is the time memory needs to deliver the 1.245 GB of weights once. The door
+    # streams the fragment-packed copy (ix_gemm_bf16_nt_decode); logits written: M * V * 2 B.
+    from isoexec_amd.ops.mm.mm_hip import pack_nt_decode
+
+    packed = pack_nt_decode(w_lm)
+    for m_small in (16, 64):
+        ms = _events_ms(lambda: linear_nt(h[:m_small], packed), 4, max(steps, 20))
+        by = Vv * Kd * 2 + m_small * (Vv + Kd) * 2
+        out[f"lm_head_gemm_M{m_small}_K4096"] = {
+            "bound": "hbm", "kernel": "k_gemm_dec (weights streamed from the packed copy)", "kernel_ms": ms,
+            "achieved": by / ms / 1e6, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": by / ms / 1e6 / PEAK_HBM_GBS,
+            "traffic": None}
+    del packed
     logits, row_max = gemm()
     ms = _events_ms(lambda: sampled_forward(logits, target, 8, row_max=row_max), 3, max(steps, 20))
     by = M * Vv * 2

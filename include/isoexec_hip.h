@@ -156,6 +156,19 @@ long ix_gemm_bf16_n_tiles(long M, long N, long K, int tile);
 int ix_gemm_bf16_nt_batched(const void* A, long lda, long stride_a, const void* W, long ldw, long stride_w, void* C,
                             long ldc, long stride_c, long batch, long M, long N, long K, int tile, void* stream);
 
+/* The same product for M <= 64 (the M in {1, 7, 64} cases of the override, mm_tiles.py:232-326, where the product is the
+ * time memory needs to deliver W once): W is read from a fragment-packed copy made once per weight version, streamed
+ * through registers; the activations are staged in LDS per workgroup. Same bits as ix_gemm_bf16_nt (same matrix
+ * instruction, same K order, one accumulator per element, one rounding).
+ * ix_gemm_pack_decode: Wf (N * K bf16, 16-byte aligned) <- W [N,K] with row pitch ldw. Serves N a multiple of 32 and
+ * K in {1024, 2048, 3072, 4096}; ix_gemm_decode_serves_shape(N, K) says so without touching memory (1 = served).
+ * ix_gemm_bf16_nt_decode: C [M,N] bf16 (row pitch ldc, a multiple of 4; C 8-byte aligned) = A [M,K] (row pitch lda, a
+ * multiple of 8; A 16-byte aligned) . W^T; no bias, no row maxima, M <= 64: declines (IX_DECLINED) anything else. */
+int ix_gemm_decode_serves_shape(long N, long K);
+int ix_gemm_pack_decode(const void* W, long ldw, void* Wf, long N, long K, void* stream);
+int ix_gemm_bf16_nt_decode(const void* A, long lda, const void* Wf, void* C, long ldc, long M, long N, long K,
+                           void* stream);
+
 /* Router gating GEMM (moe/_register.py:59-66): C fp32 [M,N] = A[M,K] . W[N,K]^T with W fp32 and
  * A fp32 or bf16 (a_dtype), fp32 accumulate in a fixed K order. */
 int ix_gemm_f32_nt(const void* A, int a_dtype, long lda, const void* W, long ldw, void* C, long ldc, long M,

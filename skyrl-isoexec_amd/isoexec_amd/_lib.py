@@ -64,6 +64,9 @@ SIGNATURES = {
         c_int,
         [P, c_long, c_long, P, c_long, c_long, P, c_long, c_long, c_long, c_long, c_long, c_long, c_int, P],
     ),
+    "ix_gemm_decode_serves_shape": (c_int, [c_long, c_long]),
+    "ix_gemm_pack_decode": (c_int, [P, c_long, P, c_long, c_long, P]),
+    "ix_gemm_bf16_nt_decode": (c_int, [P, c_long, P, P, c_long, c_long, c_long, c_long, P]),
     "ix_gemm_f32_nt": (c_int, [P, c_int, c_long, P, c_long, P, c_long, c_long, c_long, c_long, P]),
     "ix_gdn_scan": (
         c_int,

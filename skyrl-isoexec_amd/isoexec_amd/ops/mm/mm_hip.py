@@ -27,13 +27,71 @@ def reset_stats() -> None:
         _COUNTS[key] = 0
 
 
-def linear_nt(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *, tile: int = 0,
+DECODE_ROWS = 64  # the streaming form serves products of at most this many rows
+
+
+class PackedWeight:
+    """A weight ``[N, K]`` and its fragment-packed copy for products of at most ``DECODE_ROWS`` rows. The copy is made
+    by ``pack_nt_decode`` and is as large as the weight; it has to be made again when the weight changes."""
+
+    __slots__ = ("weight", "packed")
+
+    def __init__(self, weight: torch.Tensor, packed: torch.Tensor):
+        self.weight, self.packed = weight, packed
+
+    @property
+    def shape(self):
+        return self.weight.shape
+
+
+def pack_nt_decode(weight: torch.Tensor):
+    """``PackedWeight`` for ``weight [N, K]`` (bf16, rows K-contiguous), or ``None`` for a shape the streaming form does
+    not serve (N a multiple of 32, K in {1024, 2048, 3072, 4096})."""
+    _lib.require_device(weight)
+    if weight.dtype is not torch.bfloat16 or weight.ndim != 2 or weight.stride(1) != 1:
+        return None
+    n, k = weight.shape
+    L = _lib.lib()
+    if not L.ix_gemm_decode_serves_shape(n, k):
+        return None
+    packed = torch.empty(n * k, dtype=torch.bfloat16, device=weight.device)
+    rc = _lib.check(L.ix_gemm_pack_decode(weight.data_ptr(), weight.stride(0), packed.data_ptr(), n, k,
+                                          _lib.current_stream(weight.device)), "ix_gemm_pack_decode")
+    return PackedWeight(weight, packed) if rc == _lib.IX_OK else None
+
+
+def linear_nt_decode(x: torch.Tensor, packed: PackedWeight):
+    """``x [M <= 64, K] @ weight^T`` from the packed copy (bf16 out, same bits as ``linear_nt``); ``None`` if declined."""
+    _lib.require_device(x, packed.packed)
+    if x.dtype is not torch.bfloat16 or x.ndim != 2 or x.stride(1) != 1 or x.shape[1] != packed.weight.shape[1]:
+        return None
+    m, k = x.shape
+    if m > DECODE_ROWS:
+        return None
+    n = packed.weight.shape[0]
+    out = torch.empty(m, n, dtype=torch.bfloat16, device=x.device)
+    rc = _lib.check(_lib.lib().ix_gemm_bf16_nt_decode(x.data_ptr(), x.stride(0), packed.packed.data_ptr(), out.data_ptr(),
+                                                      out.stride(0), m, n, k, _lib.current_stream(x.device)),
+                    "ix_gemm_bf16_nt_decode")
+    return out if rc == _lib.IX_OK else None
+
+
+def linear_nt(x: torch.Tensor, weight, bias: torch.Tensor | None = None, *, tile: int = 0,
               out_dtype: torch.dtype = torch.bfloat16, want_row_max: bool = False):
     """``x [M, K] @ weight [N, K]^T (+ bias)``, bf16 operands, fp32 accumulate; ``None`` if declined.
 
     ``out_dtype=torch.float32`` returns the fp32 accumulator unrounded. ``want_row_max`` also returns
     each row's exact maximum over the N outputs (taken in the kernel's epilogue), as ``(out, row_max)``.
+    ``weight`` may be a ``PackedWeight``: a plain product (no bias, bf16 out, no row maximum, tile 0) of at most
+    ``DECODE_ROWS`` rows then streams the packed copy; every other call uses the weight itself. Same bits either way.
     """
+    if isinstance(weight, PackedWeight):
+        if (bias is None and tile == 0 and out_dtype is torch.bfloat16 and not want_row_max
+                and 0 < x.shape[0] <= DECODE_ROWS):
+            out = linear_nt_decode(x, weight)
+            if out is not None:
+                return out
+        weight = weight.weight
     _lib.require_device(x, weight, bias)
     if x.dtype is not torch.bfloat16 or weight.dtype is not torch.bfloat16:
         return None
