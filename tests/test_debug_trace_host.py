@@ -259,3 +259,54 @@ def test_the_tool_runs_on_the_standard_library_alone(tmp_path):
                                env=dict(os.environ, PYTHONPATH=PKG_PARENT))
     assert as_module.returncode == 0, as_module.stderr
     assert "CLEAN" in as_module.stdout
+
+
+# ---- the installer ---------------------------------------------------------------------------------------------------
+
+def test_every_registry_region_is_accounted_for():
+    from isoexec_amd.debug import install
+
+    cov = install.coverage()
+    assert not [r for r, e in cov.items() if e["status"] == "unknown"]
+    assert cov["gdn.core"]["status"] == "hooked" and "ops.gdn.gdn_ops:gdn_recurrent_kernel" in cov["gdn.core"]["doors"]
+    assert cov["gdn.state"]["status"] == "partial" and cov["moe.weights"]["status"] == "not_hooked" and cov["moe.weights"]["note"]
+    assert install.coverage(["made.up"])["made.up"]["status"] == "unknown"
+    for region, module, attr, _ in install.DOORS:                      # every door of the table exists
+        assert install._resolve(module, attr) is not None, (region, module, attr)
+
+
+def test_install_wraps_the_definition_and_every_imported_binding(tmp_path, monkeypatch):
+    from isoexec_amd.debug import install
+    from isoexec_amd.ops.norms import fused_outnorm
+    from isoexec_amd.runtimes import hybrid
+
+    T._forget_for_tests()
+    monkeypatch.delenv(T.ENV_TRACE, raising=False)
+    assert install.install_debug_hooks() == 0                          # tracing off: nothing is touched
+    original = fused_outnorm.fused_rms_norm_gamma
+    assert hybrid.fused_rms_norm_gamma is original
+
+    T._forget_for_tests()
+    monkeypatch.setenv(T.ENV_TRACE, str(tmp_path / "t"))
+    monkeypatch.setenv(T.ENV_SIDE, "trainer")
+    try:
+        T.get_tracer()._log = HostLog()
+        changed = install.install_debug_hooks()
+        wrapped = fused_outnorm.fused_rms_norm_gamma
+        assert changed > len(install.DOORS) // 2 and wrapped is not original and wrapped.__wrapped__ is original
+        assert hybrid.fused_rms_norm_gamma is wrapped                  # the binding `from ... import` left behind
+        assert fused_outnorm.ZeroCenteredRMSNorm.forward._ix_traced_region == "norms.rms"
+        from isoexec_amd.ops.mm import mm_hip
+
+        assert not hasattr(mm_hip.linear_nt, "_ix_traced_region")      # `mm` is off unless the allow list names it
+        assert install.install_debug_hooks() == 0                      # a second call finds everything wrapped
+        monkeypatch.setattr(fused_outnorm, "fused_rms_norm_gamma", lambda x, w, eps, **kw: ("normed", x))
+        T.wrap_region("norms.rms", fused_outnorm.fused_rms_norm_gamma)("x", None, 1e-6)
+        T.flush()
+        assert [r["region"] for r in C.load_dir(str(tmp_path / "t"))] == ["norms.rms"]
+    finally:
+        monkeypatch.undo()
+        assert install.uninstall_debug_hooks() > 0
+        T._forget_for_tests()
+    assert fused_outnorm.fused_rms_norm_gamma is original and hybrid.fused_rms_norm_gamma is original
+    assert not hasattr(fused_outnorm.ZeroCenteredRMSNorm.forward, "_ix_traced_region")

@@ -172,3 +172,37 @@ def test_the_environment_switch_reaches_the_runtime(tmp_path, monkeypatch):
         assert all(r["side"] == "trainer" and r["layer_src"] == "caller" for r in records)
     finally:
         trace._forget_for_tests()
+
+
+def test_installed_doors_record_what_the_runtime_calls_and_change_nothing(tmp_path, monkeypatch):
+    from isoexec_amd.debug import install, trace
+    from isoexec_amd.debug.compare import load_dir
+
+    cfg, w, prompts, lens, TrainerModel, _, _ = setup(prompt_lens=(33, 7))
+    trace._forget_for_tests()
+    monkeypatch.delenv(trace.ENV_TRACE, raising=False)
+    plain = TrainerModel(cfg, w).hidden_states(prompts, lens)
+    trace._forget_for_tests()
+    monkeypatch.setenv(trace.ENV_TRACE, str(tmp_path / "doors"))
+    monkeypatch.setenv(trace.ENV_SIDE, "trainer")
+    try:
+        assert install.install_debug_hooks() > 0
+        traced = TrainerModel(cfg, w).hidden_states(prompts, lens)
+        trace.flush()
+        assert torch.equal(traced, plain)
+        records = load_dir(str(tmp_path / "doors"))
+        by_region = {}
+        for r in records:
+            by_region.setdefault(r["region"], []).append(r)
+        # the doors the pass goes through, once per layer of their kind (no layer: the door does not know it) ...
+        gdn_layers = sum(not cfg.is_attention(i) for i in range(cfg.layers))
+        assert len([r for r in by_region["gdn.conv"] if r["layer"] is None]) == gdn_layers
+        assert len([r for r in by_region["attention.varlen"] if r["layer"] is None]) == cfg.layers - gdn_layers
+        assert len([r for r in by_region["moe.router"] if r["out"] == "0"]) == cfg.layers
+        assert {"gdn.core", "gdn.l2norm", "gdn.gating", "norms.gated_out", "norms.rms", "rope.rope", "moe.experts"} <= set(by_region)
+        assert "mm" not in by_region
+        # ... beside the runtime's own per-layer records
+        assert len([r for r in by_region["gdn.core"] if r["layer"] is not None]) == gdn_layers
+    finally:
+        install.uninstall_debug_hooks()
+        trace._forget_for_tests()
