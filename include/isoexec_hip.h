@@ -174,6 +174,27 @@ int ix_gemm_bf16_nt_decode(const void* A, long lda, const void* Wf, void* C, lon
 int ix_gemm_f32_nt(const void* A, int a_dtype, long lda, const void* W, long ldw, void* C, long ldc, long M,
                    long N, long K, void* stream);
 
+/* ---- Device memory that sleeps: ops/gdn/gdn_cpr_sleep.py --------------------------------------- */
+
+/* An arena is a range of device addresses that keeps its place while the memory behind it is given back and taken again
+ * (alloc_cpr_arena / cpr_sleep / cpr_wake_up, gdn_cpr_sleep.py:45-124, 217-282: the engine state of the boundary-form
+ * GatedDeltaNet layers is discarded at sleep without a host copy and mapped again at the same address at wake, so captured
+ * decode graphs stay valid). Built on the HIP virtual-memory calls; IX_DECLINED where the device does not support them.
+ * Set-up calls, not hot-path ones: they allocate, and release synchronises the device.
+ * ix_arena_create: `bytes` (rounded up to the allocation granularity) mapped and zeroed on `stream`, for the current
+ * device; IX_ERR_SIZE if the memory or the address range is not to be had.
+ * ix_arena_release_memory: device synchronised, memory unmapped and released; the addresses stay reserved. Touching the
+ * range before ix_arena_restore_memory has returned is a memory fault: the caller keeps tensors and graph replays away.
+ * ix_arena_restore_memory: fresh memory mapped at the same addresses and zeroed on `stream`.
+ * ix_arena_destroy: releases memory and addresses. Calls on an arena come from one thread at a time. */
+int ix_arena_create(size_t bytes, void** arena_out, void* stream);
+void* ix_arena_base(const void* arena);
+size_t ix_arena_bytes(const void* arena);
+int ix_arena_is_mapped(const void* arena);
+int ix_arena_release_memory(void* arena);
+int ix_arena_restore_memory(void* arena, void* stream);
+int ix_arena_destroy(void* arena);
+
 /* ---- GatedDeltaNet: ops/gdn/gdn_ops.py ----------------------------------------------------- */
 
 /* gdn_recurrent_kernel (gdn_ops.py:400-441): the delta-rule scan over packed tokens, state pool

@@ -64,6 +64,13 @@ SIGNATURES = {
         c_int,
         [P, c_long, c_long, P, c_long, c_long, P, c_long, c_long, c_long, c_long, c_long, c_long, c_int, P],
     ),
+    "ix_arena_create": (c_int, [c_size_t, P, P]),
+    "ix_arena_base": (P, [P]),
+    "ix_arena_bytes": (c_size_t, [P]),
+    "ix_arena_is_mapped": (c_int, [P]),
+    "ix_arena_release_memory": (c_int, [P]),
+    "ix_arena_restore_memory": (c_int, [P, P]),
+    "ix_arena_destroy": (c_int, [P]),
     "ix_gemm_decode_serves_shape": (c_int, [c_long, c_long]),
     "ix_gemm_pack_decode": (c_int, [P, c_long, P, c_long, c_long, P]),
     "ix_gemm_bf16_nt_decode": (c_int, [P, c_long, P, P, c_long, c_long, c_long, c_long, P]),

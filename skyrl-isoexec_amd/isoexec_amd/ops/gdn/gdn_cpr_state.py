@@ -25,9 +25,11 @@ Around that state, as in the reference:
   scheduler step. A miss is never a correctness event: the prompt is prefilled cold.
 * sleep (gdn_cpr_sleep.py:45-282): every layer's seven state tensors are views into one flat allocation, which
   ``cpr_sleep`` gives back to the device with no host copy and ``cpr_wake`` makes anew, zeroed, with every row released.
-  The store is dropped first, so nothing advertises a checkpoint no layer could continue from. The new allocation has a
-  new address: a decode graph captured before the sleep must be captured again (the reference's arena keeps its
-  virtual address through the engine's allocator; there is no such allocator in this package).
+  The store is dropped first, so nothing advertises a checkpoint no layer could continue from. With
+  ``SKYRL_ISOEXEC_GDN_CPR_SLEEP=1`` (the reference's switch) the allocation is a ``DeviceArena``: a reserved range of
+  device addresses whose memory is unmapped at sleep and mapped again at wake (``ix_arena_*``), so the state keeps its
+  address and a decode graph captured before the sleep replays after the wake. Without the switch it is an ordinary
+  allocation, the wake makes a new one at a new address, and such a graph has to be captured again.
 
 The reference's lazy boundary resync (``host_resync`` / ``layer_batched_resync``, gdn_cpr_state.py:295-358, 581-648)
 has no counterpart: it exists to keep a host-side position read out of the captured decode step, and here the boundary
@@ -269,18 +271,75 @@ def cpr_arena_specs(*, rows, C, HV, K, V, Hk, dt, gdt, conv_shape) -> list:
             ("v_buf", (rows, C, HV, V), dt), ("g_buf", (rows, C, HV), gdt), ("b_buf", (rows, C, HV), dt)]
 
 
-def _carve(specs, device):
-    """One zeroed flat allocation and the views the specs name, each on a 256-byte boundary."""
+_CPR_SLEEP_ENV = "SKYRL_ISOEXEC_GDN_CPR_SLEEP"
+
+
+def cpr_sleep_enabled() -> bool:
+    """True when the layers' state lives in an arena that keeps its address over a sleep (gdn_cpr_sleep.py:28-30)."""
+    return os.environ.get(_CPR_SLEEP_ENV, "0").strip().lower() not in _OFF
+
+
+class DeviceArena:
+    """A reserved range of device addresses; its memory can be released and restored (zeroed) in place."""
+
+    def __init__(self, nbytes: int, device):
+        self.device = torch.device(device)
+        handle = _lib.ctypes.c_void_p()
+        with torch.cuda.device(self.device):
+            rc = _lib.check(_lib.lib().ix_arena_create(int(nbytes), _lib.ctypes.byref(handle),
+                                                       _lib.current_stream(self.device)), "ix_arena_create")
+        if rc != _lib.IX_OK:
+            raise RuntimeError("[isoexec-gdn] this device does not support virtual-memory arenas; unset "
+                               f"{_CPR_SLEEP_ENV}")
+        self._handle = handle
+        self.base = int(_lib.lib().ix_arena_base(handle))
+        self.nbytes = int(_lib.lib().ix_arena_bytes(handle))
+
+    @property
+    def mapped(self) -> bool:
+        return bool(_lib.lib().ix_arena_is_mapped(self._handle))
+
+    @property
+    def __cuda_array_interface__(self):
+        return {"shape": (self.nbytes,), "typestr": "|u1", "data": (self.base, False), "version": 2}
+
+    def tensor(self) -> torch.Tensor:
+        """The arena's bytes as a tensor (no copy). Valid only while the memory is mapped."""
+        if not self.mapped:
+            raise RuntimeError("[isoexec-gdn] the arena's memory is released")
+        return torch.as_tensor(self, device=self.device)
+
+    def release_memory(self) -> None:
+        with torch.cuda.device(self.device):
+            _lib.check(_lib.lib().ix_arena_release_memory(self._handle), "ix_arena_release_memory")
+
+    def restore_memory(self) -> None:
+        with torch.cuda.device(self.device):
+            _lib.check(_lib.lib().ix_arena_restore_memory(self._handle, _lib.current_stream(self.device)),
+                       "ix_arena_restore_memory")
+
+    def destroy(self) -> None:
+        if self._handle is not None:
+            with torch.cuda.device(self.device):
+                _lib.check(_lib.lib().ix_arena_destroy(self._handle), "ix_arena_destroy")
+            self._handle = None
+
+
+def _carve(specs, device, arena: Optional[DeviceArena] = None, make_arena: bool = False):
+    """One zeroed flat allocation (an ordinary one, or a ``DeviceArena``'s bytes) and the views the specs name, each on a
+    256-byte boundary. Returns ``(flat, views, arena)``."""
     offsets, at = [], 0
     for _name, shape, dtype in specs:
         offsets.append(at)
         at += (int(np.prod(shape)) * torch.empty((), dtype=dtype).element_size() + 255) // 256 * 256
-    flat = torch.zeros(at, dtype=torch.uint8, device=device)
+    if arena is None and make_arena:
+        arena = DeviceArena(at, device)
+    flat = arena.tensor()[:at] if arena is not None else torch.zeros(at, dtype=torch.uint8, device=device)
     views = {}
     for (name, shape, dtype), off in zip(specs, offsets):
         n = int(np.prod(shape)) * torch.empty((), dtype=dtype).element_size()
         views[name] = flat[off:off + n].view(dtype).view(shape)
-    return flat, views
+    return flat, views, arena
 
 
 def cpr_arena_bytes(layers=None) -> int:
@@ -329,6 +388,8 @@ class CprGDN(RecurrentGDN):
                                             conv_shape=self.conv_state.shape)
         self._arena_device = dev
         self._flat_arena = None
+        self._device_arena = None              # a DeviceArena when the state keeps its address over a sleep
+        self._stable_address = cpr_sleep_enabled()
         self._restore_arena(release_rows=False)
         # row -> [(boundary position, fp32 entry state, convolution window)] stashed by the last prefill
         self._apc = cpr_apc_enabled()
@@ -353,12 +414,17 @@ class CprGDN(RecurrentGDN):
         for name, _shape, _dtype in self._arena_specs:
             setattr(self, name, None)
         self._apc_pending.clear()
+        if self._device_arena is not None:
+            self._device_arena.release_memory()  # synchronises the device first
         return size
 
     def _restore_arena(self, release_rows: bool = True) -> int:
         if self._flat_arena is not None:
             return 0
-        self._flat_arena, views = _carve(self._arena_specs, self._arena_device)
+        if self._device_arena is not None:
+            self._device_arena.restore_memory()  # the same addresses, fresh zeroed memory
+        self._flat_arena, views, self._device_arena = _carve(self._arena_specs, self._arena_device, self._device_arena,
+                                                             make_arena=self._stable_address)
         for name, view in views.items():
             setattr(self, name, view)
         if release_rows:  # what the rows held is gone: nobody may resume from them

@@ -351,3 +351,82 @@ def test_sleep_gives_the_state_back_and_wake_starts_from_nothing(monkeypatch):
         with pytest.raises(RuntimeError):
             ly.prefill(st, [1], *(t[32:] for t in req), [0, 8], has_initial_state=[True])   # nobody resumes over a sleep
         assert same_bits(ly.prefill(st, [1], *req, [0, 40]), o)    # the same request, cold, gives the same bits
+
+
+def test_arena_keeps_its_address_and_a_captured_step_replays_after_the_wake(monkeypatch):
+    """With SKYRL_ISOEXEC_GDN_CPR_SLEEP=1 the state lives in a reserved address range: sleep unmaps its memory (the
+    device's free memory grows by the arena), wake maps fresh zeroed memory at the same addresses, and a decode step
+    captured into a graph BEFORE the sleep replays AFTER the wake with the bits of an eager twin."""
+    from isoexec_amd.ops.gdn import gdn_cpr_state as cpr
+
+    monkeypatch.setenv("SKYRL_ISOEXEC_GDN_CPR_SLEEP", "1")
+    monkeypatch.setattr(cpr, "CPR_APC_STORE", cpr.CprBoundaryStore(1 << 20))
+    graphed = make_layer()
+    monkeypatch.delenv("SKYRL_ISOEXEC_GDN_CPR_SLEEP")
+    eager = make_layer()
+    assert graphed._device_arena is not None and eager._device_arena is None
+    names = ("ssm_state", "conv_state", "entry_state", "k_buf", "v_buf", "g_buf", "b_buf")
+    where = {n: getattr(graphed, n).data_ptr() for n in names}
+    assert where["ssm_state"] == graphed._device_arena.base and all(p % 256 == 0 for p in where.values())
+
+    slots, lens, total = [0, 1, 2], [5, 14, 16], 40
+    reqs = {s: request(500 + s, total) for s in slots}
+    st = torch.tensor(slots, dtype=torch.int64, device=DEV)
+    qsl = [0] + list(np.cumsum(lens))
+    packed = [torch.cat([reqs[s][j][:n] for s, n in zip(slots, lens)]) for j in range(3)]
+
+    def prefill(layer):
+        return layer.prefill(st, slots, *packed, qsl)
+
+    assert same_bits(prefill(graphed), prefill(eager))
+    have = dict(zip(slots, lens))
+    feed = lambda: tuple(torch.stack([reqs[s][j][have[s]] for s in slots]).contiguous() for j in range(3))
+    xs, as_, bs = feed()
+    assert same_bits(graphed.decode(st, xs.clone(), as_.clone(), bs.clone()), eager.decode(st, xs, as_, bs))  # warm
+    for s in slots:
+        have[s] += 1
+    sx, sa, sb = (t.clone() for t in feed())
+    graphed.flush_slot_map()
+    keep = [getattr(graphed, n).clone() for n in names] + [graphed.pos.clone(), graphed.last_used.clone(), graphed._clock.clone()]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = graphed.decode(st, sx, sa, sb)
+    for t, k in zip([getattr(graphed, n) for n in names] + [graphed.pos, graphed.last_used, graphed._clock], keep):
+        t.copy_(k)
+
+    def replay_steps(n):
+        for step in range(n):
+            xs, as_, bs = feed()
+            sx.copy_(xs); sa.copy_(as_); sb.copy_(bs)
+            graph.replay()
+            want = eager.decode(st, xs, as_, bs)
+            torch.cuda.synchronize()
+            assert same_bits(out, want), step
+            for s in slots:
+                have[s] += 1
+
+    replay_steps(6)
+    # ---- sleep: the memory goes back to the device, the addresses stay
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    size = cpr.cpr_sleep([graphed])
+    assert size > 0 and graphed.asleep and not graphed._device_arena.mapped
+    assert torch.cuda.mem_get_info()[0] >= free_before + graphed._device_arena.nbytes - (2 << 20)
+    with pytest.raises(RuntimeError, match="cpr_wake"):
+        graphed.decode(st, sx, sa, sb)
+    # ---- wake: zeroed state at the same addresses, every row released; the same requests start over on both layers
+    assert cpr.cpr_wake([graphed]) == size and graphed._device_arena.mapped
+    assert {n: getattr(graphed, n).data_ptr() for n in names} == where
+    assert not graphed.ssm_state.any() and not graphed.k_buf.any() and len(graphed.table) == 0
+    eager.reset()
+    assert same_bits(prefill(graphed), prefill(eager))
+    for s, n in zip(slots, lens):
+        have[s] = n
+    graphed.flush_slot_map()
+    replay_steps(20)                                               # the graph captured before the sleep, across boundaries
+    for t, u in ((graphed.ssm_state, eager.ssm_state), (graphed.entry_state, eager.entry_state), (graphed.pos, eager.pos)):
+        assert same_bits(t, u)
+    # ---- the arena ends with an explicit call (nothing may view it any more)
+    arena = graphed._device_arena
+    cpr.cpr_sleep([graphed])
+    arena.destroy()
