@@ -298,6 +298,15 @@ int ix_gdn_conv(const void* x, long x_pitch, const void* weight, const void* bia
                 const int* cu_seqlens, const int* state_rows_in, const int* state_rows_out, long N,
                 long total_tokens, long D, long W, int silu, void* stream);
 
+/* ix_gdn_conv with gdn_l2norm (gdn_ops.py:173-188) of the q and k heads folded into its epilogue, as the fused core does
+ * in front of its scan (gdn_ops.py:513-558): channels [0, qk_channels) of y are heads of K channels and leave normalised
+ * with `eps`, the others as ix_gdn_conv leaves them. The bits of ix_gdn_conv followed by ix_gdn_l2norm on those columns.
+ * Serves K = 128, W = 4, D and qk_channels multiples of 128, x_pitch a multiple of 8, 16-byte aligned operands; IX_DECLINED
+ * otherwise (the caller makes the two calls). */
+int ix_gdn_conv_l2norm(const void* x, long x_pitch, const void* weight, const void* bias, void* y, void* conv_pool,
+                       const int* cu_seqlens, const int* state_rows_in, const int* state_rows_out, long N,
+                       long total_tokens, long D, long W, int silu, long qk_channels, long K, float eps, void* stream);
+
 /* ---- MoE: ops/moe ------------------------------------------------------------------------- */
 
 /* fused_router_dense / ref_router_dense (moe_router_o2_kernel.py:272-311,369-386) with mode 0;

@@ -785,12 +785,31 @@ __device__ __forceinline__ void ix_conv8_finish(const float (&xv)[W][8], const f
 }
 
 
-template <int W, int TOK>
+// The l2norm of a q or k head (K = 128: sixteen lanes of eight channels) on the bf16 values the convolution just
+// rounded -- k_gdn_l2norm<16>'s expression on what it would have read back: squares, ix_tree8, the adjacent-pairwise
+// tree over the sixteen lanes, one IEEE rsqrt, bf16(x * r). Every lane of the sixteen must be here.
+__device__ __forceinline__ void ix_l2norm8_of16(bf16_t* __restrict__ yrow, float eps) {
+  float v8[8], sq[8];
+  ix_unpack8(*reinterpret_cast<const uint4*>(yrow), v8);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) sq[i] = v8[i] * v8[i];
+  const float ssum = ix_lane_tree<16>(ix_tree8(sq));
+  const float rn = ix_rsqrt_ieee(ssum + eps);
+  __attribute__((aligned(16))) bf16_t out[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) out[i] = ix_f2bf(v8[i] * rn);
+  *reinterpret_cast<uint4*>(yrow) = *reinterpret_cast<const uint4*>(out);
+}
+
+// NORM: channels below qk_channels are q and k heads of 128 and leave normalised (ix_gdn_conv_l2norm); a head's sixteen
+// threads are consecutive and share the token group, so they take the same path through the kernel.
+template <int W, int TOK, bool NORM>
 __global__ __launch_bounds__(256) void k_gdn_conv8(const bf16_t* __restrict__ x, long x_pitch,
                                                    const bf16_t* __restrict__ w, const bf16_t* __restrict__ bias,
                                                    bf16_t* __restrict__ y, const bf16_t* __restrict__ pool,
                                                    const int* __restrict__ cu, const int* __restrict__ rows_in,
-                                                   int N, long D, int silu, int T, long total) {
+                                                   int N, long D, int silu, int T, long total, long qk_channels,
+                                                   float eps) {
   const long i = ((long)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
   if (i >= total) return;
   const long D8 = D >> 3;
@@ -834,7 +853,14 @@ __global__ __launch_bounds__(256) void k_gdn_conv8(const bf16_t* __restrict__ x,
       float xv[W][8];
 #pragma unroll
       for (int j = 0; j < W; ++j) ix_unpack8(xr[q + j], xv[j]);
-      ix_conv8_finish<W>(xv, wv, has_bias, bv, silu, y + (long)(t0 + q) * D + d);
+      if constexpr (NORM) {
+        __attribute__((aligned(16))) bf16_t yv[8];
+        ix_conv8_finish<W>(xv, wv, has_bias, bv, silu, yv);
+        if (d < qk_channels) ix_l2norm8_of16(yv, eps);
+        *reinterpret_cast<uint4*>(y + (long)(t0 + q) * D + d) = *reinterpret_cast<const uint4*>(yv);
+      } else {
+        ix_conv8_finish<W>(xv, wv, has_bias, bv, silu, y + (long)(t0 + q) * D + d);
+      }
     }
     return;
   }
@@ -857,7 +883,14 @@ __global__ __launch_bounds__(256) void k_gdn_conv8(const bf16_t* __restrict__ x,
           xv[j][c] = srow > 0 ? ix_bf2f(pool[((long)srow * D + d + c) * (W - 1) + (W - 1 + r)]) : 0.0f;
       }
     }
-    ix_conv8_finish<W>(xv, wv, has_bias, bv, silu, y + (long)t * D + d);
+    if constexpr (NORM) {
+      __attribute__((aligned(16))) bf16_t yv[8];
+      ix_conv8_finish<W>(xv, wv, has_bias, bv, silu, yv);
+      if (d < qk_channels) ix_l2norm8_of16(yv, eps);
+      *reinterpret_cast<uint4*>(y + (long)t * D + d) = *reinterpret_cast<const uint4*>(yv);
+    } else {
+      ix_conv8_finish<W>(xv, wv, has_bias, bv, silu, y + (long)t * D + d);
+    }
   }
 }
 
@@ -883,10 +916,10 @@ __global__ __launch_bounds__(256) void k_gdn_conv_state(const bf16_t* __restrict
   for (int j = 0; j < W - 1; ++j) pool[((long)orow * D + d) * (W - 1) + j] = tmp[j];
 }
 
-extern "C" int ix_gdn_conv(const void* x, long x_pitch, const void* weight, const void* bias, void* y,
-                           void* conv_pool, const int* cu_seqlens, const int* state_rows_in,
-                           const int* state_rows_out, long N, long total_tokens, long D, long W, int silu,
-                           void* stream) {
+static int ix_gdn_conv_impl(const void* x, long x_pitch, const void* weight, const void* bias, void* y,
+                            void* conv_pool, const int* cu_seqlens, const int* state_rows_in,
+                            const int* state_rows_out, long N, long total_tokens, long D, long W, int silu,
+                            long qk_channels, float eps, void* stream) {
   if (!x || !weight || !y || !cu_seqlens || N < 0 || total_tokens < 0 || D <= 0 || x_pitch < D) return IX_ERR_ARG;
   if (W < 1 || W > 8) return IX_DECLINED;
   if ((state_rows_in || state_rows_out) && !conv_pool) return IX_ERR_ARG;
@@ -899,6 +932,7 @@ extern "C" int ix_gdn_conv(const void* x, long x_pitch, const void* weight, cons
     // Outputs per thread: long sequences amortise the W - 1 rows of history over 16 outputs; short ones (a decode
     // step has one token per sequence) keep one output per thread so the launch stays wide. Every output is
     // computed by the same expression whichever is chosen.
+    if (qk_channels > 0 && !vec8) return IX_DECLINED;  // the normalising form is the eight-channel kernel's
     const long avg_len = total_tokens / N;
     const int TOK = !vec8 ? 1 : avg_len >= 64 ? 16 : avg_len >= 8 ? 4 : 1;
     const long work = vec8 ? ((total_tokens + TOK - 1) / TOK) * (D / 8) : total;
@@ -906,14 +940,19 @@ extern "C" int ix_gdn_conv(const void* x, long x_pitch, const void* weight, cons
     const long gx = blocks < (1L << 22) ? blocks : (1L << 22);
     const long gy = (blocks + gx - 1) / gx;
     if (gy > 65535) return IX_DECLINED;
-#define IX_CONV8(TOK_)                                                                                              \
-  hipLaunchKernelGGL((k_gdn_conv8<4, TOK_>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st, (const bf16_t*)x,  \
-                     x_pitch, (const bf16_t*)weight, (const bf16_t*)bias, (bf16_t*)y, (const bf16_t*)conv_pool,     \
-                     cu_seqlens, state_rows_in, (int)N, D, silu, (int)total_tokens, work)
-    if (vec8) {
-      if (TOK == 16) IX_CONV8(16);
-      else if (TOK == 4) IX_CONV8(4);
-      else IX_CONV8(1);
+#define IX_CONV8(TOK_, NORM_)                                                                                       \
+  hipLaunchKernelGGL((k_gdn_conv8<4, TOK_, NORM_>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,             \
+                     (const bf16_t*)x, x_pitch, (const bf16_t*)weight, (const bf16_t*)bias, (bf16_t*)y,             \
+                     (const bf16_t*)conv_pool, cu_seqlens, state_rows_in, (int)N, D, silu, (int)total_tokens, work, \
+                     qk_channels, eps)
+    if (vec8 && qk_channels > 0) {
+      if (TOK == 16) IX_CONV8(16, true);
+      else if (TOK == 4) IX_CONV8(4, true);
+      else IX_CONV8(1, true);
+    } else if (vec8) {
+      if (TOK == 16) IX_CONV8(16, false);
+      else if (TOK == 4) IX_CONV8(4, false);
+      else IX_CONV8(1, false);
     }
 #undef IX_CONV8
     else
@@ -928,6 +967,28 @@ extern "C" int ix_gdn_conv(const void* x, long x_pitch, const void* weight, cons
                        (bf16_t*)conv_pool, cu_seqlens, state_rows_in, state_rows_out, (int)N, D, (int)W);
   }
   return ix_launch_status();
+}
+
+extern "C" int ix_gdn_conv(const void* x, long x_pitch, const void* weight, const void* bias, void* y,
+                           void* conv_pool, const int* cu_seqlens, const int* state_rows_in,
+                           const int* state_rows_out, long N, long total_tokens, long D, long W, int silu,
+                           void* stream) {
+  return ix_gdn_conv_impl(x, x_pitch, weight, bias, y, conv_pool, cu_seqlens, state_rows_in, state_rows_out, N,
+                          total_tokens, D, W, silu, 0, 0.0f, stream);
+}
+
+// ix_gdn_conv with the l2norm of the q and k heads folded into its epilogue: channels [0, qk_channels) of y are heads of
+// K = 128 and leave normalised (the bits of ix_gdn_conv followed by ix_gdn_l2norm over those columns), the rest (v) as
+// ix_gdn_conv leaves them. Serves the eight-channel form only: W = 4, D and x_pitch multiples of 8, 16-byte aligned
+// operands, qk_channels a multiple of 128; bf16.
+extern "C" int ix_gdn_conv_l2norm(const void* x, long x_pitch, const void* weight, const void* bias, void* y,
+                                  void* conv_pool, const int* cu_seqlens, const int* state_rows_in,
+                                  const int* state_rows_out, long N, long total_tokens, long D, long W, int silu,
+                                  long qk_channels, long K, float eps, void* stream) {
+  if (qk_channels <= 0 || qk_channels > D || K <= 0) return IX_ERR_ARG;
+  if (K != 128 || (qk_channels % 128) || (D % 128) || W != 4) return IX_DECLINED;
+  return ix_gdn_conv_impl(x, x_pitch, weight, bias, y, conv_pool, cu_seqlens, state_rows_in, state_rows_out, N,
+                          total_tokens, D, W, silu, qk_channels, eps, stream);
 }
 
 // ---------------------------------------------------------------------------------------------

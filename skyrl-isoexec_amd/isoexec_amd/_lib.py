@@ -88,6 +88,8 @@ SIGNATURES = {
     "ix_gdn_decode_prep": (c_int, [P, c_long, P, c_long, P, c_long, P, P, P, P, P, P, P, P, P, c_long, c_long, c_long, c_long,
                                    c_long, c_long, c_int, c_float, P]),
     "ix_gdn_conv": (c_int, [P, c_long, P, P, P, P, P, P, P, c_long, c_long, c_long, c_long, c_int, P]),
+    "ix_gdn_conv_l2norm": (c_int, [P, c_long, P, P, P, P, P, P, P, c_long, c_long, c_long, c_long, c_int, c_long, c_long,
+                                   c_float, P]),
     "ix_attn_varlen": (c_int, [P, c_long, P, P, c_long, P, P, P, P, c_long, c_long, c_long, c_long, c_long, c_float, P]),
     "ix_rope_inplace": (c_int, [P, c_long, P, P, c_long, P, c_long, c_long, c_long, c_long, P]),
     "ix_moe_router_topk": (c_int, [P, c_long, c_long, c_long, c_long, c_int, c_float, P, P, P, P, P]),

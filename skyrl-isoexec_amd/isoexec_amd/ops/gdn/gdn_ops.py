@@ -215,8 +215,13 @@ def decode_prep(x, a, b, conv_weight, conv_bias, A_log, dt_bias, conv_state, row
     return (y, g, beta) if rc == _lib.IX_OK else None
 
 
-def conv_packed(x, weight, bias, *, cu_seqlens, conv_state=None, rows_in=None, rows_out=None, activation="silu"):
-    """Packed varlen conv: ``x [T, D]`` -> ``y [T, D]``; optional pool rows for history in/out."""
+def conv_packed(x, weight, bias, *, cu_seqlens, conv_state=None, rows_in=None, rows_out=None, activation="silu",
+                l2norm_qk: int = 0, head_k_dim: int = 0):
+    """Packed varlen conv: ``x [T, D]`` -> ``y [T, D]``; optional pool rows for history in/out.
+
+    ``l2norm_qk`` > 0: channels ``[0, l2norm_qk)`` of ``y`` are q and k heads of ``head_k_dim`` channels and leave
+    L2-normalised, in the same launch (the bits of ``gdn_l2norm`` on those columns of the plain result); ``None`` is
+    returned when the library does not serve that form for these shapes (the caller makes the two calls)."""
     _lib.require_device(x, weight, bias, cu_seqlens, conv_state, rows_in, rows_out)
     if activation not in (None, "silu", "swish"):
         raise ValueError(f"unsupported activation {activation!r}")
@@ -231,9 +236,16 @@ def conv_packed(x, weight, bias, *, cu_seqlens, conv_state=None, rows_in=None, r
     wc = weight.contiguous()
     y = torch.empty(T, D, dtype=x.dtype, device=x.device)
     n_seq = cu_seqlens.numel() - 1
+    bc = None if bias is None else bias.contiguous()
+    if l2norm_qk:
+        rc = _lib.check(
+            _lib.lib().ix_gdn_conv_l2norm(xc.data_ptr(), xc.stride(0), wc.data_ptr(), _lib.ptr(bc), y.data_ptr(),
+                                          _lib.ptr(conv_state), cu_seqlens.data_ptr(), _lib.ptr(rows_in), _lib.ptr(rows_out),
+                                          n_seq, T, D, W, int(activation is not None), int(l2norm_qk), int(head_k_dim),
+                                          L2NORM_EPS, _lib.current_stream(x.device)), "ix_gdn_conv_l2norm")
+        return y if rc == _lib.IX_OK else None
     rc = _lib.check(
-        _lib.lib().ix_gdn_conv(xc.data_ptr(), xc.stride(0), wc.data_ptr(),
-                               _lib.ptr(None if bias is None else bias.contiguous()), y.data_ptr(), _lib.ptr(conv_state),
+        _lib.lib().ix_gdn_conv(xc.data_ptr(), xc.stride(0), wc.data_ptr(), _lib.ptr(bc), y.data_ptr(), _lib.ptr(conv_state),
                                cu_seqlens.data_ptr(), _lib.ptr(rows_in), _lib.ptr(rows_out), n_seq, T, D, W,
                                int(activation is not None), _lib.current_stream(x.device)), "ix_gdn_conv")
     if rc != _lib.IX_OK:
@@ -372,6 +384,18 @@ def gdn_native_core_kernel(q, k, v, a, b, A_log, dt_bias, *, ssm_state, state_in
     lead = v.shape[:2]
     return gdn_recurrent_kernel(qn, kn, v, g.view(*lead, HV), beta.view(*lead, HV), ssm_state=ssm_state,
                                 state_indices=state_indices, cu_seqlens=cu_seqlens)
+
+
+def gdn_native_core_normed(qn, kn, v, a, b, A_log, dt_bias, *, cu_seqlens=None):
+    """``gdn_native_core`` for q and k that are normalised already (``conv_packed(..., l2norm_qk=...)``): the gating and
+    the scan of the same composition, without its two l2norm launches. Same bits as ``gdn_native_core`` on the raw heads."""
+    with torch.no_grad():
+        ssm_state, idx = _recurrent_scratch_state(qn, v, cu_seqlens)
+        HV = v.shape[-2]
+        g, beta = gate_and_beta_fp32(a.reshape(-1, HV), b.reshape(-1, HV), A_log, dt_bias)
+        lead = v.shape[:2]
+        return gdn_recurrent_kernel(qn, kn, v, g.view(*lead, HV), beta.view(*lead, HV), ssm_state=ssm_state,
+                                    state_indices=idx, cu_seqlens=cu_seqlens)
 
 
 def gdn_native_core(q, k, v, a, b, A_log, dt_bias, *, cu_seqlens=None):

@@ -518,9 +518,16 @@ class RecurrentGDN:
             cu = torch.from_numpy(np.asarray(qsl, dtype=np.int32)).to(dev, non_blocking=True)
         # A fresh row must start from zero; a resumed row keeps what the previous chunk left.
         self._zero_fresh_rows(meta_t[2].long())
+        # q and k leave the convolution's launch normalised where the library serves that form (the same bits)
         y = conv_packed(x, self.conv_weight, self.conv_bias, cu_seqlens=cu, conv_state=self.conv_state,
-                        rows_in=rows_in, rows_out=rows_out, activation=self.activation)
-        q, k, v = self._split_qkv(y)
+                        rows_in=rows_in, rows_out=rows_out, activation=self.activation,
+                        l2norm_qk=2 * self.num_k_heads * self.head_k_dim, head_k_dim=self.head_k_dim)
+        if y is not None:
+            q, k, v = self._split_qkv_raw(y)
+        else:
+            y = conv_packed(x, self.conv_weight, self.conv_bias, cu_seqlens=cu, conv_state=self.conv_state,
+                            rows_in=rows_in, rows_out=rows_out, activation=self.activation)
+            q, k, v = self._split_qkv(y)
         g, beta = self._gate_and_beta(a, b)
         return rows, is_cont, rows_out, cu, q, k, v, g, beta
 

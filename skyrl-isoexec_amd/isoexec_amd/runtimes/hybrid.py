@@ -24,7 +24,7 @@ import torch
 
 from ..debug.trace import get_tracer
 from ..ops.attention.varlen_attn import KVCache, varlen_attention
-from ..ops.gdn.gdn_ops import conv_packed, gdn_native_core
+from ..ops.gdn.gdn_ops import conv_packed, gdn_native_core, gdn_native_core_normed
 from ..ops.gdn.gdn_cpr import gdn_native_cpr_fwd
 from ..ops.gdn.gdn_cpr_state import CprGDN
 from ..ops.gdn.gdn_recurrent_state import RecurrentGDN
@@ -351,8 +351,13 @@ class TrainerModel:
                 q, k, v = b.attn_qkv(i, x, positions)
                 return b.attn_out(i, varlen_attention(q, k, v, cu, max_len))
             qkv, z, bb, a = b.gdn_in(i, x)
-            y = conv_packed(qkv, lw["conv_weight"], lw["conv_bias"], cu_seqlens=cu)
             kd = c.gdn_k_heads * c.gdn_head_dim
+            # the recurrent form takes q and k normalised by the convolution's own launch where the library serves it
+            normed = None
+            if c.gdn_kernel != "cpr":
+                normed = conv_packed(qkv, lw["conv_weight"], lw["conv_bias"], cu_seqlens=cu, l2norm_qk=2 * kd,
+                                     head_k_dim=c.gdn_head_dim)
+            y = normed if normed is not None else conv_packed(qkv, lw["conv_weight"], lw["conv_bias"], cu_seqlens=cu)
             q = y[:, :kd].unflatten(1, (c.gdn_k_heads, c.gdn_head_dim))
             k = y[:, kd : 2 * kd].unflatten(1, (c.gdn_k_heads, c.gdn_head_dim))
             v = y[:, 2 * kd :].unflatten(1, (c.gdn_v_heads, c.gdn_head_dim))
@@ -360,7 +365,8 @@ class TrainerModel:
                 o = gdn_native_cpr_fwd(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), a, bb, lw["A_log"], lw["dt_bias"],
                                        cu_seqlens=cu, chunk_size=c.gdn_chunk)
             else:
-                o = gdn_native_core(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), a, bb, lw["A_log"], lw["dt_bias"], cu_seqlens=cu)
+                core = gdn_native_core_normed if normed is not None else gdn_native_core
+                o = core(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), a, bb, lw["A_log"], lw["dt_bias"], cu_seqlens=cu)
             return b.gdn_out(i, o[0], z)
 
         return b.run_layers(b.embed(tokens), mixer)

@@ -309,3 +309,47 @@ def test_fused_decode_prep_equals_the_three_launches_bit_for_bit():
     assert decode_prep(x.float(), a_in, b_in, cw, cb, A_log, dt_bias, pool_b, rows, H=H, K=K, HV=HV, V=V) is None
     assert decode_prep(x[:, :2 * 2 * 64 + HV * V], a_in, b_in, cw[:2 * 2 * 64 + HV * V], None, A_log, dt_bias, pool_b, rows,
                        H=2, K=64, HV=HV, V=V) is None
+
+
+@pytest.mark.parametrize("H,HV", [(2, 2), (16, 32)])
+def test_conv_with_the_l2norm_folded_in_equals_the_two_launches(H, HV):
+    """``conv_packed(..., l2norm_qk=...)``: q and k heads leave the convolution's launch normalised. Against the plain
+    convolution followed by ``gdn_l2norm`` on those columns, bit for bit: long and very short sequences in one packed
+    batch (both paths through the kernel), an input that is a column slice of a wider buffer, history rows in and out."""
+    from isoexec_amd.ops.gdn.gdn_ops import conv_packed, gdn_l2norm, gdn_native_core, gdn_native_core_normed
+
+    K = V = 128
+    W = 4
+    kd = H * K
+    D = 2 * kd + HV * V
+    g = cpu_gen(70 + H)
+    lens = [300, 1, 2, 70, 3, 5, 129]
+    T = sum(lens)
+    wide = torch.randn(T, D + 64, generator=g).to(torch.bfloat16).to(DEV)
+    x = wide[:, :D]
+    weight = (torch.randn(D, W, generator=g) * 0.4).to(torch.bfloat16).to(DEV)
+    bias = (torch.randn(D, generator=g) * 0.1).to(torch.bfloat16).to(DEV)
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32, device=DEV)
+    n = len(lens)
+    pools = [(torch.randn(n + 1, D, W - 1, generator=cpu_gen(9)).to(torch.bfloat16).to(DEV)) for _ in range(2)]
+    rows_in = torch.tensor([1, 0, 3, 0, 5, 6, 0], dtype=torch.int32, device=DEV)   # some sequences continue a stored window
+    rows_out = torch.arange(1, n + 1, dtype=torch.int32, device=DEV)
+    plain = conv_packed(x, weight, bias, cu_seqlens=cu, conv_state=pools[0], rows_in=rows_in, rows_out=rows_out)
+    fused = conv_packed(x, weight, bias, cu_seqlens=cu, conv_state=pools[1], rows_in=rows_in, rows_out=rows_out,
+                        l2norm_qk=2 * kd, head_k_dim=K)
+    assert fused is not None and same_bits(pools[0], pools[1])
+    want_qk = gdn_l2norm(plain[:, :2 * kd].unflatten(1, (2 * H, K)))
+    assert same_bits(fused[:, :2 * kd].unflatten(1, (2 * H, K)).contiguous(), want_qk)
+    assert same_bits(fused[:, 2 * kd:].contiguous(), plain[:, 2 * kd:].contiguous())
+    # the composition the trainer runs: raw heads through gdn_native_core == normalised heads through its _normed form
+    a = torch.randn(T, HV, generator=g).to(torch.bfloat16).to(DEV)
+    b = torch.randn(T, HV, generator=g).to(torch.bfloat16).to(DEV)
+    A_log = (torch.randn(HV, generator=g) * 0.3).to(DEV)
+    dt_bias = (torch.randn(HV, generator=g) * 0.3).to(DEV)
+    split = lambda y: (y[:, :kd].unflatten(1, (H, K)).unsqueeze(0), y[:, kd:2 * kd].unflatten(1, (H, K)).unsqueeze(0),
+                       y[:, 2 * kd:].unflatten(1, (HV, V)).unsqueeze(0))
+    o_raw = gdn_native_core(*split(plain), a, b, A_log, dt_bias, cu_seqlens=cu)
+    o_normed = gdn_native_core_normed(*split(fused), a, b, A_log, dt_bias, cu_seqlens=cu)
+    assert same_bits(o_raw, o_normed)
+    # heads of another size are not served: the caller makes the two calls
+    assert conv_packed(x, weight, bias, cu_seqlens=cu, l2norm_qk=2 * kd, head_k_dim=64) is None
