@@ -22,7 +22,6 @@
 #define IX_MOE_EC 8  // experts per lane: E <= 512
 #define IX_MOE_TILE_T 256
 #define IX_MOE_EMAX 512
-#define IX_MOE_SCAN_TILES 16
 
 // ---------------------------------------------------------------------------------------------
 __device__ __forceinline__ bool ix_beats(float av, int ai, float bv, int bi, int sentinel) {
@@ -344,39 +343,42 @@ __global__ __launch_bounds__(256) void k_moe_tile_counts(const int* __restrict__
   }
 }
 
+// Per expert, the running sum of its counts over the token tiles (tile_base[t][e] = rows of expert e in tiles before t)
+// and its total. One wave per expert: a lane owns a run of consecutive tiles, sums it, the lanes' sums are scanned across
+// the wave, then the lane walks its run again writing the bases. Integer only.
+__global__ __launch_bounds__(256) void k_moe_tile_prefix(const int* __restrict__ tile_counts, int ntiles, int E,
+                                                         int* __restrict__ tile_base, int* __restrict__ counts) {
+  const int e = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (e >= E) return;  // whole waves leave together
+  const int lane = threadIdx.x & 63;
+  const int per = (ntiles + 63) >> 6;
+  const int t_lo = min(lane * per, ntiles), t_hi = min(t_lo + per, ntiles);
+  int mine = 0;
+  for (int t = t_lo; t < t_hi; ++t) mine += tile_counts[(long)t * E + e];
+  int incl = mine;  // inclusive scan over the lanes
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int up = __shfl_up(incl, d, 64);
+    if (lane >= d) incl += up;
+  }
+  int run = incl - mine;
+  for (int t = t_lo; t < t_hi; ++t) {
+    const int c = tile_counts[(long)t * E + e];
+    tile_base[(long)t * E + e] = run;
+    run += c;
+  }
+  if (lane == 63) counts[e] = incl;
+}
+
 // meta layout: [0] = number of m-tiles, then tile_expert[max_tiles], tile_row0[max_tiles],
-// tile_nrows[max_tiles]. One workgroup: per-expert running sums over the token tiles (staged
-// through LDS 64 tiles at a time), an exclusive scan over the experts in LDS, then every expert
-// writes its own row tiles.
-__global__ __launch_bounds__(256) void k_moe_offsets(const int* __restrict__ tile_counts, int ntiles, int E,
-                                                     int BM, int max_tiles, int* __restrict__ tile_base,
-                                                     int* __restrict__ counts, int* __restrict__ offsets,
-                                                     int* __restrict__ meta) {
-  __shared__ int s_stage[IX_MOE_SCAN_TILES * IX_MOE_EMAX];
+// tile_nrows[max_tiles]. One workgroup, after k_moe_tile_prefix has left every expert's row count in `counts`: an
+// exclusive scan over the experts in LDS, then every expert writes its own row tiles.
+__global__ __launch_bounds__(256) void k_moe_offsets(int E, int BM, int max_tiles, const int* __restrict__ counts,
+                                                     int* __restrict__ offsets, int* __restrict__ meta) {
   __shared__ int s_cnt[IX_MOE_EMAX], s_off[IX_MOE_EMAX + 1], s_toff[IX_MOE_EMAX + 1];
   const int tid = threadIdx.x;
-  for (int e = tid; e < E; e += 256) s_cnt[e] = 0;
+  for (int e = tid; e < E; e += 256) s_cnt[e] = counts[e];
   __syncthreads();
-  // as many token tiles per stage as the staging array holds for this E (64 for 128 experts): each stage costs a
-  // round trip to memory and three barriers
-  const int stage_tiles = (IX_MOE_SCAN_TILES * IX_MOE_EMAX) / E;
-  for (int t0 = 0; t0 < ntiles; t0 += stage_tiles) {
-    const int nt = min(stage_tiles, ntiles - t0);
-    for (int i = tid; i < nt * E; i += 256) s_stage[i] = tile_counts[(long)t0 * E + i];
-    __syncthreads();
-    for (int e = tid; e < E; e += 256) {
-      int run = s_cnt[e];
-      for (int t = 0; t < nt; ++t) {
-        const int c = s_stage[t * E + e];
-        s_stage[t * E + e] = run;
-        run += c;
-      }
-      s_cnt[e] = run;
-    }
-    __syncthreads();
-    for (int i = tid; i < nt * E; i += 256) tile_base[(long)t0 * E + i] = s_stage[i];
-    __syncthreads();
-  }
   // exclusive scan over the experts (rows and row tiles): lane owns experts 2 tid and 2 tid + 1 (E <= 512)
   {
     __shared__ int s_rows[256], s_tiles[256];
@@ -420,7 +422,6 @@ __global__ __launch_bounds__(256) void k_moe_offsets(const int* __restrict__ til
   int* tile_nrows = tile_row0 + max_tiles;
   for (int e = tid; e < E; e += 256) {
     const int c = s_cnt[e];
-    counts[e] = c;
     offsets[e] = s_off[e];
     int nt = s_toff[e];
     for (int r0 = 0; r0 < c && nt < max_tiles; r0 += BM, ++nt) {
@@ -715,8 +716,10 @@ extern "C" int ix_moe_permute(const int* topk_idx, const float* topk_prob, long 
   if (ntiles > 0)
     hipLaunchKernelGGL(k_moe_tile_counts, dim3((unsigned)ntiles), dim3(256), 0, st, topk_idx, (int)T, (int)E, (int)k,
                        tile_counts);
-  hipLaunchKernelGGL(k_moe_offsets, dim3(1), dim3(256), 0, st, tile_counts, (int)ntiles, (int)E, (int)BM,
-                     (int)max_tiles, tile_base, counts, offsets, tile_meta);
+  hipLaunchKernelGGL(k_moe_tile_prefix, dim3((unsigned)((E + 3) / 4)), dim3(256), 0, st, tile_counts, (int)ntiles, (int)E,
+                     tile_base, counts);
+  hipLaunchKernelGGL(k_moe_offsets, dim3(1), dim3(256), 0, st, (int)E, (int)BM, (int)max_tiles, counts, offsets,
+                     tile_meta);
   if (ntiles > 0)
     hipLaunchKernelGGL(k_moe_scatter, dim3((unsigned)ntiles), dim3(256), 0, st, topk_idx, topk_prob, (int)T, (int)E,
                        (int)k, tile_base, offsets, sorted_token, permuted_prob, combine_rows);
@@ -748,7 +751,7 @@ extern "C" int ix_moe_route_one_tile(const float* logits, long ld, long T, long 
 // the library runs on holds its own copy of the array, at its own address, until the process ends; the address is
 // resolved once per device, with that device current, on the first call there. Kernels receive that address as an
 // argument, exactly as they receive the caller's workspace in ix_moe_permute. Both tables are fully rewritten by
-// every call before they are read (k_moe_tile_counts writes [ntiles, E], k_moe_offsets writes the bases), so nothing
+// every call before they are read (k_moe_tile_counts writes [ntiles, E], k_moe_tile_prefix writes the bases), so nothing
 // has to start at zero; two calls that overlap on one GPU share the array and race.
 #define IX_MOE_STATIC_SCRATCH_INTS (256 * 1024)  // 1 MiB: 2 * ceil(T / 256) * E ints, e.g. 262,144 tokens at E = 128
 #define IX_MAX_DEVICES 64
