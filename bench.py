@@ -402,7 +402,8 @@ def north_star_kernels(w, dev, steps):
         out[f"lm_head_gemm_M{m_small}_K4096"] = {
             "bound": "hbm", "kernel": "k_gemm_dec (weights streamed from the packed copy)", "kernel_ms": ms,
             "achieved": by / ms / 1e6, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": by / ms / 1e6 / PEAK_HBM_GBS,
-            "traffic": None}
+            "traffic": {16: 1.255e9, 64: 1.285e9}[m_small],
+            "traffic_source": "profiles/gemm_dec__lm_head_M16_M64_K4096.txt (not measured in this run)"}
     del packed
     logits, row_max = gemm()
     ms = _events_ms(lambda: sampled_forward(logits, target, 8, row_max=row_max), 3, max(steps, 20))
@@ -513,17 +514,28 @@ def gemm(args):
     profiles of the large products run): ``value`` = TFLOP/s, HIP events around each call."""
     import torch
 
-    from isoexec_amd.ops.mm.mm_hip import linear_nt
+    from isoexec_amd.ops.mm.mm_hip import linear_nt, pack_nt_decode
 
     dev = "cuda:0"
     g = host_gen(21)
     M, K, N = args.m, args.k, args.n
     a = hrandn((M, K), g, dev)
     w = hrandn((N, K), g, dev, std=0.02)
+    if args.packed:  # at most 64 rows: the weight is streamed from its fragment-packed copy
+        w = pack_nt_decode(w)
+        if w is None or M > 64:
+            raise SystemExit("--packed serves m <= 64, n a multiple of 32 and k in {1024, 2048, 3072, 4096}")
     fn = lambda: linear_nt(a, w, tile=args.tile, want_row_max=args.row_max)
     ms = _events_ms(fn, args.warmup, args.steps)
     fl = 2.0 * M * N * K
     algo = 2.0 * (M * K + N * K + M * N)
+    if args.packed:
+        return {"metric": "dense GEMM GB/s (weights streamed)", "value": algo / ms / 1e6, "unit": "GB/s", "n_gpus": 1,
+                "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
+                "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+                "config": {"workload": f"gemm_bf16_nt_decode {M} x {K} x {N} (packed weight)"},
+                "roofline": {"bound": "hbm", "achieved": algo / ms / 1e6, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                             "frac": algo / ms / 1e6 / PEAK_HBM_GBS, "traffic": None, "algorithmic_bytes": algo}}
     return {"metric": "dense GEMM TFLOP/s", "value": fl / ms / 1e9, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
             "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16", "data": "synthetic",
@@ -710,6 +722,7 @@ def main():
     ap.add_argument("--k", type=int, default=2048)
     ap.add_argument("--n", type=int, default=151936)
     ap.add_argument("--row-max", type=int, default=0)
+    ap.add_argument("--packed", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=2048)
     ap.add_argument("--cpu-seqs", type=int, default=4)
     ap.add_argument("--cpu-prompt", type=int, default=160)
