@@ -288,6 +288,18 @@ int ix_gdn_cpr_scatter(const void* k, long k_pitch, const void* v, long v_pitch,
 int ix_gdn_cpr_handoff(const float* entry_state, float* running_state, int* due, long rows, long elems,
                        int snapshot_dtype, void* stream);
 
+/* ix_gdn_scan whose output leaves through the layer's gated output norm in the same launch (the composition of
+ * runtimes/megatron/gdn_fla_shim.py:390-425 `_eager_apply_gated_norm` after the core, ops/norms/fused_outnorm.py:189-271):
+ * o [tokens, HV, V] bf16 receives ix_gated_out_norm(o_scan, gate, norm_weight) instead of o_scan; the bits of the two
+ * calls. gate bf16 with token pitch gate_stride_t (elements, a multiple of 8), norm_weight bf16 [V]. Served where the
+ * lane-pair layout of the scan runs: one state row per sequence (state_indices [N]), K = V = 128, bf16, N * HV >= 512, no
+ * forced time tile of 1 or row code; IX_DECLINED otherwise, before the state is touched (the caller makes the two calls). */
+int ix_gdn_scan_gated_norm(const void* q, const void* k, const void* v, const float* g, const void* beta, void* o,
+                           long q_pitch, long k_pitch, long v_pitch, float* state_pool, const int* cu_seqlens,
+                           const int* state_indices, long N, long H, long HV, long K, long V, float scale,
+                           int time_tile, const void* gate, long gate_stride_t, const void* norm_weight,
+                           float norm_eps, int zero_centered, void* stream);
+
 /* gdn_causal_conv / gdn_causal_conv_batched (gdn_ops.py:74-170) over packed tokens, and the
  * engine's window-slide update (gdn_recurrent_state.py:686-707,814-825) when every sequence has
  * one token. x bf16 [tokens, D] with token pitch x_pitch (elements; a slice of a wider projection buffer needs

@@ -225,7 +225,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3)))
 void k_gdn_scan_pairs(const TIO* __restrict__ q, const TIO* __restrict__ k, const TIO* __restrict__ v,
                       const float* __restrict__ g, const TIO* __restrict__ beta, TIO* __restrict__ o,
                       float* __restrict__ state, const int* __restrict__ cu, const int* __restrict__ sidx,
-                      long q_pitch, long k_pitch, long v_pitch, int H, int HV, int V, float scale, int TT) {
+                      long q_pitch, long k_pitch, long v_pitch, int H, int HV, int V, float scale, int TT,
+                      const bf16_t* __restrict__ gate, long gate_stride_t, const bf16_t* __restrict__ norm_w,
+                      float norm_eps, int zero_centered) {
   constexpr int K = 128;
   constexpr int R = 128;  // state rows per workgroup: 4 waves x 32 rows
   extern __shared__ __align__(16) char ix_lds[];
@@ -253,12 +255,50 @@ void k_gdn_scan_pairs(const TIO* __restrict__ q, const TIO* __restrict__ k, cons
   const int len = t_end - t_begin;
   if (len <= 0) return;
   const int row0 = sidx[n];
-  if (row0 <= 0) {  // null lane: no state, outputs defined as zero
-    if (!o) return;
-    for (int i = tid; i < len * R; i += 256) {
-      const int tt = i / R, rr = i % R;
-      ix_st(o + ((long)(t_begin + tt) * HV + hv) * V + vb * R + rr, 0.0f);
+  // What leaves for the nt tokens of the tile at t0 whose outputs stand in `of`: the outputs themselves, or, with a gate,
+  // the layer's gated output norm of them (ix_gated_out_norm: RMSNorm over the head's V = 128 values, bf16(1 + w),
+  // silu(gate)) instead of a launch that reads them back. A token's head is sixteen consecutive threads of eight
+  // values, k_rmsnorm_reg<16, 1, 1>'s layout, and the statements are its statements on the bf16 values this kernel
+  // would have stored. V == 128 there (one row block per head).
+  auto emit = [&](int t0, int nt) __attribute__((always_inline)) {
+    if (gate) {
+      for (int i0 = 0; i0 < nt * 16; i0 += 256) {
+        const int i = i0 + tid;
+        const bool live_row = i < nt * 16;
+        const int tt = live_row ? i >> 4 : nt - 1, sub = i & 15;  // rows past the tile run the shuffles, never store
+        const long tok = t_begin + t0 + tt;
+        float xv[8], wv[8], gv[8], acc[8], ov[8];
+        ix_unpack8(*reinterpret_cast<const uint4*>(gate + tok * gate_stride_t + (long)hv * V + sub * 8), gv);
+        ix_unpack8(*reinterpret_cast<const uint4*>(norm_w + sub * 8), wv);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          xv[j] = ix_rbf(of[tt * R + sub * 8 + j]);  // the scan's output is a bf16 tensor
+          const float sq = xv[j] * xv[j];
+          acc[j] = 0.0f + sq;
+        }
+        const float ssum = ix_lane_tree<16>(ix_tree8(acc));
+        const float ms = ssum / 128.0f;
+        const float rstd = ix_rsqrt_ieee(ms + norm_eps);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float nb = ix_rbf(xv[j] * rstd);
+          const float gam = zero_centered ? ix_rbf(1.0f + wv[j]) : wv[j];
+          ov[j] = ix_rbf(nb * gam) * ix_silu_div(gv[j]);
+        }
+        if (live_row) ix_store8_bf16(reinterpret_cast<bf16_t*>(o) + (tok * HV + hv) * V + sub * 8, 8, true, ov);
+      }
+    } else {
+      for (int i = tid; i < nt * R; i += 256) {
+        const int tt = i / R, rr = i % R;
+        ix_st(o + ((long)(t_begin + t0 + tt) * HV + hv) * V + vb * R + rr, of[i]);
+      }
     }
+  };
+  if (row0 <= 0) {  // null lane: no state, outputs defined as zero (and what the norm makes of zeros)
+    if (!o) return;
+    for (int i = tid; i < TT * R; i += 256) of[i] = 0.0f;
+    __syncthreads();
+    for (int t0 = 0; t0 < len; t0 += TT) emit(t0, min(TT, len - t0));
     return;
   }
   constexpr long AL = 16 * sizeof(TIO) / 2;
@@ -357,12 +397,7 @@ void k_gdn_scan_pairs(const TIO* __restrict__ q, const TIO* __restrict__ k, cons
         *reinterpret_cast<float4*>(srow + 4 * c) = make_float4(S[4 * c], S[4 * c + 1], S[4 * c + 2], S[4 * c + 3]);
     }
     __syncthreads();
-    if (o) {
-      for (int i = tid; i < nt * R; i += 256) {
-        const int tt = i / R, rr = i % R;
-        ix_st(o + ((long)(t_begin + t0 + tt) * HV + hv) * V + vb * R + rr, of[i]);
-      }
-    }
+    if (o) emit(t0, nt);
   }
 }
 
@@ -421,10 +456,11 @@ static int ix_gdn_scan_launch(const void* q, const void* k, const void* v, const
 #undef IX_RPL_CASE
 }
 
-extern "C" int ix_gdn_scan(const void* q, const void* k, const void* v, const float* g, const void* beta, void* o,
-                           int io_dtype, long q_pitch, long k_pitch, long v_pitch, float* state_pool,
-                           const int* cu_seqlens, const int* state_indices, long state_indices_stride, long N,
-                           long H, long HV, long K, long V, float scale, int time_tile, void* stream) {
+static int ix_gdn_scan_impl(const void* q, const void* k, const void* v, const float* g, const void* beta, void* o,
+                            int io_dtype, long q_pitch, long k_pitch, long v_pitch, float* state_pool,
+                            const int* cu_seqlens, const int* state_indices, long state_indices_stride, long N,
+                            long H, long HV, long K, long V, float scale, int time_tile, const bf16_t* gate,
+                            long gate_stride_t, const bf16_t* norm_w, float norm_eps, int zero_centered, void* stream) {
   if (!q || !k || !v || !g || !beta || !state_pool || !cu_seqlens || !state_indices) return IX_ERR_ARG;
   if (N < 0 || H <= 0 || HV <= 0 || K <= 0 || V <= 0 || HV % H != 0 || state_indices_stride < 0) return IX_ERR_ARG;
   if (q_pitch < H * K || k_pitch < H * K || v_pitch < HV * V) return IX_ERR_ARG;
@@ -451,13 +487,16 @@ extern "C" int ix_gdn_scan(const void* q, const void* k, const void* v, const fl
     if (io_dtype == IX_DT_BF16)
       hipLaunchKernelGGL((k_gdn_scan_pairs<bf16_t>), dim3((unsigned)grid), dim3(256), lds, st, (const bf16_t*)q,
                          (const bf16_t*)k, (const bf16_t*)v, g, (const bf16_t*)beta, (bf16_t*)o, state_pool,
-                         cu_seqlens, state_indices, q_pitch, k_pitch, v_pitch, (int)H, (int)HV, (int)V, scale, tt);
+                         cu_seqlens, state_indices, q_pitch, k_pitch, v_pitch, (int)H, (int)HV, (int)V, scale, tt, gate,
+                         gate_stride_t, norm_w, norm_eps, zero_centered);
     else
       hipLaunchKernelGGL((k_gdn_scan_pairs<float>), dim3((unsigned)grid), dim3(256), lds, st, (const float*)q,
                          (const float*)k, (const float*)v, g, (const float*)beta, (float*)o, state_pool, cu_seqlens,
-                         state_indices, q_pitch, k_pitch, v_pitch, (int)H, (int)HV, (int)V, scale, tt);
+                         state_indices, q_pitch, k_pitch, v_pitch, (int)H, (int)HV, (int)V, scale, tt,
+                         (const bf16_t*)nullptr, 0L, (const bf16_t*)nullptr, 0.0f, 0);
     return ix_launch_status();
   }
+  if (gate) return IX_DECLINED;       // the norm rides on the lane-pair layout only
   if (rpl == 16) return IX_DECLINED;  // the lane-pair layout was asked for and does not apply
 #define IX_SCAN_CASE(KSV)                                                                                         \
   if (K == KSV * 8) {                                                                                             \
@@ -475,6 +514,32 @@ extern "C" int ix_gdn_scan(const void* q, const void* k, const void* v, const fl
   IX_SCAN_CASE(32)
 #undef IX_SCAN_CASE
   return IX_DECLINED;
+}
+
+extern "C" int ix_gdn_scan(const void* q, const void* k, const void* v, const float* g, const void* beta, void* o,
+                           int io_dtype, long q_pitch, long k_pitch, long v_pitch, float* state_pool,
+                           const int* cu_seqlens, const int* state_indices, long state_indices_stride, long N,
+                           long H, long HV, long K, long V, float scale, int time_tile, void* stream) {
+  return ix_gdn_scan_impl(q, k, v, g, beta, o, io_dtype, q_pitch, k_pitch, v_pitch, state_pool, cu_seqlens, state_indices,
+                          state_indices_stride, N, H, HV, K, V, scale, time_tile, nullptr, 0, nullptr, 0.0f, 0, stream);
+}
+
+// ix_gdn_scan whose output leaves through the layer's gated output norm (ix_gated_out_norm with N = V) in the same
+// launch: o receives bf16(norm(o_scan) * silu(gate)) instead of o_scan -- the bits of the two calls. Served where the
+// lane-pair layout runs (one state row per sequence, K = V = 128, bf16, at least 512 (sequence, head) pairs) with
+// 16-byte aligned gate rows and weight; IX_DECLINED otherwise, before anything is launched or the state is touched.
+extern "C" int ix_gdn_scan_gated_norm(const void* q, const void* k, const void* v, const float* g, const void* beta,
+                                      void* o, long q_pitch, long k_pitch, long v_pitch, float* state_pool,
+                                      const int* cu_seqlens, const int* state_indices, long N, long H, long HV, long K,
+                                      long V, float scale, int time_tile, const void* gate, long gate_stride_t,
+                                      const void* norm_weight, float norm_eps, int zero_centered, void* stream) {
+  if (!o || !gate || !norm_weight || gate_stride_t < HV * V) return IX_ERR_ARG;
+  if (K != 128 || V != 128 || (gate_stride_t % 8) || !ix_aligned(gate, 16) || !ix_aligned(norm_weight, 16) ||
+      !ix_aligned(o, 16) || (time_tile & 0xff) == 1 || (time_tile >> 8) != 0 || N * HV < 512)
+    return IX_DECLINED;
+  return ix_gdn_scan_impl(q, k, v, g, beta, o, IX_DT_BF16, q_pitch, k_pitch, v_pitch, state_pool, cu_seqlens,
+                          state_indices, 0, N, H, HV, K, V, scale, time_tile, (const bf16_t*)gate, gate_stride_t,
+                          (const bf16_t*)norm_weight, norm_eps, zero_centered, stream);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -87,6 +87,11 @@ SIGNATURES = {
     "ix_gdn_gate": (c_int, [P, c_long, P, c_long, P, P, P, P, c_int, c_long, c_long, c_int, P]),
     "ix_gdn_decode_prep": (c_int, [P, c_long, P, c_long, P, c_long, P, P, P, P, P, P, P, P, P, c_long, c_long, c_long, c_long,
                                    c_long, c_long, c_int, c_float, P]),
+    "ix_gdn_scan_gated_norm": (
+        c_int,
+        [P, P, P, P, P, P, c_long, c_long, c_long, P, P, P, c_long, c_long, c_long, c_long, c_long, c_float, c_int, P,
+         c_long, P, c_float, c_int, P],
+    ),
     "ix_gdn_conv": (c_int, [P, c_long, P, P, P, P, P, P, P, c_long, c_long, c_long, c_long, c_int, P]),
     "ix_gdn_conv_l2norm": (c_int, [P, c_long, P, P, P, P, P, P, P, c_long, c_long, c_long, c_long, c_int, c_long, c_long,
                                    c_float, P]),

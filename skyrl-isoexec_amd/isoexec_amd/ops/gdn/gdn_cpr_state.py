@@ -533,12 +533,14 @@ class CprGDN(RecurrentGDN):
         return o[0]
 
     @torch.no_grad()
-    def prefill(self, slots, slots_cpu, x, a, b, qsl, has_initial_state=None, prefill_query_start_loc=None):
+    def prefill(self, slots, slots_cpu, x, a, b, qsl, has_initial_state=None, prefill_query_start_loc=None,
+                fuse_l2norm: bool = True):
         """Prefill a packed batch of N prompts or prompt chunks (a resumed row continues at its stored position,
-        which may be inside an open chunk). Returns ``o [T, HV, V]``."""
+        which may be inside an open chunk). Returns ``o [T, HV, V]``. ``fuse_l2norm=False`` keeps the convolution and
+        the l2norm apart (a traced run: each op's output is a region of its own); the same bits."""
         self._awake()
         rows, is_cont, _rows_out, cu, q, k, v, g, beta = self._prefill_prepare(
-            slots_cpu, x, a, b, qsl, has_initial_state, prefill_query_start_loc)
+            slots_cpu, x, a, b, qsl, has_initial_state, prefill_query_start_loc, fuse_l2norm=fuse_l2norm)
         C = self.chunk_size
         dev = x.device
         N = len(rows)

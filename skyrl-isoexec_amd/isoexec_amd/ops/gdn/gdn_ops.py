@@ -64,9 +64,14 @@ def gdn_recurrent_kernel(
     cu_seqlens: torch.Tensor | None = None,
     time_tile: int = 0,
     want_output: bool = True,
+    gated_norm: tuple | None = None,
 ) -> torch.Tensor:
     """The delta-rule scan. Advances ``ssm_state`` IN PLACE. Returns ``o`` shaped like ``v`` (``None`` for a
     state-only pass, ``want_output=False``: nothing but the state pool is written).
+
+    ``gated_norm = (gate [T, HV, V], weight [V], eps, zero_centered)``: the output leaves through the layer's gated
+    output norm -- in the scan's own launch where the library serves that form (it declines before the state is
+    touched), else by ``fused_gated_out_norm`` on the scan's output: the same bits either way, in ``o``'s shape.
 
     ``q, k``: ``[B, T, H, K]`` already L2-normalised (H may be GQA-compressed: ``HV % H == 0``);
     ``v``: ``[B, T, HV, V]``; ``g`` (fp32), ``beta``: ``[B, T, HV]``; ``ssm_state`` fp32 pool
@@ -112,6 +117,23 @@ def gdn_recurrent_kernel(
     o = torch.empty(qf.shape[0], HV, V, dtype=io, device=dev) if want_output else None
     if time_tile == 0 and cu_seqlens is None and T == 1:
         time_tile = 1
+    if gated_norm is not None:
+        gate, weight, eps, zero_centered = gated_norm
+        _lib.require_device(gate, weight)
+        if not want_output or tuple(gate.shape) != (qf.shape[0], HV, V):
+            raise RuntimeError("[isoexec-amd] gated_norm needs an output and a gate [tokens, HV, V]")
+        fusable = (io is torch.bfloat16 and idx_stride == 0 and gate.dtype is io and weight.dtype is io
+                   and gate.stride(2) == 1 and gate.stride(1) == V and weight.is_contiguous() and weight.numel() == V)
+        rc = _lib.IX_DECLINED
+        if fusable:
+            rc = _lib.check(
+                _lib.lib().ix_gdn_scan_gated_norm(
+                    qf.data_ptr(), kf.data_ptr(), vf.data_ptr(), gf.data_ptr(), bf.data_ptr(), o.data_ptr(),
+                    _token_pitch(qf), _token_pitch(kf), _token_pitch(vf), ssm_state.data_ptr(), cu.data_ptr(),
+                    idx.data_ptr(), n_seq, H, HV, K, V, float(K) ** -0.5, time_tile, gate.data_ptr(), gate.stride(0),
+                    weight.data_ptr(), float(eps), int(zero_centered), _lib.current_stream(dev)), "ix_gdn_scan_gated_norm")
+        if rc == _lib.IX_OK:
+            return o.view(B, T, HV, V) if cu_seqlens is None else o.unsqueeze(0)
     rc = _lib.check(
         _lib.lib().ix_gdn_scan(
             qf.data_ptr(), kf.data_ptr(), vf.data_ptr(), gf.data_ptr(), bf.data_ptr(), _lib.ptr(o),
@@ -122,6 +144,11 @@ def gdn_recurrent_kernel(
         raise RuntimeError(f"[isoexec-amd] ix_gdn_scan declined K={K} V={V} dtype={io}")
     if o is None:
         return None
+    if gated_norm is not None:  # the fused form was declined (nothing launched): the two calls
+        from ..norms.fused_outnorm import fused_gated_out_norm
+
+        gate, weight, eps, zero_centered = gated_norm
+        o = fused_gated_out_norm(o, gate, weight, eps, zero_centered=zero_centered).view(-1, HV, V)
     return o.view(B, T, HV, V) if cu_seqlens is None else o.unsqueeze(0)
 
 
@@ -220,8 +247,8 @@ def conv_packed(x, weight, bias, *, cu_seqlens, conv_state=None, rows_in=None, r
     """Packed varlen conv: ``x [T, D]`` -> ``y [T, D]``; optional pool rows for history in/out.
 
     ``l2norm_qk`` > 0: channels ``[0, l2norm_qk)`` of ``y`` are q and k heads of ``head_k_dim`` channels and leave
-    L2-normalised, in the same launch (the bits of ``gdn_l2norm`` on those columns of the plain result); ``None`` is
-    returned when the library does not serve that form for these shapes (the caller makes the two calls)."""
+    L2-normalised -- in the same launch where the library serves that form, else by ``gdn_l2norm`` on those columns of
+    the plain result: the same bits either way."""
     _lib.require_device(x, weight, bias, cu_seqlens, conv_state, rows_in, rows_out)
     if activation not in (None, "silu", "swish"):
         raise ValueError(f"unsupported activation {activation!r}")
@@ -243,13 +270,17 @@ def conv_packed(x, weight, bias, *, cu_seqlens, conv_state=None, rows_in=None, r
                                           _lib.ptr(conv_state), cu_seqlens.data_ptr(), _lib.ptr(rows_in), _lib.ptr(rows_out),
                                           n_seq, T, D, W, int(activation is not None), int(l2norm_qk), int(head_k_dim),
                                           L2NORM_EPS, _lib.current_stream(x.device)), "ix_gdn_conv_l2norm")
-        return y if rc == _lib.IX_OK else None
+        if rc == _lib.IX_OK:
+            return y
     rc = _lib.check(
         _lib.lib().ix_gdn_conv(xc.data_ptr(), xc.stride(0), wc.data_ptr(), _lib.ptr(bc), y.data_ptr(), _lib.ptr(conv_state),
                                cu_seqlens.data_ptr(), _lib.ptr(rows_in), _lib.ptr(rows_out), n_seq, T, D, W,
                                int(activation is not None), _lib.current_stream(x.device)), "ix_gdn_conv")
     if rc != _lib.IX_OK:
         raise RuntimeError(f"[isoexec-amd] ix_gdn_conv declined W={W}")
+    if l2norm_qk:  # the fused form was declined (nothing launched): the two calls
+        heads = int(l2norm_qk) // int(head_k_dim)
+        y[:, :l2norm_qk] = gdn_l2norm(y[:, :l2norm_qk].unflatten(1, (heads, int(head_k_dim)))).flatten(1)
     return y
 
 
@@ -386,16 +417,17 @@ def gdn_native_core_kernel(q, k, v, a, b, A_log, dt_bias, *, ssm_state, state_in
                                 state_indices=state_indices, cu_seqlens=cu_seqlens)
 
 
-def gdn_native_core_normed(qn, kn, v, a, b, A_log, dt_bias, *, cu_seqlens=None):
+def gdn_native_core_normed(qn, kn, v, a, b, A_log, dt_bias, *, cu_seqlens=None, gated_norm: tuple | None = None):
     """``gdn_native_core`` for q and k that are normalised already (``conv_packed(..., l2norm_qk=...)``): the gating and
-    the scan of the same composition, without its two l2norm launches. Same bits as ``gdn_native_core`` on the raw heads."""
+    the scan of the same composition, without its two l2norm launches. Same bits as ``gdn_native_core`` on the raw heads.
+    ``gated_norm`` as in ``gdn_recurrent_kernel``: the output then comes back through the layer's gated output norm."""
     with torch.no_grad():
         ssm_state, idx = _recurrent_scratch_state(qn, v, cu_seqlens)
         HV = v.shape[-2]
         g, beta = gate_and_beta_fp32(a.reshape(-1, HV), b.reshape(-1, HV), A_log, dt_bias)
         lead = v.shape[:2]
         return gdn_recurrent_kernel(qn, kn, v, g.view(*lead, HV), beta.view(*lead, HV), ssm_state=ssm_state,
-                                    state_indices=idx, cu_seqlens=cu_seqlens)
+                                    state_indices=idx, cu_seqlens=cu_seqlens, gated_norm=gated_norm)
 
 
 def gdn_native_core(q, k, v, a, b, A_log, dt_bias, *, cu_seqlens=None):

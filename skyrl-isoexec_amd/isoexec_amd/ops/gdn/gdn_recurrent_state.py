@@ -474,15 +474,17 @@ class RecurrentGDN:
         qsl: list,  # [N+1] token offsets into the packed region
         has_initial_state=None,
         prefill_query_start_loc: torch.Tensor | None = None,
+        gated_norm: tuple | None = None,
     ) -> torch.Tensor:
-        """Prefill a packed batch of N prompts (or prompt chunks). Returns ``o [T, HV, V]``."""
+        """Prefill a packed batch of N prompts (or prompt chunks). Returns ``o [T, HV, V]``; with ``gated_norm``
+        (``gdn_recurrent_kernel``'s) the output comes back through the layer's gated output norm."""
         rows, is_cont, rows_out, cu, q, k, v, g, beta = self._prefill_prepare(
-            slots_cpu, x, a, b, qsl, has_initial_state, prefill_query_start_loc)
+            slots_cpu, x, a, b, qsl, has_initial_state, prefill_query_start_loc, fuse_l2norm=gated_norm is not None)
         o = gdn_recurrent_kernel(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), g.unsqueeze(0), beta.unsqueeze(0),
-                                 ssm_state=self.ssm_state, state_indices=rows_out, cu_seqlens=cu)
+                                 ssm_state=self.ssm_state, state_indices=rows_out, cu_seqlens=cu, gated_norm=gated_norm)
         return o[0]
 
-    def _prefill_prepare(self, slots_cpu, x, a, b, qsl, has_initial_state, prefill_query_start_loc):
+    def _prefill_prepare(self, slots_cpu, x, a, b, qsl, has_initial_state, prefill_query_start_loc, fuse_l2norm=True):
         """Everything of a prefill in front of the scan: rows assigned (fresh rows zeroed), the convolution with
         its window carried in the pool, q/k normalised, gate and beta. Returns ``(rows, is_cont, rows_out int32
         device, cu int32 device, q, k, v, g, beta)`` with q, k ``[T, H, K]``, v ``[T, HV, V]``, g, beta ``[T, HV]``."""
@@ -518,13 +520,12 @@ class RecurrentGDN:
             cu = torch.from_numpy(np.asarray(qsl, dtype=np.int32)).to(dev, non_blocking=True)
         # A fresh row must start from zero; a resumed row keeps what the previous chunk left.
         self._zero_fresh_rows(meta_t[2].long())
-        # q and k leave the convolution's launch normalised where the library serves that form (the same bits)
-        y = conv_packed(x, self.conv_weight, self.conv_bias, cu_seqlens=cu, conv_state=self.conv_state,
-                        rows_in=rows_in, rows_out=rows_out, activation=self.activation,
-                        l2norm_qk=2 * self.num_k_heads * self.head_k_dim, head_k_dim=self.head_k_dim)
-        if y is not None:
+        if fuse_l2norm:  # q and k leave the convolution's launch normalised where the library serves that form
+            y = conv_packed(x, self.conv_weight, self.conv_bias, cu_seqlens=cu, conv_state=self.conv_state,
+                            rows_in=rows_in, rows_out=rows_out, activation=self.activation,
+                            l2norm_qk=2 * self.num_k_heads * self.head_k_dim, head_k_dim=self.head_k_dim)
             q, k, v = self._split_qkv_raw(y)
-        else:
+        else:  # the two ops apart (what a traced run asks for: each door's output is its own region)
             y = conv_packed(x, self.conv_weight, self.conv_bias, cu_seqlens=cu, conv_state=self.conv_state,
                             rows_in=rows_in, rows_out=rows_out, activation=self.activation)
             q, k, v = self._split_qkv(y)

@@ -227,10 +227,22 @@ class _Blocks:
         a = proj[:, c.gdn_qkv + c.gdn_z + c.gdn_v_heads :]
         return qkv, z, b, a
 
-    def gdn_out(self, layer: int, o: torch.Tensor, z: torch.Tensor) -> torch.Tensor:
+    @property
+    def fuse_ops(self) -> bool:
+        """Whether the runtimes may fold neighbouring ops into one launch (conv + l2norm, scan + gated output norm,
+        combine + add + norm). Not while a region log or the trace is attached: each op's output is then a region of its
+        own, and both sides have to cut the computation at the same points. Same bits either way."""
+        return self.region_log is None
+
+    def gdn_out(self, layer: int, o: torch.Tensor, z: torch.Tensor, normed: bool = False) -> torch.Tensor:
+        """Gated output norm (unless the scan applied it already: ``normed``) and the output projection."""
         lw = self.w.layers[layer]
-        normed = fused_gated_out_norm(o, z, lw["out_norm"], self.cfg.eps)
-        return _linear(normed.view(o.shape[0], -1), lw["out_proj"])
+        y = o if normed else fused_gated_out_norm(o, z, lw["out_norm"], self.cfg.eps)
+        return _linear(y.reshape(o.shape[0], -1), lw["out_proj"])
+
+    def gdn_gated_norm(self, layer: int, z: torch.Tensor) -> tuple:
+        """What a scan needs to apply the layer's gated output norm itself: ``(gate, weight, eps, zero_centered)``."""
+        return z, self.w.layers[layer]["out_norm"], self.cfg.eps, True
 
     def attn_qkv(self, layer: int, x: torch.Tensor, positions: torch.Tensor):
         """-> views ``q [T, HQ, D]``, ``k, v [T, HKV, D]`` of one projection buffer, q and k rotated."""
@@ -265,7 +277,7 @@ class _Blocks:
             self._note("attention.varlen" if c.is_attention(i) else "gdn.core", i, mixed)
             x, h = fused_add_rms_norm_gamma(mixed, h, lw["post_norm"], c.eps)
             nxt = self.w.layers[i + 1]["pre_norm"] if i + 1 < c.layers else self.w.final_norm
-            if self.region_log is None:
+            if self.fuse_ops:
                 x, h = self.moe(i, x, add_norm=(h, nxt, c.eps))
             else:  # the mixture's own output is a region of the comparison: keep it as a tensor
                 delta = self.moe(i, x)
@@ -352,21 +364,23 @@ class TrainerModel:
                 return b.attn_out(i, varlen_attention(q, k, v, cu, max_len))
             qkv, z, bb, a = b.gdn_in(i, x)
             kd = c.gdn_k_heads * c.gdn_head_dim
-            # the recurrent form takes q and k normalised by the convolution's own launch where the library serves it
-            normed = None
-            if c.gdn_kernel != "cpr":
-                normed = conv_packed(qkv, lw["conv_weight"], lw["conv_bias"], cu_seqlens=cu, l2norm_qk=2 * kd,
-                                     head_k_dim=c.gdn_head_dim)
-            y = normed if normed is not None else conv_packed(qkv, lw["conv_weight"], lw["conv_bias"], cu_seqlens=cu)
+            # the recurrent form takes q and k normalised by the convolution's own launch and hands its output to the
+            # gated norm inside the scan's (where the library serves those forms; the same bits as the ops apart)
+            fused = b.fuse_ops and c.gdn_kernel != "cpr"
+            y = conv_packed(qkv, lw["conv_weight"], lw["conv_bias"], cu_seqlens=cu, l2norm_qk=2 * kd if fused else 0,
+                            head_k_dim=c.gdn_head_dim)
             q = y[:, :kd].unflatten(1, (c.gdn_k_heads, c.gdn_head_dim))
             k = y[:, kd : 2 * kd].unflatten(1, (c.gdn_k_heads, c.gdn_head_dim))
             v = y[:, 2 * kd :].unflatten(1, (c.gdn_v_heads, c.gdn_head_dim))
             if c.gdn_kernel == "cpr":
                 o = gdn_native_cpr_fwd(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), a, bb, lw["A_log"], lw["dt_bias"],
                                        cu_seqlens=cu, chunk_size=c.gdn_chunk)
+            elif fused:
+                o = gdn_native_core_normed(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), a, bb, lw["A_log"],
+                                           lw["dt_bias"], cu_seqlens=cu, gated_norm=b.gdn_gated_norm(i, z))
+                return b.gdn_out(i, o[0], z, normed=True)
             else:
-                core = gdn_native_core_normed if normed is not None else gdn_native_core
-                o = core(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), a, bb, lw["A_log"], lw["dt_bias"], cu_seqlens=cu)
+                o = gdn_native_core(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), a, bb, lw["A_log"], lw["dt_bias"], cu_seqlens=cu)
             return b.gdn_out(i, o[0], z)
 
         return b.run_layers(b.embed(tokens), mixer)
@@ -459,8 +473,15 @@ class RolloutEngine:
                 kf, vf = self.kv[i].flat()
                 return b.attn_out(i, varlen_attention(q, kf, vf, cu, max_len, kv_start=kv_start))
             qkv, z, bb, a = b.gdn_in(i, x)
-            o = self.gdn[i].prefill(slots_t, slots, qkv, a, bb, qsl, prefill_query_start_loc=cu)
-            return b.gdn_out(i, o, z)
+            layer = self.gdn[i]
+            if isinstance(layer, CprGDN):
+                o = layer.prefill(slots_t, slots, qkv, a, bb, qsl, prefill_query_start_loc=cu, fuse_l2norm=b.fuse_ops)
+                return b.gdn_out(i, o, z)
+            if not b.fuse_ops:
+                return b.gdn_out(i, layer.prefill(slots_t, slots, qkv, a, bb, qsl, prefill_query_start_loc=cu), z)
+            o = layer.prefill(slots_t, slots, qkv, a, bb, qsl, prefill_query_start_loc=cu,
+                              gated_norm=b.gdn_gated_norm(i, z))
+            return b.gdn_out(i, o, z, normed=True)
 
         x = b.run_layers(b.embed(tokens), mixer)
         for s, n in zip(slots, lens):

@@ -351,5 +351,60 @@ def test_conv_with_the_l2norm_folded_in_equals_the_two_launches(H, HV):
     o_raw = gdn_native_core(*split(plain), a, b, A_log, dt_bias, cu_seqlens=cu)
     o_normed = gdn_native_core_normed(*split(fused), a, b, A_log, dt_bias, cu_seqlens=cu)
     assert same_bits(o_raw, o_normed)
-    # heads of another size are not served: the caller makes the two calls
-    assert conv_packed(x, weight, bias, cu_seqlens=cu, l2norm_qk=2 * kd, head_k_dim=64) is None
+    # heads of another size are not served by the one-launch form: the wrapper makes the two calls itself
+    y64 = conv_packed(x, weight, bias, cu_seqlens=cu, l2norm_qk=2 * kd, head_k_dim=64)
+    plain64 = conv_packed(x, weight, bias, cu_seqlens=cu)
+    assert same_bits(y64[:, :2 * kd].unflatten(1, (4 * H, 64)).contiguous(), gdn_l2norm(plain64[:, :2 * kd].unflatten(1, (4 * H, 64))))
+    assert same_bits(y64[:, 2 * kd:].contiguous(), plain64[:, 2 * kd:].contiguous())
+
+
+def test_scan_with_the_gated_output_norm_folded_in_equals_the_two_launches():
+    """``gdn_recurrent_kernel(..., gated_norm=...)``: the lane-pair scan applies the layer's gated output norm to its own
+    outputs. Against the scan followed by ``fused_gated_out_norm``: outputs and final states bit for bit, a packed batch
+    with short, long and empty sequences, null lanes (state index 0) included, a gate that is a column slice of a wider
+    buffer; where the lane-pair layout does not run the library declines the form before it touches the state and the
+    wrapper makes the two calls."""
+    from isoexec_amd.ops.gdn.gdn_ops import gdn_l2norm, gdn_recurrent_kernel
+    from isoexec_amd.ops.norms.fused_outnorm import fused_gated_out_norm
+
+    H, HV, K, V = 16, 32, 128, 128
+    g = cpu_gen(91)
+    lens = [70, 1, 0, 33, 16, 5, 129, 17, 2, 64, 48, 31, 7, 96, 3, 40, 12, 100]        # 18 sequences x 32 heads >= 512 pairs
+    T, N = sum(lens), len(lens)
+    bf = lambda t: t.to(torch.bfloat16).to(DEV)
+    q = gdn_l2norm(bf(torch.randn(T, H, K, generator=g)))
+    k = gdn_l2norm(bf(torch.randn(T, H, K, generator=g)))
+    v = bf(torch.randn(T, HV, V, generator=g))
+    gate = -torch.nn.functional.softplus(torch.randn(T, HV, generator=g)).to(DEV)
+    beta = bf(torch.sigmoid(torch.randn(T, HV, generator=g)))
+    wide = bf(torch.randn(T, HV * V + 64, generator=g))
+    z = wide[:, :HV * V].unflatten(1, (HV, V))
+    w = bf(torch.randn(V, generator=g) * 0.1)
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32, device=DEV)
+    rows = torch.arange(1, N + 1, dtype=torch.int32, device=DEV)
+    rows[4] = 0                                                                           # a null lane: outputs defined, no state
+    pool0 = torch.randn(N + 1, HV, V, K, generator=g).to(DEV) * 0.1
+    u = lambda t: t.unsqueeze(0)
+    pa, pb = pool0.clone(), pool0.clone()
+    o = gdn_recurrent_kernel(u(q), u(k), u(v), u(gate), u(beta), ssm_state=pa, state_indices=rows, cu_seqlens=cu)[0]
+    want = fused_gated_out_norm(o, z, w, 1e-6).view(T, HV, V)
+    got = gdn_recurrent_kernel(u(q), u(k), u(v), u(gate), u(beta), ssm_state=pb, state_indices=rows, cu_seqlens=cu,
+                               gated_norm=(z, w, 1e-6, True))
+    assert got is not None and same_bits(got[0], want) and same_bits(pa, pb)
+    # fewer than 512 (sequence, head) pairs: the 16-lane layout runs; the library declines the fused form untouched ...
+    from isoexec_amd import _lib
+
+    pc = pool0.clone()
+    few = torch.tensor([0, 70, 71], dtype=torch.int32, device=DEV)
+    scratch = torch.empty(71, HV, V, dtype=torch.bfloat16, device=DEV)
+    rc = _lib.lib().ix_gdn_scan_gated_norm(q.data_ptr(), k.data_ptr(), v.data_ptr(), gate.data_ptr(), beta.data_ptr(),
+                                           scratch.data_ptr(), H * K, H * K, HV * V, pc.data_ptr(), few.data_ptr(),
+                                           rows.data_ptr(), 2, H, HV, K, V, K ** -0.5, 0, z.data_ptr(), z.stride(0),
+                                           w.data_ptr(), 1e-6, 1, _lib.current_stream(torch.device(DEV)))
+    torch.cuda.synchronize()
+    assert rc == _lib.IX_DECLINED and same_bits(pc, pool0)
+    # ... and the wrapper makes the two calls: the same result
+    pd = pool0.clone()
+    got2 = gdn_recurrent_kernel(u(q[:71]), u(k[:71]), u(v[:71]), u(gate[:71]), u(beta[:71]), ssm_state=pd,
+                                state_indices=rows[:2], cu_seqlens=few, gated_norm=(z[:71], w, 1e-6, True))
+    assert same_bits(got2[0], want[:71]) and same_bits(pd[:3], pa[:3])
