@@ -860,6 +860,14 @@ __device__ __forceinline__ void ix_l2norm8_of16(bf16_t* __restrict__ yrow, float
   for (int i = 0; i < 8; ++i) sq[i] = v8[i] * v8[i];
   const float ssum = ix_lane_tree<16>(ix_tree8(sq));
   const float rn = ix_rsqrt_ieee(ssum + eps);
+  if (ssum < __builtin_inff()) {
+    // every value is finite and so is every product: the hardware pack-convert rounds them as ix_f2bf does
+    *reinterpret_cast<uint4*>(yrow) =
+        make_uint4(ix_pack_bf2_hw(v8[0] * rn, v8[1] * rn), ix_pack_bf2_hw(v8[2] * rn, v8[3] * rn),
+                   ix_pack_bf2_hw(v8[4] * rn, v8[5] * rn), ix_pack_bf2_hw(v8[6] * rn, v8[7] * rn));
+    return;
+  }
+  // an infinity or a NaN among the head's values: products can be NaN, which ix_f2bf canonicalises
   __attribute__((aligned(16))) bf16_t out[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) out[i] = ix_f2bf(v8[i] * rn);
@@ -874,10 +882,20 @@ __global__ __launch_bounds__(256) void k_gdn_conv8(const bf16_t* __restrict__ x,
                                                    bf16_t* __restrict__ y, const bf16_t* __restrict__ pool,
                                                    const int* __restrict__ cu, const int* __restrict__ rows_in,
                                                    int N, long D, int silu, int T, long total, long qk_channels,
-                                                   float eps) {
-  const long i = ((long)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
-  if (i >= total) return;
+                                                   float eps, unsigned run_blocks, unsigned run_groups) {
   const long D8 = D >> 3;
+  long i;
+  if (run_blocks) {
+    // Consecutive token groups of one 2048-channel block on one XCD, one after the other: the W - 1 rows a group
+    // shares with the group before it are then still in that XCD's L2 (dealt round-robin, neighbouring groups sit
+    // on different XCDs and every shared row is fetched twice). The host chose this only for D8 % 256 == 0.
+    unsigned pos;
+    if (!ix_xcd_run_position(blockIdx.x, run_blocks, &pos)) return;
+    i = (long)(pos % run_groups) * D8 + (long)(pos / run_groups) * 256 + threadIdx.x;
+  } else {
+    i = ((long)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
+  }
+  if (i >= total) return;
   const int t0 = (int)(i / D8) * TOK;
   const int d = (int)(i % D8) * 8;
   float wv[8][W], bv[8];
@@ -999,19 +1017,25 @@ static int ix_gdn_conv_impl(const void* x, long x_pitch, const void* weight, con
     // computed by the same expression whichever is chosen.
     if (qk_channels > 0 && !vec8) return IX_DECLINED;  // the normalising form is the eight-channel kernel's
     const long avg_len = total_tokens / N;
-    const int TOK = !vec8 ? 1 : avg_len >= 64 ? 16 : avg_len >= 8 ? 4 : 1;
+    // The normalising form stops at 8: with 16 its registers leave two waves per SIMD and the launch takes a quarter
+    // longer than the plain one; with 8 it takes the same time (1.17 ms for 163,840 tokens of 8192 channels).
+    const int TOK = !vec8 ? 1 : avg_len >= 64 ? (qk_channels > 0 ? 8 : 16) : avg_len >= 8 ? 4 : 1;
     const long work = vec8 ? ((total_tokens + TOK - 1) / TOK) * (D / 8) : total;
     const long blocks = (work + 255) / 256;
-    const long gx = blocks < (1L << 22) ? blocks : (1L << 22);
-    const long gy = (blocks + gx - 1) / gx;
+    // the XCD-run order for long sequences whose channel count fills whole workgroups
+    const bool runs = vec8 && TOK > 1 && (D / 8) % 256 == 0 && blocks < (1L << 30);
+    const unsigned run_blocks = runs ? (unsigned)blocks : 0u;
+    const unsigned run_groups = runs ? (unsigned)((total_tokens + TOK - 1) / TOK) : 1u;
+    const long gx = runs ? (long)ix_xcd_run_grid(run_blocks) : blocks < (1L << 22) ? blocks : (1L << 22);
+    const long gy = runs ? 1 : (blocks + gx - 1) / gx;
     if (gy > 65535) return IX_DECLINED;
 #define IX_CONV8(TOK_, NORM_)                                                                                       \
   hipLaunchKernelGGL((k_gdn_conv8<4, TOK_, NORM_>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,             \
                      (const bf16_t*)x, x_pitch, (const bf16_t*)weight, (const bf16_t*)bias, (bf16_t*)y,             \
                      (const bf16_t*)conv_pool, cu_seqlens, state_rows_in, (int)N, D, silu, (int)total_tokens, work, \
-                     qk_channels, eps)
+                     qk_channels, eps, run_blocks, run_groups)
     if (vec8 && qk_channels > 0) {
-      if (TOK == 16) IX_CONV8(16, true);
+      if (TOK == 8) IX_CONV8(8, true);
       else if (TOK == 4) IX_CONV8(4, true);
       else IX_CONV8(1, true);
     } else if (vec8) {
