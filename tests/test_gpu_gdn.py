@@ -351,6 +351,18 @@ def test_conv_with_the_l2norm_folded_in_equals_the_two_launches(H, HV):
     o_raw = gdn_native_core(*split(plain), a, b, A_log, dt_bias, cu_seqlens=cu)
     o_normed = gdn_native_core_normed(*split(fused), a, b, A_log, dt_bias, cu_seqlens=cu)
     assert same_bits(o_raw, o_normed)
+    # a head that holds an infinity or a NaN takes the launch's other way out (canonical NaNs, zeros): same bits again
+    spoiled = x.clone()
+    spoiled[5, 3] = float("inf")            # long sequence, first q head
+    spoiled[200, kd + 130] = float("nan")   # long sequence, a k head
+    spoiled[300, 7] = float("-inf")         # the one-token sequence
+    spoiled[T - 1, 2 * kd - 1] = float("nan")
+    plain_s = conv_packed(spoiled, weight, bias, cu_seqlens=cu)
+    fused_s = conv_packed(spoiled, weight, bias, cu_seqlens=cu, l2norm_qk=2 * kd, head_k_dim=K)
+    want_s = gdn_l2norm(plain_s[:, :2 * kd].unflatten(1, (2 * H, K)))
+    assert not torch.isfinite(want_s.float()).all()
+    assert same_bits(fused_s[:, :2 * kd].unflatten(1, (2 * H, K)).contiguous(), want_s)
+    assert same_bits(fused_s[:, 2 * kd:].contiguous(), plain_s[:, 2 * kd:].contiguous())
     # heads of another size are not served by the one-launch form: the wrapper makes the two calls itself
     y64 = conv_packed(x, weight, bias, cu_seqlens=cu, l2norm_qk=2 * kd, head_k_dim=64)
     plain64 = conv_packed(x, weight, bias, cu_seqlens=cu)
