@@ -267,12 +267,19 @@ void k_gdn_scan_pairs(const TIO* __restrict__ q, const TIO* __restrict__ k, cons
         const bool live_row = i < nt * 16;
         const int tt = live_row ? i >> 4 : nt - 1, sub = i & 15;  // rows past the tile run the shuffles, never store
         const long tok = t_begin + t0 + tt;
-        float xv[8], wv[8], gv[8], acc[8], ov[8];
+        // The roundings inside the chain are the hardware pack-convert's (ix_rbf2_hw): it differs from ix_rbf on NaNs
+        // only, a NaN stays a NaN through every operation below whatever its payload, and the values that are stored
+        // get their NaNs made canonical (ix_pack_bf2_canon_hw) -- the stored bits are the ix_rbf chain's. This kernel
+        // is bound by vector issue, so the twenty-odd instructions less per value are time.
+        float xv[8], wv[8], gv[8], acc[8];
+        uint32_t op[4];
         ix_unpack8(*reinterpret_cast<const uint4*>(gate + tok * gate_stride_t + (long)hv * V + sub * 8), gv);
         ix_unpack8(*reinterpret_cast<const uint4*>(norm_w + sub * 8), wv);
 #pragma unroll
+        for (int j = 0; j < 8; j += 2)  // the scan's output is a bf16 tensor
+          ix_rbf2_hw(of[tt * R + sub * 8 + j], of[tt * R + sub * 8 + j + 1], xv[j], xv[j + 1]);
+#pragma unroll
         for (int j = 0; j < 8; ++j) {
-          xv[j] = ix_rbf(of[tt * R + sub * 8 + j]);  // the scan's output is a bf16 tensor
           const float sq = xv[j] * xv[j];
           acc[j] = 0.0f + sq;
         }
@@ -280,12 +287,16 @@ void k_gdn_scan_pairs(const TIO* __restrict__ q, const TIO* __restrict__ k, cons
         const float ms = ssum / 128.0f;
         const float rstd = ix_rsqrt_ieee(ms + norm_eps);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const float nb = ix_rbf(xv[j] * rstd);
-          const float gam = zero_centered ? ix_rbf(1.0f + wv[j]) : wv[j];
-          ov[j] = ix_rbf(nb * gam) * ix_silu_div(gv[j]);
+        for (int j = 0; j < 8; j += 2) {
+          float nb0, nb1, g0 = wv[j], g1 = wv[j + 1], y0, y1;
+          ix_rbf2_hw(xv[j] * rstd, xv[j + 1] * rstd, nb0, nb1);
+          if (zero_centered) ix_rbf2_hw(1.0f + wv[j], 1.0f + wv[j + 1], g0, g1);
+          ix_rbf2_hw(nb0 * g0, nb1 * g1, y0, y1);
+          op[j >> 1] = ix_pack_bf2_canon_hw(y0 * ix_silu_div(gv[j]), y1 * ix_silu_div(gv[j + 1]));
         }
-        if (live_row) ix_store8_bf16(reinterpret_cast<bf16_t*>(o) + (tok * HV + hv) * V + sub * 8, 8, true, ov);
+        if (live_row)
+          *reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(o) + (tok * HV + hv) * V + sub * 8) =
+              make_uint4(op[0], op[1], op[2], op[3]);
       }
     } else {
       for (int i = tid; i < nt * R; i += 256) {

@@ -273,6 +273,10 @@ __global__ __launch_bounds__(256) void k_combine_add_rmsnorm_reg(const bf16_t* _
 #pragma unroll
     for (int r = 0; r < KC; ++r)
       ep[r] = *reinterpret_cast<const uint4*>(expert_out + src[r] * N + sub * 8 + c * LPR * 8);
+    // Roundings inside the chain go through the hardware pack-convert (ix_rbf2_hw), which differs from ix_rbf on NaNs
+    // only (it keeps a payload where ix_rbf makes 0x7fc0). A NaN stays a NaN through every add, multiply, divide and
+    // square root below whatever its payload, and everything else is the same number either way, so making the NaNs
+    // canonical where values are STORED (ix_pack_bf2_canon_hw) leaves every stored bit what the ix_rbf chain stores.
     float sum[8];
     ix_unpack8(ep[0], sum);
 #pragma unroll
@@ -280,17 +284,32 @@ __global__ __launch_bounds__(256) void k_combine_add_rmsnorm_reg(const bf16_t* _
       float e[8];
       ix_unpack8(ep[r], e);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float t = sum[i] + e[i];
-        sum[i] = fp32_acc ? t : ix_rbf(t);
+      for (int i = 0; i < 8; i += 2) {
+        const float t0 = sum[i] + e[i], t1 = sum[i + 1] + e[i + 1];
+        if (fp32_acc) {
+          sum[i] = t0;
+          sum[i + 1] = t1;
+        } else {
+          ix_rbf2_hw(t0, t1, sum[i], sum[i + 1]);
+        }
       }
     }
     float r8[8];
     ix_unpack8(ap[c], r8);
+    uint32_t hp[4];
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) {
+      float d0, d1;
+      ix_rbf2_hw(sum[i], sum[i + 1], d0, d1);      // what k_moe_combine stores
+      const uint32_t u = ix_pack_bf2_canon_hw(d0 + r8[i], d1 + r8[i + 1]);  // h = bf16(x + residual)
+      hp[i >> 1] = u;
+      xv[c][i] = __uint_as_float(u << 16);
+      xv[c][i + 1] = __uint_as_float(u & 0xffff0000u);
+    }
+    if (live)
+      *reinterpret_cast<uint4*>(h_out + row * N + sub * 8 + c * LPR * 8) = make_uint4(hp[0], hp[1], hp[2], hp[3]);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const float delta = ix_rbf(sum[i]);         // what k_moe_combine stores
-      xv[c][i] = ix_rbf(delta + r8[i]);           // h = bf16(x + residual)
       const float sq = xv[c][i] * xv[c][i];
       acc[i] = acc[i] + sq;
     }
@@ -302,16 +321,17 @@ __global__ __launch_bounds__(256) void k_combine_add_rmsnorm_reg(const bf16_t* _
   bf16_t* orow = out + row * N + sub * 8;
 #pragma unroll
   for (int c = 0; c < NG; ++c) {
-    float wv[8], o[8];
+    float wv[8];
+    uint32_t op[4];
     ix_unpack8(wp[c], wv);
-    ix_store8_bf16(h_out + row * N + sub * 8 + c * LPR * 8, 8, true, xv[c]);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float nb = ix_rbf(xv[c][i] * rstd);
-      const float gam = zero_centered ? ix_rbf(1.0f + wv[i]) : wv[i];
-      o[i] = ix_rbf(nb * gam);
+    for (int i = 0; i < 8; i += 2) {
+      float nb0, nb1, g0 = wv[i], g1 = wv[i + 1];
+      ix_rbf2_hw(xv[c][i] * rstd, xv[c][i + 1] * rstd, nb0, nb1);
+      if (zero_centered) ix_rbf2_hw(1.0f + wv[i], 1.0f + wv[i + 1], g0, g1);
+      op[i >> 1] = ix_pack_bf2_canon_hw(nb0 * g0, nb1 * g1);
     }
-    ix_store8_bf16(orow + c * LPR * 8, 8, true, o);
+    *reinterpret_cast<uint4*>(orow + c * LPR * 8) = make_uint4(op[0], op[1], op[2], op[3]);
   }
 }
 

@@ -403,6 +403,24 @@ def test_scan_with_the_gated_output_norm_folded_in_equals_the_two_launches():
     got = gdn_recurrent_kernel(u(q), u(k), u(v), u(gate), u(beta), ssm_state=pb, state_indices=rows, cu_seqlens=cu,
                                gated_norm=(z, w, 1e-6, True))
     assert got is not None and same_bits(got[0], want) and same_bits(pa, pb)
+    # NaNs and infinities in values, gate and weight: the folded norm rounds inside its chain with the hardware convert
+    # and must still store what the two launches store (canonical NaNs, signed zeros, infinities)
+    v2, wide2, w2 = v.clone(), wide.clone(), w.clone()
+    v2[3, 1, 7] = float("nan")
+    v2[80, 5, 100] = float("inf")
+    v2.view(torch.int16)[200, 9, 3] = -1                      # 0xffff: a negative NaN with a full payload
+    wide2[10, 2 * V + 5] = float("-inf")
+    wide2[11, 3 * V + 6] = float("nan")
+    wide2[12, 4 * V + 7] = -300.0                             # silu underflows to a signed zero
+    w2[9] = float("inf")
+    z2 = wide2[:, :HV * V].unflatten(1, (HV, V))
+    pe, pf = pool0.clone(), pool0.clone()
+    o2 = gdn_recurrent_kernel(u(q), u(k), u(v2), u(gate), u(beta), ssm_state=pe, state_indices=rows, cu_seqlens=cu)[0]
+    want2 = fused_gated_out_norm(o2, z2, w2, 1e-6).view(T, HV, V)
+    got_nf = gdn_recurrent_kernel(u(q), u(k), u(v2), u(gate), u(beta), ssm_state=pf, state_indices=rows, cu_seqlens=cu,
+                                  gated_norm=(z2, w2, 1e-6, True))
+    assert not torch.isfinite(want2.float()).all()
+    assert got_nf is not None and same_bits(got_nf[0], want2) and same_bits(pe, pf)
     # fewer than 512 (sequence, head) pairs: the 16-lane layout runs; the library declines the fused form untouched ...
     from isoexec_amd import _lib
 

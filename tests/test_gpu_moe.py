@@ -222,4 +222,23 @@ def test_combine_add_norm_in_one_launch_equals_the_two_calls(T, H, k):
         got = combine_add_rms_norm(eo, p, res, w, 1e-6, fp32_acc=fp32_acc)
         assert got is not None
         assert same_bits(got[0], want_y) and same_bits(got[1], want_h), fp32_acc
+    # NaNs and infinities (with payloads and signs of their own) in expert rows, residual and weight: the one launch
+    # rounds inside its chain with the hardware convert and must still store what the two calls store
+    eo2, res2, w2 = eo.clone(), res.clone(), w.clone()
+    bits = eo2.view(torch.int16)
+    bits[0, 3] = 0x7fa5                                      # a NaN with a payload
+    bits[(T * k) // 2, 9] = -1                               # 0xffff: negative NaN, full payload
+    eo2[T * k - 1, 17] = float("inf")
+    eo2[0, 40] = float("-inf")
+    res2[T - 1, 5] = float("nan")
+    res2[0, 41] = float("inf")
+    res2.view(torch.int16)[T // 2, 100] = 0x7f81             # signalling-pattern NaN
+    w2[7] = float("inf")
+    w2[200] = float("nan")
+    eo2[:, 300] = 3.0e38                                     # sums overflow to infinity on the way
+    for fp32_acc in (False, True):
+        want_y, want_h = fused_add_rms_norm_gamma(combine(eo2, p, fp32_acc=fp32_acc), res2, w2, 1e-6)
+        got = combine_add_rms_norm(eo2, p, res2, w2, 1e-6, fp32_acc=fp32_acc)
+        assert not torch.isfinite(want_y.float()).all() and not torch.isfinite(want_h.float()).all()
+        assert same_bits(got[0], want_y) and same_bits(got[1], want_h), fp32_acc
     assert combine_add_rms_norm(eo[:, :384].contiguous(), p, res[:, :384].contiguous(), w[:384].contiguous(), 1e-6) is None
