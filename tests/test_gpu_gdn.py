@@ -245,6 +245,40 @@ def test_conv_bit_exact_prefill_decode_and_state(dprims):
         assert same_bits(y2.cpu(), np_to_bf16(want_y)) and same_bits(s2.cpu(), np_to_bf16(want_s)), (D2, W2)
 
 
+@pytest.mark.parametrize("D,normed", [(2048, False), (6144, False), (2048, True), (4096, True)])
+def test_packed_conv_in_the_run_order_against_the_oracle(D, normed, dprims):
+    """Channel counts that fill whole workgroups take the convolution's XCD-run order (consecutive token groups of a
+    channel block on one XCD). Every sequence of a ragged packed batch against the oracle, stored windows in and out; the
+    normalising form against the oracle's conv followed by its l2norm."""
+    from isoexec_amd.ops.gdn.gdn_ops import conv_packed
+
+    W, K = 4, 128
+    g = cpu_gen(D + normed)
+    lens = [333, 7, 64, 1, 257, 130, 80, 16, 90]
+    T, n = sum(lens), len(lens)
+    wide = torch.randn(T, D + 72, generator=g).to(torch.bfloat16)
+    x = wide[:, 8:8 + D]                                    # a column slice: row pitch D + 72, first column 8
+    w = (0.5 * torch.randn(D, W, generator=g)).to(torch.bfloat16)
+    b = (0.1 * torch.randn(D, generator=g)).to(torch.bfloat16)
+    pool = torch.randn(n + 1, D, W - 1, generator=g).to(torch.bfloat16)
+    rows_in = torch.tensor([0, 2, 0, 4, 5, 0, 7, 0, 9], dtype=torch.int32)
+    rows_out = torch.arange(1, n + 1, dtype=torch.int32)
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    pool_d = pool.to(DEV)
+    qk = D // 2 if normed else 0
+    y = conv_packed(wide.to(DEV)[:, 8:8 + D], w.to(DEV), b.to(DEV), cu_seqlens=cu.to(DEV), conv_state=pool_d,
+                    rows_in=rows_in.to(DEV), rows_out=rows_out.to(DEV), l2norm_qk=qk, head_k_dim=K if normed else 0)
+    for i, L in enumerate(lens):
+        s0 = int(cu[i])
+        init = bf16_to_np(pool[int(rows_in[i])]) if int(rows_in[i]) else None
+        want_y, want_s = o_gdn.causal_conv(bf16_to_np(x[s0:s0 + L]), bf16_to_np(w), bf16_to_np(b), initial_state=init,
+                                           prims=dprims)
+        if normed:
+            want_y[:, :qk] = o_gdn.l2norm(want_y[:, :qk].reshape(L, qk // K, K)).reshape(L, qk)
+        assert same_bits(y[s0:s0 + L].cpu(), np_to_bf16(want_y)), (i, L)
+        assert same_bits(pool_d[i + 1].cpu(), np_to_bf16(want_s)), (i, L)
+
+
 def test_native_core_varlen_equals_decode_steps():
     """The fused-front composition (raw q/k, raw a/b): one varlen call == T sequential decode calls,
     state included (gdn_native_kernel_parity_test_gpu.py T1-T4)."""
