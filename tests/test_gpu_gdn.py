@@ -245,8 +245,10 @@ def test_conv_bit_exact_prefill_decode_and_state(dprims):
         assert same_bits(y2.cpu(), np_to_bf16(want_y)) and same_bits(s2.cpu(), np_to_bf16(want_s)), (D2, W2)
 
 
+@pytest.mark.parametrize("lens", [[333, 7, 64, 1, 257, 130, 80, 16, 90], [40, 3, 9, 1, 21, 33, 12, 2, 30]],
+                         ids=["long", "short"])
 @pytest.mark.parametrize("D,normed", [(2048, False), (6144, False), (2048, True), (4096, True)])
-def test_packed_conv_in_the_run_order_against_the_oracle(D, normed, dprims):
+def test_packed_conv_in_the_run_order_against_the_oracle(D, normed, lens, dprims):
     """Channel counts that fill whole workgroups take the convolution's XCD-run order (consecutive token groups of a
     channel block on one XCD). Every sequence of a ragged packed batch against the oracle, stored windows in and out; the
     normalising form against the oracle's conv followed by its l2norm."""
@@ -254,8 +256,7 @@ def test_packed_conv_in_the_run_order_against_the_oracle(D, normed, dprims):
 
     W, K = 4, 128
     g = cpu_gen(D + normed)
-    lens = [333, 7, 64, 1, 257, 130, 80, 16, 90]
-    T, n = sum(lens), len(lens)
+    T, n = sum(lens), len(lens)             # mean length 108 (16 or 8 tokens per thread) or 16 (4 per thread)
     wide = torch.randn(T, D + 72, generator=g).to(torch.bfloat16)
     x = wide[:, 8:8 + D]                                    # a column slice: row pitch D + 72, first column 8
     w = (0.5 * torch.randn(D, W, generator=g)).to(torch.bfloat16)
