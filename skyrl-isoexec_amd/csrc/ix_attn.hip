@@ -445,20 +445,21 @@ __global__ __launch_bounds__(256) void k_rope8(bf16_t* __restrict__ x, long x_pi
     const uint32_t* aw = &a4.x; const uint32_t* bw = &b4.x;
     const uint32_t* c0w = &c0.x; const uint32_t* c1w = &c1.x; const uint32_t* s0w = &s0.x; const uint32_t* s1w = &s1.x;
     uint32_t* low = &lo4.x; uint32_t* hiw = &hi4.x;
+    // The products are rounded by the hardware pack-convert, two at a time (ix_rbf2_hw: k_rope's ix_rbf on everything but
+    // a NaN, whose payload it keeps); a NaN stays a NaN through the add whatever its payload, and the sums are stored
+    // with their NaNs made canonical (ix_pack_bf2_canon_hw), so the stored bits are k_rope's.
+    auto lo16 = [](uint32_t u) { return __uint_as_float(u << 16); };
+    auto hi16 = [](uint32_t u) { return __uint_as_float(u & 0xffff0000u); };
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-      uint32_t lo_pair = 0, hi_pair = 0;
-#pragma unroll
-      for (int e = 0; e < 2; ++e) {
-        auto pick = [&](uint32_t u) { return e == 0 ? __uint_as_float(u << 16) : __uint_as_float(u & 0xffff0000u); };
-        const float a = pick(aw[w]), b = pick(bw[w]);
-        const float lo = ix_rbf(a * pick(c0w[w])) + ix_rbf((b * -1.0f) * pick(s0w[w]));
-        const float hi = ix_rbf(b * pick(c1w[w])) + ix_rbf(a * pick(s1w[w]));
-        lo_pair |= (uint32_t)ix_f2bf(lo) << (16 * e);
-        hi_pair |= (uint32_t)ix_f2bf(hi) << (16 * e);
-      }
-      low[w] = lo_pair;
-      hiw[w] = hi_pair;
+      const float a0 = lo16(aw[w]), a1 = hi16(aw[w]), b0 = lo16(bw[w]), b1 = hi16(bw[w]);
+      float t0, t1, u0, u1;
+      ix_rbf2_hw(a0 * lo16(c0w[w]), a1 * hi16(c0w[w]), t0, t1);
+      ix_rbf2_hw((b0 * -1.0f) * lo16(s0w[w]), (b1 * -1.0f) * hi16(s0w[w]), u0, u1);
+      low[w] = ix_pack_bf2_canon_hw(t0 + u0, t1 + u1);
+      ix_rbf2_hw(b0 * lo16(c1w[w]), b1 * hi16(c1w[w]), t0, t1);
+      ix_rbf2_hw(a0 * lo16(s1w[w]), a1 * hi16(s1w[w]), u0, u1);
+      hiw[w] = ix_pack_bf2_canon_hw(t0 + u0, t1 + u1);
     }
   }
   *reinterpret_cast<uint4*>(row) = lo4;

@@ -265,6 +265,36 @@ def test_rope_scalar_and_vector_kernels_give_the_oracle_bits(R):
     assert np.array_equal(np_bits(bf16_to_np(got)), np_bits(want))
 
 
+def test_rope_vector_kernel_stores_the_element_kernels_bits_for_nans_and_infinities():
+    """The 16-byte kernel rounds its products with the hardware convert and makes NaNs canonical at the store; the
+    element kernel rounds with integer arithmetic throughout. Same values through both (a slice that starts 8 bytes
+    into a row is not 16-byte aligned and takes the element kernel), NaNs with payloads and infinities included."""
+    from isoexec_amd.ops.rope.rope_hip import apply_rope_, rope_tables
+
+    g = cpu_gen(5)
+    T, Hh, D = 33, 4, 128
+    x = torch.randn(T, Hh * D, generator=g).to(torch.bfloat16)
+    bits = x.view(torch.int16)
+    bits[0, 3] = 0x7fa5
+    bits[1, D + 70] = -1
+    bits[2, 5] = 0x7f81
+    x[3, 9] = float("inf")
+    x[3, 9 + 64] = float("inf")
+    x[4, 2 * D + 1] = float("-inf")
+    x[5, :] = 3.0e38
+    pos = torch.randint(0, 300, (T,), generator=g, dtype=torch.int32).to(DEV)
+    cos, sin = rope_tables(300, D, 1e6, device=DEV)
+    aligned = x.clone().to(DEV).view(T, Hh, D)
+    wide = torch.zeros(T, Hh * D + 8, dtype=torch.bfloat16, device=DEV)
+    wide[:, 4:4 + Hh * D] = x.to(DEV)
+    shifted = wide[:, 4:4 + Hh * D].unflatten(1, (Hh, D))
+    assert shifted.data_ptr() % 16 == 8
+    a = apply_rope_(aligned, cos, sin, pos)
+    b = apply_rope_(shifted, cos, sin, pos)
+    assert not torch.isfinite(a.float()).all()
+    assert torch.equal(a.contiguous().view(torch.int16), b.contiguous().view(torch.int16))
+
+
 def test_rope_positions_outside_the_tables_read_nothing_and_give_nan():
     """The kernel bounds every position by the tables' row count: a position past the end (or negative) makes that
     token's rotated lanes NaN instead of reading beyond the tables; its neighbours are rotated as usual."""
